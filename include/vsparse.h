@@ -1,0 +1,152 @@
+/*
+ * vsparse — C ABI of the MI355X (gfx950) column-vector-sparse SpMM / SDDMM library.
+ *
+ * Every entry point is `extern "C"`, takes plain ints and raw pointers, and
+ * mirrors one function of the reference's operator API (cited per function,
+ * paths relative to the reference tree).  Dimension letters are the
+ * reference's, not BLAS's:
+ *
+ *   SpMM   C[m x k] = A[m x n] * B[n x k]      m = m_vec * vec_length, A sparse
+ *   SDDMM  D[nnz]   = (A[m x k] * B[n x k]^T) sampled at the mask's nonzeros
+ *
+ * Sparse operands are column-vector CSR: `row_offsets[m_vec + 1]`,
+ * `column_indices[nnz_vec]`, and `values[nnz_vec * vec_length]` fp16 where
+ * values[j * vec_length + v] is the element in scalar row i*vec_length + v,
+ * column column_indices[j], of vector row i.  Dense operands are row-major
+ * fp16; fp16 is IEEE binary16, passed as `void *`.
+ *
+ * Conventions shared by all device entry points
+ *   - all array pointers are DEVICE pointers owned by the caller; nothing is
+ *     retained after return; no workspace; no allocation inside the library;
+ *   - the output is fully overwritten (alpha = 1, beta = 0), including the
+ *     rows of empty vector rows, and nothing outside it is written;
+ *   - the launch is asynchronous on `stream` (a hipStream_t; NULL = default
+ *     stream); the functions are re-entrant;
+ *   - the return value is 0 on success, otherwise a hipError_t-valued int:
+ *     1 (hipErrorInvalidValue) for null pointers, negative sizes,
+ *     misaligned operands or unsupported vec_length / algorithm;
+ *     801 (hipErrorNotSupported) for shapes the selected path cannot take;
+ *     any other value is the launch error reported by the runtime.
+ *     On a non-zero return no kernel was launched.
+ *   - `row_indices[m_vec]` is the row swizzle: work item t processes vector
+ *     row row_indices[t].  It must be a permutation of 0..m_vec-1.
+ */
+#ifndef VSPARSE_H
+#define VSPARSE_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VS_SUCCESS 0
+#define VS_ERROR_INVALID_VALUE 1
+#define VS_ERROR_NOT_SUPPORTED 801
+
+/* Library version, major * 10000 + minor * 100 + patch. */
+int vs_version(void);
+
+/* Short text for a status returned by the functions below. */
+const char *vs_status_string(int status);
+
+/*
+ * Replaces spmm::wmmaSpmm(half in, half out) — include/wmma_spmm.cuh:15-21,
+ * src/wmma_spmm.cu:400-409.  fp16 MFMA with fp32 accumulate.
+ * vec_length in {2, 4, 8} as in the reference (1 is accepted as well).
+ * Requirements: k % 4 == 0; `values` aligned to 2*vec_length bytes,
+ * `rhs_matrix` and `output_matrix` aligned to 16 bytes.
+ */
+int vs_wmma_spmm_f16(int m_vec, int vec_length, int k, int n,
+                     const int *row_indices, const int *row_offsets,
+                     const int *column_indices, const void *values,
+                     const void *rhs_matrix, void *output_matrix, void *stream);
+
+/* fp32-output overload of the same operator — include/wmma_spmm.cuh:7-13, src/wmma_spmm.cu:388-397. */
+int vs_wmma_spmm_f16_f32out(int m_vec, int vec_length, int k, int n,
+                            const int *row_indices, const int *row_offsets,
+                            const int *column_indices, const void *values,
+                            const void *rhs_matrix, float *output_matrix, void *stream);
+
+/*
+ * Replaces spmm::cudaSpmm(half in, half out) — include/cuda_spmm.cuh:15-21,
+ * src/cuda_spmm.cu:316-325.  Fine-grained path on packed-fp16 VALU: every
+ * product is rounded to fp16 (src/spmm_utils/compute_utils.h:45) and added in
+ * fp32.  vec_length in {1, 2, 4, 8}.  Same alignment rules; k % 8 == 0.
+ */
+int vs_cuda_spmm_f16(int m_vec, int vec_length, int k, int n,
+                     const int *row_indices, const int *row_offsets,
+                     const int *column_indices, const void *values,
+                     const void *rhs_matrix, void *output_matrix, void *stream);
+
+/* fp32-output overload — include/cuda_spmm.cuh:7-13, src/cuda_spmm.cu:304-313. */
+int vs_cuda_spmm_f16_f32out(int m_vec, int vec_length, int k, int n,
+                            const int *row_indices, const int *row_offsets,
+                            const int *column_indices, const void *values,
+                            const void *rhs_matrix, float *output_matrix, void *stream);
+
+/*
+ * Replaces sddmm::wmmaSddmm(half in, half out) — include/wmma_sddmm.cuh:17-24,
+ * src/wmma_sddmm.cu:3190-3202.  fp16 MFMA, fp32 accumulate, one rounding to
+ * fp16 on store.  vec_length in {2, 4, 8} (1 accepted).  `algorithm` selects
+ * among the reference's four Volta register/shuffle schedules (0..3); they
+ * compute the same function, so 0, 1 and 2 run the one MFMA kernel here and 3
+ * (the reference's timing-only hardware simulation, whose results are wrong
+ * by design) is rejected with hipErrorInvalidValue.
+ * Requirements: k % 8 == 0 (the whole of k is contracted — the reference drops
+ * k % 64); lhs_matrix / rhs_matrix aligned to 16 bytes, output_values to
+ * 2*vec_length bytes.
+ */
+int vs_wmma_sddmm_f16(int m_vec, int k, int n, int nonzeros_vec,
+                      const int *row_indices, const int *row_offsets,
+                      const int *col_indices, const void *lhs_matrix,
+                      const void *rhs_matrix, void *output_values,
+                      int vec_length, void *stream, int algorithm);
+
+/* fp32-output overload — include/wmma_sddmm.cuh:8-15, src/wmma_sddmm.cu:3175-3187. */
+int vs_wmma_sddmm_f16_f32out(int m_vec, int k, int n, int nonzeros_vec,
+                             const int *row_indices, const int *row_offsets,
+                             const int *col_indices, const void *lhs_matrix,
+                             const void *rhs_matrix, float *output_values,
+                             int vec_length, void *stream, int algorithm);
+
+/*
+ * Replaces sddmm::cudaSddmm(half in, half out) — include/cuda_sddmm.cuh:16-23,
+ * src/cuda_sddmm.cu:1295-1331.  Per-lane slices of the contraction with a
+ * cross-lane (DPP / ds_swizzle) reduction; products rounded to fp16
+ * (src/cuda_sddmm.cu:382), fp32 adds.  vec_length in {1, 2, 4, 8}; any k >= 1
+ * (k % 8 != 0 takes a slower scalar-load kernel).
+ */
+int vs_cuda_sddmm_f16(int m_vec, int k, int n, int nonzeros_vec,
+                      const int *row_indices, const int *row_offsets,
+                      const int *col_indices, const void *lhs_matrix,
+                      const void *rhs_matrix, void *output_values,
+                      int vec_length, void *stream);
+
+/* fp32-output overload — include/cuda_sddmm.cuh:7-14, src/cuda_sddmm.cu:1281-1293. */
+int vs_cuda_sddmm_f16_f32out(int m_vec, int k, int n, int nonzeros_vec,
+                             const int *row_indices, const int *row_offsets,
+                             const int *col_indices, const void *lhs_matrix,
+                             const void *rhs_matrix, float *output_values,
+                             int vec_length, void *stream);
+
+/*
+ * Host helpers (HOST pointers).  Replace IdentityRowSwizzle / SortedRowSwizzle —
+ * include/bm_test_utils.h:196-198 and :200-215.  The sorted swizzle orders
+ * vector rows by descending length; equal lengths keep ascending row order.
+ */
+void vs_identity_row_swizzle(int rows, int *row_indices);
+void vs_sorted_row_swizzle(int rows, const int *row_offsets, int *row_indices);
+
+/*
+ * Launch-shape tuning knob (process-wide, not thread-safe against concurrent
+ * launches).  Names: "spmm_waves" (waves per workgroup, 0 = automatic),
+ * "spmm_cols_per_lane" (4, 8, 0 = automatic), "sddmm_slots" (workgroups per
+ * vector row, 0 = automatic).  Returns 0, or 1 for an unknown name / bad value.
+ * No counterpart in the reference, whose tile sizes are compile-time constants
+ * (src/wmma_spmm.cu:396).
+ */
+int vs_set_option(const char *name, int value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VSPARSE_H */

@@ -1,0 +1,91 @@
+"""The C-ABI library loads, exports what include/vsparse.h declares, and validates arguments.
+
+No kernel is launched here: every call either is a host helper or is rejected (or is a no-op)
+before any device work.
+"""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from oracle import c_oracle as co
+from vectorsparse_amd import _lib, ops
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "vsparse.h")
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(vs_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_bound():
+    names = _declared()
+    assert len(names) >= 13
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for name in names:
+        assert hasattr(raw, name), "libvsparse.so does not export %s" % name
+    assert sorted(_lib.SIGNATURES) == names
+
+
+def test_version_and_status_text():
+    L = _lib.lib()
+    assert L.vs_version() >= 100
+    assert b"success" in L.vs_status_string(0)
+    assert b"invalid" in L.vs_status_string(1)
+    assert b"not supported" in L.vs_status_string(801)
+
+
+def test_swizzles_match_oracle():
+    rng = np.random.default_rng(1)
+    lengths = rng.integers(0, 9, 300)
+    ro = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    assert np.array_equal(ops.IdentityRowSwizzle(300), co.identity_row_swizzle(300))
+    assert np.array_equal(ops.SortedRowSwizzle(300, ro), co.sorted_row_swizzle(300, ro))
+    assert ops.SortedRowSwizzle(0, np.zeros(1, np.int32)).size == 0
+
+
+def test_argument_validation_without_launch():
+    L = _lib.lib()
+    p = 0x1000  # never dereferenced: all calls below return before any device work
+    INVALID, OK = 1, 0
+    # unsupported vector length (the reference prints "Unsupported Vector Length!" and launches nothing)
+    assert L.vs_wmma_spmm_f16(4, 3, 64, 64, p, p, p, p, p, p, None) == INVALID
+    assert L.vs_cuda_spmm_f16(4, 16, 64, 64, p, p, p, p, p, p, None) == INVALID
+    assert L.vs_wmma_sddmm_f16(4, 64, 64, 10, p, p, p, p, p, p, 5, None, 1) == INVALID
+    assert L.vs_cuda_sddmm_f16(4, 64, 64, 10, p, p, p, p, p, p, 0, None) == INVALID
+    # negative sizes, null pointers, misaligned operands
+    assert L.vs_wmma_spmm_f16(-1, 8, 64, 64, p, p, p, p, p, p, None) == INVALID
+    assert L.vs_wmma_spmm_f16(4, 8, 64, 64, None, p, p, p, p, p, None) == INVALID
+    assert L.vs_wmma_spmm_f16(4, 8, 64, 64, p, p, p, p, p, None, None) == INVALID
+    assert L.vs_wmma_spmm_f16(4, 8, 64, 64, p, p, p, p + 2, p, p, None) == INVALID
+    assert L.vs_wmma_spmm_f16(4, 8, 64, 64, p, p, p, p, p + 8, p, None) == INVALID
+    assert L.vs_cuda_sddmm_f16(4, 64, 64, 10, p, p, p, None, p, p, 8, None) == INVALID
+    assert L.vs_wmma_sddmm_f16(4, 64, 64, 10, p, p, p, p, p, p + 2, 8, None, 1) == INVALID
+    # algorithm 3 is the reference's timing-only hardware simulation; unknown algorithms launch nothing
+    assert L.vs_wmma_sddmm_f16(4, 64, 64, 10, p, p, p, p, p, p, 8, None, 3) == INVALID
+    assert L.vs_wmma_sddmm_f16(4, 64, 64, 10, p, p, p, p, p, p, 8, None, -1) == INVALID
+    # shapes a path cannot take
+    assert L.vs_wmma_spmm_f16(4, 8, 66, 64, p, p, p, p, p, p, None) == 801
+    assert L.vs_cuda_spmm_f16(4, 8, 68, 64, p, p, p, p, p, p, None) == 801
+    assert L.vs_wmma_sddmm_f16(4, 60, 64, 10, p, p, p, p, p, p, 8, None, 1) == 801
+    # empty problems succeed without touching the device
+    assert L.vs_wmma_spmm_f16(0, 8, 64, 64, None, None, None, None, None, None, None) == OK
+    assert L.vs_cuda_spmm_f16(4, 8, 0, 64, None, None, None, None, None, None, None) == OK
+    assert L.vs_wmma_sddmm_f16(4, 64, 64, 0, None, None, None, None, None, None, 8, None, 1) == OK
+    assert L.vs_cuda_sddmm_f16(0, 64, 64, 0, None, None, None, None, None, None, 8, None) == OK
+
+
+def test_options():
+    _lib.set_option("spmm_waves", 4)
+    _lib.set_option("spmm_waves", 0)
+    with pytest.raises(_lib.VSparseError):
+        _lib.set_option("spmm_waves", 17)
+    with pytest.raises(_lib.VSparseError):
+        _lib.set_option("no_such_option", 1)
+    with pytest.raises(_lib.VSparseError):
+        _lib.set_option("spmm_cols_per_lane", 3)

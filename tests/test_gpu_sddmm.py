@@ -1,0 +1,158 @@
+"""SDDMM parity on the GPU: HIP kernels through the C ABI vs the CPU oracle (same seeded inputs)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle as co
+from vectorsparse_amd import _lib, ops
+from vectorsparse_amd import colvec_csr as cv
+from util import assert_parity
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(pat, A, B, kernel, sort=False, out_dtype=torch.float16, algorithm=1, device="cuda"):
+    prob = ops.DeviceProblem(pat, sort=sort, device=device)
+    Ad = torch.from_numpy(A).to(device)
+    Bd = torch.from_numpy(B).to(device)
+    V = pat.vec_length
+    pad = 128
+    buf = torch.full((pat.nnz_vec + 2 * pad, V), 777.0, dtype=out_dtype, device=device)
+    out = buf[pad:pad + pat.nnz_vec]
+    prob.sddmm(Ad, Bd, kernel=kernel, out=out, algorithm=algorithm)
+    torch.cuda.synchronize()
+    host = buf.cpu().numpy()
+    assert np.all(host[:pad] == 777.0) and np.all(host[pad + pat.nnz_vec:] == 777.0), "wrote outside the output"
+    assert np.array_equal(prob.row_offsets.cpu().numpy(), pat.row_offsets)
+    assert np.array_equal(prob.column_indices.cpu().numpy(), pat.column_indices)
+    return host[pad:pad + pat.nnz_vec].reshape(-1)
+
+
+def _oracle(pat, A, B):
+    # fp32 flavour of the host loop: the comparison tolerance covers the final fp16 rounding
+    return co.sddmm_host_ref_f32(pat.m_vec, A.shape[1], pat.vec_length, pat.row_offsets, pat.column_indices, A, B)
+
+
+@pytest.mark.parametrize("kernel", ["wmma", "cuda"])
+@pytest.mark.parametrize("K", [64, 128])
+@pytest.mark.parametrize("sparsity", [0.9, 0.95])
+def test_config4(gpu, kernel, K, sparsity):
+    # M = N = 2048, V = 8, uniform mask
+    seed = 4 + (K == 128) + 2 * (sparsity == 0.95)
+    pat = cv.uniform_pattern(256, 2048, sparsity, seed=seed, vec_length=8)
+    A = cv.dense_normal(2048, K, seed=seed + 10)
+    B = cv.dense_normal(2048, K, seed=seed + 20)
+    got = _run(pat, A, B, kernel)
+    assert_parity(got, _oracle(pat, A, B), "config4 K%d s%g %s" % (K, sparsity, kernel))
+    # the fp16 host loop itself (rounded output) agrees to within one rounding step
+    ref16 = co.sddmm_host_ref_f16(pat.m_vec, K, 8, pat.row_offsets, pat.column_indices, A, B)
+    assert_parity(got, ref16.astype(np.float32), "config4 vs fp16 host loop")
+
+
+@pytest.mark.parametrize("V", [1, 2, 4, 8])
+@pytest.mark.parametrize("K", [8, 32, 64, 72, 128, 256, 320, 512, 1024])
+def test_vec_lengths_and_contraction_sizes(gpu, V, K):
+    pat = cv.binomial_pattern(96 // V, 300, 0.85, seed=V * 1000 + K, vec_length=V)
+    A = cv.dense_normal(pat.m, K, seed=1)
+    B = cv.dense_normal(300, K, seed=2)
+    ref = _oracle(pat, A, B)
+    for kernel in ("wmma", "cuda"):
+        assert_parity(_run(pat, A, B, kernel), ref, "V%d K%d %s" % (V, K, kernel))
+
+
+@pytest.mark.parametrize("V", [1, 2, 4, 8])
+@pytest.mark.parametrize("K", [1, 7, 12, 50, 100, 130])
+def test_cuda_path_takes_any_k(gpu, V, K):
+    pat = cv.binomial_pattern(48 // V, 100, 0.8, seed=V * 100 + K, vec_length=V)
+    A = cv.dense_normal(pat.m, K, seed=3)
+    B = cv.dense_normal(100, K, seed=4)
+    assert_parity(_run(pat, A, B, "cuda"), _oracle(pat, A, B), "cuda V%d K%d" % (V, K))
+
+
+@pytest.mark.parametrize("V", [1, 2, 4, 8])
+@pytest.mark.parametrize("kernel", ["wmma", "cuda"])
+def test_ragged_and_empty_rows(gpu, V, kernel):
+    lengths = np.array([0, 1, 15, 16, 17, 0, 31, 33, 64, 65, 300, 2, 0, 128, 7, 0], dtype=np.int64)
+    rng = np.random.default_rng(5)
+    ro, ci = cv._pattern_from_lengths(rng, len(lengths), 320, lengths)
+    pat = cv.ColVecCSR(len(lengths), 320, V, ro, ci).validate()
+    A = cv.dense_normal(pat.m, 64, seed=8)
+    B = cv.dense_normal(320, 64, seed=9)
+    assert_parity(_run(pat, A, B, kernel), _oracle(pat, A, B), "ragged V%d %s" % (V, kernel))
+
+
+@pytest.mark.parametrize("kernel", ["wmma", "cuda"])
+def test_skew_swizzle_invariance_and_slots(gpu, kernel):
+    lengths = np.full(40, 20, dtype=np.int64)
+    lengths[17] = 1500
+    lengths[3] = 700
+    rng = np.random.default_rng(11)
+    ro, ci = cv._pattern_from_lengths(rng, 40, 2048, lengths)
+    pat = cv.ColVecCSR(40, 2048, 8, ro, ci)
+    A = cv.dense_normal(pat.m, 128, seed=12)
+    B = cv.dense_normal(2048, 128, seed=13)
+    ref = _oracle(pat, A, B)
+    a = _run(pat, A, B, kernel, sort=False)
+    b = _run(pat, A, B, kernel, sort=True)
+    assert_parity(a, ref, "skew " + kernel)
+    assert np.array_equal(a.view(np.uint16), b.view(np.uint16))
+    try:
+        for slots in (1, 2, 7, 64, 200):
+            _lib.set_option("sddmm_slots", slots)
+            c = _run(pat, A, B, kernel)
+            assert np.array_equal(a.view(np.uint16), c.view(np.uint16)), "slots=%d changed the bits" % slots
+    finally:
+        _lib.set_option("sddmm_slots", 0)
+
+
+@pytest.mark.parametrize("kernel", ["wmma", "cuda"])
+def test_fp32_output_overload(gpu, kernel):
+    pat = cv.uniform_pattern(32, 512, 0.9, seed=21, vec_length=4)
+    A = cv.dense_normal(pat.m, 64, seed=22)
+    B = cv.dense_normal(512, 64, seed=23)
+    got = _run(pat, A, B, kernel, out_dtype=torch.float32)
+    assert got.dtype == np.float32
+    assert_parity(got, _oracle(pat, A, B), "fp32 out " + kernel)
+
+
+def test_algorithm_argument(gpu):
+    pat = cv.uniform_pattern(16, 256, 0.9, seed=1, vec_length=8)
+    A = cv.dense_normal(pat.m, 64, seed=2)
+    B = cv.dense_normal(256, 64, seed=3)
+    ref = _oracle(pat, A, B)
+    outs = [_run(pat, A, B, "wmma", algorithm=alg) for alg in (0, 1, 2)]
+    for o in outs:
+        assert_parity(o, ref, "algorithm")
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[1], outs[2])
+    with pytest.raises(_lib.VSparseError):
+        _run(pat, A, B, "wmma", algorithm=3)
+
+
+def test_full_mask_equals_dense_product(gpu):
+    V, m_vec, n, K = 8, 8, 96, 64
+    ro = (np.arange(m_vec + 1) * n).astype(np.int32)
+    ci = np.tile(np.arange(n, dtype=np.int32), m_vec)
+    pat = cv.ColVecCSR(m_vec, n, V, ro, ci)
+    A = cv.dense_normal(m_vec * V, K, seed=3)
+    B = cv.dense_normal(n, K, seed=4)
+    got = _run(pat, A, B, "wmma").reshape(m_vec, n, V).transpose(0, 2, 1).reshape(m_vec * V, n)
+    dense = A.astype(np.float64) @ B.astype(np.float64).T
+    assert_parity(got, dense, "full mask")
+
+
+def test_sddmm_output_chains_into_spmm(gpu):
+    # the [nnz_vec][V] output layout is exactly the `values` layout of SpMM
+    V, K, N = 8, 64, 64
+    pat = cv.band_strided_pattern(512, V, band_half_width=64, stride=64)
+    Q = cv.dense_normal(512, K, seed=1)
+    Kmat = cv.dense_normal(512, K, seed=2)
+    W = cv.dense_uniform(512, N, seed=3)
+    prob = ops.DeviceProblem(pat)
+    scores = prob.sddmm(torch.from_numpy(Q).cuda(), torch.from_numpy(Kmat).cuda())
+    prob.values = scores
+    out = prob.spmm(torch.from_numpy(W).cuda())
+    torch.cuda.synchronize()
+    vals = scores.cpu().numpy()
+    assert_parity(vals.reshape(-1), _oracle(pat, Q, Kmat), "chain sddmm")
+    ref = co.spmm_host_ref_f32(pat.m_vec, V, N, 512, pat.row_offsets, pat.column_indices, vals, W)
+    assert_parity(out.cpu().numpy(), ref, "chain spmm")

@@ -1,0 +1,182 @@
+"""SpMM parity on the GPU: HIP kernels through the C ABI vs the CPU oracle (same seeded inputs).
+
+Tolerance (written in tests/util.py): max relative error <= 1e-2 with the denominator floored at
+1e-2*rms(ref), and zero elements beyond the reference's own 0.5 absolute criterion.  Pattern
+arrays must come back byte-identical.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle as co
+from vectorsparse_amd import _lib, ops
+from vectorsparse_amd import colvec_csr as cv
+from util import assert_parity
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(pat, B, kernel, sort=False, out_dtype=torch.float16, device="cuda"):
+    prob = ops.DeviceProblem(pat, sort=sort, device=device)
+    Bd = torch.from_numpy(B).to(device)
+    k = B.shape[1]
+    # canary rows either side of the output catch out-of-range writes
+    pad = 64
+    buf = torch.full((pat.m + 2 * pad, k), 12345.0, dtype=out_dtype, device=device)
+    out = buf[pad:pad + pat.m]
+    prob.spmm(Bd, kernel=kernel, out=out)
+    torch.cuda.synchronize()
+    host = buf.cpu().numpy()
+    assert np.all(host[:pad] == 12345.0) and np.all(host[pad + pat.m:] == 12345.0), "wrote outside the output"
+    assert np.array_equal(prob.row_offsets.cpu().numpy(), pat.row_offsets)
+    assert np.array_equal(prob.column_indices.cpu().numpy(), pat.column_indices)
+    return host[pad:pad + pat.m]
+
+
+def _oracle(pat, B):
+    return co.spmm_host_ref_f32(pat.m_vec, pat.vec_length, B.shape[1], pat.n, pat.row_offsets,
+                                pat.column_indices, pat.values, B)
+
+
+def _kernels(V):
+    return ["wmma", "cuda"]
+
+
+@pytest.mark.parametrize("kernel", ["wmma", "cuda"])
+def test_config1_oracle_case(gpu, kernel):
+    # M=256, K=256, V=4, N=128, 90 % sparse, exactly 26 vectors per row
+    pat = cv.random_values(cv.uniform_pattern(64, 256, 0.9, seed=0, vec_length=4), seed=100)
+    B = cv.dense_uniform(256, 128, seed=200)
+    assert_parity(_run(pat, B, kernel), _oracle(pat, B), "config1/" + kernel)
+
+
+@pytest.mark.parametrize("kernel", ["wmma", "cuda"])
+@pytest.mark.parametrize("sort", [False, True])
+def test_config2_resnet_shape(gpu, kernel, sort):
+    # M=512, K=4608, V=8, N=256, 90 % sparse, binomial row lengths
+    pat = cv.random_values(cv.binomial_pattern(64, 4608, 0.9, seed=1, vec_length=8), seed=101)
+    B = cv.dense_uniform(4608, 256, seed=201)
+    assert_parity(_run(pat, B, kernel, sort=sort), _oracle(pat, B), "config2/%s/sort=%d" % (kernel, sort))
+
+
+SWEEP = [
+    # (M, K, sparsity) subset of the ResNet-50-like grid, N = 256
+    (64, 64, 0.5), (128, 147, 0.7), (256, 576, 0.8), (1024, 1152, 0.95), (2048, 2304, 0.98), (2048, 4608, 0.9),
+]
+
+
+@pytest.mark.parametrize("V", [1, 2, 4, 8])
+@pytest.mark.parametrize("shape", SWEEP, ids=lambda s: "M%d_K%d_s%g" % s)
+def test_config3_sweep_points(gpu, V, shape):
+    M, K, s = shape
+    seed = (M * 31 + K * 7 + int(s * 100) * 3 + V) % 100000
+    pat = cv.random_values(cv.uniform_pattern(M // V, K, s, seed=seed, vec_length=V), seed=seed + 1)
+    B = cv.dense_uniform(K, 256, seed=seed + 2)
+    ref = _oracle(pat, B)
+    for kernel in _kernels(V):
+        assert_parity(_run(pat, B, kernel), ref, "sweep M%d K%d s%g V%d %s" % (M, K, s, V, kernel))
+
+
+@pytest.mark.parametrize("V", [1, 2, 4, 8])
+@pytest.mark.parametrize("kernel", ["wmma", "cuda"])
+def test_ragged_rows_and_empty_rows(gpu, V, kernel):
+    # lengths 0, 1, 15, 16, 17, 31, 33, 300 ... exercise the padded tail of every tile size
+    lengths = np.array([0, 1, 15, 16, 17, 0, 31, 33, 64, 65, 300, 2, 0, 128, 7, 0], dtype=np.int64)
+    n = 320
+    rng = np.random.default_rng(5)
+    ro, ci = cv._pattern_from_lengths(rng, len(lengths), n, lengths)
+    pat = cv.random_values(cv.ColVecCSR(len(lengths), n, V, ro, ci).validate(), seed=6)
+    B = cv.dense_uniform(n, 192, seed=7)
+    got = _run(pat, B, kernel)
+    assert_parity(got, _oracle(pat, B), "ragged V%d %s" % (V, kernel))
+    for i in np.nonzero(lengths == 0)[0]:
+        assert not got[i * V:(i + 1) * V].any(), "empty vector row %d must be written as zeros" % i
+
+
+@pytest.mark.parametrize("kernel", ["wmma", "cuda"])
+def test_all_rows_empty(gpu, kernel):
+    pat = cv.ColVecCSR(8, 64, 8, np.zeros(9, np.int32), np.zeros(0, np.int32), np.zeros((0, 8), np.float16))
+    B = cv.dense_uniform(64, 64, seed=1)
+    got = _run(pat, B, kernel)
+    assert got.shape == (64, 64) and not got.any()
+
+
+@pytest.mark.parametrize("N", [8, 24, 64, 72, 136, 512, 1000])
+@pytest.mark.parametrize("kernel", ["wmma", "cuda"])
+def test_dense_width_edges(gpu, N, kernel):
+    pat = cv.random_values(cv.binomial_pattern(24, 200, 0.8, seed=N, vec_length=8), seed=N + 1)
+    B = cv.dense_uniform(200, N, seed=N + 2)
+    assert_parity(_run(pat, B, kernel), _oracle(pat, B), "N=%d %s" % (N, kernel))
+
+
+def test_dense_width_multiple_of_4_on_mfma_path(gpu):
+    pat = cv.random_values(cv.binomial_pattern(24, 100, 0.7, seed=3, vec_length=4), seed=4)
+    for N in (4, 12, 68, 132):
+        B = cv.dense_uniform(100, N, seed=N)
+        assert_parity(_run(pat, B, "wmma"), _oracle(pat, B), "N=%d wmma" % N)
+
+
+@pytest.mark.parametrize("kernel", ["wmma", "cuda"])
+def test_skewed_rows_and_swizzle_invariance(gpu, kernel):
+    # one very long row among short ones; the result must not depend on the row swizzle at all
+    lengths = np.full(40, 20, dtype=np.int64)
+    lengths[17] = 1500
+    lengths[3] = 700
+    rng = np.random.default_rng(11)
+    ro, ci = cv._pattern_from_lengths(rng, 40, 2048, lengths)
+    pat = cv.random_values(cv.ColVecCSR(40, 2048, 8, ro, ci), seed=12)
+    B = cv.dense_uniform(2048, 256, seed=13)
+    a = _run(pat, B, kernel, sort=False)
+    b = _run(pat, B, kernel, sort=True)
+    assert_parity(a, _oracle(pat, B), "skew " + kernel)
+    assert np.array_equal(a.view(np.uint16), b.view(np.uint16)), "row swizzle changed the bits"
+
+
+@pytest.mark.parametrize("kernel", ["wmma", "cuda"])
+def test_fp32_output_overload(gpu, kernel):
+    pat = cv.random_values(cv.binomial_pattern(32, 512, 0.9, seed=21, vec_length=8), seed=22)
+    B = cv.dense_uniform(512, 128, seed=23)
+    got = _run(pat, B, kernel, out_dtype=torch.float32)
+    assert got.dtype == np.float32
+    assert_parity(got, _oracle(pat, B), "fp32 out " + kernel)
+
+
+def test_launch_shape_overrides_keep_parity(gpu):
+    pat = cv.random_values(cv.binomial_pattern(16, 1024, 0.8, seed=31, vec_length=8), seed=32)
+    B = cv.dense_uniform(1024, 256, seed=33)
+    ref = _oracle(pat, B)
+    try:
+        for cpl in (4, 8):
+            for waves in (1, 2, 3, 8, 16):
+                _lib.set_option("spmm_cols_per_lane", cpl)
+                _lib.set_option("spmm_waves", waves)
+                assert_parity(_run(pat, B, "wmma"), ref, "cpl=%d waves=%d" % (cpl, waves))
+        for waves in (1, 2, 4):
+            _lib.set_option("spmm_waves", waves)
+            assert_parity(_run(pat, B, "cuda"), ref, "cuda waves=%d" % waves)
+    finally:
+        _lib.set_option("spmm_cols_per_lane", 0)
+        _lib.set_option("spmm_waves", 0)
+
+
+def test_deterministic_and_linear(gpu):
+    pat = cv.random_values(cv.binomial_pattern(64, 4608, 0.9, seed=1, vec_length=8), seed=101)
+    B = cv.dense_uniform(4608, 256, seed=201)
+    a = _run(pat, B, "wmma")
+    b = _run(pat, B, "wmma")
+    assert np.array_equal(a.view(np.uint16), b.view(np.uint16))
+    # scaling the values by a power of two scales the result exactly
+    doubled = pat.with_values(pat.values * np.float16(2))
+    c = _run(doubled, B, "wmma")
+    normal = np.abs(a) >= 2.0 ** -13      # doubling commutes with fp16 rounding outside the subnormal range
+    assert np.array_equal(c[normal], (a * np.float16(2))[normal])
+
+
+def test_wrong_dtype_and_host_tensor_are_rejected(gpu):
+    pat = cv.random_values(cv.uniform_pattern(4, 32, 0.5, seed=1, vec_length=4), seed=2)
+    prob = ops.DeviceProblem(pat)
+    B = torch.ones((32, 64), dtype=torch.float32, device="cuda")
+    with pytest.raises(TypeError):
+        prob.spmm(B)
+    with pytest.raises(ValueError):
+        prob.spmm(torch.ones((32, 64), dtype=torch.float16))

@@ -1,0 +1,61 @@
+"""ctypes binding of libvsparse.so.  Raises if the library is missing: there is no fallback path."""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libvsparse.so")
+
+_vp = ctypes.c_void_p
+_int = ctypes.c_int
+
+# name -> argtypes, exactly the declarations of include/vsparse.h
+SIGNATURES = {
+    "vs_version": ([], _int),
+    "vs_status_string": ([_int], ctypes.c_char_p),
+    "vs_wmma_spmm_f16": ([_int] * 4 + [_vp] * 7, _int),
+    "vs_wmma_spmm_f16_f32out": ([_int] * 4 + [_vp] * 7, _int),
+    "vs_cuda_spmm_f16": ([_int] * 4 + [_vp] * 7, _int),
+    "vs_cuda_spmm_f16_f32out": ([_int] * 4 + [_vp] * 7, _int),
+    "vs_wmma_sddmm_f16": ([_int] * 4 + [_vp] * 6 + [_int, _vp, _int], _int),
+    "vs_wmma_sddmm_f16_f32out": ([_int] * 4 + [_vp] * 6 + [_int, _vp, _int], _int),
+    "vs_cuda_sddmm_f16": ([_int] * 4 + [_vp] * 6 + [_int, _vp], _int),
+    "vs_cuda_sddmm_f16_f32out": ([_int] * 4 + [_vp] * 6 + [_int, _vp], _int),
+    "vs_identity_row_swizzle": ([_int, _vp], None),
+    "vs_sorted_row_swizzle": ([_int, _vp, _vp], None),
+    "vs_set_option": ([ctypes.c_char_p, _int], _int),
+}
+
+_lib = None
+
+
+class VSparseError(RuntimeError):
+    def __init__(self, status, where):
+        self.status = status
+        msg = lib().vs_status_string(status)
+        super().__init__("%s failed with status %d: %s" % (where, status, msg.decode() if msg else "?"))
+
+
+def lib():
+    """Load the library once; a missing file is an error, never a silent fallback."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                "%s not found: build it with `python -m vectorsparse_amd.build` "
+                "(hipcc --offload-arch=gfx950)" % LIB_PATH)
+        L = ctypes.CDLL(LIB_PATH)
+        for name, (argtypes, restype) in SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.argtypes = argtypes
+            fn.restype = restype
+        _lib = L
+    return _lib
+
+
+def check(status, where):
+    if status != 0:
+        raise VSparseError(status, where)
+
+
+def set_option(name, value):
+    check(lib().vs_set_option(name.encode(), int(value)), "vs_set_option(%s)" % name)

@@ -1,0 +1,231 @@
+// Fine-grained SDDMM with per-lane slices of the contraction and a cross-lane reduction
+// (replaces src/cuda_sddmm.cu of the reference).
+//
+// A wave is G = 64/LK groups of LK lanes; a group owns one nonzero vector j per step and lane
+// cl of the group owns the slice k in [chunk*LK*VEC + cl*VEC, +VEC) of both operand rows
+// (VEC = 8 halves: one 128-bit load; VEC = 1 for K % 8 != 0).  Each lane forms the V partial dot
+// products of its slice with v_pk_mul_f16 — products rounded to fp16 as in the reference
+// (src/cuda_sddmm.cu:382) — added in fp32, then the LK lanes of a group combine them with a
+// reduce-scatter butterfly: at every stage a lane keeps half of its values and adds the
+// partner's copy of that half, so after log2(V) stages each output sits in exactly one lane.
+// Partners are reached with DPP (quad_perm, row_half_mirror, row_mirror) inside a 16-lane row,
+// ds_swizzle across rows and ds_bpermute across the two 32-lane halves.
+#include "vs_common.hpp"
+
+namespace vs {
+
+// Value held by the lane's partner in the opposite half of an aligned block of 2*STRIDE lanes.
+template <int STRIDE>
+__device__ __forceinline__ float partner(float x)
+{
+    const int xi = __builtin_bit_cast(int, x);
+    int r;
+    if constexpr (STRIDE == 1) {
+        r = __builtin_amdgcn_update_dpp(0, xi, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
+    } else if constexpr (STRIDE == 2) {
+        r = __builtin_amdgcn_update_dpp(0, xi, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
+    } else if constexpr (STRIDE == 4) {
+        r = __builtin_amdgcn_update_dpp(0, xi, 0x141, 0xF, 0xF, true);  // row_half_mirror: i <-> 7 - i
+    } else if constexpr (STRIDE == 8) {
+        r = __builtin_amdgcn_update_dpp(0, xi, 0x140, 0xF, 0xF, true);  // row_mirror: i <-> 15 - i
+    } else if constexpr (STRIDE == 16) {
+        r = __builtin_amdgcn_ds_swizzle(xi, 0x401F);                    // bit mode, xor 16
+    } else {
+        const int lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+        r = __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, xi);
+    }
+    return __builtin_bit_cast(float, r);
+}
+
+// One butterfly stage over `vals[0..NV)`.  Returns through vals[0..max(NV/2,1)).
+template <int STRIDE, int NV>
+__device__ __forceinline__ void reduce_stage(float *vals, int cl)
+{
+    if constexpr (NV > 1) {
+        const bool upper = (cl & STRIDE) != 0;
+#pragma unroll
+        for (int i = 0; i < NV / 2; ++i) {
+            const float send = upper ? vals[i] : vals[i + NV / 2];
+            const float keep = upper ? vals[i + NV / 2] : vals[i];
+            vals[i] = keep + partner<STRIDE>(send);
+        }
+    } else {
+        vals[0] += partner<STRIDE>(vals[0]);
+    }
+}
+
+template <int LK, int NV>
+__device__ __forceinline__ void reduce_group(float *vals, int cl)
+{
+    if constexpr (LK > 1) {
+        reduce_stage<LK / 2, NV>(vals, cl);
+        reduce_group<LK / 2, (NV > 1 ? NV / 2 : 1)>(vals, cl);
+    }
+}
+
+template <int VEC>
+__device__ __forceinline__ void load_slice(half_t (&dst)[VEC], const half_t *p, bool ok)
+{
+    if constexpr (VEC == 8) {
+        half8_t t = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (ok) t = *reinterpret_cast<const half8_t *>(p);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) dst[i] = t[i];
+    } else {
+        dst[0] = ok ? p[0] : (half_t)0.f;
+    }
+}
+
+template <int V, int VEC>
+__device__ __forceinline__ void slice_dot(float (&acc)[V], const half_t (&a)[V][VEC], const half_t (&b)[VEC])
+{
+#pragma clang fp contract(off)  // keep the fp16 rounding of every product
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+        if constexpr (VEC == 8) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const half2_t aa = {a[v][2 * i], a[v][2 * i + 1]};
+                const half2_t bb = {b[2 * i], b[2 * i + 1]};
+                const half2_t prod = aa * bb;  // v_pk_mul_f16
+                acc[v] += (float)prod[0];
+                acc[v] += (float)prod[1];
+            }
+        } else {
+            const half_t prod = a[v][0] * b[0];
+            acc[v] += (float)prod;
+        }
+    }
+}
+
+// SINGLE: the whole of K fits one chunk (K <= LK*VEC) and the lhs slices stay in registers.
+template <int V, int LK, int VEC, bool SINGLE, typename OutT>
+__global__ void __launch_bounds__(256)
+sddmm_valu_kernel(int m_vec, int K, int slots, const int *__restrict__ row_indices,
+                  const int *__restrict__ row_offsets, const int *__restrict__ col_indices,
+                  const half_t *__restrict__ lhs, const half_t *__restrict__ rhs, OutT *__restrict__ out)
+{
+    constexpr int G = 64 / LK;
+    constexpr int CHUNK = LK * VEC;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const long long wg = (long long)blockIdx.x * (blockDim.x >> 6) + wave;
+    if (wg >= (long long)m_vec * slots) return;
+    const int slot = (int)(wg / slots);
+    const int s = (int)(wg % slots);
+    const int row = row_indices[slot];
+    const int beg = row_offsets[row];
+    const int end = row_offsets[row + 1];
+    const int n_groups = (end - beg + G - 1) / G;
+    if (s >= n_groups) return;
+    const int cl = lane % LK;
+    const int g = lane / LK;
+    const half_t *lhs_rows = lhs + (size_t)row * V * K;
+    const int n_chunks = SINGLE ? 1 : (K + CHUNK - 1) / CHUNK;
+
+    half_t a0[V][VEC];
+    if constexpr (SINGLE) {
+        const int off = cl * VEC;
+#pragma unroll
+        for (int v = 0; v < V; ++v) load_slice<VEC>(a0[v], lhs_rows + (size_t)v * K + off, off < K);
+    }
+
+    // Every lane of the wave runs the same number of steps so the cross-lane exchanges below
+    // always see all partners; padded slots gather the row's last vector and skip the store.
+    for (int grp = s; grp < n_groups; grp += slots) {
+        const int j = beg + grp * G + g;
+        const bool valid = j < end;
+        const int jc = valid ? j : end - 1;
+        const half_t *rhs_row = rhs + (size_t)col_indices[jc] * K;
+        float acc[V];
+#pragma unroll
+        for (int v = 0; v < V; ++v) acc[v] = 0.f;
+        if constexpr (SINGLE) {
+            const int off = cl * VEC;
+            half_t b[VEC];
+            load_slice<VEC>(b, rhs_row + off, off < K);
+            slice_dot<V, VEC>(acc, a0, b);
+        } else {
+            for (int ch = 0; ch < n_chunks; ++ch) {
+                const int off = ch * CHUNK + cl * VEC;
+                const bool ok = off < K;
+                half_t a[V][VEC];
+                half_t b[VEC];
+#pragma unroll
+                for (int v = 0; v < V; ++v) load_slice<VEC>(a[v], lhs_rows + (size_t)v * K + off, ok);
+                load_slice<VEC>(b, rhs_row + off, ok);
+                slice_dot<V, VEC>(acc, a, b);
+            }
+        }
+        reduce_group<LK, V>(acc, cl);
+        // After the butterfly: V >= LK -> lane cl holds outputs v = cl*(V/LK) + i, i < V/LK;
+        //                      V <  LK -> lanes with cl % (LK/V) == 0 hold output v = cl / (LK/V).
+        if (valid) {
+            if constexpr (V >= LK) {
+                constexpr int PER = V / LK;
+                store_converted<OutT, PER>(out + (size_t)j * V + cl * PER, acc);
+            } else {
+                constexpr int REP = LK / V;
+                if (cl % REP == 0) store_converted<OutT, 1>(out + (size_t)j * V + cl / REP, acc);
+            }
+        }
+    }
+}
+
+template <int V, int LK, int VEC, bool SINGLE, typename OutT>
+static int launch_one(int m_vec, int k, int nonzeros_vec, const int *row_indices, const int *row_offsets,
+                      const int *col_indices, const half_t *lhs, const half_t *rhs, OutT *out, hipStream_t stream)
+{
+    constexpr int kWavesPerBlock = 4;
+    const int slots = sddmm_auto_slots(m_vec, nonzeros_vec, 64 / LK);
+    const long long waves = (long long)m_vec * slots;
+    const long long blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
+    if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
+    hipLaunchKernelGGL((sddmm_valu_kernel<V, LK, VEC, SINGLE, OutT>), dim3((unsigned)blocks),
+                       dim3(64 * kWavesPerBlock), 0, stream, m_vec, k, slots, row_indices, row_offsets,
+                       col_indices, lhs, rhs, out);
+    return (int)hipGetLastError();
+}
+
+template <int V, typename OutT>
+static int launch_shape(int m_vec, int k, int nonzeros_vec, const int *row_indices, const int *row_offsets,
+                        const int *col_indices, const half_t *lhs, const half_t *rhs, OutT *out, hipStream_t stream)
+{
+#define VS_GO(LK, VEC, SINGLE) \
+    return launch_one<V, LK, VEC, SINGLE, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream)
+    if (k % 8 == 0) {
+        if (k <= 32) VS_GO(4, 8, true);
+        if (k <= 64) VS_GO(8, 8, true);
+        if (k <= 128) VS_GO(16, 8, true);
+        if (k <= 256) VS_GO(32, 8, true);
+        if (k <= 512) VS_GO(64, 8, true);
+        VS_GO(64, 8, false);
+    }
+    if (k <= 16) VS_GO(16, 1, true);
+    VS_GO(64, 1, false);
+#undef VS_GO
+}
+
+template <typename OutT>
+int launch_sddmm_valu(int m_vec, int k, int n, int nonzeros_vec, const int *row_indices,
+                      const int *row_offsets, const int *col_indices, const half_t *lhs,
+                      const half_t *rhs, OutT *out, int vec_length, hipStream_t stream)
+{
+    (void)n;
+    if (m_vec == 0 || nonzeros_vec == 0) return hipSuccess;
+    if (k <= 0) return hipErrorNotSupported;
+    switch (vec_length) {
+    case 1: return launch_shape<1, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream);
+    case 2: return launch_shape<2, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream);
+    case 4: return launch_shape<4, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream);
+    case 8: return launch_shape<8, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+template int launch_sddmm_valu<half_t>(int, int, int, int, const int *, const int *, const int *, const half_t *,
+                                       const half_t *, half_t *, int, hipStream_t);
+template int launch_sddmm_valu<float>(int, int, int, int, const int *, const int *, const int *, const half_t *,
+                                      const half_t *, float *, int, hipStream_t);
+
+}  // namespace vs

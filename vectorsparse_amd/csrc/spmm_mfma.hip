@@ -1,0 +1,218 @@
+// SpMM on fp16 MFMA for column-vector CSR (replaces src/wmma_spmm.cu of the reference).
+//
+// Work item = (vector row, tile of TN = 16*CPL dense columns), one workgroup of W waves.
+// The waves of a workgroup split the row's nonzero vectors in interleaved steps of 16 and
+// their fp32 partial tiles are summed through LDS in a fixed order, so the result does not
+// depend on the launch shape's timing and no cross-workgroup reduction is needed for the
+// fp16 output.
+//
+// One step (16 nonzero vectors x TN columns) in a wave, lane = (cs = lane % 16, g = lane / 16):
+//   * the lane loads CPL consecutive halves of four gathered rhs rows j = base + 4g + e,
+//     e = 0..3, at columns tile*TN + cs*CPL.. : for each e the 16 lanes of a group read one
+//     contiguous 2*TN-byte segment (128-bit loads for CPL = 8);
+//   * v_mfma_f32_16x16x16_f16 wants, per lane, 4 consecutive k for ONE column, so the
+//     CPL x 4 block a lane holds is transposed in registers with v_perm_b32 (no LDS round
+//     trip for the dense operand);
+//   * MFMA number c (c < CPL) computes D[v][cs] += sum_k a[v][j(k)] * B[col_j(k)][tile*TN + cs*CPL + c]
+//     with the sparse vectors as the 16 x 16 A operand (rows v >= V are zero).
+//   The accumulator of lane (cs, g), register e, MFMA c is out[4g + e][tile*TN + cs*CPL + c], i.e.
+//   CPL consecutive outputs per (lane, e): one vector store each.
+#include "vs_common.hpp"
+
+namespace vs {
+
+template <int CPL>
+struct RowChunk;
+template <>
+struct RowChunk<8> {
+    uint4_t d;
+    __device__ __forceinline__ void load(const half_t *p) { d = *reinterpret_cast<const uint4_t *>(p); }
+    __device__ __forceinline__ uint32_t dword(int i) const { return d[i]; }
+};
+template <>
+struct RowChunk<4> {
+    uint2_t d;
+    __device__ __forceinline__ void load(const half_t *p) { d = *reinterpret_cast<const uint2_t *>(p); }
+    __device__ __forceinline__ uint32_t dword(int i) const { return d[i]; }
+};
+
+template <int V, int CPL, typename OutT>
+__global__ void __launch_bounds__(1024)
+spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
+                 const int *__restrict__ row_offsets, const int *__restrict__ column_indices,
+                 const half_t *__restrict__ values, const half_t *__restrict__ rhs,
+                 OutT *__restrict__ out)
+{
+    extern __shared__ float partial[];  // [W][V][TN]
+    constexpr int TN = 16 * CPL;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int n_waves = blockDim.x >> 6;
+    const int tile = blockIdx.x % n_tiles;
+    const int slot = blockIdx.x / n_tiles;
+    const int row = row_indices[slot];
+    const int beg = row_offsets[row];
+    const int end = row_offsets[row + 1];
+    const int cs = lane & 15;
+    const int g = lane >> 4;
+    const int col0 = tile * TN + cs * CPL;
+    const bool col_ok = col0 < n_cols;  // n_cols % CPL == 0: a lane's chunk is all in or all out
+    const half_t *rhs_col = rhs + (col_ok ? col0 : 0);
+
+    float4_t acc[CPL];
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) acc[c] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    for (int base = beg + 16 * wave; base < end; base += 16 * n_waves) {
+        RowChunk<CPL> chunk[4];
+        half4_t a;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int j = base + 4 * g + e;
+            const bool valid = j < end;
+            // Slots past the row's end repeat its last vector with a zero value: the gather
+            // stays in bounds and contributes nothing.
+            const int jc = valid ? j : end - 1;
+            const int col = column_indices[jc];
+            half_t av = (half_t)0.f;
+            if (valid && cs < V) av = values[(size_t)jc * V + cs];
+            a[e] = av;
+            chunk[e].load(rhs_col + (size_t)col * n_cols);
+        }
+#pragma unroll
+        for (int p = 0; p < CPL / 2; ++p) {
+            const uint32_t lo01 = pack_lo(chunk[0].dword(p), chunk[1].dword(p));
+            const uint32_t lo23 = pack_lo(chunk[2].dword(p), chunk[3].dword(p));
+            const uint32_t hi01 = pack_hi(chunk[0].dword(p), chunk[1].dword(p));
+            const uint32_t hi23 = pack_hi(chunk[2].dword(p), chunk[3].dword(p));
+            const half4_t b_even = bit_cast_u32x2<half4_t>(lo01, lo23);
+            const half4_t b_odd = bit_cast_u32x2<half4_t>(hi01, hi23);
+            acc[2 * p] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, b_even, acc[2 * p], 0, 0, 0);
+            acc[2 * p + 1] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, b_odd, acc[2 * p + 1], 0, 0, 0);
+        }
+    }
+
+    if (n_waves == 1) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int v = 4 * g + e;
+            if (v < V && col_ok) {
+                float tmp[CPL];
+#pragma unroll
+                for (int c = 0; c < CPL; ++c) tmp[c] = acc[c][e];
+                store_converted<OutT, CPL>(out + ((size_t)row * V + v) * n_cols + col0, tmp);
+            }
+        }
+        return;
+    }
+
+    float *mine = partial + (size_t)wave * V * TN;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int v = 4 * g + e;
+        if (v < V) {
+#pragma unroll
+            for (int c4 = 0; c4 < CPL / 4; ++c4) {
+                float4_t t = {acc[4 * c4][e], acc[4 * c4 + 1][e], acc[4 * c4 + 2][e], acc[4 * c4 + 3][e]};
+                *reinterpret_cast<float4_t *>(mine + v * TN + cs * CPL + 4 * c4) = t;
+            }
+        }
+    }
+    __syncthreads();
+    const int t = threadIdx.x;
+    if (t < V * 16) {
+        const int v = t >> 4;
+        const int cs2 = t & 15;
+        const int col = tile * TN + cs2 * CPL;
+        if (col < n_cols) {
+            float sum[CPL];
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) sum[c] = 0.f;
+            for (int w = 0; w < n_waves; ++w) {
+                const float *src = partial + (size_t)w * V * TN + v * TN + cs2 * CPL;
+#pragma unroll
+                for (int c4 = 0; c4 < CPL / 4; ++c4) {
+                    const float4_t x = *reinterpret_cast<const float4_t *>(src + 4 * c4);
+                    sum[4 * c4] += x[0];
+                    sum[4 * c4 + 1] += x[1];
+                    sum[4 * c4 + 2] += x[2];
+                    sum[4 * c4 + 3] += x[3];
+                }
+            }
+            store_converted<OutT, CPL>(out + ((size_t)row * V + v) * n_cols + col, sum);
+        }
+    }
+}
+
+static int next_pow2(int x)
+{
+    int p = 1;
+    while (p < x) p <<= 1;
+    return p;
+}
+
+template <int V, int CPL, typename OutT>
+static int launch_one(int m_vec, int k, int n, int waves, const int *row_indices, const int *row_offsets,
+                      const int *column_indices, const half_t *values, const half_t *rhs, OutT *out,
+                      hipStream_t stream)
+{
+    (void)n;
+    constexpr int TN = 16 * CPL;
+    const int n_tiles = ceil_div(k, TN);
+    const long long blocks = (long long)m_vec * n_tiles;
+    if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
+    const size_t lds = waves > 1 ? (size_t)waves * V * TN * sizeof(float) : 0;
+    hipLaunchKernelGGL((spmm_mfma_kernel<V, CPL, OutT>), dim3((unsigned)blocks), dim3(64 * waves), lds, stream,
+                       k, n_tiles, row_indices, row_offsets, column_indices, values, rhs, out);
+    return (int)hipGetLastError();
+}
+
+template <int CPL, typename OutT>
+static int launch_v(int vec_length, int m_vec, int k, int n, int waves, const int *row_indices,
+                    const int *row_offsets, const int *column_indices, const half_t *values,
+                    const half_t *rhs, OutT *out, hipStream_t stream)
+{
+    switch (vec_length) {
+    case 1: return launch_one<1, CPL, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
+    case 2: return launch_one<2, CPL, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
+    case 4: return launch_one<4, CPL, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
+    case 8: return launch_one<8, CPL, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+template <typename OutT>
+int launch_spmm_mfma(int m_vec, int vec_length, int k, int n, const int *row_indices,
+                     const int *row_offsets, const int *column_indices, const half_t *values,
+                     const half_t *rhs, OutT *out, hipStream_t stream)
+{
+    if (m_vec == 0 || k == 0) return hipSuccess;
+    if (k % 4 != 0) return hipErrorNotSupported;
+    constexpr int kTargetBlocks = 256;   // one workgroup per CU at least
+    constexpr int kTargetWaves = 4096;
+    int cpl = options().spmm_cols_per_lane;
+    if (cpl != 4 && cpl != 8) {
+        const long long blocks128 = (long long)m_vec * ceil_div(k, 128);
+        cpl = (k % 8 == 0 && blocks128 >= kTargetBlocks) ? 8 : 4;
+    }
+    if (cpl == 8 && k % 8 != 0) cpl = 4;
+    const long long blocks = (long long)m_vec * ceil_div(k, 16 * cpl);
+    int waves = options().spmm_waves;
+    if (waves <= 0) {
+        waves = next_pow2((int)((kTargetWaves + blocks - 1) / blocks));
+        const int max_useful = next_pow2(ceil_div(n > 0 ? n : 1, 16));  // a row holds at most n vectors
+        if (waves > max_useful) waves = max_useful;
+    }
+    if (waves < 1) waves = 1;
+    if (waves > 16) waves = 16;
+    if (cpl == 8)
+        return launch_v<8, OutT>(vec_length, m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
+    return launch_v<4, OutT>(vec_length, m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
+}
+
+template int launch_spmm_mfma<half_t>(int, int, int, int, const int *, const int *, const int *, const half_t *,
+                                      const half_t *, half_t *, hipStream_t);
+template int launch_spmm_mfma<float>(int, int, int, int, const int *, const int *, const int *, const half_t *,
+                                     const half_t *, float *, hipStream_t);
+
+}  // namespace vs

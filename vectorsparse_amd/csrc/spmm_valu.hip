@@ -1,0 +1,175 @@
+// Fine-grained SpMM on packed-fp16 VALU (replaces src/cuda_spmm.cu of the reference).
+//
+// A V x 1 vector times a gathered rhs row is a rank-1 update, not a dense contraction, so
+// this path keeps it on the vector ALU: v_pk_mul_f16 forms the products, each rounded to fp16
+// exactly as the reference does (src/spmm_utils/compute_utils.h:45), and the sum is kept in
+// fp32.  Work item = (vector row, tile of TN = 8*LR dense columns); a wave is G = 64/LR groups
+// of LR lanes, each group walks its own nonzero vectors and every lane owns 8 consecutive
+// columns (one 128-bit load per gathered row).  The W*G partial tiles are summed through LDS
+// in a fixed order.
+#include "vs_common.hpp"
+
+namespace vs {
+
+template <int V, int LR, typename OutT>
+__global__ void __launch_bounds__(1024)
+spmm_valu_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
+                 const int *__restrict__ row_offsets, const int *__restrict__ column_indices,
+                 const half_t *__restrict__ values, const half_t *__restrict__ rhs,
+                 OutT *__restrict__ out)
+{
+#pragma clang fp contract(off)  // keep the fp16 rounding of every product
+    extern __shared__ float partial[];  // [W*G][V][TN]
+    constexpr int G = 64 / LR;
+    constexpr int TN = 8 * LR;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int n_waves = blockDim.x >> 6;
+    const int tile = blockIdx.x % n_tiles;
+    const int slot = blockIdx.x / n_tiles;
+    const int row = row_indices[slot];
+    const int beg = row_offsets[row];
+    const int end = row_offsets[row + 1];
+    const int cl = lane % LR;
+    const int g = lane / LR;
+    const int col0 = tile * TN + cl * 8;
+    const bool col_ok = col0 < n_cols;  // n_cols % 8 == 0
+    const half_t *rhs_col = rhs + (col_ok ? col0 : 0);
+
+    float acc[V][8];
+#pragma unroll
+    for (int v = 0; v < V; ++v)
+#pragma unroll
+        for (int c = 0; c < 8; ++c) acc[v][c] = 0.f;
+
+    for (int j = beg + wave * G + g; j < end; j += n_waves * G) {
+        const int col = column_indices[j];
+        half_t a[V];
+        if constexpr (V == 8) {
+            const half8_t t = *reinterpret_cast<const half8_t *>(values + (size_t)j * 8);
+#pragma unroll
+            for (int v = 0; v < 8; ++v) a[v] = t[v];
+        } else if constexpr (V == 4) {
+            const half4_t t = *reinterpret_cast<const half4_t *>(values + (size_t)j * 4);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) a[v] = t[v];
+        } else if constexpr (V == 2) {
+            const half2_t t = *reinterpret_cast<const half2_t *>(values + (size_t)j * 2);
+            a[0] = t[0];
+            a[1] = t[1];
+        } else {
+            a[0] = values[j];
+        }
+        const half8_t b = *reinterpret_cast<const half8_t *>(rhs_col + (size_t)col * n_cols);
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+#pragma unroll
+            for (int c2 = 0; c2 < 4; ++c2) {
+                const half2_t bb = {b[2 * c2], b[2 * c2 + 1]};
+                const half2_t aa = {a[v], a[v]};
+                const half2_t prod = aa * bb;  // v_pk_mul_f16: products rounded to fp16
+                acc[v][2 * c2] += (float)prod[0];
+                acc[v][2 * c2 + 1] += (float)prod[1];
+            }
+        }
+    }
+
+    if (n_waves * G == 1) {
+        if (col_ok) {
+#pragma unroll
+            for (int v = 0; v < V; ++v)
+                store_converted<OutT, 8>(out + ((size_t)row * V + v) * n_cols + col0, acc[v]);
+        }
+        return;
+    }
+
+    float *mine = partial + (size_t)(wave * G + g) * V * TN;
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+        float4_t lo = {acc[v][0], acc[v][1], acc[v][2], acc[v][3]};
+        float4_t hi = {acc[v][4], acc[v][5], acc[v][6], acc[v][7]};
+        *reinterpret_cast<float4_t *>(mine + v * TN + cl * 8) = lo;
+        *reinterpret_cast<float4_t *>(mine + v * TN + cl * 8 + 4) = hi;
+    }
+    __syncthreads();
+    const int n_partials = n_waves * G;
+    for (int item = threadIdx.x; item < V * LR; item += blockDim.x) {
+        const int v = item / LR;
+        const int cl2 = item % LR;
+        const int col = tile * TN + cl2 * 8;
+        if (col >= n_cols) continue;
+        float sum[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) sum[c] = 0.f;
+        for (int p = 0; p < n_partials; ++p) {
+            const float *src = partial + (size_t)p * V * TN + v * TN + cl2 * 8;
+            const float4_t x = *reinterpret_cast<const float4_t *>(src);
+            const float4_t y = *reinterpret_cast<const float4_t *>(src + 4);
+            sum[0] += x[0]; sum[1] += x[1]; sum[2] += x[2]; sum[3] += x[3];
+            sum[4] += y[0]; sum[5] += y[1]; sum[6] += y[2]; sum[7] += y[3];
+        }
+        store_converted<OutT, 8>(out + ((size_t)row * V + v) * n_cols + col, sum);
+    }
+}
+
+template <int V, int LR, typename OutT>
+static int launch_one(int m_vec, int k, int waves, const int *row_indices, const int *row_offsets,
+                      const int *column_indices, const half_t *values, const half_t *rhs, OutT *out,
+                      hipStream_t stream)
+{
+    constexpr int G = 64 / LR;
+    constexpr int TN = 8 * LR;
+    const int n_tiles = ceil_div(k, TN);
+    const long long blocks = (long long)m_vec * n_tiles;
+    if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
+    // LDS for the partial tiles: waves * 64 lanes * V * 8 floats; stay within 64 KiB.
+    const int max_waves = (64 * 1024) / (64 * V * 8 * (int)sizeof(float));
+    if (waves > max_waves) waves = max_waves;
+    if (waves < 1) waves = 1;
+    const size_t lds = (waves * G > 1) ? (size_t)waves * G * V * TN * sizeof(float) : 0;
+    hipLaunchKernelGGL((spmm_valu_kernel<V, LR, OutT>), dim3((unsigned)blocks), dim3(64 * waves), lds, stream,
+                       k, n_tiles, row_indices, row_offsets, column_indices, values, rhs, out);
+    return (int)hipGetLastError();
+}
+
+template <int V, typename OutT>
+static int launch_lr(int m_vec, int k, int waves, const int *row_indices, const int *row_offsets,
+                     const int *column_indices, const half_t *values, const half_t *rhs, OutT *out,
+                     hipStream_t stream)
+{
+    if (k <= 64) return launch_one<V, 8, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
+    if (k <= 128) return launch_one<V, 16, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
+    if (k <= 256) return launch_one<V, 32, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
+    return launch_one<V, 64, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
+}
+
+template <typename OutT>
+int launch_spmm_valu(int m_vec, int vec_length, int k, int n, const int *row_indices,
+                     const int *row_offsets, const int *column_indices, const half_t *values,
+                     const half_t *rhs, OutT *out, hipStream_t stream)
+{
+    (void)n;
+    if (m_vec == 0 || k == 0) return hipSuccess;
+    if (k % 8 != 0) return hipErrorNotSupported;
+    int waves = options().spmm_waves;
+    if (waves <= 0) {
+        const long long blocks = (long long)m_vec * ceil_div(k, 512);
+        waves = 1;
+        while (waves < 8 && blocks * waves < 2048) waves <<= 1;
+    }
+    if (waves > 16) waves = 16;
+    switch (vec_length) {
+    case 1: return launch_lr<1, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
+    case 2: return launch_lr<2, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
+    case 4: return launch_lr<4, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
+    case 8: return launch_lr<8, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+template int launch_spmm_valu<half_t>(int, int, int, int, const int *, const int *, const int *, const half_t *,
+                                      const half_t *, half_t *, hipStream_t);
+template int launch_spmm_valu<float>(int, int, int, int, const int *, const int *, const int *, const half_t *,
+                                     const half_t *, float *, hipStream_t);
+
+}  // namespace vs

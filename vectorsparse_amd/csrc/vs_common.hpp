@@ -1,0 +1,131 @@
+// Shared device/host helpers for the gfx950 SpMM / SDDMM kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace vs {
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+// 4-byte aligned vector views: row starts inside the CSR arrays are only int-aligned.
+typedef int32_t int4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+
+constexpr int kWave = 64;
+
+// v_perm_b32 selectors: pick the low (high) halves of two dwords, first operand in the low half.
+constexpr uint32_t kPermLoLo = 0x05040100u;
+constexpr uint32_t kPermHiHi = 0x07060302u;
+
+__device__ __forceinline__ uint32_t pack_lo(uint32_t first, uint32_t second)
+{
+    return __builtin_amdgcn_perm(second, first, kPermLoLo);
+}
+__device__ __forceinline__ uint32_t pack_hi(uint32_t first, uint32_t second)
+{
+    return __builtin_amdgcn_perm(second, first, kPermHiHi);
+}
+
+template <typename T>
+__device__ __forceinline__ T bit_cast_u32x2(uint32_t a, uint32_t b)
+{
+    uint2_t u = {a, b};
+    return __builtin_bit_cast(T, u);
+}
+
+template <typename OutT>
+struct OutVec;
+
+// Store `Count` consecutive outputs converted from fp32 (Count in {1,2,4,8}).
+template <typename OutT, int Count>
+__device__ __forceinline__ void store_converted(OutT *dst, const float *src);
+
+template <>
+__device__ __forceinline__ void store_converted<half_t, 8>(half_t *dst, const float *src)
+{
+    half8_t h;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) h[i] = (half_t)src[i];
+    *reinterpret_cast<half8_t *>(dst) = h;
+}
+template <>
+__device__ __forceinline__ void store_converted<half_t, 4>(half_t *dst, const float *src)
+{
+    half4_t h;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) h[i] = (half_t)src[i];
+    *reinterpret_cast<half4_t *>(dst) = h;
+}
+template <>
+__device__ __forceinline__ void store_converted<half_t, 2>(half_t *dst, const float *src)
+{
+    half2_t h = {(half_t)src[0], (half_t)src[1]};
+    *reinterpret_cast<half2_t *>(dst) = h;
+}
+template <>
+__device__ __forceinline__ void store_converted<half_t, 1>(half_t *dst, const float *src)
+{
+    *dst = (half_t)src[0];
+}
+template <>
+__device__ __forceinline__ void store_converted<float, 8>(float *dst, const float *src)
+{
+    float4_t a = {src[0], src[1], src[2], src[3]};
+    float4_t b = {src[4], src[5], src[6], src[7]};
+    reinterpret_cast<float4_t *>(dst)[0] = a;
+    reinterpret_cast<float4_t *>(dst)[1] = b;
+}
+template <>
+__device__ __forceinline__ void store_converted<float, 4>(float *dst, const float *src)
+{
+    float4_t a = {src[0], src[1], src[2], src[3]};
+    *reinterpret_cast<float4_t *>(dst) = a;
+}
+template <>
+__device__ __forceinline__ void store_converted<float, 2>(float *dst, const float *src)
+{
+    dst[0] = src[0];
+    dst[1] = src[1];
+}
+template <>
+__device__ __forceinline__ void store_converted<float, 1>(float *dst, const float *src)
+{
+    dst[0] = src[0];
+}
+
+// Process-wide launch-shape overrides (0 = automatic).
+struct Options {
+    int spmm_waves = 0;
+    int spmm_cols_per_lane = 0;
+    int sddmm_slots = 0;
+};
+Options &options();
+
+inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// Waves per vector row for the SDDMM kernels; `group` = nonzero vectors a wave covers per step.
+int sddmm_auto_slots(int m_vec, int nonzeros_vec, int group);
+
+// Launchers (one per kernel family); return a hipError_t-valued int.
+template <typename OutT>
+int launch_spmm_mfma(int m_vec, int vec_length, int k, int n, const int *row_indices,
+                     const int *row_offsets, const int *column_indices, const half_t *values,
+                     const half_t *rhs, OutT *out, hipStream_t stream);
+template <typename OutT>
+int launch_spmm_valu(int m_vec, int vec_length, int k, int n, const int *row_indices,
+                     const int *row_offsets, const int *column_indices, const half_t *values,
+                     const half_t *rhs, OutT *out, hipStream_t stream);
+template <typename OutT>
+int launch_sddmm_mfma(int m_vec, int k, int n, int nonzeros_vec, const int *row_indices,
+                      const int *row_offsets, const int *col_indices, const half_t *lhs,
+                      const half_t *rhs, OutT *out, int vec_length, hipStream_t stream);
+template <typename OutT>
+int launch_sddmm_valu(int m_vec, int k, int n, int nonzeros_vec, const int *row_indices,
+                      const int *row_offsets, const int *col_indices, const half_t *lhs,
+                      const half_t *rhs, OutT *out, int vec_length, hipStream_t stream);
+
+}  // namespace vs

@@ -1,0 +1,209 @@
+// C ABI of the library: argument validation and dispatch to the kernel launchers.
+#include "../../include/vsparse.h"
+
+#include <algorithm>
+#include <cstring>
+#include <numeric>
+#include <vector>
+
+#include "vs_common.hpp"
+
+namespace vs {
+Options &options()
+{
+    static Options opts;
+    return opts;
+}
+}  // namespace vs
+
+namespace {
+
+using vs::half_t;
+
+bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+bool vec_ok(int v) { return v == 1 || v == 2 || v == 4 || v == 8; }
+
+int check_spmm(int m_vec, int vec_length, int k, int n, const int *row_indices, const int *row_offsets,
+               const int *column_indices, const void *values, const void *rhs, const void *out, size_t out_elem)
+{
+    if (m_vec < 0 || k < 0 || n < 0 || !vec_ok(vec_length)) return VS_ERROR_INVALID_VALUE;
+    if (m_vec == 0 || k == 0) return VS_SUCCESS;
+    if (!row_indices || !row_offsets || !out) return VS_ERROR_INVALID_VALUE;
+    // column_indices / values / rhs may legitimately be null only if the pattern is empty, which the
+    // host cannot see; require them whenever the sparse matrix has columns at all.
+    if (n > 0 && (!column_indices || !values || !rhs)) return VS_ERROR_INVALID_VALUE;
+    if (!aligned(values, 2 * (size_t)vec_length) || !aligned(rhs, 16) || !aligned(out, 8 * out_elem))
+        return VS_ERROR_INVALID_VALUE;
+    return VS_SUCCESS;
+}
+
+int check_sddmm(int m_vec, int k, int n, int nonzeros_vec, const int *row_indices, const int *row_offsets,
+                const int *col_indices, const void *lhs, const void *rhs, const void *out, int vec_length,
+                size_t out_elem)
+{
+    if (m_vec < 0 || k < 0 || n < 0 || nonzeros_vec < 0 || !vec_ok(vec_length)) return VS_ERROR_INVALID_VALUE;
+    if (m_vec == 0 || nonzeros_vec == 0) return VS_SUCCESS;
+    if (!row_indices || !row_offsets || !col_indices || !lhs || !rhs || !out) return VS_ERROR_INVALID_VALUE;
+    if (!aligned(out, out_elem * (size_t)vec_length)) return VS_ERROR_INVALID_VALUE;
+    if (k % 8 == 0 && (!aligned(lhs, 16) || !aligned(rhs, 16))) return VS_ERROR_INVALID_VALUE;
+    return VS_SUCCESS;
+}
+
+}  // namespace
+
+extern "C" {
+
+int vs_version(void) { return 100; }
+
+const char *vs_status_string(int status)
+{
+    switch (status) {
+    case VS_SUCCESS: return "success";
+    case VS_ERROR_INVALID_VALUE: return "invalid value (null pointer, negative size, misaligned operand, or unsupported vec_length/algorithm)";
+    case VS_ERROR_NOT_SUPPORTED: return "shape not supported by the selected path";
+    default: return hipGetErrorString(static_cast<hipError_t>(status));
+    }
+}
+
+int vs_wmma_spmm_f16(int m_vec, int vec_length, int k, int n, const int *row_indices, const int *row_offsets,
+                     const int *column_indices, const void *values, const void *rhs_matrix, void *output_matrix,
+                     void *stream)
+{
+    int st = check_spmm(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices, values, rhs_matrix,
+                        output_matrix, sizeof(half_t));
+    if (st != VS_SUCCESS) return st;
+    return vs::launch_spmm_mfma<half_t>(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices,
+                                        static_cast<const half_t *>(values), static_cast<const half_t *>(rhs_matrix),
+                                        static_cast<half_t *>(output_matrix), static_cast<hipStream_t>(stream));
+}
+
+int vs_wmma_spmm_f16_f32out(int m_vec, int vec_length, int k, int n, const int *row_indices,
+                            const int *row_offsets, const int *column_indices, const void *values,
+                            const void *rhs_matrix, float *output_matrix, void *stream)
+{
+    int st = check_spmm(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices, values, rhs_matrix,
+                        output_matrix, sizeof(float));
+    if (st != VS_SUCCESS) return st;
+    return vs::launch_spmm_mfma<float>(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices,
+                                       static_cast<const half_t *>(values), static_cast<const half_t *>(rhs_matrix),
+                                       output_matrix, static_cast<hipStream_t>(stream));
+}
+
+int vs_cuda_spmm_f16(int m_vec, int vec_length, int k, int n, const int *row_indices, const int *row_offsets,
+                     const int *column_indices, const void *values, const void *rhs_matrix, void *output_matrix,
+                     void *stream)
+{
+    int st = check_spmm(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices, values, rhs_matrix,
+                        output_matrix, sizeof(half_t));
+    if (st != VS_SUCCESS) return st;
+    return vs::launch_spmm_valu<half_t>(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices,
+                                        static_cast<const half_t *>(values), static_cast<const half_t *>(rhs_matrix),
+                                        static_cast<half_t *>(output_matrix), static_cast<hipStream_t>(stream));
+}
+
+int vs_cuda_spmm_f16_f32out(int m_vec, int vec_length, int k, int n, const int *row_indices,
+                            const int *row_offsets, const int *column_indices, const void *values,
+                            const void *rhs_matrix, float *output_matrix, void *stream)
+{
+    int st = check_spmm(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices, values, rhs_matrix,
+                        output_matrix, sizeof(float));
+    if (st != VS_SUCCESS) return st;
+    return vs::launch_spmm_valu<float>(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices,
+                                       static_cast<const half_t *>(values), static_cast<const half_t *>(rhs_matrix),
+                                       output_matrix, static_cast<hipStream_t>(stream));
+}
+
+int vs_wmma_sddmm_f16(int m_vec, int k, int n, int nonzeros_vec, const int *row_indices, const int *row_offsets,
+                      const int *col_indices, const void *lhs_matrix, const void *rhs_matrix, void *output_values,
+                      int vec_length, void *stream, int algorithm)
+{
+    if (algorithm < 0 || algorithm > 2) return VS_ERROR_INVALID_VALUE;
+    int st = check_sddmm(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices, lhs_matrix, rhs_matrix,
+                         output_values, vec_length, sizeof(half_t));
+    if (st != VS_SUCCESS) return st;
+    return vs::launch_sddmm_mfma<half_t>(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices,
+                                         static_cast<const half_t *>(lhs_matrix),
+                                         static_cast<const half_t *>(rhs_matrix),
+                                         static_cast<half_t *>(output_values), vec_length,
+                                         static_cast<hipStream_t>(stream));
+}
+
+int vs_wmma_sddmm_f16_f32out(int m_vec, int k, int n, int nonzeros_vec, const int *row_indices,
+                             const int *row_offsets, const int *col_indices, const void *lhs_matrix,
+                             const void *rhs_matrix, float *output_values, int vec_length, void *stream,
+                             int algorithm)
+{
+    if (algorithm < 0 || algorithm > 2) return VS_ERROR_INVALID_VALUE;
+    int st = check_sddmm(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices, lhs_matrix, rhs_matrix,
+                         output_values, vec_length, sizeof(float));
+    if (st != VS_SUCCESS) return st;
+    return vs::launch_sddmm_mfma<float>(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices,
+                                        static_cast<const half_t *>(lhs_matrix),
+                                        static_cast<const half_t *>(rhs_matrix), output_values, vec_length,
+                                        static_cast<hipStream_t>(stream));
+}
+
+int vs_cuda_sddmm_f16(int m_vec, int k, int n, int nonzeros_vec, const int *row_indices, const int *row_offsets,
+                      const int *col_indices, const void *lhs_matrix, const void *rhs_matrix, void *output_values,
+                      int vec_length, void *stream)
+{
+    int st = check_sddmm(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices, lhs_matrix, rhs_matrix,
+                         output_values, vec_length, sizeof(half_t));
+    if (st != VS_SUCCESS) return st;
+    return vs::launch_sddmm_valu<half_t>(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices,
+                                         static_cast<const half_t *>(lhs_matrix),
+                                         static_cast<const half_t *>(rhs_matrix),
+                                         static_cast<half_t *>(output_values), vec_length,
+                                         static_cast<hipStream_t>(stream));
+}
+
+int vs_cuda_sddmm_f16_f32out(int m_vec, int k, int n, int nonzeros_vec, const int *row_indices,
+                             const int *row_offsets, const int *col_indices, const void *lhs_matrix,
+                             const void *rhs_matrix, float *output_values, int vec_length, void *stream)
+{
+    int st = check_sddmm(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices, lhs_matrix, rhs_matrix,
+                         output_values, vec_length, sizeof(float));
+    if (st != VS_SUCCESS) return st;
+    return vs::launch_sddmm_valu<float>(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices,
+                                        static_cast<const half_t *>(lhs_matrix),
+                                        static_cast<const half_t *>(rhs_matrix), output_values, vec_length,
+                                        static_cast<hipStream_t>(stream));
+}
+
+void vs_identity_row_swizzle(int rows, int *row_indices)
+{
+    if (rows <= 0 || !row_indices) return;
+    std::iota(row_indices, row_indices + rows, 0);
+}
+
+void vs_sorted_row_swizzle(int rows, const int *row_offsets, int *row_indices)
+{
+    if (rows <= 0 || !row_offsets || !row_indices) return;
+    std::iota(row_indices, row_indices + rows, 0);
+    // Longest rows first so they are dispatched first; a stable sort keeps equal-length rows in
+    // ascending order, which makes the swizzle reproducible.
+    std::stable_sort(row_indices, row_indices + rows, [row_offsets](int a, int b) {
+        return row_offsets[a + 1] - row_offsets[a] > row_offsets[b + 1] - row_offsets[b];
+    });
+}
+
+int vs_set_option(const char *name, int value)
+{
+    if (!name || value < 0) return VS_ERROR_INVALID_VALUE;
+    vs::Options &o = vs::options();
+    if (std::strcmp(name, "spmm_waves") == 0) {
+        if (value > 16) return VS_ERROR_INVALID_VALUE;
+        o.spmm_waves = value;
+    } else if (std::strcmp(name, "spmm_cols_per_lane") == 0) {
+        if (value != 0 && value != 4 && value != 8) return VS_ERROR_INVALID_VALUE;
+        o.spmm_cols_per_lane = value;
+    } else if (std::strcmp(name, "sddmm_slots") == 0) {
+        o.sddmm_slots = value;
+    } else {
+        return VS_ERROR_INVALID_VALUE;
+    }
+    return VS_SUCCESS;
+}
+
+}  // extern "C"
