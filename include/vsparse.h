@@ -68,9 +68,12 @@ int vs_wmma_spmm_f16_f32out(int m_vec, int vec_length, int k, int n,
 
 /*
  * Replaces spmm::cudaSpmm(half in, half out) — include/cuda_spmm.cuh:15-21,
- * src/cuda_spmm.cu:316-325.  Fine-grained path on packed-fp16 VALU: every
- * product is rounded to fp16 (src/spmm_utils/compute_utils.h:45) and added in
- * fp32.  vec_length in {1, 2, 4, 8}.  Same alignment rules; k % 8 == 0.
+ * src/cuda_spmm.cu:316-325.  Fine-grained path on the fp16 vector ALU
+ * (mixed-precision FMA: exact fp16 x fp16 products, fp32 accumulate).  The
+ * reference rounds each product to fp16 (src/spmm_utils/compute_utils.h:45);
+ * that rounding is deliberately not reproduced because it alone breaks the
+ * 1e-2 relative-error contract against the host loop.
+ * vec_length in {1, 2, 4, 8}.  Same alignment rules; k % 8 == 0.
  */
 int vs_cuda_spmm_f16(int m_vec, int vec_length, int k, int n,
                      const int *row_indices, const int *row_offsets,
@@ -111,8 +114,9 @@ int vs_wmma_sddmm_f16_f32out(int m_vec, int k, int n, int nonzeros_vec,
 /*
  * Replaces sddmm::cudaSddmm(half in, half out) — include/cuda_sddmm.cuh:16-23,
  * src/cuda_sddmm.cu:1295-1331.  Per-lane slices of the contraction with a
- * cross-lane (DPP / ds_swizzle) reduction; products rounded to fp16
- * (src/cuda_sddmm.cu:382), fp32 adds.  vec_length in {1, 2, 4, 8}; any k >= 1
+ * cross-lane (DPP / ds_swizzle) reduction; packed-fp16 dot products with
+ * exact products and fp32 sums (the reference's fp16 rounding of each product,
+ * src/cuda_sddmm.cu:382, is deliberately not reproduced).  vec_length in {1, 2, 4, 8}; any k >= 1
  * (k % 8 != 0 takes a slower scalar-load kernel).
  */
 int vs_cuda_sddmm_f16(int m_vec, int k, int n, int nonzeros_vec,

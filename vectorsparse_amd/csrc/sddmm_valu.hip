@@ -4,9 +4,10 @@
 // A wave is G = 64/LK groups of LK lanes; a group owns one nonzero vector j per step and lane
 // cl of the group owns the slice k in [chunk*LK*VEC + cl*VEC, +VEC) of both operand rows
 // (VEC = 8 halves: one 128-bit load; VEC = 1 for K % 8 != 0).  Each lane forms the V partial dot
-// products of its slice with v_pk_mul_f16 — products rounded to fp16 as in the reference
-// (src/cuda_sddmm.cu:382) — added in fp32, then the LK lanes of a group combine them with a
-// reduce-scatter butterfly: at every stage a lane keeps half of its values and adds the
+// products of its slice with v_dot2_f32_f16 (packed fp16 pairs, exact products, fp32 sum; the
+// reference rounds each product to fp16 first, src/cuda_sddmm.cu:382, which by itself exceeds the
+// 1e-2 relative-error budget against the host loop on near-zero outputs and is not reproduced),
+// then the LK lanes of a group combine them with a reduce-scatter butterfly: at every stage a lane keeps half of its values and adds the
 // partner's copy of that half, so after log2(V) stages each output sits in exactly one lane.
 // Partners are reached with DPP (quad_perm, row_half_mirror, row_mirror) inside a 16-lane row,
 // ds_swizzle across rows and ds_bpermute across the two 32-lane halves.
@@ -79,7 +80,6 @@ __device__ __forceinline__ void load_slice(half_t (&dst)[VEC], const half_t *p, 
 template <int V, int VEC>
 __device__ __forceinline__ void slice_dot(float (&acc)[V], const half_t (&a)[V][VEC], const half_t (&b)[VEC])
 {
-#pragma clang fp contract(off)  // keep the fp16 rounding of every product
 #pragma unroll
     for (int v = 0; v < V; ++v) {
         if constexpr (VEC == 8) {
@@ -87,13 +87,10 @@ __device__ __forceinline__ void slice_dot(float (&acc)[V], const half_t (&a)[V][
             for (int i = 0; i < 4; ++i) {
                 const half2_t aa = {a[v][2 * i], a[v][2 * i + 1]};
                 const half2_t bb = {b[2 * i], b[2 * i + 1]};
-                const half2_t prod = aa * bb;  // v_pk_mul_f16
-                acc[v] += (float)prod[0];
-                acc[v] += (float)prod[1];
+                acc[v] = __builtin_amdgcn_fdot2(aa, bb, acc[v], false);  // v_dot2_f32_f16
             }
         } else {
-            const half_t prod = a[v][0] * b[0];
-            acc[v] += (float)prod;
+            acc[v] = __builtin_fmaf((float)a[v][0], (float)b[0], acc[v]);
         }
     }
 }

@@ -1,9 +1,11 @@
-// Fine-grained SpMM on packed-fp16 VALU (replaces src/cuda_spmm.cu of the reference).
+// Fine-grained SpMM on the fp16 vector ALU (replaces src/cuda_spmm.cu of the reference).
 //
 // A V x 1 vector times a gathered rhs row is a rank-1 update, not a dense contraction, so
-// this path keeps it on the vector ALU: v_pk_mul_f16 forms the products, each rounded to fp16
-// exactly as the reference does (src/spmm_utils/compute_utils.h:45), and the sum is kept in
-// fp32.  Work item = (vector row, tile of TN = 8*LR dense columns); a wave is G = 64/LR groups
+// this path keeps it on the vector ALU: one mixed-precision v_fma_mix_f32 per multiply-add
+// (fp16 operands, exact product, fp32 accumulate).  The reference rounds every product to fp16
+// first (src/spmm_utils/compute_utils.h:45); that rounding alone costs up to ~9e-2 of the
+// 1e-2 relative-error budget against the host loop on near-zero outputs, so it is not
+// reproduced.  Work item = (vector row, tile of TN = 8*LR dense columns); a wave is G = 64/LR groups
 // of LR lanes, each group walks its own nonzero vectors and every lane owns 8 consecutive
 // columns (one 128-bit load per gathered row).  The W*G partial tiles are summed through LDS
 // in a fixed order.
@@ -18,7 +20,6 @@ spmm_valu_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
                  const half_t *__restrict__ values, const half_t *__restrict__ rhs,
                  OutT *__restrict__ out)
 {
-#pragma clang fp contract(off)  // keep the fp16 rounding of every product
     extern __shared__ float partial[];  // [W*G][V][TN]
     constexpr int G = 64 / LR;
     constexpr int TN = 8 * LR;
@@ -64,13 +65,7 @@ spmm_valu_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
 #pragma unroll
         for (int v = 0; v < V; ++v) {
 #pragma unroll
-            for (int c2 = 0; c2 < 4; ++c2) {
-                const half2_t bb = {b[2 * c2], b[2 * c2 + 1]};
-                const half2_t aa = {a[v], a[v]};
-                const half2_t prod = aa * bb;  // v_pk_mul_f16: products rounded to fp16
-                acc[v][2 * c2] += (float)prod[0];
-                acc[v][2 * c2 + 1] += (float)prod[1];
-            }
+            for (int c = 0; c < 8; ++c) acc[v][c] = __builtin_fmaf((float)a[v], (float)b[c], acc[v][c]);
         }
     }
 

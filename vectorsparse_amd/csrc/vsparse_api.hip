@@ -30,9 +30,9 @@ int check_spmm(int m_vec, int vec_length, int k, int n, const int *row_indices, 
     if (m_vec < 0 || k < 0 || n < 0 || !vec_ok(vec_length)) return VS_ERROR_INVALID_VALUE;
     if (m_vec == 0 || k == 0) return VS_SUCCESS;
     if (!row_indices || !row_offsets || !out) return VS_ERROR_INVALID_VALUE;
-    // column_indices / values / rhs may legitimately be null only if the pattern is empty, which the
-    // host cannot see; require them whenever the sparse matrix has columns at all.
-    if (n > 0 && (!column_indices || !values || !rhs)) return VS_ERROR_INVALID_VALUE;
+    // column_indices / values may be null when the pattern has no nonzero at all (an empty device
+    // allocation); the host cannot see the pattern, so only the dense operand is required here.
+    if (n > 0 && !rhs) return VS_ERROR_INVALID_VALUE;
     if (!aligned(values, 2 * (size_t)vec_length) || !aligned(rhs, 16) || !aligned(out, 8 * out_elem))
         return VS_ERROR_INVALID_VALUE;
     return VS_SUCCESS;
