@@ -123,6 +123,9 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--pmc", action="store_true",
+                    help="counter-collection mode for `rocprofv3 --pmc`: a 64 MiB device copy of known size "
+                         "(calibration), then a few eager launches of the headline kernel, nothing else")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the SpMM/SDDMM path has no multi-GPU leg (rows shard with no "
@@ -152,6 +155,19 @@ def main():
 
     def step():
         prob.spmm(Bd, kernel="wmma", out=out)
+
+    if args.pmc:
+        src = torch.zeros(32 * 1024 * 1024, dtype=torch.float16, device="cuda")   # 64 MiB read + 64 MiB written
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        for _ in range(10):
+            step()
+        torch.cuda.synchronize()
+        print(json.dumps({"pmc_mode": True, "copy_bytes_each_way": src.numel() * 2,
+                          "algorithmic_bytes": alg_bytes}))
+        return
 
     wall_ms, ev_ms = time_graph(torch, step, args.steps, args.warmup)
     eager_wall_ms, _ = time_eager(torch, step, args.steps, args.warmup)

@@ -133,6 +133,58 @@ int vs_cuda_sddmm_f16_f32out(int m_vec, int k, int n, int nonzeros_vec,
                              int vec_length, void *stream);
 
 /*
+ * Batched forms: `batch` independent problems that share one sparsity pattern
+ * (row_indices, row_offsets, column indices) in a single launch; problem b uses
+ * each operand pointer advanced by b * its stride (strides in ELEMENTS; a stride
+ * of 0 shares the operand).  batch <= 65535.  Everything else is as in the
+ * unbatched entry points.  No counterpart in the reference, which launches one
+ * problem per process; they exist because sparse attention runs one mask over
+ * many heads (the reference only links an external sparse-transformer repository,
+ * README.md:76).
+ */
+int vs_wmma_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n,
+                             const int *row_indices, const int *row_offsets,
+                             const int *column_indices,
+                             const void *values, long long stride_values,
+                             const void *rhs_matrix, long long stride_rhs,
+                             void *output_matrix, long long stride_output, void *stream);
+int vs_cuda_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n,
+                             const int *row_indices, const int *row_offsets,
+                             const int *column_indices,
+                             const void *values, long long stride_values,
+                             const void *rhs_matrix, long long stride_rhs,
+                             void *output_matrix, long long stride_output, void *stream);
+int vs_wmma_sddmm_f16_batched(int batch, int m_vec, int k, int n, int nonzeros_vec,
+                              const int *row_indices, const int *row_offsets,
+                              const int *col_indices,
+                              const void *lhs_matrix, long long stride_lhs,
+                              const void *rhs_matrix, long long stride_rhs,
+                              void *output_values, long long stride_output,
+                              int vec_length, void *stream, int algorithm);
+int vs_cuda_sddmm_f16_batched(int batch, int m_vec, int k, int n, int nonzeros_vec,
+                              const int *row_indices, const int *row_offsets,
+                              const int *col_indices,
+                              const void *lhs_matrix, long long stride_lhs,
+                              const void *rhs_matrix, long long stride_rhs,
+                              void *output_values, long long stride_output,
+                              int vec_length, void *stream);
+
+/*
+ * Row-wise softmax over the nonzeros of each SCALAR row of a column-vector CSR
+ * matrix, on the [nnz_vec][vec_length] fp16 value layout SDDMM writes and SpMM
+ * reads:  out = softmax_row(scale * in), computed in fp32.  `values_out` may
+ * equal `values_in`.  Batched like the entry points above (batch = 1 and zero
+ * strides for a single problem).  The reference does not ship this operator (it
+ * includes Sputnik's sparse_softmax.h, include/sputnik.h:22, from an external
+ * library); it is the middle step of SDDMM -> softmax -> SpMM sparse attention.
+ */
+int vs_sparse_softmax_f16(int batch, int m_vec, int vec_length,
+                          const int *row_indices, const int *row_offsets,
+                          const void *values_in, long long stride_in,
+                          void *values_out, long long stride_out,
+                          float scale, void *stream);
+
+/*
  * Host helpers (HOST pointers).  Replace IdentityRowSwizzle / SortedRowSwizzle —
  * include/bm_test_utils.h:196-198 and :200-215.  The sorted swizzle orders
  * vector rows by descending length; equal lengths keep ascending row order.

@@ -51,6 +51,25 @@ def sddmm_host_ref(m_vec, k, vec_length, row_offsets, col_indices, lhs_matrix, r
     return acc.astype(out_dtype).reshape(-1)
 
 
+def sparse_softmax_ref(m_vec, vec_length, row_offsets, values, scale=1.0):
+    """Row-wise softmax over the nonzeros of every scalar row, [nnz_vec, V] layout, in float64.
+
+    The reference does not ship this operator (it includes Sputnik's sparse_softmax.h,
+    include/sputnik.h:22, from an external library that is not in its tree), so this is the textbook
+    definition: out = exp(s*x - max) / sum(exp(s*x - max)) over the row's stored elements.
+    """
+    row_offsets = np.asarray(row_offsets)
+    x = np.asarray(values, dtype=np.float64).reshape(-1, vec_length) * float(scale)
+    out = np.empty_like(x)
+    for i in range(m_vec):
+        lo, hi = int(row_offsets[i]), int(row_offsets[i + 1])
+        if hi > lo:
+            blk = x[lo:hi]
+            e = np.exp(blk - blk.max(axis=0, keepdims=True))
+            out[lo:hi] = e / e.sum(axis=0, keepdims=True)
+    return out
+
+
 def identity_row_swizzle(rows):
     """include/bm_test_utils.h:196-198."""
     return np.arange(rows, dtype=np.int32)

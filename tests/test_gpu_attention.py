@@ -1,0 +1,117 @@
+"""Batched entry points, sparse softmax and the fixed-mask attention layer on the GPU."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle as co
+from oracle import numpy_oracle as no
+from vectorsparse_amd import ops
+from vectorsparse_amd import colvec_csr as cv
+from util import assert_parity
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("V", [1, 2, 4, 8])
+def test_sparse_softmax_parity(gpu, V):
+    # ragged rows incl. empty ones, a row longer than the register-cached limit (512 vectors)
+    lengths = np.array([0, 1, 3, 64, 65, 200, 513, 700, 0, 17], dtype=np.int64)
+    rng = np.random.default_rng(V)
+    ro, ci = cv._pattern_from_lengths(rng, len(lengths), 1024, lengths)
+    pat = cv.random_values(cv.ColVecCSR(len(lengths), 1024, V, ro, ci), seed=V + 1, scale=3.0)
+    prob = ops.DeviceProblem(pat, sort=True)
+    scale = 0.125
+    out = ops.sparse_softmax(pat.m_vec, V, prob.row_indices, prob.row_offsets, prob.values, scale=scale)
+    torch.cuda.synchronize()
+    ref = no.sparse_softmax_ref(pat.m_vec, V, pat.row_offsets, pat.values, scale)
+    assert_parity(out.cpu().numpy(), ref, "softmax V%d" % V)
+    # in place
+    vals = prob.values.clone()
+    ops.sparse_softmax(pat.m_vec, V, prob.row_indices, prob.row_offsets, vals, vals, scale=scale)
+    torch.cuda.synchronize()
+    assert np.array_equal(vals.cpu().numpy(), out.cpu().numpy())
+
+
+@pytest.mark.parametrize("kernel", ["wmma", "cuda"])
+def test_batched_equals_unbatched(gpu, kernel):
+    V, heads, K, N = 8, 5, 64, 64
+    pat = cv.binomial_pattern(24, 192, 0.8, seed=2, vec_length=V)
+    prob = ops.DeviceProblem(pat)
+    g = torch.Generator(device="cuda").manual_seed(0)
+    lhs = torch.randn((heads, pat.m, K), device="cuda", generator=g).half()
+    rhs = torch.randn((heads, 192, K), device="cuda", generator=g).half()
+    dense = torch.rand((heads, 192, N), device="cuda", generator=g).half()
+    scores = torch.empty((heads, pat.nnz_vec, V), dtype=torch.float16, device="cuda")
+    ops.sddmm_batched(pat.m_vec, K, 192, pat.nnz_vec, prob.row_indices, prob.row_offsets, prob.column_indices,
+                      lhs, rhs, scores, V, kernel=kernel)
+    out = torch.empty((heads, pat.m, N), dtype=torch.float16, device="cuda")
+    ops.spmm_batched(pat.m_vec, V, N, 192, prob.row_indices, prob.row_offsets, prob.column_indices, scores, dense,
+                     out, kernel=kernel)
+    torch.cuda.synchronize()
+    for h in range(heads):
+        one = prob.sddmm(lhs[h], rhs[h], kernel=kernel)
+        assert torch.equal(one, scores[h]), "head %d sddmm" % h
+        prob.values = scores[h]
+        assert torch.equal(prob.spmm(dense[h], kernel=kernel), out[h]), "head %d spmm" % h
+    # a shared (stride 0) dense operand
+    shared = torch.empty_like(out)
+    ops.spmm_batched(pat.m_vec, V, N, 192, prob.row_indices, prob.row_offsets, prob.column_indices, scores,
+                     dense[0], shared, kernel=kernel)
+    torch.cuda.synchronize()
+    prob.values = scores[3]
+    assert torch.equal(prob.spmm(dense[0], kernel=kernel), shared[3])
+
+
+@pytest.mark.parametrize("kernel", ["wmma", "cuda"])
+def test_attention_layer_vs_dense_masked_attention(gpu, kernel):
+    # config-5 structure at a size the float64 brute force finishes quickly: band + strided column mask
+    V, heads, seq, d = 8, 3, 512, 64
+    mask = cv.band_strided_pattern(seq, V, band_half_width=64, stride=64)
+    layer = ops.SparseAttention(mask)
+    rng = np.random.default_rng(5)
+    q, k, v = (rng.standard_normal((heads, seq, d)).astype(np.float16) for _ in range(3))
+    out = layer.forward(torch.from_numpy(q).cuda(), torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda(),
+                        kernel=kernel)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    dense_mask = np.zeros((seq, seq), dtype=bool)
+    for i in range(mask.m_vec):
+        cols = mask.column_indices[mask.row_offsets[i]:mask.row_offsets[i + 1]]
+        dense_mask[i * V:(i + 1) * V, cols] = True
+    for h in range(heads):
+        s = q[h].astype(np.float64) @ k[h].astype(np.float64).T / np.sqrt(d)
+        s[~dense_mask] = -np.inf
+        p = np.exp(s - s.max(axis=1, keepdims=True))
+        p /= p.sum(axis=1, keepdims=True)
+        ref = p @ v[h].astype(np.float64)
+        # End to end against an unrounded float64 layer: the chain rounds to fp16 three times (scores,
+        # probabilities, output), so the per-element 1e-2 criterion of a single operator does not apply
+        # to near-zero outputs; the bound here is max |error| <= 1e-2 * rms(ref).  The per-operator
+        # criterion is checked step by step in test_attention_steps_match_the_oracle_chain.
+        rms = float(np.sqrt(np.mean(ref * ref)))
+        err = float(np.max(np.abs(got[h].astype(np.float64) - ref))) / rms
+        assert err <= 1e-2, "attention head %d %s: max |err| / rms = %.3e" % (h, kernel, err)
+
+
+def test_attention_steps_match_the_oracle_chain(gpu):
+    # the same layer step by step against the three oracles (exact intermediate layout)
+    V, seq, d = 8, 256, 64
+    mask = cv.band_strided_pattern(seq, V, band_half_width=32, stride=32)
+    prob = ops.DeviceProblem(mask)
+    rng = np.random.default_rng(7)
+    q, k, v = (rng.standard_normal((seq, d)).astype(np.float16) for _ in range(3))
+    scores = prob.sddmm(torch.from_numpy(q).cuda(), torch.from_numpy(k).cuda())
+    torch.cuda.synchronize()
+    s_host = scores.cpu().numpy()
+    assert_parity(s_host.reshape(-1),
+                  co.sddmm_host_ref_f32(mask.m_vec, d, V, mask.row_offsets, mask.column_indices, q, k), "scores")
+    probs = ops.sparse_softmax(mask.m_vec, V, prob.row_indices, prob.row_offsets, scores, scale=0.125)
+    torch.cuda.synchronize()
+    p_host = probs.cpu().numpy()
+    assert_parity(p_host, no.sparse_softmax_ref(mask.m_vec, V, mask.row_offsets, s_host, 0.125), "probs")
+    prob.values = probs
+    out = prob.spmm(torch.from_numpy(v).cuda())
+    torch.cuda.synchronize()
+    assert_parity(out.cpu().numpy(),
+                  co.spmm_host_ref_f32(mask.m_vec, V, d, seq, mask.row_offsets, mask.column_indices, p_host, v),
+                  "context")

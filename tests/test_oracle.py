@@ -216,3 +216,29 @@ def test_row_swizzles():
     assert np.array_equal(srt, no.sorted_row_swizzle(200, ro))        # same tie rule in both restatements
     for L in np.unique(lengths):                                      # ties keep ascending row order
         assert np.all(np.diff(srt[lengths[srt] == L]) > 0)
+
+
+# ------------------------------------------------------------------ sparse softmax (attention middle step)
+
+def test_sparse_softmax_oracle_vs_dense_masked_softmax():
+    from scipy.special import softmax
+    V = 4
+    pat = cv.random_values(cv.binomial_pattern(6, 40, 0.6, seed=3, vec_length=V), seed=4)
+    scale = 0.37
+    got = no.sparse_softmax_ref(pat.m_vec, V, pat.row_offsets, pat.values, scale)
+    dense = np.full((pat.m, pat.n), -np.inf)
+    for i in range(pat.m_vec):
+        for j in range(pat.row_offsets[i], pat.row_offsets[i + 1]):
+            dense[i * V:(i + 1) * V, pat.column_indices[j]] = pat.values[j].astype(np.float64) * scale
+    full = softmax(dense, axis=1)
+    for i in range(pat.m_vec):
+        for j in range(pat.row_offsets[i], pat.row_offsets[i + 1]):
+            np.testing.assert_allclose(got[j], full[i * V:(i + 1) * V, pat.column_indices[j]], rtol=1e-12)
+    # every scalar row sums to one; uniform inputs give 1 / row length
+    for i in range(pat.m_vec):
+        blk = got[pat.row_offsets[i]:pat.row_offsets[i + 1]]
+        if blk.size:
+            np.testing.assert_allclose(blk.sum(axis=0), 1.0, rtol=1e-12)
+    ones = no.sparse_softmax_ref(pat.m_vec, V, pat.row_offsets, np.ones_like(pat.values), 5.0)
+    L = np.repeat(pat.row_lengths(), pat.row_lengths())
+    np.testing.assert_allclose(ones, (1.0 / L)[:, None] * np.ones((1, V)), rtol=1e-12)

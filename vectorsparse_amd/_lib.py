@@ -7,6 +7,7 @@ LIB_PATH = os.path.join(_HERE, "libvsparse.so")
 
 _vp = ctypes.c_void_p
 _int = ctypes.c_int
+_ll = ctypes.c_longlong
 
 # name -> argtypes, exactly the declarations of include/vsparse.h
 SIGNATURES = {
@@ -20,6 +21,11 @@ SIGNATURES = {
     "vs_wmma_sddmm_f16_f32out": ([_int] * 4 + [_vp] * 6 + [_int, _vp, _int], _int),
     "vs_cuda_sddmm_f16": ([_int] * 4 + [_vp] * 6 + [_int, _vp], _int),
     "vs_cuda_sddmm_f16_f32out": ([_int] * 4 + [_vp] * 6 + [_int, _vp], _int),
+    "vs_wmma_spmm_f16_batched": ([_int] * 5 + [_vp] * 3 + [_vp, _ll, _vp, _ll, _vp, _ll, _vp], _int),
+    "vs_cuda_spmm_f16_batched": ([_int] * 5 + [_vp] * 3 + [_vp, _ll, _vp, _ll, _vp, _ll, _vp], _int),
+    "vs_wmma_sddmm_f16_batched": ([_int] * 5 + [_vp] * 3 + [_vp, _ll, _vp, _ll, _vp, _ll, _int, _vp, _int], _int),
+    "vs_cuda_sddmm_f16_batched": ([_int] * 5 + [_vp] * 3 + [_vp, _ll, _vp, _ll, _vp, _ll, _int, _vp], _int),
+    "vs_sparse_softmax_f16": ([_int] * 3 + [_vp] * 2 + [_vp, _ll, _vp, _ll, ctypes.c_float, _vp], _int),
     "vs_identity_row_swizzle": ([_int, _vp], None),
     "vs_sorted_row_swizzle": ([_int, _vp, _vp], None),
     "vs_set_option": ([ctypes.c_char_p, _int], _int),

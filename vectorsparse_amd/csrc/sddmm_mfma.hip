@@ -33,8 +33,12 @@ template <int V, int KS, typename OutT>
 __global__ void __launch_bounds__(256)
 sddmm_mfma_kernel(int m_vec, int K, int slots, const int *__restrict__ row_indices,
                   const int *__restrict__ row_offsets, const int *__restrict__ col_indices,
-                  const half_t *__restrict__ lhs, const half_t *__restrict__ rhs, OutT *__restrict__ out)
+                  const half_t *__restrict__ lhs, const half_t *__restrict__ rhs, OutT *__restrict__ out,
+                  long long stride_lhs, long long stride_rhs, long long stride_out)
 {
+    lhs += blockIdx.y * stride_lhs;  // batch: shared mask, per-problem operands
+    rhs += blockIdx.y * stride_rhs;
+    out += blockIdx.y * stride_out;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const long long wg = (long long)blockIdx.x * (blockDim.x >> 6) + wave;
@@ -102,26 +106,29 @@ sddmm_mfma_kernel(int m_vec, int K, int slots, const int *__restrict__ row_indic
 
 template <int V, int KS, typename OutT>
 static int launch_one(int m_vec, int k, int slots, const int *row_indices, const int *row_offsets,
-                      const int *col_indices, const half_t *lhs, const half_t *rhs, OutT *out, hipStream_t stream)
+                      const int *col_indices, const half_t *lhs, const half_t *rhs, OutT *out, hipStream_t stream,
+                      const Batch &batch)
 {
     constexpr int kWavesPerBlock = 4;
     const long long waves = (long long)m_vec * slots;
     const long long blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
-    hipLaunchKernelGGL((sddmm_mfma_kernel<V, KS, OutT>), dim3((unsigned)blocks), dim3(64 * kWavesPerBlock), 0, stream,
-                       m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out);
+    hipLaunchKernelGGL((sddmm_mfma_kernel<V, KS, OutT>), dim3((unsigned)blocks, (unsigned)batch.count), dim3(64 * kWavesPerBlock), 0, stream,
+                       m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out,
+                       batch.stride_a, batch.stride_b, batch.stride_out);
     return (int)hipGetLastError();
 }
 
 template <int V, typename OutT>
 static int launch_ks(int m_vec, int k, int slots, const int *row_indices, const int *row_offsets,
-                     const int *col_indices, const half_t *lhs, const half_t *rhs, OutT *out, hipStream_t stream)
+                     const int *col_indices, const half_t *lhs, const half_t *rhs, OutT *out, hipStream_t stream,
+                      const Batch &batch)
 {
-    if (k <= 32) return launch_one<V, 1, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream);
-    if (k <= 64) return launch_one<V, 2, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream);
-    if (k <= 128) return launch_one<V, 4, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream);
-    if (k <= 256) return launch_one<V, 8, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream);
-    return launch_one<V, 0, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream);
+    if (k <= 32) return launch_one<V, 1, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    if (k <= 64) return launch_one<V, 2, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    if (k <= 128) return launch_one<V, 4, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    if (k <= 256) return launch_one<V, 8, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    return launch_one<V, 0, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
 }
 
 // Workgroups per vector row: enough waves to fill the chip, at most one per 16-vector group of an
@@ -140,24 +147,25 @@ int sddmm_auto_slots(int m_vec, int nonzeros_vec, int group)
 template <typename OutT>
 int launch_sddmm_mfma(int m_vec, int k, int n, int nonzeros_vec, const int *row_indices,
                       const int *row_offsets, const int *col_indices, const half_t *lhs,
-                      const half_t *rhs, OutT *out, int vec_length, hipStream_t stream)
+                      const half_t *rhs, OutT *out, int vec_length, hipStream_t stream, const Batch &batch)
 {
     (void)n;
-    if (m_vec == 0 || nonzeros_vec == 0) return hipSuccess;
+    if (m_vec == 0 || nonzeros_vec == 0 || batch.count == 0) return hipSuccess;
+    if (batch.count > 65535) return hipErrorNotSupported;
     if (k <= 0 || k % 8 != 0) return hipErrorNotSupported;
-    const int slots = sddmm_auto_slots(m_vec, nonzeros_vec, 16);
+    const int slots = sddmm_auto_slots(m_vec * batch.count, nonzeros_vec * batch.count, 16);
     switch (vec_length) {
-    case 1: return launch_ks<1, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream);
-    case 2: return launch_ks<2, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream);
-    case 4: return launch_ks<4, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream);
-    case 8: return launch_ks<8, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream);
+    case 1: return launch_ks<1, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    case 2: return launch_ks<2, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    case 4: return launch_ks<4, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    case 8: return launch_ks<8, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
     default: return hipErrorInvalidValue;
     }
 }
 
 template int launch_sddmm_mfma<half_t>(int, int, int, int, const int *, const int *, const int *, const half_t *,
-                                       const half_t *, half_t *, int, hipStream_t);
+                                       const half_t *, half_t *, int, hipStream_t, const Batch &);
 template int launch_sddmm_mfma<float>(int, int, int, int, const int *, const int *, const int *, const half_t *,
-                                      const half_t *, float *, int, hipStream_t);
+                                      const half_t *, float *, int, hipStream_t, const Batch &);
 
 }  // namespace vs

@@ -15,29 +15,6 @@
 
 namespace vs {
 
-// Value held by the lane's partner in the opposite half of an aligned block of 2*STRIDE lanes.
-template <int STRIDE>
-__device__ __forceinline__ float partner(float x)
-{
-    const int xi = __builtin_bit_cast(int, x);
-    int r;
-    if constexpr (STRIDE == 1) {
-        r = __builtin_amdgcn_update_dpp(0, xi, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
-    } else if constexpr (STRIDE == 2) {
-        r = __builtin_amdgcn_update_dpp(0, xi, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
-    } else if constexpr (STRIDE == 4) {
-        r = __builtin_amdgcn_update_dpp(0, xi, 0x141, 0xF, 0xF, true);  // row_half_mirror: i <-> 7 - i
-    } else if constexpr (STRIDE == 8) {
-        r = __builtin_amdgcn_update_dpp(0, xi, 0x140, 0xF, 0xF, true);  // row_mirror: i <-> 15 - i
-    } else if constexpr (STRIDE == 16) {
-        r = __builtin_amdgcn_ds_swizzle(xi, 0x401F);                    // bit mode, xor 16
-    } else {
-        const int lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-        r = __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, xi);
-    }
-    return __builtin_bit_cast(float, r);
-}
-
 // One butterfly stage over `vals[0..NV)`.  Returns through vals[0..max(NV/2,1)).
 template <int STRIDE, int NV>
 __device__ __forceinline__ void reduce_stage(float *vals, int cl)
@@ -100,8 +77,12 @@ template <int V, int LK, int VEC, bool SINGLE, typename OutT>
 __global__ void __launch_bounds__(256)
 sddmm_valu_kernel(int m_vec, int K, int slots, const int *__restrict__ row_indices,
                   const int *__restrict__ row_offsets, const int *__restrict__ col_indices,
-                  const half_t *__restrict__ lhs, const half_t *__restrict__ rhs, OutT *__restrict__ out)
+                  const half_t *__restrict__ lhs, const half_t *__restrict__ rhs, OutT *__restrict__ out,
+                  long long stride_lhs, long long stride_rhs, long long stride_out)
 {
+    lhs += blockIdx.y * stride_lhs;  // batch: shared mask, per-problem operands
+    rhs += blockIdx.y * stride_rhs;
+    out += blockIdx.y * stride_out;
     constexpr int G = 64 / LK;
     constexpr int CHUNK = LK * VEC;
     const int lane = threadIdx.x & 63;
@@ -171,25 +152,28 @@ sddmm_valu_kernel(int m_vec, int K, int slots, const int *__restrict__ row_indic
 
 template <int V, int LK, int VEC, bool SINGLE, typename OutT>
 static int launch_one(int m_vec, int k, int nonzeros_vec, const int *row_indices, const int *row_offsets,
-                      const int *col_indices, const half_t *lhs, const half_t *rhs, OutT *out, hipStream_t stream)
+                      const int *col_indices, const half_t *lhs, const half_t *rhs, OutT *out, hipStream_t stream,
+                      const Batch &batch)
 {
     constexpr int kWavesPerBlock = 4;
-    const int slots = sddmm_auto_slots(m_vec, nonzeros_vec, 64 / LK);
+    const int slots = sddmm_auto_slots(m_vec * batch.count, nonzeros_vec * batch.count, 64 / LK);
     const long long waves = (long long)m_vec * slots;
     const long long blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
-    hipLaunchKernelGGL((sddmm_valu_kernel<V, LK, VEC, SINGLE, OutT>), dim3((unsigned)blocks),
+    hipLaunchKernelGGL((sddmm_valu_kernel<V, LK, VEC, SINGLE, OutT>), dim3((unsigned)blocks, (unsigned)batch.count),
                        dim3(64 * kWavesPerBlock), 0, stream, m_vec, k, slots, row_indices, row_offsets,
-                       col_indices, lhs, rhs, out);
+                       col_indices, lhs, rhs, out,
+                       batch.stride_a, batch.stride_b, batch.stride_out);
     return (int)hipGetLastError();
 }
 
 template <int V, typename OutT>
 static int launch_shape(int m_vec, int k, int nonzeros_vec, const int *row_indices, const int *row_offsets,
-                        const int *col_indices, const half_t *lhs, const half_t *rhs, OutT *out, hipStream_t stream)
+                        const int *col_indices, const half_t *lhs, const half_t *rhs, OutT *out, hipStream_t stream,
+                      const Batch &batch)
 {
 #define VS_GO(LK, VEC, SINGLE) \
-    return launch_one<V, LK, VEC, SINGLE, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream)
+    return launch_one<V, LK, VEC, SINGLE, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch)
     if (k % 8 == 0) {
         if (k <= 32) VS_GO(4, 8, true);
         if (k <= 64) VS_GO(8, 8, true);
@@ -206,23 +190,24 @@ static int launch_shape(int m_vec, int k, int nonzeros_vec, const int *row_indic
 template <typename OutT>
 int launch_sddmm_valu(int m_vec, int k, int n, int nonzeros_vec, const int *row_indices,
                       const int *row_offsets, const int *col_indices, const half_t *lhs,
-                      const half_t *rhs, OutT *out, int vec_length, hipStream_t stream)
+                      const half_t *rhs, OutT *out, int vec_length, hipStream_t stream, const Batch &batch)
 {
     (void)n;
-    if (m_vec == 0 || nonzeros_vec == 0) return hipSuccess;
+    if (m_vec == 0 || nonzeros_vec == 0 || batch.count == 0) return hipSuccess;
+    if (batch.count > 65535) return hipErrorNotSupported;
     if (k <= 0) return hipErrorNotSupported;
     switch (vec_length) {
-    case 1: return launch_shape<1, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream);
-    case 2: return launch_shape<2, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream);
-    case 4: return launch_shape<4, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream);
-    case 8: return launch_shape<8, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream);
+    case 1: return launch_shape<1, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    case 2: return launch_shape<2, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    case 4: return launch_shape<4, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    case 8: return launch_shape<8, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
     default: return hipErrorInvalidValue;
     }
 }
 
 template int launch_sddmm_valu<half_t>(int, int, int, int, const int *, const int *, const int *, const half_t *,
-                                       const half_t *, half_t *, int, hipStream_t);
+                                       const half_t *, half_t *, int, hipStream_t, const Batch &);
 template int launch_sddmm_valu<float>(int, int, int, int, const int *, const int *, const int *, const half_t *,
-                                      const half_t *, float *, int, hipStream_t);
+                                      const half_t *, float *, int, hipStream_t, const Batch &);
 
 }  // namespace vs

@@ -1,20 +1,21 @@
 // SpMM on fp16 MFMA for column-vector CSR (replaces src/wmma_spmm.cu of the reference).
 //
 // Work item = (vector row, tile of TN = 16*CPL dense columns), one workgroup of W waves.
-// The waves of a workgroup split the row's nonzero vectors in interleaved steps of 16 and
+// The waves of a workgroup split the row's nonzero vectors in interleaved steps of 32 and
 // their fp32 partial tiles are summed through LDS in a fixed order, so the result does not
-// depend on the launch shape's timing and no cross-workgroup reduction is needed for the
-// fp16 output.
+// depend on timing and no cross-workgroup reduction is needed for the fp16 output.
 //
-// One step (16 nonzero vectors x TN columns) in a wave, lane = (cs = lane % 16, g = lane / 16):
-//   * the lane loads CPL consecutive halves of four gathered rhs rows j = base + 4g + e,
-//     e = 0..3, at columns tile*TN + cs*CPL.. : for each e the 16 lanes of a group read one
-//     contiguous 2*TN-byte segment (128-bit loads for CPL = 8);
-//   * v_mfma_f32_16x16x16_f16 wants, per lane, 4 consecutive k for ONE column, so the
-//     CPL x 4 block a lane holds is transposed in registers with v_perm_b32 (no LDS round
-//     trip for the dense operand);
+// One step (32 nonzero vectors x TN columns) in a wave, lane = (cs = lane % 16, g = lane / 16):
+//   * lanes 0..31 fetch one column index and one V-vector each (coalesced) and park them in a
+//     wave-private LDS slot, the vectors transposed to [v][nonzero]; no workgroup barrier;
+//   * every lane then issues eight loads of CPL consecutive halves, one per gathered rhs row
+//     j = base + 8g + e, e = 0..7, at columns tile*TN + cs*CPL.. : for each e the 16 lanes of a
+//     group read one contiguous 2*TN-byte segment (128-bit loads for CPL = 8), 8 rows in flight;
+//   * v_mfma_f32_16x16x32_f16 wants, per lane, 8 consecutive k for ONE column, so the CPL x 8
+//     block a lane holds is transposed in registers with v_perm_b32 (the dense operand never
+//     goes through LDS);
 //   * MFMA number c (c < CPL) computes D[v][cs] += sum_k a[v][j(k)] * B[col_j(k)][tile*TN + cs*CPL + c]
-//     with the sparse vectors as the 16 x 16 A operand (rows v >= V are zero).
+//     with the sparse vectors as the 16 x 32 A operand (rows v >= V are zero).
 //   The accumulator of lane (cs, g), register e, MFMA c is out[4g + e][tile*TN + cs*CPL + c], i.e.
 //   CPL consecutive outputs per (lane, e): one vector store each.
 #include "vs_common.hpp"
@@ -36,15 +37,56 @@ struct RowChunk<4> {
     __device__ __forceinline__ uint32_t dword(int i) const { return d[i]; }
 };
 
+// The V halves of one nonzero vector, fetched with one load.
+template <int V>
+__device__ __forceinline__ void load_vector(half_t (&dst)[V], const half_t *p)
+{
+    if constexpr (V == 8) {
+        const half8_t t = *reinterpret_cast<const half8_t *>(p);
+#pragma unroll
+        for (int v = 0; v < 8; ++v) dst[v] = t[v];
+    } else if constexpr (V == 4) {
+        const half4_t t = *reinterpret_cast<const half4_t *>(p);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) dst[v] = t[v];
+    } else if constexpr (V == 2) {
+        const half2_t t = *reinterpret_cast<const half2_t *>(p);
+        dst[0] = t[0];
+        dst[1] = t[1];
+    } else {
+        dst[0] = p[0];
+    }
+}
+
+__device__ __forceinline__ void wave_lds_fence()
+{
+    // LDS operations of one wave execute in order; this only stops the compiler from moving
+    // LDS accesses of different lanes' data across the hand-off point.
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+constexpr int kStep = 32;  // nonzero vectors per MFMA step
+
+template <int V>
+constexpr int stage_bytes()
+{
+    return kStep * (int)sizeof(int) + V * kStep * (int)sizeof(half_t);  // indices + transposed vectors
+}
+
 template <int V, int CPL, typename OutT>
 __global__ void __launch_bounds__(1024)
 spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
                  const int *__restrict__ row_offsets, const int *__restrict__ column_indices,
                  const half_t *__restrict__ values, const half_t *__restrict__ rhs,
-                 OutT *__restrict__ out)
+                 OutT *__restrict__ out, long long stride_values, long long stride_rhs, long long stride_out)
 {
-    extern __shared__ float partial[];  // [W][V][TN]
+    values += blockIdx.y * stride_values;  // batch: shared pattern, per-problem operands
+    rhs += blockIdx.y * stride_rhs;
+    out += blockIdx.y * stride_out;
+    extern __shared__ __align__(16) unsigned char smem[];  // [W] staging slots, then [W][V][TN] partials
     constexpr int TN = 16 * CPL;
+    constexpr int kStage = stage_bytes<V>();
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int n_waves = blockDim.x >> 6;
@@ -59,36 +101,52 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
     const bool col_ok = col0 < n_cols;  // n_cols % CPL == 0: a lane's chunk is all in or all out
     const half_t *rhs_col = rhs + (col_ok ? col0 : 0);
 
+    int *idx_s = reinterpret_cast<int *>(smem + (size_t)wave * kStage);
+    half_t *vec_s = reinterpret_cast<half_t *>(idx_s + kStep);  // [V][kStep]
+    float *partial = reinterpret_cast<float *>(smem + (size_t)n_waves * kStage);
+
     float4_t acc[CPL];
 #pragma unroll
     for (int c = 0; c < CPL; ++c) acc[c] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    for (int base = beg + 16 * wave; base < end; base += 16 * n_waves) {
-        RowChunk<CPL> chunk[4];
-        half4_t a;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int j = base + 4 * g + e;
+    for (int base = beg + kStep * wave; base < end; base += kStep * n_waves) {
+        if (lane < kStep) {
+            const int j = base + lane;
             const bool valid = j < end;
-            // Slots past the row's end repeat its last vector with a zero value: the gather
-            // stays in bounds and contributes nothing.
+            // Slots past the row's end repeat its last vector with a zero value: the gather stays
+            // in bounds and contributes nothing.
             const int jc = valid ? j : end - 1;
-            const int col = column_indices[jc];
-            half_t av = (half_t)0.f;
-            if (valid && cs < V) av = values[(size_t)jc * V + cs];
-            a[e] = av;
+            idx_s[lane] = column_indices[jc];
+            half_t av[V];
+            load_vector<V>(av, values + (size_t)jc * V);
+#pragma unroll
+            for (int v = 0; v < V; ++v) vec_s[v * kStep + lane] = valid ? av[v] : (half_t)0.f;
+        }
+        wave_lds_fence();
+        const int4_t i_lo = *reinterpret_cast<const int4_t *>(idx_s + 8 * g);
+        const int4_t i_hi = *reinterpret_cast<const int4_t *>(idx_s + 8 * g + 4);
+        half8_t a = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (cs < V) a = *reinterpret_cast<const half8_t *>(vec_s + cs * kStep + 8 * g);
+        wave_lds_fence();
+
+        RowChunk<CPL> chunk[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int col = e < 4 ? i_lo[e] : i_hi[e - 4];
             chunk[e].load(rhs_col + (size_t)col * n_cols);
         }
 #pragma unroll
         for (int p = 0; p < CPL / 2; ++p) {
-            const uint32_t lo01 = pack_lo(chunk[0].dword(p), chunk[1].dword(p));
-            const uint32_t lo23 = pack_lo(chunk[2].dword(p), chunk[3].dword(p));
-            const uint32_t hi01 = pack_hi(chunk[0].dword(p), chunk[1].dword(p));
-            const uint32_t hi23 = pack_hi(chunk[2].dword(p), chunk[3].dword(p));
-            const half4_t b_even = bit_cast_u32x2<half4_t>(lo01, lo23);
-            const half4_t b_odd = bit_cast_u32x2<half4_t>(hi01, hi23);
-            acc[2 * p] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, b_even, acc[2 * p], 0, 0, 0);
-            acc[2 * p + 1] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, b_odd, acc[2 * p + 1], 0, 0, 0);
+            uint4_t even, odd;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                even[q] = pack_lo(chunk[2 * q].dword(p), chunk[2 * q + 1].dword(p));
+                odd[q] = pack_hi(chunk[2 * q].dword(p), chunk[2 * q + 1].dword(p));
+            }
+            const half8_t b_even = __builtin_bit_cast(half8_t, even);
+            const half8_t b_odd = __builtin_bit_cast(half8_t, odd);
+            acc[2 * p] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b_even, acc[2 * p], 0, 0, 0);
+            acc[2 * p + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b_odd, acc[2 * p + 1], 0, 0, 0);
         }
     }
 
@@ -154,29 +212,34 @@ static int next_pow2(int x)
 template <int V, int CPL, typename OutT>
 static int launch_one(int m_vec, int k, int n, int waves, const int *row_indices, const int *row_offsets,
                       const int *column_indices, const half_t *values, const half_t *rhs, OutT *out,
-                      hipStream_t stream)
+                      hipStream_t stream, const Batch &batch)
 {
     (void)n;
     constexpr int TN = 16 * CPL;
     const int n_tiles = ceil_div(k, TN);
     const long long blocks = (long long)m_vec * n_tiles;
     if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
-    const size_t lds = waves > 1 ? (size_t)waves * V * TN * sizeof(float) : 0;
-    hipLaunchKernelGGL((spmm_mfma_kernel<V, CPL, OutT>), dim3((unsigned)blocks), dim3(64 * waves), lds, stream,
-                       k, n_tiles, row_indices, row_offsets, column_indices, values, rhs, out);
+    const size_t lds = (size_t)waves * stage_bytes<V>() + (waves > 1 ? (size_t)waves * V * TN * sizeof(float) : 0);
+    auto kernel = spmm_mfma_kernel<V, CPL, OutT>;
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+    if (attr != hipSuccess) return (int)attr;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)batch.count), dim3(64 * waves), lds, stream,
+                       k, n_tiles, row_indices, row_offsets, column_indices, values, rhs, out,
+                       batch.stride_a, batch.stride_b, batch.stride_out);
     return (int)hipGetLastError();
 }
 
 template <int CPL, typename OutT>
 static int launch_v(int vec_length, int m_vec, int k, int n, int waves, const int *row_indices,
                     const int *row_offsets, const int *column_indices, const half_t *values,
-                    const half_t *rhs, OutT *out, hipStream_t stream)
+                    const half_t *rhs, OutT *out, hipStream_t stream, const Batch &batch)
 {
     switch (vec_length) {
-    case 1: return launch_one<1, CPL, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
-    case 2: return launch_one<2, CPL, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
-    case 4: return launch_one<4, CPL, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
-    case 8: return launch_one<8, CPL, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
+    case 1: return launch_one<1, CPL, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
+    case 2: return launch_one<2, CPL, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
+    case 4: return launch_one<4, CPL, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
+    case 8: return launch_one<8, CPL, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
     default: return hipErrorInvalidValue;
     }
 }
@@ -184,35 +247,35 @@ static int launch_v(int vec_length, int m_vec, int k, int n, int waves, const in
 template <typename OutT>
 int launch_spmm_mfma(int m_vec, int vec_length, int k, int n, const int *row_indices,
                      const int *row_offsets, const int *column_indices, const half_t *values,
-                     const half_t *rhs, OutT *out, hipStream_t stream)
+                     const half_t *rhs, OutT *out, hipStream_t stream, const Batch &batch)
 {
-    if (m_vec == 0 || k == 0) return hipSuccess;
-    if (k % 4 != 0) return hipErrorNotSupported;
+    if (m_vec == 0 || k == 0 || batch.count == 0) return hipSuccess;
+    if (k % 4 != 0 || batch.count > 65535) return hipErrorNotSupported;
     constexpr int kTargetBlocks = 256;   // one workgroup per CU at least
     constexpr int kTargetWaves = 4096;
     int cpl = options().spmm_cols_per_lane;
     if (cpl != 4 && cpl != 8) {
-        const long long blocks128 = (long long)m_vec * ceil_div(k, 128);
+        const long long blocks128 = (long long)m_vec * ceil_div(k, 128) * batch.count;
         cpl = (k % 8 == 0 && blocks128 >= kTargetBlocks) ? 8 : 4;
     }
     if (cpl == 8 && k % 8 != 0) cpl = 4;
-    const long long blocks = (long long)m_vec * ceil_div(k, 16 * cpl);
+    const long long blocks = (long long)m_vec * ceil_div(k, 16 * cpl) * batch.count;
     int waves = options().spmm_waves;
     if (waves <= 0) {
         waves = next_pow2((int)((kTargetWaves + blocks - 1) / blocks));
-        const int max_useful = next_pow2(ceil_div(n > 0 ? n : 1, 16));  // a row holds at most n vectors
+        const int max_useful = next_pow2(ceil_div(n > 0 ? n : 1, kStep));  // a row holds at most n vectors
         if (waves > max_useful) waves = max_useful;
     }
     if (waves < 1) waves = 1;
     if (waves > 16) waves = 16;
     if (cpl == 8)
-        return launch_v<8, OutT>(vec_length, m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
-    return launch_v<4, OutT>(vec_length, m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
+        return launch_v<8, OutT>(vec_length, m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
+    return launch_v<4, OutT>(vec_length, m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
 }
 
 template int launch_spmm_mfma<half_t>(int, int, int, int, const int *, const int *, const int *, const half_t *,
-                                      const half_t *, half_t *, hipStream_t);
+                                      const half_t *, half_t *, hipStream_t, const Batch &);
 template int launch_spmm_mfma<float>(int, int, int, int, const int *, const int *, const int *, const half_t *,
-                                     const half_t *, float *, hipStream_t);
+                                     const half_t *, float *, hipStream_t, const Batch &);
 
 }  // namespace vs

@@ -18,8 +18,11 @@ __global__ void __launch_bounds__(1024)
 spmm_valu_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
                  const int *__restrict__ row_offsets, const int *__restrict__ column_indices,
                  const half_t *__restrict__ values, const half_t *__restrict__ rhs,
-                 OutT *__restrict__ out)
+                 OutT *__restrict__ out, long long stride_values, long long stride_rhs, long long stride_out)
 {
+    values += blockIdx.y * stride_values;  // batch: shared pattern, per-problem operands
+    rhs += blockIdx.y * stride_rhs;
+    out += blockIdx.y * stride_out;
     extern __shared__ float partial[];  // [W*G][V][TN]
     constexpr int G = 64 / LR;
     constexpr int TN = 8 * LR;
@@ -110,7 +113,7 @@ spmm_valu_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
 template <int V, int LR, typename OutT>
 static int launch_one(int m_vec, int k, int waves, const int *row_indices, const int *row_offsets,
                       const int *column_indices, const half_t *values, const half_t *rhs, OutT *out,
-                      hipStream_t stream)
+                      hipStream_t stream, const Batch &batch)
 {
     constexpr int G = 64 / LR;
     constexpr int TN = 8 * LR;
@@ -122,49 +125,50 @@ static int launch_one(int m_vec, int k, int waves, const int *row_indices, const
     if (waves > max_waves) waves = max_waves;
     if (waves < 1) waves = 1;
     const size_t lds = (waves * G > 1) ? (size_t)waves * G * V * TN * sizeof(float) : 0;
-    hipLaunchKernelGGL((spmm_valu_kernel<V, LR, OutT>), dim3((unsigned)blocks), dim3(64 * waves), lds, stream,
-                       k, n_tiles, row_indices, row_offsets, column_indices, values, rhs, out);
+    hipLaunchKernelGGL((spmm_valu_kernel<V, LR, OutT>), dim3((unsigned)blocks, (unsigned)batch.count),
+                       dim3(64 * waves), lds, stream, k, n_tiles, row_indices, row_offsets, column_indices, values,
+                       rhs, out, batch.stride_a, batch.stride_b, batch.stride_out);
     return (int)hipGetLastError();
 }
 
 template <int V, typename OutT>
 static int launch_lr(int m_vec, int k, int waves, const int *row_indices, const int *row_offsets,
                      const int *column_indices, const half_t *values, const half_t *rhs, OutT *out,
-                     hipStream_t stream)
+                     hipStream_t stream, const Batch &batch)
 {
-    if (k <= 64) return launch_one<V, 8, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
-    if (k <= 128) return launch_one<V, 16, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
-    if (k <= 256) return launch_one<V, 32, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
-    return launch_one<V, 64, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
+    if (k <= 64) return launch_one<V, 8, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
+    if (k <= 128) return launch_one<V, 16, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
+    if (k <= 256) return launch_one<V, 32, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
+    return launch_one<V, 64, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
 }
 
 template <typename OutT>
 int launch_spmm_valu(int m_vec, int vec_length, int k, int n, const int *row_indices,
                      const int *row_offsets, const int *column_indices, const half_t *values,
-                     const half_t *rhs, OutT *out, hipStream_t stream)
+                     const half_t *rhs, OutT *out, hipStream_t stream, const Batch &batch)
 {
     (void)n;
-    if (m_vec == 0 || k == 0) return hipSuccess;
-    if (k % 8 != 0) return hipErrorNotSupported;
+    if (m_vec == 0 || k == 0 || batch.count == 0) return hipSuccess;
+    if (k % 8 != 0 || batch.count > 65535) return hipErrorNotSupported;
     int waves = options().spmm_waves;
     if (waves <= 0) {
-        const long long blocks = (long long)m_vec * ceil_div(k, 512);
+        const long long blocks = (long long)m_vec * ceil_div(k, 512) * batch.count;
         waves = 1;
         while (waves < 8 && blocks * waves < 2048) waves <<= 1;
     }
     if (waves > 16) waves = 16;
     switch (vec_length) {
-    case 1: return launch_lr<1, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
-    case 2: return launch_lr<2, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
-    case 4: return launch_lr<4, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
-    case 8: return launch_lr<8, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream);
+    case 1: return launch_lr<1, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
+    case 2: return launch_lr<2, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
+    case 4: return launch_lr<4, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
+    case 8: return launch_lr<8, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
     default: return hipErrorInvalidValue;
     }
 }
 
 template int launch_spmm_valu<half_t>(int, int, int, int, const int *, const int *, const int *, const half_t *,
-                                      const half_t *, half_t *, hipStream_t);
+                                      const half_t *, half_t *, hipStream_t, const Batch &);
 template int launch_spmm_valu<float>(int, int, int, int, const int *, const int *, const int *, const half_t *,
-                                     const half_t *, float *, hipStream_t);
+                                     const half_t *, float *, hipStream_t, const Batch &);
 
 }  // namespace vs

@@ -12,6 +12,7 @@ typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
 typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+typedef int32_t int4_t __attribute__((ext_vector_type(4)));
 // 4-byte aligned vector views: row starts inside the CSR arrays are only int-aligned.
 typedef int32_t int4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 
@@ -37,8 +38,29 @@ __device__ __forceinline__ T bit_cast_u32x2(uint32_t a, uint32_t b)
     return __builtin_bit_cast(T, u);
 }
 
-template <typename OutT>
-struct OutVec;
+// Value held by the lane's partner in the opposite half of an aligned block of 2*STRIDE lanes.
+template <int STRIDE>
+__device__ __forceinline__ float partner(float x)
+{
+    const int xi = __builtin_bit_cast(int, x);
+    int r;
+    if constexpr (STRIDE == 1) {
+        r = __builtin_amdgcn_update_dpp(0, xi, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
+    } else if constexpr (STRIDE == 2) {
+        r = __builtin_amdgcn_update_dpp(0, xi, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
+    } else if constexpr (STRIDE == 4) {
+        r = __builtin_amdgcn_update_dpp(0, xi, 0x141, 0xF, 0xF, true);  // row_half_mirror: i <-> 7 - i
+    } else if constexpr (STRIDE == 8) {
+        r = __builtin_amdgcn_update_dpp(0, xi, 0x140, 0xF, 0xF, true);  // row_mirror: i <-> 15 - i
+    } else if constexpr (STRIDE == 16) {
+        r = __builtin_amdgcn_ds_swizzle(xi, 0x401F);                    // bit mode, xor 16
+    } else {
+        const int lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+        r = __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, xi);
+    }
+    return __builtin_bit_cast(float, r);
+}
+
 
 // Store `Count` consecutive outputs converted from fp32 (Count in {1,2,4,8}).
 template <typename OutT, int Count>
@@ -110,22 +132,37 @@ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 // Waves per vector row for the SDDMM kernels; `group` = nonzero vectors a wave covers per step.
 int sddmm_auto_slots(int m_vec, int nonzeros_vec, int group);
 
+// Batched launches: problem b of `count` uses operand pointers advanced by b * stride (in elements);
+// the sparsity pattern (row_indices, row_offsets, column indices) is shared by the whole batch.
+struct Batch {
+    int count = 1;
+    long long stride_a = 0;    // SpMM: values        SDDMM: lhs_matrix
+    long long stride_b = 0;    // SpMM: rhs_matrix    SDDMM: rhs_matrix
+    long long stride_out = 0;  // SpMM: output_matrix SDDMM: output_values
+};
+
 // Launchers (one per kernel family); return a hipError_t-valued int.
 template <typename OutT>
 int launch_spmm_mfma(int m_vec, int vec_length, int k, int n, const int *row_indices,
                      const int *row_offsets, const int *column_indices, const half_t *values,
-                     const half_t *rhs, OutT *out, hipStream_t stream);
+                     const half_t *rhs, OutT *out, hipStream_t stream, const Batch &batch = Batch());
 template <typename OutT>
 int launch_spmm_valu(int m_vec, int vec_length, int k, int n, const int *row_indices,
                      const int *row_offsets, const int *column_indices, const half_t *values,
-                     const half_t *rhs, OutT *out, hipStream_t stream);
+                     const half_t *rhs, OutT *out, hipStream_t stream, const Batch &batch = Batch());
 template <typename OutT>
 int launch_sddmm_mfma(int m_vec, int k, int n, int nonzeros_vec, const int *row_indices,
                       const int *row_offsets, const int *col_indices, const half_t *lhs,
-                      const half_t *rhs, OutT *out, int vec_length, hipStream_t stream);
+                      const half_t *rhs, OutT *out, int vec_length, hipStream_t stream,
+                      const Batch &batch = Batch());
 template <typename OutT>
 int launch_sddmm_valu(int m_vec, int k, int n, int nonzeros_vec, const int *row_indices,
                       const int *row_offsets, const int *col_indices, const half_t *lhs,
-                      const half_t *rhs, OutT *out, int vec_length, hipStream_t stream);
+                      const half_t *rhs, OutT *out, int vec_length, hipStream_t stream,
+                      const Batch &batch = Batch());
+
+int launch_sparse_softmax(int m_vec, int vec_length, const int *row_indices, const int *row_offsets,
+                          const half_t *values_in, half_t *values_out, float scale, hipStream_t stream,
+                          const Batch &batch = Batch());
 
 }  // namespace vs

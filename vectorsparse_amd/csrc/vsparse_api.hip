@@ -171,6 +171,109 @@ int vs_cuda_sddmm_f16_f32out(int m_vec, int k, int n, int nonzeros_vec, const in
                                         static_cast<hipStream_t>(stream));
 }
 
+static vs::Batch make_batch(int batch, long long a, long long b, long long out)
+{
+    vs::Batch x;
+    x.count = batch;
+    x.stride_a = a;
+    x.stride_b = b;
+    x.stride_out = out;
+    return x;
+}
+
+// Strides keep every problem's operand as aligned as the first one.
+static bool stride_ok(long long stride, long long multiple) { return stride >= 0 && stride % multiple == 0; }
+
+int vs_wmma_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n, const int *row_indices,
+                             const int *row_offsets, const int *column_indices, const void *values,
+                             long long stride_values, const void *rhs_matrix, long long stride_rhs,
+                             void *output_matrix, long long stride_output, void *stream)
+{
+    if (batch < 0) return VS_ERROR_INVALID_VALUE;
+    int st = check_spmm(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices, values, rhs_matrix,
+                        output_matrix, sizeof(half_t));
+    if (st != VS_SUCCESS) return st;
+    if (!stride_ok(stride_values, vec_length) || !stride_ok(stride_rhs, 8) || !stride_ok(stride_output, 8))
+        return VS_ERROR_INVALID_VALUE;
+    return vs::launch_spmm_mfma<half_t>(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices,
+                                        static_cast<const half_t *>(values), static_cast<const half_t *>(rhs_matrix),
+                                        static_cast<half_t *>(output_matrix), static_cast<hipStream_t>(stream),
+                                        make_batch(batch, stride_values, stride_rhs, stride_output));
+}
+
+int vs_cuda_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n, const int *row_indices,
+                             const int *row_offsets, const int *column_indices, const void *values,
+                             long long stride_values, const void *rhs_matrix, long long stride_rhs,
+                             void *output_matrix, long long stride_output, void *stream)
+{
+    if (batch < 0) return VS_ERROR_INVALID_VALUE;
+    int st = check_spmm(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices, values, rhs_matrix,
+                        output_matrix, sizeof(half_t));
+    if (st != VS_SUCCESS) return st;
+    if (!stride_ok(stride_values, vec_length) || !stride_ok(stride_rhs, 8) || !stride_ok(stride_output, 8))
+        return VS_ERROR_INVALID_VALUE;
+    return vs::launch_spmm_valu<half_t>(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices,
+                                        static_cast<const half_t *>(values), static_cast<const half_t *>(rhs_matrix),
+                                        static_cast<half_t *>(output_matrix), static_cast<hipStream_t>(stream),
+                                        make_batch(batch, stride_values, stride_rhs, stride_output));
+}
+
+int vs_wmma_sddmm_f16_batched(int batch, int m_vec, int k, int n, int nonzeros_vec, const int *row_indices,
+                              const int *row_offsets, const int *col_indices, const void *lhs_matrix,
+                              long long stride_lhs, const void *rhs_matrix, long long stride_rhs,
+                              void *output_values, long long stride_output, int vec_length, void *stream,
+                              int algorithm)
+{
+    if (batch < 0 || algorithm < 0 || algorithm > 2) return VS_ERROR_INVALID_VALUE;
+    int st = check_sddmm(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices, lhs_matrix, rhs_matrix,
+                         output_values, vec_length, sizeof(half_t));
+    if (st != VS_SUCCESS) return st;
+    if (!stride_ok(stride_lhs, 8) || !stride_ok(stride_rhs, 8) || !stride_ok(stride_output, vec_length))
+        return VS_ERROR_INVALID_VALUE;
+    return vs::launch_sddmm_mfma<half_t>(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices,
+                                         static_cast<const half_t *>(lhs_matrix),
+                                         static_cast<const half_t *>(rhs_matrix),
+                                         static_cast<half_t *>(output_values), vec_length,
+                                         static_cast<hipStream_t>(stream),
+                                         make_batch(batch, stride_lhs, stride_rhs, stride_output));
+}
+
+int vs_cuda_sddmm_f16_batched(int batch, int m_vec, int k, int n, int nonzeros_vec, const int *row_indices,
+                              const int *row_offsets, const int *col_indices, const void *lhs_matrix,
+                              long long stride_lhs, const void *rhs_matrix, long long stride_rhs,
+                              void *output_values, long long stride_output, int vec_length, void *stream)
+{
+    if (batch < 0) return VS_ERROR_INVALID_VALUE;
+    int st = check_sddmm(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices, lhs_matrix, rhs_matrix,
+                         output_values, vec_length, sizeof(half_t));
+    if (st != VS_SUCCESS) return st;
+    const long long in_mult = (k % 8 == 0) ? 8 : 1;
+    if (!stride_ok(stride_lhs, in_mult) || !stride_ok(stride_rhs, in_mult) || !stride_ok(stride_output, vec_length))
+        return VS_ERROR_INVALID_VALUE;
+    return vs::launch_sddmm_valu<half_t>(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices,
+                                         static_cast<const half_t *>(lhs_matrix),
+                                         static_cast<const half_t *>(rhs_matrix),
+                                         static_cast<half_t *>(output_values), vec_length,
+                                         static_cast<hipStream_t>(stream),
+                                         make_batch(batch, stride_lhs, stride_rhs, stride_output));
+}
+
+int vs_sparse_softmax_f16(int batch, int m_vec, int vec_length, const int *row_indices, const int *row_offsets,
+                          const void *values_in, long long stride_in, void *values_out, long long stride_out,
+                          float scale, void *stream)
+{
+    if (batch < 0 || m_vec < 0 || !vec_ok(vec_length)) return VS_ERROR_INVALID_VALUE;
+    if (batch == 0 || m_vec == 0) return VS_SUCCESS;
+    if (!row_indices || !row_offsets) return VS_ERROR_INVALID_VALUE;
+    if (!aligned(values_in, 2 * (size_t)vec_length) || !aligned(values_out, 2 * (size_t)vec_length))
+        return VS_ERROR_INVALID_VALUE;
+    if (!stride_ok(stride_in, vec_length) || !stride_ok(stride_out, vec_length)) return VS_ERROR_INVALID_VALUE;
+    return vs::launch_sparse_softmax(m_vec, vec_length, row_indices, row_offsets,
+                                     static_cast<const half_t *>(values_in), static_cast<half_t *>(values_out),
+                                     scale, static_cast<hipStream_t>(stream),
+                                     make_batch(batch, stride_in, 0, stride_out));
+}
+
 void vs_identity_row_swizzle(int rows, int *row_indices)
 {
     if (rows <= 0 || !row_indices) return;

@@ -110,6 +110,107 @@ class sddmm:
                       lhs_matrix, rhs_matrix, output_values, vec_length, stream)
 
 
+def _stride(t, batch):
+    """Element stride between consecutive problems of a [batch, ...] tensor (0 when shared)."""
+    if batch == 1 or t.dim() < 3:
+        return 0
+    return t.stride(0)
+
+
+def spmm_batched(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices, values, rhs_matrix,
+                 output_matrix, kernel="wmma", stream=None):
+    """`batch` SpMMs sharing one pattern in one launch.
+
+    values: [batch, nnz_vec, V] (or [nnz_vec, V] shared), rhs_matrix: [batch, n, k] (or [n, k] shared),
+    output_matrix: [batch, m, k], all fp16 and contiguous in their trailing dimensions.
+    """
+    batch = output_matrix.shape[0]
+    for t, nm in ((values, "values"), (rhs_matrix, "rhs_matrix"), (output_matrix, "output_matrix")):
+        _expect_batched(t, torch.float16, nm)
+    entry = "vs_wmma_spmm_f16_batched" if kernel == "wmma" else "vs_cuda_spmm_f16_batched"
+    st = getattr(_lib.lib(), entry)(batch, m_vec, vec_length, k, n, _ptr(row_indices), _ptr(row_offsets),
+                                    _ptr(column_indices), _ptr(values), _stride(values, batch), _ptr(rhs_matrix),
+                                    _stride(rhs_matrix, batch), _ptr(output_matrix), _stride(output_matrix, batch),
+                                    _stream(stream))
+    _lib.check(st, entry)
+    return output_matrix
+
+
+def sddmm_batched(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices, lhs_matrix, rhs_matrix,
+                  output_values, vec_length, kernel="wmma", stream=None, algorithm=1):
+    """`batch` SDDMMs sharing one mask in one launch.
+
+    lhs_matrix: [batch, m, k], rhs_matrix: [batch, n, k], output_values: [batch, nnz_vec, V], fp16.
+    """
+    batch = output_values.shape[0]
+    for t, nm in ((lhs_matrix, "lhs_matrix"), (rhs_matrix, "rhs_matrix"), (output_values, "output_values")):
+        _expect_batched(t, torch.float16, nm)
+    args = [batch, m_vec, k, n, nonzeros_vec, _ptr(row_indices), _ptr(row_offsets), _ptr(col_indices),
+            _ptr(lhs_matrix), _stride(lhs_matrix, batch), _ptr(rhs_matrix), _stride(rhs_matrix, batch),
+            _ptr(output_values), _stride(output_values, batch), vec_length, _stream(stream)]
+    if kernel == "wmma":
+        entry = "vs_wmma_sddmm_f16_batched"
+        args.append(algorithm)
+    else:
+        entry = "vs_cuda_sddmm_f16_batched"
+    _lib.check(getattr(_lib.lib(), entry)(*args), entry)
+    return output_values
+
+
+def sparse_softmax(m_vec, vec_length, row_indices, row_offsets, values_in, values_out=None, scale=1.0,
+                   stream=None):
+    """Row-wise softmax(scale * x) over each scalar row's nonzeros, [nnz_vec, V] or [batch, nnz_vec, V]."""
+    if values_out is None:
+        values_out = torch.empty_like(values_in)
+    _expect_batched(values_in, torch.float16, "values_in")
+    _expect_batched(values_out, torch.float16, "values_out")
+    batch = values_in.shape[0] if values_in.dim() == 3 else 1
+    st = _lib.lib().vs_sparse_softmax_f16(batch, m_vec, vec_length, _ptr(row_indices), _ptr(row_offsets),
+                                          _ptr(values_in), _stride(values_in, batch), _ptr(values_out),
+                                          _stride(values_out, batch), float(scale), _stream(stream))
+    _lib.check(st, "vs_sparse_softmax_f16")
+    return values_out
+
+
+def _expect_batched(t, dtype, name):
+    if t.dtype != dtype:
+        raise TypeError("%s must be %s, got %s" % (name, dtype, t.dtype))
+    if not t.is_cuda:
+        raise ValueError("%s must live in device memory" % name)
+    inner = t[0] if t.dim() == 3 else t
+    if not inner.is_contiguous():
+        raise ValueError("%s must be contiguous in its trailing dimensions" % name)
+
+
+class SparseAttention:
+    """One fixed-mask sparse attention layer: SDDMM (QK^T on the mask) -> row softmax -> SpMM (P V).
+
+    The mask is a column-vector CSR pattern over [seq, seq] shared by all heads; the three steps are
+    one batched launch each, chained on one stream with no host synchronisation and no re-layout (the
+    SDDMM output layout is the SpMM value layout).
+    """
+
+    def __init__(self, mask, device="cuda", sort=True):
+        self.prob = DeviceProblem(mask, sort=sort, device=device)
+
+    def forward(self, q, k, v, scale=None, kernel="wmma", stream=None, scores=None, out=None):
+        """q, k, v: fp16 [heads, seq, d] on the device.  Returns fp16 [heads, seq, d]."""
+        p = self.prob
+        heads, seq, d = q.shape
+        if scale is None:
+            scale = 1.0 / float(d) ** 0.5
+        if scores is None:
+            scores = torch.empty((heads, p.nnz_vec, p.vec_length), dtype=torch.float16, device=q.device)
+        if out is None:
+            out = torch.empty((heads, seq, v.shape[2]), dtype=torch.float16, device=q.device)
+        sddmm_batched(p.m_vec, d, p.n, p.nnz_vec, p.row_indices, p.row_offsets, p.column_indices, q, k, scores,
+                      p.vec_length, kernel=kernel, stream=stream)
+        sparse_softmax(p.m_vec, p.vec_length, p.row_indices, p.row_offsets, scores, scores, scale, stream=stream)
+        spmm_batched(p.m_vec, p.vec_length, v.shape[2], p.n, p.row_indices, p.row_offsets, p.column_indices,
+                     scores, v, out, kernel=kernel, stream=stream)
+        return out
+
+
 def IdentityRowSwizzle(rows):
     """include/bm_test_utils.h:196-198 through the C ABI (host arrays)."""
     out = np.empty(rows, dtype=np.int32)
