@@ -73,6 +73,39 @@ def time_graph(torch, fn, steps, warmup):
     return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
 
 
+def time_cold(torch, fn, samples=20):
+    """Device time of single launches with the caches thrashed in between: a 1 GiB fill evicts the 256 MB
+    Infinity Cache and the L2s before every timed launch (the reference measures with Nsight's
+    --cache-control all, i.e. flushed caches)."""
+    thrash = torch.empty(512 * 1024 * 1024, dtype=torch.float16, device="cuda")
+    times = []
+    for i in range(samples):
+        thrash.fill_(float(i))
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn()
+        e1.record()
+        torch.cuda.synchronize()
+        times.append(e0.elapsed_time(e1))
+    del thrash
+    times.sort()
+    return times[len(times) // 2]
+
+
+def measured_traffic(path):
+    """HBM-side bytes per launch of the headline kernel, from the committed rocprofv3 --pmc summary
+    (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a copy of known size)."""
+    try:
+        with open(path) as f:
+            for ln in f:
+                if ln.startswith("traffic_bytes_per_launch"):
+                    return float(ln.split()[1])
+    except OSError:
+        pass
+    return None
+
+
 def time_eager(torch, fn, steps, warmup):
     for _ in range(warmup):
         fn()
@@ -195,7 +228,28 @@ def main():
     sddmm_flops = 2.0 * mask.nnz * 64
     sddmm_bytes = sddmm_algorithmic_bytes(mask, 64)
 
+    # ---- fixed-mask sparse attention layer (config 5: 16 heads, seq 4096, d 64, V = 8 band + strided mask)
+    heads, seq, dim = 16, 4096, 64
+    amask = cv.band_strided_pattern(seq, 8, band_half_width=128, stride=128)
+    layer = ops.SparseAttention(amask)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    q, kk_, vv = (torch.randn((heads, seq, dim), device="cuda", generator=gen).half() for _ in range(3))
+    scores = torch.empty((heads, amask.nnz_vec, 8), dtype=torch.float16, device="cuda")
+    ctx = torch.empty((heads, seq, dim), dtype=torch.float16, device="cuda")
+    attn_steps = max(5, args.steps // 10)
+    _, attn_ms = time_graph(torch, lambda: layer.forward(q, kk_, vv, scores=scores, out=ctx), attn_steps, 3)
+
+    def dense_attention():
+        s_ = torch.matmul(q, kk_.transpose(1, 2))
+        return torch.matmul(torch.softmax(s_ * 0.125, dim=-1), vv)
+
+    _, dense_attn_ms = time_graph(torch, dense_attention, 5, 2)
+    attn_flops = 2.0 * amask.nnz * heads * dim * 2
+
+    cold_ms = time_cold(torch, step)
+
     achieved = alg_bytes / (ev_ms * 1e-3) * 1e-9
+    traffic = measured_traffic(os.path.join(ROOT, "profiles", "spmm_mfma_config2_pmc.txt"))
     line = {
         "metric": "SpMM effective TFLOP/s (2*nnz*N), fp16 V=8, 90% sparse",
         "value": flops / (wall_ms * 1e-3) * 1e-12,
@@ -213,7 +267,7 @@ def main():
                                "sorted row swizzle, fp16 out / fp32 accumulate",
                    "nnz_vec": pat.nnz_vec, "launch": "HIP graph of `steps` operator calls"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "kernel": "spmm_mfma_kernel<V=8>", "algorithmic_bytes": alg_bytes,
                      "avg_launch_us": ev_ms * 1e3},
         "parity": {"max_rel_err": max_rel, "errors_gt_0.5": errors},
@@ -221,6 +275,11 @@ def main():
             "eager_ms_per_step": eager_wall_ms,
             "dense_gemm_ms": dense_ms,
             "speedup_vs_dense_gemm": dense_ms / ev_ms,
+            "cold_cache_launch_us": cold_ms * 1e3,
+            "attention_config5": {"layer_ms": attn_ms, "density": 1.0 - amask.sparsity,
+                                  "tflops": attn_flops / (attn_ms * 1e-3) * 1e-12,
+                                  "dense_masked_attention_ms": dense_attn_ms,
+                                  "speedup_vs_dense": dense_attn_ms / attn_ms},
             "sddmm_config4_k64": {"ms": sddmm_ms, "tflops": sddmm_flops / (sddmm_ms * 1e-3) * 1e-12,
                                   "hbm_gbs": sddmm_bytes / (sddmm_ms * 1e-3) * 1e-9,
                                   "hbm_frac": sddmm_bytes / (sddmm_ms * 1e-3) * 1e-9 / HBM_PEAK_GBS},

@@ -2,15 +2,18 @@
 //
 // out[j*V + v] = sum_l lhs[(i*V + v)*K + l] * rhs[col_j*K + l]   for every nonzero vector j of vector row i.
 //
-// Both operands are contiguous along the contraction index, which is exactly the per-lane layout
-// v_mfma_f32_16x16x32_f16 wants (8 consecutive k per lane), so operands go from global memory
-// straight into MFMA registers with 128-bit loads; there is no LDS stage and no barrier.
-// Lane = (c = lane % 16, g = lane / 16).  One wave step covers 16 nonzero vectors of a row:
-//   A operand: lhs row i*V + c (zero for c >= V), k slice [32*kk + 8g, +8)
-//   B operand: rhs row col_{j0 + c},               same k slice
+// Both operands are contiguous along the contraction index, which is the per-lane layout
+// v_mfma_f32_16x16x32_f16 wants (8 consecutive k per lane).  One wave step covers 16 nonzero vectors:
+//   A operand: lhs row i*V + c (zero for c >= V), k slice [32*kk + 8g, +8)        lane = (c = lane % 16,
+//   B operand: rhs row col_{j0 + c},               same k slice                           g = lane / 16)
 //   D[v][c]  : lane (c, g), register e  ->  out[(j0 + c)*V + 4g + e]   (4 consecutive outputs per lane)
-// A wave owns (vector row, slot s) and walks the row's 16-vector groups s, s + slots, ...; the lhs
-// slices of the vector row stay in registers across groups when K <= 256.
+// Loading in that layout would make the four lanes of every quad touch four different rows (four cache
+// lines for 64 bytes), which caps the gather at a quarter of the L1 rate.  So the 128-bit loads are issued
+// in the row-major lane order instead - lane n reads slice n % 4 of row n / 4, a quad reads 64 contiguous
+// bytes - and the registers are moved to the MFMA lane order with ds_bpermute (LDS crossbar only, no LDS
+// storage, no barrier).  A wave owns (vector row, slot s) and walks super-groups of GRP*16 vectors
+// s, s + slots, ... with all GRP*KS loads of a super-group in flight together; the lhs slices of the
+// vector row stay in registers across super-groups when K <= 256.
 #include "vs_common.hpp"
 
 namespace vs {
@@ -28,8 +31,26 @@ __device__ __forceinline__ void store_group(OutT *out, int j, int g, const float
     }
 }
 
-// KS > 0: K <= 32*KS, lhs slices preloaded; KS == 0: any K % 8 == 0, lhs re-read per group.
-template <int V, int KS, typename OutT>
+// Row-major lane order -> MFMA lane order: lane (c, g) takes the registers of lane 4c + g.
+__device__ __forceinline__ half8_t to_mfma_order(const uint4_t &x, int src_lane_bytes)
+{
+    uint4_t y;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) y[i] = (uint32_t)__builtin_amdgcn_ds_bpermute(src_lane_bytes, (int)x[i]);
+    return __builtin_bit_cast(half8_t, y);
+}
+
+// Slice q (8 halves at k = 32*kk + 8q) of `row`, zero past K.
+__device__ __forceinline__ uint4_t load_slice16(const half_t *row, int kk, int q, int K, bool ok)
+{
+    const int off = 32 * kk + 8 * q;
+    uint4_t x = {0u, 0u, 0u, 0u};
+    if (ok && off < K) x = *reinterpret_cast<const uint4_t *>(row + off);
+    return x;
+}
+
+// KS > 0: K <= 32*KS, lhs slices preloaded; KS == 0: any K % 8 == 0, lhs re-read per super-group.
+template <int V, int KS, int GRP, typename OutT>
 __global__ void __launch_bounds__(256)
 sddmm_mfma_kernel(int m_vec, int K, int slots, const int *__restrict__ row_indices,
                   const int *__restrict__ row_offsets, const int *__restrict__ col_indices,
@@ -39,6 +60,7 @@ sddmm_mfma_kernel(int m_vec, int K, int slots, const int *__restrict__ row_indic
     lhs += blockIdx.y * stride_lhs;  // batch: shared mask, per-problem operands
     rhs += blockIdx.y * stride_rhs;
     out += blockIdx.y * stride_out;
+    constexpr int SUPER = 16 * GRP;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const long long wg = (long long)blockIdx.x * (blockDim.x >> 6) + wave;
@@ -48,91 +70,101 @@ sddmm_mfma_kernel(int m_vec, int K, int slots, const int *__restrict__ row_indic
     const int row = row_indices[slot];
     const int beg = row_offsets[row];
     const int end = row_offsets[row + 1];
-    const int n_groups = (end - beg + 15) >> 4;
-    if (s >= n_groups) return;
-    const int c = lane & 15;
-    const int g = lane >> 4;
-    const bool a_row_ok = c < V;
-    const half_t *lhs_row = lhs + ((size_t)row * V + (a_row_ok ? c : 0)) * K;
-    const half8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    const int n_super = (end - beg + SUPER - 1) / SUPER;
+    if (s >= n_super) return;
+    const int c = lane & 15;        // MFMA order: column (nonzero vector) index
+    const int g = lane >> 4;        //             k group
+    const int r = lane >> 2;        // load order: row within the group of 16
+    const int q = lane & 3;         //             16-byte slice within a 64-byte k step
+    const int src = (4 * c + g) << 2;
+    const bool a_row_ok = r < V;
+    const half_t *lhs_row = lhs + ((size_t)row * V + (a_row_ok ? r : 0)) * K;
 
     if constexpr (KS > 0) {
         half8_t a[KS];
 #pragma unroll
-        for (int kk = 0; kk < KS; ++kk) {
-            const int off = 32 * kk + 8 * g;
-            a[kk] = zero8;
-            if (a_row_ok && off < K) a[kk] = *reinterpret_cast<const half8_t *>(lhs_row + off);
-        }
-        for (int grp = s; grp < n_groups; grp += slots) {
-            const int j = beg + 16 * grp + c;
-            const bool valid = j < end;
-            const int jc = valid ? j : end - 1;  // in-bounds gather for the padded slots; result discarded
-            const half_t *rhs_row = rhs + (size_t)col_indices[jc] * K;
-            half8_t b[KS];
+        for (int kk = 0; kk < KS; ++kk) a[kk] = to_mfma_order(load_slice16(lhs_row, kk, q, K, a_row_ok), src);
+        for (int sg = s; sg < n_super; sg += slots) {
+            const int j0 = beg + SUPER * sg;
+            uint4_t raw[GRP][KS];
 #pragma unroll
-            for (int kk = 0; kk < KS; ++kk) {
-                const int off = 32 * kk + 8 * g;
-                b[kk] = zero8;
-                if (off < K) b[kk] = *reinterpret_cast<const half8_t *>(rhs_row + off);
+            for (int u = 0; u < GRP; ++u) {
+                const int jl = j0 + 16 * u + r;
+                // slots past the row's end gather its last vector (in bounds); their results are dropped
+                const half_t *rhs_row = rhs + (size_t)col_indices[jl < end ? jl : end - 1] * K;
+#pragma unroll
+                for (int kk = 0; kk < KS; ++kk) raw[u][kk] = load_slice16(rhs_row, kk, q, K, true);
             }
-            float4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int kk = 0; kk < KS; ++kk)
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[kk], b[kk], acc, 0, 0, 0);
-            if (valid) store_group<V, OutT>(out, j, g, acc);
+            for (int u = 0; u < GRP; ++u) {
+                float4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int kk = 0; kk < KS; ++kk)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[kk], to_mfma_order(raw[u][kk], src), acc, 0, 0, 0);
+                const int j = j0 + 16 * u + c;
+                if (j < end) store_group<V, OutT>(out, j, g, acc);
+            }
         }
     } else {
         const int k_steps = (K + 31) >> 5;
-        for (int grp = s; grp < n_groups; grp += slots) {
-            const int j = beg + 16 * grp + c;
-            const bool valid = j < end;
-            const int jc = valid ? j : end - 1;
-            const half_t *rhs_row = rhs + (size_t)col_indices[jc] * K;
-            float4_t acc = {0.f, 0.f, 0.f, 0.f};
-            for (int kk = 0; kk < k_steps; ++kk) {
-                const int off = 32 * kk + 8 * g;
-                half8_t a = zero8, b = zero8;
-                if (off < K) {
-                    b = *reinterpret_cast<const half8_t *>(rhs_row + off);
-                    if (a_row_ok) a = *reinterpret_cast<const half8_t *>(lhs_row + off);
-                }
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
+        for (int sg = s; sg < n_super; sg += slots) {
+            const int j0 = beg + SUPER * sg;
+            const half_t *rhs_row[GRP];
+            float4_t acc[GRP];
+#pragma unroll
+            for (int u = 0; u < GRP; ++u) {
+                const int jl = j0 + 16 * u + r;
+                rhs_row[u] = rhs + (size_t)col_indices[jl < end ? jl : end - 1] * K;
+                acc[u] = float4_t{0.f, 0.f, 0.f, 0.f};
             }
-            if (valid) store_group<V, OutT>(out, j, g, acc);
+            for (int kk = 0; kk < k_steps; ++kk) {
+                const half8_t a = to_mfma_order(load_slice16(lhs_row, kk, q, K, a_row_ok), src);
+                uint4_t raw[GRP];
+#pragma unroll
+                for (int u = 0; u < GRP; ++u) raw[u] = load_slice16(rhs_row[u], kk, q, K, true);
+#pragma unroll
+                for (int u = 0; u < GRP; ++u)
+                    acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, to_mfma_order(raw[u], src), acc[u], 0, 0, 0);
+            }
+#pragma unroll
+            for (int u = 0; u < GRP; ++u) {
+                const int j = j0 + 16 * u + c;
+                if (j < end) store_group<V, OutT>(out, j, g, acc[u]);
+            }
         }
     }
 }
 
-template <int V, int KS, typename OutT>
-static int launch_one(int m_vec, int k, int slots, const int *row_indices, const int *row_offsets,
+template <int V, int KS, int GRP, typename OutT>
+static int launch_one(int m_vec, int k, int nonzeros_vec, const int *row_indices, const int *row_offsets,
                       const int *col_indices, const half_t *lhs, const half_t *rhs, OutT *out, hipStream_t stream,
                       const Batch &batch)
 {
     constexpr int kWavesPerBlock = 4;
+    const int slots = sddmm_auto_slots(m_vec * batch.count, nonzeros_vec * batch.count, 16 * GRP);
     const long long waves = (long long)m_vec * slots;
     const long long blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
-    hipLaunchKernelGGL((sddmm_mfma_kernel<V, KS, OutT>), dim3((unsigned)blocks, (unsigned)batch.count), dim3(64 * kWavesPerBlock), 0, stream,
+    hipLaunchKernelGGL((sddmm_mfma_kernel<V, KS, GRP, OutT>), dim3((unsigned)blocks, (unsigned)batch.count), dim3(64 * kWavesPerBlock), 0, stream,
                        m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out,
                        batch.stride_a, batch.stride_b, batch.stride_out);
     return (int)hipGetLastError();
 }
 
 template <int V, typename OutT>
-static int launch_ks(int m_vec, int k, int slots, const int *row_indices, const int *row_offsets,
+static int launch_ks(int m_vec, int k, int nonzeros_vec, const int *row_indices, const int *row_offsets,
                      const int *col_indices, const half_t *lhs, const half_t *rhs, OutT *out, hipStream_t stream,
                       const Batch &batch)
 {
-    if (k <= 32) return launch_one<V, 1, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
-    if (k <= 64) return launch_one<V, 2, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
-    if (k <= 128) return launch_one<V, 4, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
-    if (k <= 256) return launch_one<V, 8, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
-    return launch_one<V, 0, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    if (k <= 32) return launch_one<V, 1, 4, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    if (k <= 64) return launch_one<V, 2, 4, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    if (k <= 128) return launch_one<V, 4, 2, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    if (k <= 256) return launch_one<V, 8, 1, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    return launch_one<V, 0, 4, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
 }
 
-// Workgroups per vector row: enough waves to fill the chip, at most one per 16-vector group of an
-// average row (longer rows loop).
+// Waves per vector row: enough waves to fill the chip, at most one per super-group of an average row
+// (longer rows loop).
 int sddmm_auto_slots(int m_vec, int nonzeros_vec, int group)
 {
     int slots = options().sddmm_slots;
@@ -153,12 +185,11 @@ int launch_sddmm_mfma(int m_vec, int k, int n, int nonzeros_vec, const int *row_
     if (m_vec == 0 || nonzeros_vec == 0 || batch.count == 0) return hipSuccess;
     if (batch.count > 65535) return hipErrorNotSupported;
     if (k <= 0 || k % 8 != 0) return hipErrorNotSupported;
-    const int slots = sddmm_auto_slots(m_vec * batch.count, nonzeros_vec * batch.count, 16);
     switch (vec_length) {
-    case 1: return launch_ks<1, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
-    case 2: return launch_ks<2, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
-    case 4: return launch_ks<4, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
-    case 8: return launch_ks<8, OutT>(m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    case 1: return launch_ks<1, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    case 2: return launch_ks<2, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    case 4: return launch_ks<4, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    case 8: return launch_ks<8, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
     default: return hipErrorInvalidValue;
     }
 }

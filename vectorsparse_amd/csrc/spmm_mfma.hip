@@ -109,7 +109,13 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
 #pragma unroll
     for (int c = 0; c < CPL; ++c) acc[c] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    for (int base = beg + kStep * wave; base < end; base += kStep * n_waves) {
+    // Short rows do not need every wave: with fewer than two steps per wave the partial-tile
+    // reduction costs more than the split saves, so only `active` waves take steps.
+    const int steps = (end - beg + kStep - 1) / kStep;
+    int active = (steps + 1) >> 1;
+    active = active < 1 ? 1 : (active > n_waves ? n_waves : active);
+
+    for (int base = beg + kStep * wave; wave < active && base < end; base += kStep * active) {
         if (lane < kStep) {
             const int j = base + lane;
             const bool valid = j < end;
@@ -168,7 +174,7 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         const int v = 4 * g + e;
-        if (v < V) {
+        if (v < V && wave < active) {
 #pragma unroll
             for (int c4 = 0; c4 < CPL / 4; ++c4) {
                 float4_t t = {acc[4 * c4][e], acc[4 * c4 + 1][e], acc[4 * c4 + 2][e], acc[4 * c4 + 3][e]};
@@ -186,7 +192,7 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
             float sum[CPL];
 #pragma unroll
             for (int c = 0; c < CPL; ++c) sum[c] = 0.f;
-            for (int w = 0; w < n_waves; ++w) {
+            for (int w = 0; w < active; ++w) {
                 const float *src = partial + (size_t)w * V * TN + v * TN + cs2 * CPL;
 #pragma unroll
                 for (int c4 = 0; c4 < CPL / 4; ++c4) {
@@ -256,7 +262,7 @@ int launch_spmm_mfma(int m_vec, int vec_length, int k, int n, const int *row_ind
     int cpl = options().spmm_cols_per_lane;
     if (cpl != 4 && cpl != 8) {
         const long long blocks128 = (long long)m_vec * ceil_div(k, 128) * batch.count;
-        cpl = (k % 8 == 0 && blocks128 >= kTargetBlocks) ? 8 : 4;
+        cpl = (k % 8 == 0 && k > 64 && blocks128 >= kTargetBlocks) ? 8 : 4;  // k <= 64 fits one 64-column tile
     }
     if (cpl == 8 && k % 8 != 0) cpl = 4;
     const long long blocks = (long long)m_vec * ceil_div(k, 16 * cpl) * batch.count;
@@ -265,6 +271,8 @@ int launch_spmm_mfma(int m_vec, int vec_length, int k, int n, const int *row_ind
         waves = next_pow2((int)((kTargetWaves + blocks - 1) / blocks));
         const int max_useful = next_pow2(ceil_div(n > 0 ? n : 1, kStep));  // a row holds at most n vectors
         if (waves > max_useful) waves = max_useful;
+        // two waves per row even on a full chip: measured 30 % faster than one on 8192 rows of ~280 vectors
+        if (waves < 2 && n >= 4 * kStep) waves = 2;
     }
     if (waves < 1) waves = 1;
     if (waves > 16) waves = 16;
