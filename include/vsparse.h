@@ -185,6 +185,22 @@ int vs_sparse_softmax_f16(int batch, int m_vec, int vec_length,
                           float scale, void *stream);
 
 /*
+ * Softmax fused into SpMM:  out = softmax_row(scale * scores) * rhs_matrix, where `scores` has the
+ * layout of `values` (for example the raw output of SDDMM).  Equivalent to vs_sparse_softmax_f16
+ * followed by vs_wmma_spmm_f16_batched without writing the probabilities to memory: the kernel finds
+ * each scalar row's maximum, exponentiates while staging the sparse operand and divides the
+ * accumulated tile by the row sum.  Same requirements as vs_wmma_spmm_f16_batched.  No counterpart in
+ * the reference (see vs_sparse_softmax_f16).
+ */
+int vs_wmma_spmm_softmax_f16_batched(int batch, int m_vec, int vec_length, int k, int n,
+                                     const int *row_indices, const int *row_offsets,
+                                     const int *column_indices,
+                                     const void *scores, long long stride_scores,
+                                     const void *rhs_matrix, long long stride_rhs,
+                                     void *output_matrix, long long stride_output,
+                                     float scale, void *stream);
+
+/*
  * Host helpers (HOST pointers).  Replace IdentityRowSwizzle / SortedRowSwizzle —
  * include/bm_test_utils.h:196-198 and :200-215.  The sorted swizzle orders
  * vector rows by descending length; equal lengths keep ascending row order.

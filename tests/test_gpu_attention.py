@@ -93,6 +93,58 @@ def test_attention_layer_vs_dense_masked_attention(gpu, kernel):
         assert err <= 1e-2, "attention head %d %s: max |err| / rms = %.3e" % (h, kernel, err)
 
 
+@pytest.mark.parametrize("V", [1, 2, 4, 8])
+@pytest.mark.parametrize("N", [64, 256])
+def test_softmax_fused_into_spmm(gpu, V, N):
+    # ragged rows incl. empty ones and rows long enough for several waves; scores with a wide range
+    lengths = np.array([0, 1, 31, 32, 33, 64, 200, 513, 0, 17, 90, 300], dtype=np.int64)
+    rng = np.random.default_rng(V + N)
+    ro, ci = cv._pattern_from_lengths(rng, len(lengths), 640, lengths)
+    pat = cv.random_values(cv.ColVecCSR(len(lengths), 640, V, ro, ci), seed=V, scale=4.0)
+    W = cv.dense_uniform(640, N, seed=9)
+    scale = 0.3
+    prob = ops.DeviceProblem(pat, sort=True)
+    out = torch.full((pat.m, N), 7.0, dtype=torch.float16, device="cuda")
+    ops.spmm_softmax_batched(pat.m_vec, V, N, 640, prob.row_indices, prob.row_offsets, prob.column_indices,
+                             prob.values, torch.from_numpy(W).cuda(), out, scale)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().astype(np.float64)
+    # (1) against the exact float64 definition softmax(scale*x) @ W.  The probabilities enter the MFMA as
+    # fp16 (as they do when the separate softmax kernel stores them), so outputs that cancel to nearly
+    # zero carry that rounding; the bound for the fused operator is max |err| <= 1e-2 * rms(ref) per row.
+    probs = no.sparse_softmax_ref(pat.m_vec, V, pat.row_offsets, pat.values, scale)
+    # (2) against the same definition with the exponentials rounded to fp16 where the kernel rounds them
+    # (before the normalisation): here the per-element 1e-2 criterion of a single operator applies.
+    x = pat.values.astype(np.float64) * scale
+    exact = np.zeros((pat.m, N))
+    rounded = np.zeros((pat.m, N))
+    for i in range(pat.m_vec):
+        lo, hi = int(ro[i]), int(ro[i + 1])
+        if hi > lo:
+            rows = W[ci[lo:hi]].astype(np.float64)
+            exact[i * V:(i + 1) * V] = probs[lo:hi].T @ rows
+            e = np.exp(x[lo:hi] - x[lo:hi].max(axis=0, keepdims=True))
+            rounded[i * V:(i + 1) * V] = (e.astype(np.float16).astype(np.float64).T @ rows) / e.sum(axis=0)[:, None]
+    assert_parity(got, rounded, "softmax+spmm V%d N%d" % (V, N))
+    rms = np.sqrt(np.mean(exact * exact, axis=1, keepdims=True))
+    nonempty = rms[:, 0] > 0
+    assert float(np.max(np.abs(got - exact)[nonempty] / rms[nonempty])) <= 1e-2
+    for i in np.nonzero(lengths == 0)[0]:
+        assert not out[i * V:(i + 1) * V].any()
+
+
+def test_fused_and_unfused_layers_agree(gpu):
+    V, heads, seq, d = 8, 4, 1024, 64
+    mask = cv.band_strided_pattern(seq, V, band_half_width=128, stride=128)
+    layer = ops.SparseAttention(mask)
+    g = torch.Generator(device="cuda").manual_seed(1)
+    q, k, v = (torch.randn((heads, seq, d), device="cuda", generator=g).half() for _ in range(3))
+    a = layer.forward(q, k, v, fused=True).float().cpu().numpy()
+    b = layer.forward(q, k, v, fused=False).float().cpu().numpy()
+    rms = float(np.sqrt(np.mean(b * b)))
+    assert float(np.max(np.abs(a - b))) <= 1e-2 * rms
+
+
 def test_attention_steps_match_the_oracle_chain(gpu):
     # the same layer step by step against the three oracles (exact intermediate layout)
     V, seq, d = 8, 256, 64

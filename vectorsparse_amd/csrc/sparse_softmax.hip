@@ -46,29 +46,6 @@ __device__ __forceinline__ void store_vec(half_t *p, const float (&src)[V])
     store_converted<half_t, V>(p, src);
 }
 
-__device__ __forceinline__ float wave_max(float x)
-{
-    x = fmaxf(x, partner<1>(x));
-    x = fmaxf(x, partner<2>(x));
-    x = fmaxf(x, partner<4>(x));
-    x = fmaxf(x, partner<8>(x));
-    x = fmaxf(x, partner<16>(x));
-    x = fmaxf(x, partner<32>(x));
-    return x;
-}
-
-__device__ __forceinline__ float wave_sum(float x)
-{
-    x += partner<1>(x);
-    x += partner<2>(x);
-    x += partner<4>(x);
-    x += partner<8>(x);
-    x += partner<16>(x);
-    x += partner<32>(x);
-    return x;
-}
-
-constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kCached = 8;  // vectors per lane kept in registers: rows of up to 64 * 8 vectors
 
 template <int V>

@@ -74,12 +74,16 @@ constexpr int stage_bytes()
     return kStep * (int)sizeof(int) + V * kStep * (int)sizeof(half_t);  // indices + transposed vectors
 }
 
-template <int V, int CPL, typename OutT>
+// SOFTMAX: the sparse values are raw scores and the kernel multiplies by softmax_row(scale * values)
+// instead: a pre-pass finds each scalar row's maximum, the staging step turns every score into
+// exp2(s*x - max) (and sums them), and the accumulated tile is divided by the row sum at the end.
+template <int V, int CPL, bool SOFTMAX, typename OutT>
 __global__ void __launch_bounds__(1024)
 spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
                  const int *__restrict__ row_offsets, const int *__restrict__ column_indices,
                  const half_t *__restrict__ values, const half_t *__restrict__ rhs,
-                 OutT *__restrict__ out, long long stride_values, long long stride_rhs, long long stride_out)
+                 OutT *__restrict__ out, long long stride_values, long long stride_rhs, long long stride_out,
+                 float scale)
 {
     values += blockIdx.y * stride_values;  // batch: shared pattern, per-problem operands
     rhs += blockIdx.y * stride_rhs;
@@ -104,6 +108,25 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
     int *idx_s = reinterpret_cast<int *>(smem + (size_t)wave * kStage);
     half_t *vec_s = reinterpret_cast<half_t *>(idx_s + kStep);  // [V][kStep]
     float *partial = reinterpret_cast<float *>(smem + (size_t)n_waves * kStage);
+    float *sums_s = partial + (size_t)n_waves * V * TN;  // [W][V] softmax denominators (SOFTMAX only)
+
+    const float s2 = scale * kLog2e;
+    float row_max[V], row_sum[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+        row_max[v] = -__builtin_inff();
+        row_sum[v] = 0.f;
+    }
+    if constexpr (SOFTMAX) {
+        for (int j = beg + lane; j < end; j += 64) {
+            half_t x[V];
+            load_vector<V>(x, values + (size_t)j * V);
+#pragma unroll
+            for (int v = 0; v < V; ++v) row_max[v] = fmaxf(row_max[v], (float)x[v] * s2);
+        }
+#pragma unroll
+        for (int v = 0; v < V; ++v) row_max[v] = wave_max(row_max[v]);
+    }
 
     float4_t acc[CPL];
 #pragma unroll
@@ -126,7 +149,15 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
             half_t av[V];
             load_vector<V>(av, values + (size_t)jc * V);
 #pragma unroll
-            for (int v = 0; v < V; ++v) vec_s[v * kStep + lane] = valid ? av[v] : (half_t)0.f;
+            for (int v = 0; v < V; ++v) {
+                half_t staged = valid ? av[v] : (half_t)0.f;
+                if constexpr (SOFTMAX) {
+                    const float p = valid ? __builtin_amdgcn_exp2f((float)av[v] * s2 - row_max[v]) : 0.f;
+                    row_sum[v] += p;
+                    staged = (half_t)p;
+                }
+                vec_s[v * kStep + lane] = staged;
+            }
         }
         wave_lds_fence();
         const int4_t i_lo = *reinterpret_cast<const int4_t *>(idx_s + 8 * g);
@@ -156,14 +187,26 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
         }
     }
 
+    if constexpr (SOFTMAX) {
+#pragma unroll
+        for (int v = 0; v < V; ++v) row_sum[v] = wave_sum(row_sum[v]);
+    }
+
     if (n_waves == 1) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const int v = 4 * g + e;
             if (v < V && col_ok) {
+                float norm = 1.f;
+                if constexpr (SOFTMAX) {
+                    float total = 1.f;
+#pragma unroll
+                    for (int vv = 0; vv < V; ++vv) total = (vv == v) ? row_sum[vv] : total;
+                    norm = end > beg ? 1.f / total : 0.f;
+                }
                 float tmp[CPL];
 #pragma unroll
-                for (int c = 0; c < CPL; ++c) tmp[c] = acc[c][e];
+                for (int c = 0; c < CPL; ++c) tmp[c] = acc[c][e] * norm;
                 store_converted<OutT, CPL>(out + ((size_t)row * V + v) * n_cols + col0, tmp);
             }
         }
@@ -180,6 +223,14 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
                 float4_t t = {acc[4 * c4][e], acc[4 * c4 + 1][e], acc[4 * c4 + 2][e], acc[4 * c4 + 3][e]};
                 *reinterpret_cast<float4_t *>(mine + v * TN + cs * CPL + 4 * c4) = t;
             }
+        }
+    }
+    if constexpr (SOFTMAX) {
+        if (lane < V && wave < active) {
+            float mine_sum = 0.f;
+#pragma unroll
+            for (int v = 0; v < V; ++v) mine_sum = (v == lane) ? row_sum[v] : mine_sum;
+            sums_s[wave * V + lane] = mine_sum;
         }
     }
     __syncthreads();
@@ -203,6 +254,13 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
                     sum[4 * c4 + 3] += x[3];
                 }
             }
+            if constexpr (SOFTMAX) {
+                float total = 0.f;
+                for (int w = 0; w < active; ++w) total += sums_s[w * V + v];
+                const float norm = end > beg ? 1.f / total : 0.f;
+#pragma unroll
+                for (int c = 0; c < CPL; ++c) sum[c] *= norm;
+            }
             store_converted<OutT, CPL>(out + ((size_t)row * V + v) * n_cols + col, sum);
         }
     }
@@ -215,45 +273,47 @@ static int next_pow2(int x)
     return p;
 }
 
-template <int V, int CPL, typename OutT>
+template <int V, int CPL, bool SOFTMAX, typename OutT>
 static int launch_one(int m_vec, int k, int n, int waves, const int *row_indices, const int *row_offsets,
                       const int *column_indices, const half_t *values, const half_t *rhs, OutT *out,
-                      hipStream_t stream, const Batch &batch)
+                      hipStream_t stream, const Batch &batch, float scale)
 {
     (void)n;
     constexpr int TN = 16 * CPL;
     const int n_tiles = ceil_div(k, TN);
     const long long blocks = (long long)m_vec * n_tiles;
     if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
-    const size_t lds = (size_t)waves * stage_bytes<V>() + (waves > 1 ? (size_t)waves * V * TN * sizeof(float) : 0);
-    auto kernel = spmm_mfma_kernel<V, CPL, OutT>;
+    const size_t lds = (size_t)waves * stage_bytes<V>() +
+                       (waves > 1 ? (size_t)waves * V * (TN + 1) * sizeof(float) : 0);
+    auto kernel = spmm_mfma_kernel<V, CPL, SOFTMAX, OutT>;
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
     if (attr != hipSuccess) return (int)attr;
     hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)batch.count), dim3(64 * waves), lds, stream,
                        k, n_tiles, row_indices, row_offsets, column_indices, values, rhs, out,
-                       batch.stride_a, batch.stride_b, batch.stride_out);
+                       batch.stride_a, batch.stride_b, batch.stride_out, scale);
     return (int)hipGetLastError();
 }
 
-template <int CPL, typename OutT>
+template <int CPL, bool SOFTMAX, typename OutT>
 static int launch_v(int vec_length, int m_vec, int k, int n, int waves, const int *row_indices,
                     const int *row_offsets, const int *column_indices, const half_t *values,
-                    const half_t *rhs, OutT *out, hipStream_t stream, const Batch &batch)
+                    const half_t *rhs, OutT *out, hipStream_t stream, const Batch &batch,
+                    float scale)
 {
     switch (vec_length) {
-    case 1: return launch_one<1, CPL, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
-    case 2: return launch_one<2, CPL, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
-    case 4: return launch_one<4, CPL, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
-    case 8: return launch_one<8, CPL, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
+    case 1: return launch_one<1, CPL, SOFTMAX, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
+    case 2: return launch_one<2, CPL, SOFTMAX, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
+    case 4: return launch_one<4, CPL, SOFTMAX, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
+    case 8: return launch_one<8, CPL, SOFTMAX, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
     default: return hipErrorInvalidValue;
     }
 }
 
-template <typename OutT>
-int launch_spmm_mfma(int m_vec, int vec_length, int k, int n, const int *row_indices,
-                     const int *row_offsets, const int *column_indices, const half_t *values,
-                     const half_t *rhs, OutT *out, hipStream_t stream, const Batch &batch)
+template <bool SOFTMAX, typename OutT>
+static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_indices,
+                      const int *row_offsets, const int *column_indices, const half_t *values,
+                      const half_t *rhs, OutT *out, hipStream_t stream, const Batch &batch, float scale)
 {
     if (m_vec == 0 || k == 0 || batch.count == 0) return hipSuccess;
     if (k % 4 != 0 || batch.count > 65535) return hipErrorNotSupported;
@@ -277,8 +337,25 @@ int launch_spmm_mfma(int m_vec, int vec_length, int k, int n, const int *row_ind
     if (waves < 1) waves = 1;
     if (waves > 16) waves = 16;
     if (cpl == 8)
-        return launch_v<8, OutT>(vec_length, m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
-    return launch_v<4, OutT>(vec_length, m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
+        return launch_v<8, SOFTMAX, OutT>(vec_length, m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
+    return launch_v<4, SOFTMAX, OutT>(vec_length, m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
+}
+
+template <typename OutT>
+int launch_spmm_mfma(int m_vec, int vec_length, int k, int n, const int *row_indices,
+                     const int *row_offsets, const int *column_indices, const half_t *values,
+                     const half_t *rhs, OutT *out, hipStream_t stream, const Batch &batch)
+{
+    return launch_any<false, OutT>(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices, values, rhs,
+                                   out, stream, batch, 1.f);
+}
+
+int launch_spmm_softmax_mfma(int m_vec, int vec_length, int k, int n, const int *row_indices,
+                             const int *row_offsets, const int *column_indices, const half_t *scores,
+                             const half_t *rhs, half_t *out, float scale, hipStream_t stream, const Batch &batch)
+{
+    return launch_any<true, half_t>(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices, scores, rhs,
+                                    out, stream, batch, scale);
 }
 
 template int launch_spmm_mfma<half_t>(int, int, int, int, const int *, const int *, const int *, const half_t *,

@@ -62,6 +62,30 @@ __device__ __forceinline__ float partner(float x)
 }
 
 
+// All-lane max / sum over the 64 lanes of a wave (every lane must be active).
+__device__ __forceinline__ float wave_max(float x)
+{
+    x = fmaxf(x, partner<1>(x));
+    x = fmaxf(x, partner<2>(x));
+    x = fmaxf(x, partner<4>(x));
+    x = fmaxf(x, partner<8>(x));
+    x = fmaxf(x, partner<16>(x));
+    x = fmaxf(x, partner<32>(x));
+    return x;
+}
+
+__device__ __forceinline__ float wave_sum(float x)
+{
+    x += partner<1>(x);
+    x += partner<2>(x);
+    x += partner<4>(x);
+    x += partner<8>(x);
+    x += partner<16>(x);
+    x += partner<32>(x);
+    return x;
+}
+
+constexpr float kLog2e = 1.4426950408889634f;
 // Store `Count` consecutive outputs converted from fp32 (Count in {1,2,4,8}).
 template <typename OutT, int Count>
 __device__ __forceinline__ void store_converted(OutT *dst, const float *src);
@@ -161,6 +185,10 @@ int launch_sddmm_valu(int m_vec, int k, int n, int nonzeros_vec, const int *row_
                       const half_t *rhs, OutT *out, int vec_length, hipStream_t stream,
                       const Batch &batch = Batch());
 
+int launch_spmm_softmax_mfma(int m_vec, int vec_length, int k, int n, const int *row_indices,
+                             const int *row_offsets, const int *column_indices, const half_t *scores,
+                             const half_t *rhs, half_t *out, float scale, hipStream_t stream,
+                             const Batch &batch = Batch());
 int launch_sparse_softmax(int m_vec, int vec_length, const int *row_indices, const int *row_offsets,
                           const half_t *values_in, half_t *values_out, float scale, hipStream_t stream,
                           const Batch &batch = Batch());

@@ -258,6 +258,24 @@ int vs_cuda_sddmm_f16_batched(int batch, int m_vec, int k, int n, int nonzeros_v
                                          make_batch(batch, stride_lhs, stride_rhs, stride_output));
 }
 
+int vs_wmma_spmm_softmax_f16_batched(int batch, int m_vec, int vec_length, int k, int n, const int *row_indices,
+                                     const int *row_offsets, const int *column_indices, const void *scores,
+                                     long long stride_scores, const void *rhs_matrix, long long stride_rhs,
+                                     void *output_matrix, long long stride_output, float scale, void *stream)
+{
+    if (batch < 0) return VS_ERROR_INVALID_VALUE;
+    int st = check_spmm(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices, scores, rhs_matrix,
+                        output_matrix, sizeof(half_t));
+    if (st != VS_SUCCESS) return st;
+    if (!stride_ok(stride_scores, vec_length) || !stride_ok(stride_rhs, 8) || !stride_ok(stride_output, 8))
+        return VS_ERROR_INVALID_VALUE;
+    return vs::launch_spmm_softmax_mfma(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices,
+                                        static_cast<const half_t *>(scores), static_cast<const half_t *>(rhs_matrix),
+                                        static_cast<half_t *>(output_matrix), scale,
+                                        static_cast<hipStream_t>(stream),
+                                        make_batch(batch, stride_scores, stride_rhs, stride_output));
+}
+
 int vs_sparse_softmax_f16(int batch, int m_vec, int vec_length, const int *row_indices, const int *row_offsets,
                           const void *values_in, long long stride_in, void *values_out, long long stride_out,
                           float scale, void *stream)

@@ -136,6 +136,22 @@ def spmm_batched(m_vec, vec_length, k, n, row_indices, row_offsets, column_indic
     return output_matrix
 
 
+def spmm_softmax_batched(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices, scores, rhs_matrix,
+                         output_matrix, scale=1.0, stream=None):
+    """out[b] = softmax_row(scale * scores[b]) @ rhs_matrix[b] in one launch (softmax fused into SpMM)."""
+    if output_matrix.dim() == 2:
+        output_matrix = output_matrix.unsqueeze(0)
+    batch = output_matrix.shape[0]
+    for t, nm in ((scores, "scores"), (rhs_matrix, "rhs_matrix"), (output_matrix, "output_matrix")):
+        _expect_batched(t, torch.float16, nm)
+    st = _lib.lib().vs_wmma_spmm_softmax_f16_batched(
+        batch, m_vec, vec_length, k, n, _ptr(row_indices), _ptr(row_offsets), _ptr(column_indices), _ptr(scores),
+        _stride(scores, batch), _ptr(rhs_matrix), _stride(rhs_matrix, batch), _ptr(output_matrix),
+        _stride(output_matrix, batch), float(scale), _stream(stream))
+    _lib.check(st, "vs_wmma_spmm_softmax_f16_batched")
+    return output_matrix
+
+
 def sddmm_batched(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices, lhs_matrix, rhs_matrix,
                   output_values, vec_length, kernel="wmma", stream=None, algorithm=1):
     """`batch` SDDMMs sharing one mask in one launch.
@@ -193,8 +209,12 @@ class SparseAttention:
     def __init__(self, mask, device="cuda", sort=True):
         self.prob = DeviceProblem(mask, sort=sort, device=device)
 
-    def forward(self, q, k, v, scale=None, kernel="wmma", stream=None, scores=None, out=None):
-        """q, k, v: fp16 [heads, seq, d] on the device.  Returns fp16 [heads, seq, d]."""
+    def forward(self, q, k, v, scale=None, kernel="wmma", stream=None, scores=None, out=None, fused=None):
+        """q, k, v: fp16 [heads, seq, d] on the device.  Returns fp16 [heads, seq, d].
+
+        fused (default: True on the MFMA path) folds the softmax into the SpMM launch, so the layer is
+        two launches and the probabilities never go to memory.
+        """
         p = self.prob
         heads, seq, d = q.shape
         if scale is None:
@@ -205,6 +225,11 @@ class SparseAttention:
             out = torch.empty((heads, seq, v.shape[2]), dtype=torch.float16, device=q.device)
         sddmm_batched(p.m_vec, d, p.n, p.nnz_vec, p.row_indices, p.row_offsets, p.column_indices, q, k, scores,
                       p.vec_length, kernel=kernel, stream=stream)
+        if fused is None:
+            fused = kernel == "wmma"
+        if fused:
+            return spmm_softmax_batched(p.m_vec, p.vec_length, v.shape[2], p.n, p.row_indices, p.row_offsets,
+                                        p.column_indices, scores, v, out, scale, stream=stream)
         sparse_softmax(p.m_vec, p.vec_length, p.row_indices, p.row_offsets, scores, scores, scale, stream=stream)
         spmm_batched(p.m_vec, p.vec_length, v.shape[2], p.n, p.row_indices, p.row_offsets, p.column_indices,
                      scores, v, out, kernel=kernel, stream=stream)
