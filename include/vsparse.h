@@ -201,6 +201,24 @@ int vs_wmma_spmm_softmax_f16_batched(int batch, int m_vec, int vec_length, int k
                                      float scale, void *stream);
 
 /*
+ * One fixed-mask sparse attention layer in a single launch:
+ *     out[b] = softmax_row(scale * (q[b] k[b]^T sampled on the mask)) v[b]
+ * q: [m_vec*vec_length, d_qk], k: [n, d_qk], v: [n, d_v], out: [m_vec*vec_length, d_v], all fp16
+ * row-major; the mask is a column-vector CSR pattern over [m, n] shared by the batch (heads).
+ * Scores and probabilities stay in LDS (never written to memory); rows of any length are handled with
+ * a running maximum / sum over chunks of the row.  Requirements: d_qk % 8 == 0, d_qk <= 128;
+ * d_v % 4 == 0 and d_v <= 64, or d_v % 8 == 0 and d_v <= 128; operands aligned to 16 bytes, strides
+ * multiples of 8 elements.  Empty rows produce zeros.  No counterpart in the reference (it links an
+ * external sparse-transformer repository, README.md:76); same result as vs_wmma_sddmm_f16_batched ->
+ * vs_sparse_softmax_f16 -> vs_wmma_spmm_f16_batched up to the fp16 rounding of the intermediates.
+ */
+int vs_sparse_attention_f16(int batch, int m_vec, int vec_length, int n, int d_qk, int d_v,
+                            const int *row_indices, const int *row_offsets, const int *col_indices,
+                            const void *q, long long stride_q, const void *k, long long stride_k,
+                            const void *v, long long stride_v, void *out, long long stride_out,
+                            float scale, void *stream);
+
+/*
  * Host helpers (HOST pointers).  Replace IdentityRowSwizzle / SortedRowSwizzle —
  * include/bm_test_utils.h:196-198 and :200-215.  The sorted swizzle orders
  * vector rows by descending length; equal lengths keep ascending row order.
@@ -211,8 +229,9 @@ void vs_sorted_row_swizzle(int rows, const int *row_offsets, int *row_indices);
 /*
  * Launch-shape tuning knob (process-wide, not thread-safe against concurrent
  * launches).  Names: "spmm_waves" (waves per workgroup, 0 = automatic),
- * "spmm_cols_per_lane" (4, 8, 0 = automatic), "sddmm_slots" (workgroups per
- * vector row, 0 = automatic).  Returns 0, or 1 for an unknown name / bad value.
+ * "spmm_cols_per_lane" (4, 8, 0 = automatic), "sddmm_slots" (waves per
+ * vector row, 0 = automatic), "attention_waves" (1..8, 0 = automatic),
+ * "attention_chunk" (nonzero vectors per LDS chunk, 0 = automatic).  Returns 0, or 1 for an unknown name / bad value.
  * No counterpart in the reference, whose tile sizes are compile-time constants
  * (src/wmma_spmm.cu:396).
  */

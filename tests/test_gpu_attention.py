@@ -167,3 +167,96 @@ def test_attention_steps_match_the_oracle_chain(gpu):
     assert_parity(out.cpu().numpy(),
                   co.spmm_host_ref_f32(mask.m_vec, V, d, seq, mask.row_offsets, mask.column_indices, p_host, v),
                   "context")
+
+
+def _dense_attention(mask, q, k, v, scale):
+    V = mask.vec_length
+    allowed = np.zeros((mask.m, mask.n), dtype=bool)
+    for i in range(mask.m_vec):
+        cols = mask.column_indices[mask.row_offsets[i]:mask.row_offsets[i + 1]]
+        allowed[i * V:(i + 1) * V, cols] = True
+    out = np.zeros((q.shape[0], mask.m, v.shape[2]))
+    for h in range(q.shape[0]):
+        s = q[h].astype(np.float64) @ k[h].astype(np.float64).T * scale
+        s[~allowed] = -np.inf
+        with np.errstate(invalid="ignore"):
+            p = np.exp(s - np.where(allowed.any(axis=1, keepdims=True), s.max(axis=1, keepdims=True), 0.0))
+        p[~allowed] = 0.0
+        denom = p.sum(axis=1, keepdims=True)
+        p = np.divide(p, denom, out=np.zeros_like(p), where=denom > 0)
+        out[h] = p @ v[h].astype(np.float64)
+    return out
+
+
+def _check_layer(got, ref, what):
+    # end-to-end bound for a chain with fp16 operands in both MFMA stages: max |err| <= 1e-2 * rms(ref)
+    rms = float(np.sqrt(np.mean(ref * ref)))
+    err = float(np.max(np.abs(got.astype(np.float64) - ref))) / rms
+    assert np.all(np.isfinite(got)), what
+    assert err <= 1e-2, "%s: max |err| / rms = %.3e" % (what, err)
+
+
+@pytest.mark.parametrize("V", [1, 2, 4, 8])
+@pytest.mark.parametrize("dims", [(64, 64), (32, 128), (128, 40), (72, 64)], ids=lambda d: "dqk%d_dv%d" % d)
+def test_single_launch_attention(gpu, V, dims):
+    d_qk, d_v = dims
+    heads = 3
+    lengths = np.array([0, 1, 15, 16, 17, 31, 32, 33, 64, 130, 300, 5, 0, 48, 7, 100], dtype=np.int64)
+    rng = np.random.default_rng(V * 7 + d_qk)
+    n = 384
+    ro, ci = cv._pattern_from_lengths(rng, len(lengths), n, lengths)
+    mask = cv.ColVecCSR(len(lengths), n, V, ro, ci).validate()
+    prob = ops.DeviceProblem(mask, sort=True)
+    q = rng.standard_normal((heads, mask.m, d_qk)).astype(np.float16)
+    k = rng.standard_normal((heads, n, d_qk)).astype(np.float16)
+    v = rng.standard_normal((heads, n, d_v)).astype(np.float16)
+    scale = 1.0 / np.sqrt(d_qk)
+    ref = _dense_attention(mask, q, k, v, scale)
+    qd, kd, vd = (torch.from_numpy(x).cuda() for x in (q, k, v))
+    try:
+        for chunk, waves in ((0, 0), (64, 3), (32, 8), (96, 1)):      # one chunk / several chunks per long row
+            _lib_set("attention_chunk", chunk)
+            _lib_set("attention_waves", waves)
+            pad = torch.full((heads, mask.m + 16, d_v), 3.0, dtype=torch.float16, device="cuda")
+            out = pad[:, 8:8 + mask.m]
+            ops.sparse_attention(mask.m_vec, V, n, prob.row_indices, prob.row_offsets, prob.column_indices,
+                                 qd, kd, vd, out=out, scale=scale)
+            torch.cuda.synchronize()
+            host = pad.cpu().numpy()
+            assert np.all(host[:, :8] == 3.0) and np.all(host[:, 8 + mask.m:] == 3.0), "wrote outside the output"
+            _check_layer(host[:, 8:8 + mask.m], ref, "V%d dqk%d dv%d chunk%d waves%d" % (V, d_qk, d_v, chunk, waves))
+            for i in np.nonzero(lengths == 0)[0]:
+                assert not host[:, 8 + i * V:8 + (i + 1) * V].any(), "an empty row must produce zeros"
+    finally:
+        _lib_set("attention_chunk", 0)
+        _lib_set("attention_waves", 0)
+
+
+def _lib_set(name, value):
+    from vectorsparse_amd import _lib
+    _lib.set_option(name, value)
+
+
+def test_single_launch_layer_matches_three_launch_layer(gpu):
+    V, heads, seq, d = 8, 4, 1024, 64
+    mask = cv.band_strided_pattern(seq, V, band_half_width=128, stride=128)
+    layer = ops.SparseAttention(mask)
+    g = torch.Generator(device="cuda").manual_seed(2)
+    q, k, v = (torch.randn((heads, seq, d), device="cuda", generator=g).half() for _ in range(3))
+    a = layer.forward(q, k, v, fused="layer").float().cpu().numpy()
+    b = layer.forward(q, k, v, fused=False).float().cpu().numpy()
+    rms = float(np.sqrt(np.mean(b * b)))
+    assert float(np.max(np.abs(a - b))) <= 1e-2 * rms
+    again = layer.forward(q, k, v, fused="layer").float().cpu().numpy()
+    assert np.array_equal(a, again)       # deterministic
+
+
+def test_single_launch_attention_rejects_unsupported_shapes(gpu):
+    from vectorsparse_amd import _lib
+    mask = cv.uniform_pattern(4, 64, 0.5, seed=1, vec_length=8)
+    prob = ops.DeviceProblem(mask)
+    q = torch.zeros((1, 32, 256), dtype=torch.float16, device="cuda")
+    k = torch.zeros((1, 64, 256), dtype=torch.float16, device="cuda")
+    v = torch.zeros((1, 64, 64), dtype=torch.float16, device="cuda")
+    with pytest.raises(_lib.VSparseError):     # d_qk > 128: use the three-operator chain
+        ops.sparse_attention(4, 8, 64, prob.row_indices, prob.row_offsets, prob.column_indices, q, k, v)

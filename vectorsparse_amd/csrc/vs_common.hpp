@@ -148,6 +148,8 @@ struct Options {
     int spmm_waves = 0;
     int spmm_cols_per_lane = 0;
     int sddmm_slots = 0;
+    int attention_waves = 0;
+    int attention_chunk = 0;
 };
 Options &options();
 
@@ -189,6 +191,10 @@ int launch_spmm_softmax_mfma(int m_vec, int vec_length, int k, int n, const int 
                              const int *row_offsets, const int *column_indices, const half_t *scores,
                              const half_t *rhs, half_t *out, float scale, hipStream_t stream,
                              const Batch &batch = Batch());
+int launch_sparse_attention(int m_vec, int vec_length, int d_qk, int d_v, const int *row_indices,
+                            const int *row_offsets, const int *col_indices, const half_t *q, const half_t *k,
+                            const half_t *v, half_t *out, float scale, hipStream_t stream, const Batch &batch,
+                            long long stride_v);
 int launch_sparse_softmax(int m_vec, int vec_length, const int *row_indices, const int *row_offsets,
                           const half_t *values_in, half_t *values_out, float scale, hipStream_t stream,
                           const Batch &batch = Batch());

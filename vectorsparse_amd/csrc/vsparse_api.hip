@@ -276,6 +276,25 @@ int vs_wmma_spmm_softmax_f16_batched(int batch, int m_vec, int vec_length, int k
                                         make_batch(batch, stride_scores, stride_rhs, stride_output));
 }
 
+int vs_sparse_attention_f16(int batch, int m_vec, int vec_length, int n, int d_qk, int d_v, const int *row_indices,
+                            const int *row_offsets, const int *col_indices, const void *q, long long stride_q,
+                            const void *k, long long stride_k, const void *v, long long stride_v, void *out,
+                            long long stride_out, float scale, void *stream)
+{
+    if (batch < 0 || m_vec < 0 || n < 0 || d_qk < 0 || d_v < 0 || !vec_ok(vec_length)) return VS_ERROR_INVALID_VALUE;
+    if (batch == 0 || m_vec == 0 || d_v == 0) return VS_SUCCESS;
+    if (!row_indices || !row_offsets || !q || !out) return VS_ERROR_INVALID_VALUE;
+    if (n > 0 && (!k || !v)) return VS_ERROR_INVALID_VALUE;
+    if (!aligned(q, 16) || !aligned(k, 16) || !aligned(v, 16) || !aligned(out, 16)) return VS_ERROR_INVALID_VALUE;
+    if (!stride_ok(stride_q, 8) || !stride_ok(stride_k, 8) || !stride_ok(stride_v, 8) || !stride_ok(stride_out, 8))
+        return VS_ERROR_INVALID_VALUE;
+    return vs::launch_sparse_attention(m_vec, vec_length, d_qk, d_v, row_indices, row_offsets, col_indices,
+                                       static_cast<const half_t *>(q), static_cast<const half_t *>(k),
+                                       static_cast<const half_t *>(v), static_cast<half_t *>(out), scale,
+                                       static_cast<hipStream_t>(stream), make_batch(batch, stride_q, stride_k, stride_out),
+                                       stride_v);
+}
+
 int vs_sparse_softmax_f16(int batch, int m_vec, int vec_length, const int *row_indices, const int *row_offsets,
                           const void *values_in, long long stride_in, void *values_out, long long stride_out,
                           float scale, void *stream)
@@ -321,6 +340,11 @@ int vs_set_option(const char *name, int value)
         o.spmm_cols_per_lane = value;
     } else if (std::strcmp(name, "sddmm_slots") == 0) {
         o.sddmm_slots = value;
+    } else if (std::strcmp(name, "attention_waves") == 0) {
+        if (value > 8) return VS_ERROR_INVALID_VALUE;
+        o.attention_waves = value;
+    } else if (std::strcmp(name, "attention_chunk") == 0) {
+        o.attention_chunk = value;
     } else {
         return VS_ERROR_INVALID_VALUE;
     }

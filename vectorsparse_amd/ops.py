@@ -152,6 +152,32 @@ def spmm_softmax_batched(m_vec, vec_length, k, n, row_indices, row_offsets, colu
     return output_matrix
 
 
+def sparse_attention(m_vec, vec_length, n, row_indices, row_offsets, col_indices, q, k, v, out=None, scale=None,
+                     stream=None):
+    """Single-launch fixed-mask attention: out = softmax(scale * mask(q k^T)) v.
+
+    q: [heads, m, d_qk], k: [heads, n, d_qk], v: [heads, n, d_v] (or 2-D for one head), fp16.
+    """
+    if q.dim() == 2:
+        q, k, v = q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0)
+        if out is not None:
+            out = out.unsqueeze(0)
+    heads, m, d_qk = q.shape
+    d_v = v.shape[2]
+    if scale is None:
+        scale = 1.0 / float(d_qk) ** 0.5
+    if out is None:
+        out = torch.empty((heads, m, d_v), dtype=torch.float16, device=q.device)
+    for t, nm in ((q, "q"), (k, "k"), (v, "v"), (out, "out")):
+        _expect_batched(t, torch.float16, nm)
+    st = _lib.lib().vs_sparse_attention_f16(heads, m_vec, vec_length, n, d_qk, d_v, _ptr(row_indices),
+                                            _ptr(row_offsets), _ptr(col_indices), _ptr(q), _stride(q, heads),
+                                            _ptr(k), _stride(k, heads), _ptr(v), _stride(v, heads), _ptr(out),
+                                            _stride(out, heads), float(scale), _stream(stream))
+    _lib.check(st, "vs_sparse_attention_f16")
+    return out
+
+
 def sddmm_batched(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices, lhs_matrix, rhs_matrix,
                   output_values, vec_length, kernel="wmma", stream=None, algorithm=1):
     """`batch` SDDMMs sharing one mask in one launch.
@@ -212,8 +238,9 @@ class SparseAttention:
     def forward(self, q, k, v, scale=None, kernel="wmma", stream=None, scores=None, out=None, fused=None):
         """q, k, v: fp16 [heads, seq, d] on the device.  Returns fp16 [heads, seq, d].
 
-        fused (default: True on the MFMA path) folds the softmax into the SpMM launch, so the layer is
-        two launches and the probabilities never go to memory.
+        fused: "layer" (default on the MFMA path) runs the whole layer in one launch with scores and
+        probabilities kept in LDS; True folds only the softmax into the SpMM launch (two launches, raw
+        scores go through memory); False runs the three operators one after the other.
         """
         p = self.prob
         heads, seq, d = q.shape
@@ -223,10 +250,13 @@ class SparseAttention:
             scores = torch.empty((heads, p.nnz_vec, p.vec_length), dtype=torch.float16, device=q.device)
         if out is None:
             out = torch.empty((heads, seq, v.shape[2]), dtype=torch.float16, device=q.device)
+        if fused is None:
+            fused = "layer" if kernel == "wmma" else False
+        if fused == "layer":
+            return sparse_attention(p.m_vec, p.vec_length, p.n, p.row_indices, p.row_offsets, p.column_indices,
+                                    q, k, v, out=out, scale=scale, stream=stream)
         sddmm_batched(p.m_vec, d, p.n, p.nnz_vec, p.row_indices, p.row_offsets, p.column_indices, q, k, scores,
                       p.vec_length, kernel=kernel, stream=stream)
-        if fused is None:
-            fused = kernel == "wmma"
         if fused:
             return spmm_softmax_batched(p.m_vec, p.vec_length, v.shape[2], p.n, p.row_indices, p.row_offsets,
                                         p.column_indices, scores, v, out, scale, stream=stream)
