@@ -77,7 +77,7 @@ constexpr int stage_bytes()
 // SOFTMAX: the sparse values are raw scores and the kernel multiplies by softmax_row(scale * values)
 // instead: a pre-pass finds each scalar row's maximum, the staging step turns every score into
 // exp2(s*x - max) (and sums them), and the accumulated tile is divided by the row sum at the end.
-template <int V, int CPL, bool SOFTMAX, typename OutT>
+template <int V, int CPL, bool SOFTMAX, bool IDX32, typename OutT>
 __global__ void __launch_bounds__(1024)
 spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
                  const int *__restrict__ row_offsets, const int *__restrict__ column_indices,
@@ -103,7 +103,7 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
     const int g = lane >> 4;
     const int col0 = tile * TN + cs * CPL;
     const bool col_ok = col0 < n_cols;  // n_cols % CPL == 0: a lane's chunk is all in or all out
-    const half_t *rhs_col = rhs + (col_ok ? col0 : 0);
+    const uint32_t col_off = col_ok ? col0 : 0;
 
     int *idx_s = reinterpret_cast<int *>(smem + (size_t)wave * kStage);
     half_t *vec_s = reinterpret_cast<half_t *>(idx_s + kStep);  // [V][kStep]
@@ -138,21 +138,37 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
     int active = (steps + 1) >> 1;
     active = active < 1 ? 1 : (active > n_waves ? n_waves : active);
 
-    for (int base = beg + kStep * wave; wave < active && base < end; base += kStep * active) {
+    // The column index and the vector of the NEXT step are fetched into registers while the gathered
+    // rows of the current step are in flight, so a wave pays one memory round trip per step, not two.
+    const int stride = kStep * active;
+    int base = beg + kStep * wave;
+    const bool has_work = wave < active && base < end;
+    int next_idx = 0;
+    bool next_valid = false;
+    half_t next_vec[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) next_vec[v] = (half_t)0.f;
+    auto fetch = [&](int b) {
         if (lane < kStep) {
-            const int j = base + lane;
-            const bool valid = j < end;
+            const int j = b + lane;
+            next_valid = j < end;
             // Slots past the row's end repeat its last vector with a zero value: the gather stays
             // in bounds and contributes nothing.
-            const int jc = valid ? j : end - 1;
-            idx_s[lane] = column_indices[jc];
-            half_t av[V];
-            load_vector<V>(av, values + (size_t)jc * V);
+            const int jc = next_valid ? j : end - 1;
+            next_idx = column_indices[jc];
+            load_vector<V>(next_vec, values + (size_t)jc * V);
+        }
+    };
+    if (has_work) fetch(base);
+
+    for (; has_work && base < end; base += stride) {
+        if (lane < kStep) {
+            idx_s[lane] = next_idx;
 #pragma unroll
             for (int v = 0; v < V; ++v) {
-                half_t staged = valid ? av[v] : (half_t)0.f;
+                half_t staged = next_valid ? next_vec[v] : (half_t)0.f;
                 if constexpr (SOFTMAX) {
-                    const float p = valid ? __builtin_amdgcn_exp2f((float)av[v] * s2 - row_max[v]) : 0.f;
+                    const float p = next_valid ? __builtin_amdgcn_exp2f((float)next_vec[v] * s2 - row_max[v]) : 0.f;
                     row_sum[v] += p;
                     staged = (half_t)p;
                 }
@@ -170,8 +186,14 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const int col = e < 4 ? i_lo[e] : i_hi[e - 4];
-            chunk[e].load(rhs_col + (size_t)col * n_cols);
+            if constexpr (IDX32) {
+                // rhs has fewer than 2^31 elements: 32-bit offsets from a uniform base
+                chunk[e].load(rhs + ((uint32_t)col * (uint32_t)n_cols + col_off));
+            } else {
+                chunk[e].load(rhs + ((size_t)col * n_cols + col_off));
+            }
         }
+        if (base + stride < end) fetch(base + stride);
 #pragma unroll
         for (int p = 0; p < CPL / 2; ++p) {
             uint4_t even, odd;
@@ -273,8 +295,8 @@ static int next_pow2(int x)
     return p;
 }
 
-template <int V, int CPL, bool SOFTMAX, typename OutT>
-static int launch_one(int m_vec, int k, int n, int waves, const int *row_indices, const int *row_offsets,
+template <int V, int CPL, bool SOFTMAX, bool IDX32, typename OutT>
+static int launch_idx(int m_vec, int k, int n, int waves, const int *row_indices, const int *row_offsets,
                       const int *column_indices, const half_t *values, const half_t *rhs, OutT *out,
                       hipStream_t stream, const Batch &batch, float scale)
 {
@@ -285,7 +307,7 @@ static int launch_one(int m_vec, int k, int n, int waves, const int *row_indices
     if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
     const size_t lds = (size_t)waves * stage_bytes<V>() +
                        (waves > 1 ? (size_t)waves * V * (TN + 1) * sizeof(float) : 0);
-    auto kernel = spmm_mfma_kernel<V, CPL, SOFTMAX, OutT>;
+    auto kernel = spmm_mfma_kernel<V, CPL, SOFTMAX, IDX32, OutT>;
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
     if (attr != hipSuccess) return (int)attr;
@@ -293,6 +315,18 @@ static int launch_one(int m_vec, int k, int n, int waves, const int *row_indices
                        k, n_tiles, row_indices, row_offsets, column_indices, values, rhs, out,
                        batch.stride_a, batch.stride_b, batch.stride_out, scale);
     return (int)hipGetLastError();
+}
+
+template <int V, int CPL, bool SOFTMAX, typename OutT>
+static int launch_one(int m_vec, int k, int n, int waves, const int *row_indices, const int *row_offsets,
+                      const int *column_indices, const half_t *values, const half_t *rhs, OutT *out,
+                      hipStream_t stream, const Batch &batch, float scale)
+{
+    if ((long long)n * k < (1LL << 31))
+        return launch_idx<V, CPL, SOFTMAX, true, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices,
+                                                        values, rhs, out, stream, batch, scale);
+    return launch_idx<V, CPL, SOFTMAX, false, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices,
+                                                     values, rhs, out, stream, batch, scale);
 }
 
 template <int CPL, bool SOFTMAX, typename OutT>
