@@ -84,17 +84,27 @@ sddmm_mfma_kernel(int m_vec, int K, int slots, const int *__restrict__ row_indic
         half8_t a[KS];
 #pragma unroll
         for (int kk = 0; kk < KS; ++kk) a[kk] = to_mfma_order(load_slice16(lhs_row, kk, q, K, a_row_ok), src);
+        // the column indices of the next super-group are fetched while this one's rows are in flight
+        int col[GRP];
+        auto fetch = [&](int sg) {
+#pragma unroll
+            for (int u = 0; u < GRP; ++u) {
+                const int jl = beg + SUPER * sg + 16 * u + r;
+                // slots past the row's end gather its last vector (in bounds); their results are dropped
+                col[u] = col_indices[jl < end ? jl : end - 1];
+            }
+        };
+        fetch(s);
         for (int sg = s; sg < n_super; sg += slots) {
             const int j0 = beg + SUPER * sg;
             uint4_t raw[GRP][KS];
 #pragma unroll
             for (int u = 0; u < GRP; ++u) {
-                const int jl = j0 + 16 * u + r;
-                // slots past the row's end gather its last vector (in bounds); their results are dropped
-                const half_t *rhs_row = rhs + (size_t)col_indices[jl < end ? jl : end - 1] * K;
+                const half_t *rhs_row = rhs + (size_t)col[u] * K;
 #pragma unroll
                 for (int kk = 0; kk < KS; ++kk) raw[u][kk] = load_slice16(rhs_row, kk, q, K, true);
             }
+            if (sg + slots < n_super) fetch(sg + slots);
 #pragma unroll
             for (int u = 0; u < GRP; ++u) {
                 float4_t acc = {0.f, 0.f, 0.f, 0.f};
