@@ -1,0 +1,69 @@
+"""Randomised differential parity: many small random shapes, every kernel path, against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle as co
+from vectorsparse_amd import ops
+from vectorsparse_amd import colvec_csr as cv
+from util import assert_parity
+
+pytestmark = pytest.mark.gpu
+
+
+def _random_pattern(rng, V):
+    m_vec = int(rng.integers(1, 70))
+    n = int(rng.integers(1, 700))
+    kind = rng.integers(0, 4)
+    if kind == 0:      # uniform density
+        lengths = rng.binomial(n, rng.uniform(0.02, 0.6), size=m_vec)
+    elif kind == 1:    # heavy tail
+        lengths = np.minimum((rng.pareto(1.2, m_vec) + 0.1) * n * 0.05, n).astype(np.int64)
+    elif kind == 2:    # many empty rows
+        lengths = np.where(rng.random(m_vec) < 0.6, 0, rng.integers(1, n + 1, m_vec))
+    else:              # dense rows
+        lengths = np.full(m_vec, n)
+    ro, ci = cv._pattern_from_lengths(rng, m_vec, n, lengths.astype(np.int64))
+    return cv.ColVecCSR(m_vec, n, V, ro, ci).validate()
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_spmm_random(gpu, seed):
+    rng = np.random.default_rng(1000 + seed)
+    V = int(rng.choice([1, 2, 4, 8]))
+    pat = cv.random_values(_random_pattern(rng, V), seed=seed)
+    N = int(rng.choice([4, 8, 16, 40, 64, 96, 128, 200, 256, 264, 384, 520]))
+    B = cv.dense_uniform(pat.n, N, seed=seed + 1)
+    ref = co.spmm_host_ref_f32(pat.m_vec, V, N, pat.n, pat.row_offsets, pat.column_indices, pat.values, B)
+    prob = ops.DeviceProblem(pat, sort=bool(seed % 2))
+    Bd = torch.from_numpy(B).cuda()
+    what = "seed %d V%d m_vec%d n%d N%d nnz_vec%d" % (seed, V, pat.m_vec, pat.n, N, pat.nnz_vec)
+    print(what, flush=True)
+    assert_parity(prob.spmm(Bd, kernel="wmma").cpu().numpy(), ref, "wmma " + what)
+    if N % 8 == 0:
+        assert_parity(prob.spmm(Bd, kernel="cuda").cpu().numpy(), ref, "cuda " + what)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_sddmm_random(gpu, seed):
+    rng = np.random.default_rng(2000 + seed)
+    V = int(rng.choice([1, 2, 4, 8]))
+    pat = _random_pattern(rng, V)
+    K = int(rng.choice([8, 16, 24, 32, 40, 64, 96, 128, 136, 256, 264, 520]))
+    A = cv.dense_normal(pat.m, K, seed=seed + 1)
+    B = cv.dense_normal(pat.n, K, seed=seed + 2)
+    ref = co.sddmm_host_ref_f32(pat.m_vec, K, V, pat.row_offsets, pat.column_indices, A, B)
+    prob = ops.DeviceProblem(pat, sort=bool(seed % 2))
+    Ad, Bd = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+    what = "seed %d V%d m_vec%d n%d K%d nnz_vec%d" % (seed, V, pat.m_vec, pat.n, K, pat.nnz_vec)
+    print(what, flush=True)
+    for kernel in ("wmma", "cuda"):
+        got = prob.sddmm(Ad, Bd, kernel=kernel).cpu().numpy().reshape(-1)
+        assert_parity(got, ref, kernel + " " + what)
+    if seed % 4 == 0:       # the cross-lane path with a contraction length that is not a multiple of 8
+        K2 = K + int(rng.integers(1, 8))
+        A2 = cv.dense_normal(pat.m, K2, seed=seed + 3)
+        B2 = cv.dense_normal(pat.n, K2, seed=seed + 4)
+        ref2 = co.sddmm_host_ref_f32(pat.m_vec, K2, V, pat.row_offsets, pat.column_indices, A2, B2)
+        got = prob.sddmm(torch.from_numpy(A2).cuda(), torch.from_numpy(B2).cuda(), kernel="cuda")
+        assert_parity(got.cpu().numpy().reshape(-1), ref2, "cuda K%d " % K2 + what)
