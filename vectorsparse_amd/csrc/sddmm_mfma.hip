@@ -51,7 +51,7 @@ __device__ __forceinline__ uint4_t load_slice16(const half_t *row, int kk, int q
 
 // KS > 0: K <= 32*KS, lhs slices preloaded; KS == 0: any K % 8 == 0, lhs re-read per super-group.
 template <int V, int KS, int GRP, typename OutT>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 sddmm_mfma_kernel(int m_vec, int K, int slots, const int *__restrict__ row_indices,
                   const int *__restrict__ row_offsets, const int *__restrict__ col_indices,
                   const half_t *__restrict__ lhs, const half_t *__restrict__ rhs, OutT *__restrict__ out,
@@ -150,7 +150,7 @@ static int launch_one(int m_vec, int k, int nonzeros_vec, const int *row_indices
                       const int *col_indices, const half_t *lhs, const half_t *rhs, OutT *out, hipStream_t stream,
                       const Batch &batch)
 {
-    constexpr int kWavesPerBlock = 4;
+    const int kWavesPerBlock = options().sddmm_block_waves > 0 ? options().sddmm_block_waves : 8;
     const int slots = sddmm_auto_slots(m_vec * batch.count, nonzeros_vec * batch.count, 16 * GRP);
     const long long waves = (long long)m_vec * slots;
     const long long blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
@@ -173,8 +173,11 @@ static int launch_ks(int m_vec, int k, int nonzeros_vec, const int *row_indices,
     return launch_one<V, 0, 4, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
 }
 
-// Waves per vector row: enough waves to fill the chip, at most one per super-group of an average row
-// (longer rows loop).
+// Waves per vector row.  Waves are independent (no reduction): twice as many as an average row has
+// super-groups, so that a row twice the average still gets one super-group per wave (longer rows loop),
+// capped so that the launch stays near the number of wave slots of the chip.  A wave that finds no
+// super-group of its own exits after two scalar loads; what it costs is its share of a workgroup
+// dispatch, which is why workgroups are eight waves wide.
 int sddmm_auto_slots(int m_vec, int nonzeros_vec, int group)
 {
     int slots = options().sddmm_slots;
@@ -182,7 +185,7 @@ int sddmm_auto_slots(int m_vec, int nonzeros_vec, int group)
     const long long avg = ((long long)nonzeros_vec + m_vec - 1) / (m_vec > 0 ? m_vec : 1);
     const int avg_groups = (int)((avg + group - 1) / group);
     const int want = ceil_div(8192, m_vec > 0 ? m_vec : 1);
-    slots = avg_groups < want ? avg_groups : want;
+    slots = 2 * avg_groups < want ? 2 * avg_groups : want;
     return slots < 1 ? 1 : slots;
 }
 

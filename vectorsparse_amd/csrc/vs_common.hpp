@@ -148,6 +148,7 @@ struct Options {
     int spmm_waves = 0;
     int spmm_cols_per_lane = 0;
     int sddmm_slots = 0;
+    int sddmm_block_waves = 0;
     int attention_waves = 0;
     int attention_chunk = 0;
 };

@@ -340,6 +340,9 @@ int vs_set_option(const char *name, int value)
         o.spmm_cols_per_lane = value;
     } else if (std::strcmp(name, "sddmm_slots") == 0) {
         o.sddmm_slots = value;
+    } else if (std::strcmp(name, "sddmm_block_waves") == 0) {
+        if (value > 16) return VS_ERROR_INVALID_VALUE;
+        o.sddmm_block_waves = value;
     } else if (std::strcmp(name, "attention_waves") == 0) {
         if (value > 8) return VS_ERROR_INVALID_VALUE;
         o.attention_waves = value;
