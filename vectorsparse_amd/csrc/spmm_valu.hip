@@ -7,11 +7,31 @@
 // 1e-2 relative-error budget against the host loop on near-zero outputs, so it is not
 // reproduced.  Work item = (vector row, tile of TN = 8*LR dense columns); a wave is G = 64/LR groups
 // of LR lanes, each group walks its own nonzero vectors and every lane owns 8 consecutive
-// columns (one 128-bit load per gathered row).  The W*G partial tiles are summed through LDS
-// in a fixed order.
+// columns (one 128-bit load per gathered row, four rows in flight per lane).  The W*G partial tiles
+// are summed through LDS in a fixed order.
 #include "vs_common.hpp"
 
 namespace vs {
+
+template <int V>
+__device__ __forceinline__ void load_values(half_t (&dst)[V], const half_t *p)
+{
+    if constexpr (V == 8) {
+        const half8_t t = *reinterpret_cast<const half8_t *>(p);
+#pragma unroll
+        for (int v = 0; v < 8; ++v) dst[v] = t[v];
+    } else if constexpr (V == 4) {
+        const half4_t t = *reinterpret_cast<const half4_t *>(p);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) dst[v] = t[v];
+    } else if constexpr (V == 2) {
+        const half2_t t = *reinterpret_cast<const half2_t *>(p);
+        dst[0] = t[0];
+        dst[1] = t[1];
+    } else {
+        dst[0] = p[0];
+    }
+}
 
 template <int V, int LR, typename OutT>
 __global__ void __launch_bounds__(1024)
@@ -46,29 +66,33 @@ spmm_valu_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
 #pragma unroll
         for (int c = 0; c < 8; ++c) acc[v][c] = 0.f;
 
-    for (int j = beg + wave * G + g; j < end; j += n_waves * G) {
-        const int col = column_indices[j];
-        half_t a[V];
-        if constexpr (V == 8) {
-            const half8_t t = *reinterpret_cast<const half8_t *>(values + (size_t)j * 8);
+    // U nonzero vectors per group and iteration, so that U gathered rows are in flight per lane
+    constexpr int U = 4;
+    for (int j0 = beg + (wave * G + g) * U; j0 < end; j0 += n_waves * G * U) {
+        int col[U];
+        half_t a[U][V];
 #pragma unroll
-            for (int v = 0; v < 8; ++v) a[v] = t[v];
-        } else if constexpr (V == 4) {
-            const half4_t t = *reinterpret_cast<const half4_t *>(values + (size_t)j * 4);
+        for (int u = 0; u < U; ++u) {
+            const int j = j0 + u;
+            const bool valid = j < end;
+            const int jc = valid ? j : end - 1;  // padded slots repeat the last vector with zero values
+            col[u] = column_indices[jc];
+            load_values<V>(a[u], values + (size_t)jc * V);
+            if (!valid) {
 #pragma unroll
-            for (int v = 0; v < 4; ++v) a[v] = t[v];
-        } else if constexpr (V == 2) {
-            const half2_t t = *reinterpret_cast<const half2_t *>(values + (size_t)j * 2);
-            a[0] = t[0];
-            a[1] = t[1];
-        } else {
-            a[0] = values[j];
+                for (int v = 0; v < V; ++v) a[u][v] = (half_t)0.f;
+            }
         }
-        const half8_t b = *reinterpret_cast<const half8_t *>(rhs_col + (size_t)col * n_cols);
+        half8_t b[U];
 #pragma unroll
-        for (int v = 0; v < V; ++v) {
+        for (int u = 0; u < U; ++u) b[u] = *reinterpret_cast<const half8_t *>(rhs_col + (size_t)col[u] * n_cols);
 #pragma unroll
-            for (int c = 0; c < 8; ++c) acc[v][c] = __builtin_fmaf((float)a[v], (float)b[c], acc[v][c]);
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+#pragma unroll
+                for (int c = 0; c < 8; ++c) acc[v][c] = __builtin_fmaf((float)a[u][v], (float)b[u][c], acc[v][c]);
+            }
         }
     }
 
@@ -153,8 +177,8 @@ int launch_spmm_valu(int m_vec, int vec_length, int k, int n, const int *row_ind
     int waves = options().spmm_waves;
     if (waves <= 0) {
         const long long blocks = (long long)m_vec * ceil_div(k, 512) * batch.count;
-        waves = 1;
-        while (waves < 8 && blocks * waves < 2048) waves <<= 1;
+        waves = 2;
+        while (waves < 8 && blocks * waves < 8192) waves <<= 1;
     }
     if (waves > 16) waves = 16;
     switch (vec_length) {
