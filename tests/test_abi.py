@@ -89,3 +89,33 @@ def test_options():
         _lib.set_option("no_such_option", 1)
     with pytest.raises(_lib.VSparseError):
         _lib.set_option("spmm_cols_per_lane", 3)
+
+
+def test_header_is_plain_c_and_cxx(tmp_path):
+    """include/vsparse.h compiles as C99 and as C++ with nothing but itself."""
+    import subprocess
+    src_c = tmp_path / "use.c"
+    src_c.write_text('#include "vsparse.h"\nint main(void) { return vs_version() > 0 ? 0 : 1; }\n')
+    subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic", "-fsyntax-only",
+                           "-I", os.path.join(ROOT, "include"), str(src_c)])
+    src_cpp = tmp_path / "use.cpp"
+    src_cpp.write_text('#include "vsparse.h"\nint main() { return vs_version() > 0 ? 0 : 1; }\n')
+    subprocess.check_call(["g++", "-std=c++17", "-Wall", "-Werror", "-fsyntax-only",
+                           "-I", os.path.join(ROOT, "include"), str(src_cpp)])
+
+
+def test_reference_side_shim_compiles(tmp_path):
+    """The C++ binding shown in INTEGRATION.md (same namespaces and signatures as the reference's
+    operator headers) is valid against the header: extracted from the document and syntax-checked."""
+    import subprocess
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    start = text.index("```cpp") + len("```cpp")
+    shim = text[start:text.index("```", start)]
+    assert "namespace spmm" in shim and "namespace sddmm" in shim
+    src = tmp_path / "vsparse_shim.cpp"
+    src.write_text(shim)
+    hipcc = "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc not installed")
+    subprocess.check_call([hipcc, "-x", "hip", "--offload-arch=gfx950", "-std=c++17", "-fsyntax-only",
+                           "-I", os.path.join(ROOT, "include"), str(src)])
