@@ -231,7 +231,11 @@ void vs_sorted_row_swizzle(int rows, const int *row_offsets, int *row_indices);
  * launches).  Names: "spmm_waves" (waves per workgroup, 0 = automatic),
  * "spmm_cols_per_lane" (4, 8, 0 = automatic), "sddmm_slots" (waves per
  * vector row, 0 = automatic), "sddmm_block_waves" (1..16, 0 = automatic), "attention_waves" (1..8, 0 = automatic),
- * "attention_chunk" (nonzero vectors per LDS chunk, 0 = automatic).  Returns 0, or 1 for an unknown name / bad value.
+ * "attention_chunk" (nonzero vectors per LDS chunk, 0 = automatic),
+ * "attention_rows" (0 or 1: one vector row per workgroup, gathers from memory;
+ * 2..8: that many consecutive vector rows per workgroup with the K / V rows they
+ * share gathered once into LDS - faster when neighbouring rows share most of
+ * their columns, e.g. banded masks, slower on random masks).  Returns 0, or 1 for an unknown name / bad value.
  * No counterpart in the reference, whose tile sizes are compile-time constants
  * (src/wmma_spmm.cu:396).
  */

@@ -214,9 +214,12 @@ def test_single_launch_attention(gpu, V, dims):
     ref = _dense_attention(mask, q, k, v, scale)
     qd, kd, vd = (torch.from_numpy(x).cuda() for x in (q, k, v))
     try:
-        for chunk, waves in ((0, 0), (64, 3), (32, 8), (96, 1)):      # one chunk / several chunks per long row
+        # (chunk, waves, rows per workgroup): one chunk / several chunks per long row; rows = 1 is the
+        # one-row-per-workgroup kernel, anything else the union-gather kernel (LDS copy or global fallback)
+        for chunk, waves, rows in ((0, 0, 1), (64, 3, 1), (32, 8, 1), (96, 1, 0), (0, 0, 8), (64, 0, 3), (32, 0, 16)):
             _lib_set("attention_chunk", chunk)
             _lib_set("attention_waves", waves)
+            _lib_set("attention_rows", rows)
             pad = torch.full((heads, mask.m + 16, d_v), 3.0, dtype=torch.float16, device="cuda")
             out = pad[:, 8:8 + mask.m]
             ops.sparse_attention(mask.m_vec, V, n, prob.row_indices, prob.row_offsets, prob.column_indices,
@@ -224,12 +227,42 @@ def test_single_launch_attention(gpu, V, dims):
             torch.cuda.synchronize()
             host = pad.cpu().numpy()
             assert np.all(host[:, :8] == 3.0) and np.all(host[:, 8 + mask.m:] == 3.0), "wrote outside the output"
-            _check_layer(host[:, 8:8 + mask.m], ref, "V%d dqk%d dv%d chunk%d waves%d" % (V, d_qk, d_v, chunk, waves))
+            _check_layer(host[:, 8:8 + mask.m], ref,
+                         "V%d dqk%d dv%d chunk%d waves%d rows%d" % (V, d_qk, d_v, chunk, waves, rows))
             for i in np.nonzero(lengths == 0)[0]:
                 assert not host[:, 8 + i * V:8 + (i + 1) * V].any(), "an empty row must produce zeros"
     finally:
         _lib_set("attention_chunk", 0)
         _lib_set("attention_waves", 0)
+        _lib_set("attention_rows", 0)
+
+
+@pytest.mark.parametrize("V", [2, 8])
+def test_union_gather_on_structured_and_random_masks(gpu, V):
+    heads, seq, d = 2, 1024, 64
+    rng = np.random.default_rng(V)
+    q, k, v = (rng.standard_normal((heads, seq, d)).astype(np.float16) for _ in range(3))
+    qd, kd, vd = (torch.from_numpy(x).cuda() for x in (q, k, v))
+    masks = {
+        "band": cv.band_strided_pattern(seq, V, band_half_width=64, stride=128),     # union fits LDS
+        "random": cv.uniform_pattern(seq // V, seq, 0.7, seed=3, vec_length=V),      # union too large: fallback
+    }
+    try:
+        for name, mask in masks.items():
+            prob = ops.DeviceProblem(mask)
+            ref = _dense_attention(mask, q, k, v, 0.125)
+            outs = {}
+            for rows in (1, 4, 8, 32):
+                _lib_set("attention_rows", rows)
+                out = ops.sparse_attention(mask.m_vec, V, seq, prob.row_indices, prob.row_offsets,
+                                           prob.column_indices, qd, kd, vd, scale=0.125)
+                torch.cuda.synchronize()
+                outs[rows] = out.cpu().numpy()
+                _check_layer(outs[rows], ref, "%s mask V%d rows%d" % (name, V, rows))
+            # same arithmetic in the same order whatever the source of the gathered rows
+            assert np.array_equal(outs[4], outs[8]) and np.array_equal(outs[8], outs[32])
+    finally:
+        _lib_set("attention_rows", 0)
 
 
 def _lib_set(name, value):

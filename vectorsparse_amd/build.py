@@ -10,7 +10,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_HERE, "libvsparse.so")
 SOURCES = ["vsparse_api.hip", "spmm_mfma.hip", "spmm_valu.hip", "sddmm_mfma.hip", "sddmm_valu.hip",
-           "sparse_softmax.hip", "sparse_attention.hip"]
+           "sparse_softmax.hip", "sparse_attention.hip",
+           "sparse_attention_union.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared",

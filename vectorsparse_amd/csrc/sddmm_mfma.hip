@@ -31,24 +31,6 @@ __device__ __forceinline__ void store_group(OutT *out, int j, int g, const float
     }
 }
 
-// Row-major lane order -> MFMA lane order: lane (c, g) takes the registers of lane 4c + g.
-__device__ __forceinline__ half8_t to_mfma_order(const uint4_t &x, int src_lane_bytes)
-{
-    uint4_t y;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) y[i] = (uint32_t)__builtin_amdgcn_ds_bpermute(src_lane_bytes, (int)x[i]);
-    return __builtin_bit_cast(half8_t, y);
-}
-
-// Slice q (8 halves at k = 32*kk + 8q) of `row`, zero past K.
-__device__ __forceinline__ uint4_t load_slice16(const half_t *row, int kk, int q, int K, bool ok)
-{
-    const int off = 32 * kk + 8 * q;
-    uint4_t x = {0u, 0u, 0u, 0u};
-    if (ok && off < K) x = *reinterpret_cast<const uint4_t *>(row + off);
-    return x;
-}
-
 // KS > 0: K <= 32*KS, lhs slices preloaded; KS == 0: any K % 8 == 0, lhs re-read per super-group.
 template <int V, int KS, int GRP, typename OutT>
 __global__ void __launch_bounds__(1024)

@@ -20,41 +20,6 @@
 
 namespace vs {
 
-namespace {
-
-template <int CPL>
-struct Chunk;
-template <>
-struct Chunk<8> {
-    uint4_t d;
-    __device__ __forceinline__ void load(const half_t *p) { d = *reinterpret_cast<const uint4_t *>(p); }
-    __device__ __forceinline__ uint32_t dword(int i) const { return d[i]; }
-};
-template <>
-struct Chunk<4> {
-    uint2_t d;
-    __device__ __forceinline__ void load(const half_t *p) { d = *reinterpret_cast<const uint2_t *>(p); }
-    __device__ __forceinline__ uint32_t dword(int i) const { return d[i]; }
-};
-
-__device__ __forceinline__ half8_t relayout(const uint4_t &x, int src_lane_bytes)
-{
-    uint4_t y;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) y[i] = (uint32_t)__builtin_amdgcn_ds_bpermute(src_lane_bytes, (int)x[i]);
-    return __builtin_bit_cast(half8_t, y);
-}
-
-__device__ __forceinline__ uint4_t slice16(const half_t *row, int kk, int q, int d, bool ok)
-{
-    const int off = 32 * kk + 8 * q;
-    uint4_t x = {0u, 0u, 0u, 0u};
-    if (ok && off < d) x = *reinterpret_cast<const uint4_t *>(row + off);
-    return x;
-}
-
-}  // namespace
-
 // V: vector length; KS: d_qk <= 32*KS; CPL: d_v <= 16*CPL.
 template <int V, int KS, int CPL>
 __global__ void __launch_bounds__(512)
@@ -106,7 +71,7 @@ sparse_attention_kernel(int d_qk, int d_v, int chunk, const int *__restrict__ ro
         const bool ok = r < V;
         const half_t *q_row = q + ((size_t)row * V + (ok ? r : 0)) * d_qk;
 #pragma unroll
-        for (int kk = 0; kk < KS; ++kk) qa[kk] = relayout(slice16(q_row, kk, qs, d_qk, ok), src);
+        for (int kk = 0; kk < KS; ++kk) qa[kk] = to_mfma_order(load_slice16(q_row, kk, qs, d_qk, ok), src);
     }
 
     float4_t acc[CPL];
@@ -125,11 +90,11 @@ sparse_attention_kernel(int d_qk, int d_v, int chunk, const int *__restrict__ ro
             const half_t *k_row = k + (size_t)col_indices[c0 + (jl < len ? jl : len - 1)] * d_qk;
             uint4_t raw[KS];
 #pragma unroll
-            for (int kk = 0; kk < KS; ++kk) raw[kk] = slice16(k_row, kk, qs, d_qk, true);
+            for (int kk = 0; kk < KS; ++kk) raw[kk] = load_slice16(k_row, kk, qs, d_qk, true);
             float4_t s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int kk = 0; kk < KS; ++kk)
-                s = __builtin_amdgcn_mfma_f32_16x16x32_f16(qa[kk], relayout(raw[kk], src), s, 0, 0, 0);
+                s = __builtin_amdgcn_mfma_f32_16x16x32_f16(qa[kk], to_mfma_order(raw[kk], src), s, 0, 0, 0);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int vv = 4 * g + e;
@@ -177,7 +142,7 @@ sparse_attention_kernel(int d_qk, int d_v, int chunk, const int *__restrict__ ro
             const int4_t i_hi = *reinterpret_cast<const int4_t *>(idx + 32 * st + 8 * g + 4);
             half8_t a = {0, 0, 0, 0, 0, 0, 0, 0};
             if (c < V) a = *reinterpret_cast<const half8_t *>(pr + (size_t)c * chunk + 32 * st + 8 * g);
-            Chunk<CPL> rows[8];
+            RowChunk<CPL> rows[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const int col = e < 4 ? i_lo[e] : i_hi[e - 4];

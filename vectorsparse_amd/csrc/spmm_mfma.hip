@@ -22,21 +22,6 @@
 
 namespace vs {
 
-template <int CPL>
-struct RowChunk;
-template <>
-struct RowChunk<8> {
-    uint4_t d;
-    __device__ __forceinline__ void load(const half_t *p) { d = *reinterpret_cast<const uint4_t *>(p); }
-    __device__ __forceinline__ uint32_t dword(int i) const { return d[i]; }
-};
-template <>
-struct RowChunk<4> {
-    uint2_t d;
-    __device__ __forceinline__ void load(const half_t *p) { d = *reinterpret_cast<const uint2_t *>(p); }
-    __device__ __forceinline__ uint32_t dword(int i) const { return d[i]; }
-};
-
 // The V halves of one nonzero vector, fetched with one load.
 template <int V>
 __device__ __forceinline__ void load_vector(half_t (&dst)[V], const half_t *p)

@@ -62,6 +62,44 @@ __device__ __forceinline__ float partner(float x)
 }
 
 
+// CPL consecutive halves of one gathered row, fetched with one load (CPL = 8: 128 bits, 4: 64 bits).
+template <int CPL>
+struct RowChunk;
+template <>
+struct RowChunk<8> {
+    uint4_t d;
+    __device__ __forceinline__ void load(const half_t *p) { d = *reinterpret_cast<const uint4_t *>(p); }
+    __device__ __forceinline__ uint32_t dword(int i) const { return d[i]; }
+};
+template <>
+struct RowChunk<4> {
+    uint2_t d;
+    __device__ __forceinline__ void load(const half_t *p) { d = *reinterpret_cast<const uint2_t *>(p); }
+    __device__ __forceinline__ uint32_t dword(int i) const { return d[i]; }
+};
+
+// Row-major lane order -> MFMA lane order for a 16-row x 64-byte block: lane (c = lane % 16, g = lane / 16)
+// takes the four registers of lane 4c + g (`src_lane_bytes` = (4c + g) * 4) through the LDS crossbar.
+__device__ __forceinline__ half8_t to_mfma_order(const uint4_t &x, int src_lane_bytes)
+{
+    uint4_t y;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) y[i] = (uint32_t)__builtin_amdgcn_ds_bpermute(src_lane_bytes, (int)x[i]);
+    return __builtin_bit_cast(half8_t, y);
+}
+
+// Slice q (8 halves at k = 32*kk + 8q) of `row`, zero past K or when !ok.  Branch-free: a slice that
+// does not exist is read at offset 0 (always valid) and replaced by zeros, so the load can be
+// scheduled with its neighbours instead of sitting in its own exec-masked block.
+__device__ __forceinline__ uint4_t load_slice16(const half_t *row, int kk, int q, int K, bool ok)
+{
+    const int off = 32 * kk + 8 * q;
+    const bool take = ok && off < K;
+    const uint4_t x = *reinterpret_cast<const uint4_t *>(row + (take ? off : 0));
+    const uint4_t zero = {0u, 0u, 0u, 0u};
+    return take ? x : zero;
+}
+
 // All-lane max / sum over the 64 lanes of a wave (every lane must be active).
 __device__ __forceinline__ float wave_max(float x)
 {
@@ -151,6 +189,7 @@ struct Options {
     int sddmm_block_waves = 0;
     int attention_waves = 0;
     int attention_chunk = 0;
+    int attention_rows = 0;
 };
 Options &options();
 
@@ -196,6 +235,10 @@ int launch_sparse_attention(int m_vec, int vec_length, int d_qk, int d_v, const 
                             const int *row_offsets, const int *col_indices, const half_t *q, const half_t *k,
                             const half_t *v, half_t *out, float scale, hipStream_t stream, const Batch &batch,
                             long long stride_v);
+int launch_sparse_attention_union(int m_vec, int vec_length, int n, int d_qk, int d_v, const int *row_offsets,
+                                  const int *col_indices, const half_t *q, const half_t *k, const half_t *v,
+                                  half_t *out, float scale, hipStream_t stream, const Batch &batch,
+                                  long long stride_v);
 int launch_sparse_softmax(int m_vec, int vec_length, const int *row_indices, const int *row_offsets,
                           const half_t *values_in, half_t *values_out, float scale, hipStream_t stream,
                           const Batch &batch = Batch());

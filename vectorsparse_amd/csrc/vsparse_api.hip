@@ -288,6 +288,12 @@ int vs_sparse_attention_f16(int batch, int m_vec, int vec_length, int n, int d_q
     if (!aligned(q, 16) || !aligned(k, 16) || !aligned(v, 16) || !aligned(out, 16)) return VS_ERROR_INVALID_VALUE;
     if (!stride_ok(stride_q, 8) || !stride_ok(stride_k, 8) || !stride_ok(stride_v, 8) || !stride_ok(stride_out, 8))
         return VS_ERROR_INVALID_VALUE;
+    if (vs::options().attention_rows > 1)  // union-gather kernel: pays off when neighbouring rows share columns
+        return vs::launch_sparse_attention_union(m_vec, vec_length, n, d_qk, d_v, row_offsets, col_indices,
+                                                 static_cast<const half_t *>(q), static_cast<const half_t *>(k),
+                                                 static_cast<const half_t *>(v), static_cast<half_t *>(out), scale,
+                                                 static_cast<hipStream_t>(stream),
+                                                 make_batch(batch, stride_q, stride_k, stride_out), stride_v);
     return vs::launch_sparse_attention(m_vec, vec_length, d_qk, d_v, row_indices, row_offsets, col_indices,
                                        static_cast<const half_t *>(q), static_cast<const half_t *>(k),
                                        static_cast<const half_t *>(v), static_cast<half_t *>(out), scale,
@@ -348,6 +354,9 @@ int vs_set_option(const char *name, int value)
         o.attention_waves = value;
     } else if (std::strcmp(name, "attention_chunk") == 0) {
         o.attention_chunk = value;
+    } else if (std::strcmp(name, "attention_rows") == 0) {
+        if (value > 64) return VS_ERROR_INVALID_VALUE;
+        o.attention_rows = value;
     } else {
         return VS_ERROR_INVALID_VALUE;
     }

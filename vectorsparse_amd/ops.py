@@ -234,6 +234,21 @@ class SparseAttention:
 
     def __init__(self, mask, device="cuda", sort=True):
         self.prob = DeviceProblem(mask, sort=sort, device=device)
+        self.union_rows = self._union_rows(mask)
+
+    @staticmethod
+    def _union_rows(mask, rows=8, budget_rows=400, max_len=320):
+        """Rows per workgroup for the single-launch kernel: 8 when every block of 8 consecutive vector
+        rows touches few enough distinct columns for their K / V rows to sit in LDS (banded, blocky or
+        strided masks) and no row is too long for the register-resident scores, else 1."""
+        ro, ci = mask.row_offsets, mask.column_indices
+        if mask.m_vec == 0 or int(np.max(np.diff(ro))) > max_len:
+            return 1
+        for first in range(0, mask.m_vec, rows):
+            last = min(first + rows, mask.m_vec)
+            if np.unique(ci[ro[first]:ro[last]]).size > budget_rows:
+                return 1
+        return rows
 
     def forward(self, q, k, v, scale=None, kernel="wmma", stream=None, scores=None, out=None, fused=None):
         """q, k, v: fp16 [heads, seq, d] on the device.  Returns fp16 [heads, seq, d].
@@ -253,6 +268,7 @@ class SparseAttention:
         if fused is None:
             fused = "layer" if kernel == "wmma" else False
         if fused == "layer":
+            _lib.set_option("attention_rows", self.union_rows)
             return sparse_attention(p.m_vec, p.vec_length, p.n, p.row_indices, p.row_offsets, p.column_indices,
                                     q, k, v, out=out, scale=scale, stream=stream)
         sddmm_batched(p.m_vec, d, p.n, p.nnz_vec, p.row_indices, p.row_offsets, p.column_indices, q, k, scores,
