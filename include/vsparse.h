@@ -211,12 +211,17 @@ int vs_wmma_spmm_softmax_f16_batched(int batch, int m_vec, int vec_length, int k
  * multiples of 8 elements.  Empty rows produce zeros.  No counterpart in the reference (it links an
  * external sparse-transformer repository, README.md:76); same result as vs_wmma_sddmm_f16_batched ->
  * vs_sparse_softmax_f16 -> vs_wmma_spmm_f16_batched up to the fp16 rounding of the intermediates.
+ * rows_per_workgroup: 0 or 1 = one vector row per workgroup, K / V rows gathered from memory per row
+ * (any mask); 2..8 = that many consecutive vector rows per workgroup with the K / V rows they share
+ * gathered once into LDS - faster when neighbouring rows share most of their columns (banded, blocky,
+ * strided masks), slower on random masks, same results up to summation order; row_indices is then only
+ * validated, rows are taken in their natural order.
  */
 int vs_sparse_attention_f16(int batch, int m_vec, int vec_length, int n, int d_qk, int d_v,
                             const int *row_indices, const int *row_offsets, const int *col_indices,
                             const void *q, long long stride_q, const void *k, long long stride_k,
                             const void *v, long long stride_v, void *out, long long stride_out,
-                            float scale, void *stream);
+                            float scale, int rows_per_workgroup, void *stream);
 
 /*
  * Host helpers (HOST pointers).  Replace IdentityRowSwizzle / SortedRowSwizzle —
@@ -231,11 +236,7 @@ void vs_sorted_row_swizzle(int rows, const int *row_offsets, int *row_indices);
  * launches).  Names: "spmm_waves" (waves per workgroup, 0 = automatic),
  * "spmm_cols_per_lane" (4, 8, 0 = automatic), "sddmm_slots" (waves per
  * vector row, 0 = automatic), "sddmm_block_waves" (1..16, 0 = automatic), "attention_waves" (1..8, 0 = automatic),
- * "attention_chunk" (nonzero vectors per LDS chunk, 0 = automatic),
- * "attention_rows" (0 or 1: one vector row per workgroup, gathers from memory;
- * 2..8: that many consecutive vector rows per workgroup with the K / V rows they
- * share gathered once into LDS - faster when neighbouring rows share most of
- * their columns, e.g. banded masks, slower on random masks).  Returns 0, or 1 for an unknown name / bad value.
+ * "attention_chunk" (nonzero vectors per LDS chunk, 0 = automatic).  Returns 0, or 1 for an unknown name / bad value.
  * No counterpart in the reference, whose tile sizes are compile-time constants
  * (src/wmma_spmm.cu:396).
  */

@@ -216,14 +216,13 @@ def test_single_launch_attention(gpu, V, dims):
     try:
         # (chunk, waves, rows per workgroup): one chunk / several chunks per long row; rows = 1 is the
         # one-row-per-workgroup kernel, anything else the union-gather kernel (LDS copy or global fallback)
-        for chunk, waves, rows in ((0, 0, 1), (64, 3, 1), (32, 8, 1), (96, 1, 0), (0, 0, 8), (64, 0, 3), (32, 0, 16)):
+        for chunk, waves, rows in ((0, 0, 1), (64, 3, 1), (32, 8, 1), (96, 1, 0), (0, 0, 8), (64, 0, 3), (32, 0, 5)):
             _lib_set("attention_chunk", chunk)
             _lib_set("attention_waves", waves)
-            _lib_set("attention_rows", rows)
             pad = torch.full((heads, mask.m + 16, d_v), 3.0, dtype=torch.float16, device="cuda")
             out = pad[:, 8:8 + mask.m]
             ops.sparse_attention(mask.m_vec, V, n, prob.row_indices, prob.row_offsets, prob.column_indices,
-                                 qd, kd, vd, out=out, scale=scale)
+                                 qd, kd, vd, out=out, scale=scale, rows_per_workgroup=rows)
             torch.cuda.synchronize()
             host = pad.cpu().numpy()
             assert np.all(host[:, :8] == 3.0) and np.all(host[:, 8 + mask.m:] == 3.0), "wrote outside the output"
@@ -234,7 +233,6 @@ def test_single_launch_attention(gpu, V, dims):
     finally:
         _lib_set("attention_chunk", 0)
         _lib_set("attention_waves", 0)
-        _lib_set("attention_rows", 0)
 
 
 @pytest.mark.parametrize("V", [2, 8])
@@ -247,22 +245,19 @@ def test_union_gather_on_structured_and_random_masks(gpu, V):
         "band": cv.band_strided_pattern(seq, V, band_half_width=64, stride=128),     # union fits LDS
         "random": cv.uniform_pattern(seq // V, seq, 0.7, seed=3, vec_length=V),      # union too large: fallback
     }
-    try:
-        for name, mask in masks.items():
-            prob = ops.DeviceProblem(mask)
-            ref = _dense_attention(mask, q, k, v, 0.125)
-            outs = {}
-            for rows in (1, 4, 8, 32):
-                _lib_set("attention_rows", rows)
-                out = ops.sparse_attention(mask.m_vec, V, seq, prob.row_indices, prob.row_offsets,
-                                           prob.column_indices, qd, kd, vd, scale=0.125)
-                torch.cuda.synchronize()
-                outs[rows] = out.cpu().numpy()
-                _check_layer(outs[rows], ref, "%s mask V%d rows%d" % (name, V, rows))
-            # same arithmetic in the same order whatever the source of the gathered rows
-            assert np.array_equal(outs[4], outs[8]) and np.array_equal(outs[8], outs[32])
-    finally:
-        _lib_set("attention_rows", 0)
+    for name, mask in masks.items():
+        prob = ops.DeviceProblem(mask)
+        ref = _dense_attention(mask, q, k, v, 0.125)
+        outs = {}
+        for rows in (1, 2, 4, 8):
+            out = ops.sparse_attention(mask.m_vec, V, seq, prob.row_indices, prob.row_offsets,
+                                       prob.column_indices, qd, kd, vd, scale=0.125, rows_per_workgroup=rows)
+            torch.cuda.synchronize()
+            outs[rows] = out.cpu().numpy()
+            _check_layer(outs[rows], ref, "%s mask V%d rows%d" % (name, V, rows))
+        # same arithmetic in the same order whatever the source of the gathered rows
+        assert np.array_equal(outs[2], outs[4]) and np.array_equal(outs[4], outs[8])
+        assert ops.SparseAttention(mask).union_rows == (8 if name == "band" else 1)
 
 
 def _lib_set(name, value):

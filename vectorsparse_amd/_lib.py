@@ -27,7 +27,8 @@ SIGNATURES = {
     "vs_cuda_sddmm_f16_batched": ([_int] * 5 + [_vp] * 3 + [_vp, _ll, _vp, _ll, _vp, _ll, _int, _vp], _int),
     "vs_wmma_spmm_softmax_f16_batched": ([_int] * 5 + [_vp] * 3 + [_vp, _ll, _vp, _ll, _vp, _ll, ctypes.c_float, _vp],
                                          _int),
-    "vs_sparse_attention_f16": ([_int] * 6 + [_vp] * 3 + [_vp, _ll, _vp, _ll, _vp, _ll, _vp, _ll, ctypes.c_float, _vp],
+    "vs_sparse_attention_f16": ([_int] * 6 + [_vp] * 3 + [_vp, _ll, _vp, _ll, _vp, _ll, _vp, _ll, ctypes.c_float, _int,
+                                 _vp],
                                 _int),
     "vs_sparse_softmax_f16": ([_int] * 3 + [_vp] * 2 + [_vp, _ll, _vp, _ll, ctypes.c_float, _vp], _int),
     "vs_identity_row_swizzle": ([_int, _vp], None),

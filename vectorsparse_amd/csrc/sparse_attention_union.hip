@@ -402,15 +402,15 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int rows_per_
 }
 
 template <int V, int KS, int CPL>
-static int launch_one(int m_vec, int n, int d_qk, int d_v, const int *row_offsets, const int *col_indices,
+static int launch_one(int m_vec, int n, int d_qk, int d_v, int rows, const int *row_offsets, const int *col_indices,
                       const half_t *q, const half_t *k, const half_t *v, half_t *out, float scale,
                       hipStream_t stream, const Batch &batch, long long stride_v)
 {
     // Half of a CU's LDS per workgroup, so that two workgroups overlap each other's memory phases.
     constexpr size_t kLdsBudget = 72 * 1024;
     const int waves = 8;
-    int rows = options().attention_rows > 1 ? options().attention_rows : 8;
     if (rows > waves) rows = waves;  // one wave per row
+    if (rows < 1) rows = 1;
     const int n_words = (((n + 31) / 32) + 3) & ~3;
     const size_t fixed = 2 * (size_t)n_words * sizeof(unsigned) + 16 * sizeof(int);
     const int rk_cap = rows * 32 * kMaxSteps;  // ranks of the block's nonzeros, 16 bits each
@@ -432,12 +432,12 @@ static int launch_one(int m_vec, int n, int d_qk, int d_v, const int *row_offset
 }
 
 template <int V>
-static int launch_shape(int m_vec, int n, int d_qk, int d_v, const int *row_offsets, const int *col_indices,
+static int launch_shape(int m_vec, int n, int d_qk, int d_v, int rows, const int *row_offsets, const int *col_indices,
                         const half_t *q, const half_t *k, const half_t *v, half_t *out, float scale,
                         hipStream_t stream, const Batch &batch, long long stride_v)
 {
 #define VS_ATT(KS, CPL) \
-    return launch_one<V, KS, CPL>(m_vec, n, d_qk, d_v, row_offsets, col_indices, q, k, v, out, scale, stream, batch, stride_v)
+    return launch_one<V, KS, CPL>(m_vec, n, d_qk, d_v, rows, row_offsets, col_indices, q, k, v, out, scale, stream, batch, stride_v)
     if (d_v <= 64) {
         if (d_qk <= 32) VS_ATT(1, 4);
         if (d_qk <= 64) VS_ATT(2, 4);
@@ -449,7 +449,7 @@ static int launch_shape(int m_vec, int n, int d_qk, int d_v, const int *row_offs
 #undef VS_ATT
 }
 
-int launch_sparse_attention_union(int m_vec, int vec_length, int n, int d_qk, int d_v, const int *row_offsets,
+int launch_sparse_attention_union(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, const int *row_offsets,
                                   const int *col_indices, const half_t *q, const half_t *k, const half_t *v,
                                   half_t *out, float scale, hipStream_t stream, const Batch &batch,
                                   long long stride_v)
@@ -460,10 +460,10 @@ int launch_sparse_attention_union(int m_vec, int vec_length, int n, int d_qk, in
     if (d_v % 4 != 0 || d_v > 128 || (d_v > 64 && d_v % 8 != 0)) return hipErrorNotSupported;
     if (n > 1024 * 1024) return hipErrorNotSupported;  // the column bitmap lives in LDS
     switch (vec_length) {
-    case 1: return launch_shape<1>(m_vec, n, d_qk, d_v, row_offsets, col_indices, q, k, v, out, scale, stream, batch, stride_v);
-    case 2: return launch_shape<2>(m_vec, n, d_qk, d_v, row_offsets, col_indices, q, k, v, out, scale, stream, batch, stride_v);
-    case 4: return launch_shape<4>(m_vec, n, d_qk, d_v, row_offsets, col_indices, q, k, v, out, scale, stream, batch, stride_v);
-    case 8: return launch_shape<8>(m_vec, n, d_qk, d_v, row_offsets, col_indices, q, k, v, out, scale, stream, batch, stride_v);
+    case 1: return launch_shape<1>(m_vec, n, d_qk, d_v, rows, row_offsets, col_indices, q, k, v, out, scale, stream, batch, stride_v);
+    case 2: return launch_shape<2>(m_vec, n, d_qk, d_v, rows, row_offsets, col_indices, q, k, v, out, scale, stream, batch, stride_v);
+    case 4: return launch_shape<4>(m_vec, n, d_qk, d_v, rows, row_offsets, col_indices, q, k, v, out, scale, stream, batch, stride_v);
+    case 8: return launch_shape<8>(m_vec, n, d_qk, d_v, rows, row_offsets, col_indices, q, k, v, out, scale, stream, batch, stride_v);
     default: return hipErrorInvalidValue;
     }
 }

@@ -189,7 +189,6 @@ struct Options {
     int sddmm_block_waves = 0;
     int attention_waves = 0;
     int attention_chunk = 0;
-    int attention_rows = 0;
 };
 Options &options();
 
@@ -235,7 +234,7 @@ int launch_sparse_attention(int m_vec, int vec_length, int d_qk, int d_v, const 
                             const int *row_offsets, const int *col_indices, const half_t *q, const half_t *k,
                             const half_t *v, half_t *out, float scale, hipStream_t stream, const Batch &batch,
                             long long stride_v);
-int launch_sparse_attention_union(int m_vec, int vec_length, int n, int d_qk, int d_v, const int *row_offsets,
+int launch_sparse_attention_union(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, const int *row_offsets,
                                   const int *col_indices, const half_t *q, const half_t *k, const half_t *v,
                                   half_t *out, float scale, hipStream_t stream, const Batch &batch,
                                   long long stride_v);

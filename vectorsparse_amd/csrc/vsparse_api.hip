@@ -279,17 +279,18 @@ int vs_wmma_spmm_softmax_f16_batched(int batch, int m_vec, int vec_length, int k
 int vs_sparse_attention_f16(int batch, int m_vec, int vec_length, int n, int d_qk, int d_v, const int *row_indices,
                             const int *row_offsets, const int *col_indices, const void *q, long long stride_q,
                             const void *k, long long stride_k, const void *v, long long stride_v, void *out,
-                            long long stride_out, float scale, void *stream)
+                            long long stride_out, float scale, int rows_per_workgroup, void *stream)
 {
     if (batch < 0 || m_vec < 0 || n < 0 || d_qk < 0 || d_v < 0 || !vec_ok(vec_length)) return VS_ERROR_INVALID_VALUE;
+    if (rows_per_workgroup < 0 || rows_per_workgroup > 8) return VS_ERROR_INVALID_VALUE;
     if (batch == 0 || m_vec == 0 || d_v == 0) return VS_SUCCESS;
     if (!row_indices || !row_offsets || !q || !out) return VS_ERROR_INVALID_VALUE;
     if (n > 0 && (!k || !v)) return VS_ERROR_INVALID_VALUE;
     if (!aligned(q, 16) || !aligned(k, 16) || !aligned(v, 16) || !aligned(out, 16)) return VS_ERROR_INVALID_VALUE;
     if (!stride_ok(stride_q, 8) || !stride_ok(stride_k, 8) || !stride_ok(stride_v, 8) || !stride_ok(stride_out, 8))
         return VS_ERROR_INVALID_VALUE;
-    if (vs::options().attention_rows > 1)  // union-gather kernel: pays off when neighbouring rows share columns
-        return vs::launch_sparse_attention_union(m_vec, vec_length, n, d_qk, d_v, row_offsets, col_indices,
+    if (rows_per_workgroup > 1)  // union-gather kernel: pays off when neighbouring rows share columns
+        return vs::launch_sparse_attention_union(m_vec, vec_length, n, d_qk, d_v, rows_per_workgroup, row_offsets, col_indices,
                                                  static_cast<const half_t *>(q), static_cast<const half_t *>(k),
                                                  static_cast<const half_t *>(v), static_cast<half_t *>(out), scale,
                                                  static_cast<hipStream_t>(stream),
@@ -354,9 +355,7 @@ int vs_set_option(const char *name, int value)
         o.attention_waves = value;
     } else if (std::strcmp(name, "attention_chunk") == 0) {
         o.attention_chunk = value;
-    } else if (std::strcmp(name, "attention_rows") == 0) {
-        if (value > 64) return VS_ERROR_INVALID_VALUE;
-        o.attention_rows = value;
+
     } else {
         return VS_ERROR_INVALID_VALUE;
     }

@@ -153,10 +153,12 @@ def spmm_softmax_batched(m_vec, vec_length, k, n, row_indices, row_offsets, colu
 
 
 def sparse_attention(m_vec, vec_length, n, row_indices, row_offsets, col_indices, q, k, v, out=None, scale=None,
-                     stream=None):
+                     stream=None, rows_per_workgroup=0):
     """Single-launch fixed-mask attention: out = softmax(scale * mask(q k^T)) v.
 
     q: [heads, m, d_qk], k: [heads, n, d_qk], v: [heads, n, d_v] (or 2-D for one head), fp16.
+    rows_per_workgroup: 0 / 1 = one vector row per workgroup; 2..8 = union-gather kernel for masks whose
+    neighbouring rows share columns.
     """
     if q.dim() == 2:
         q, k, v = q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0)
@@ -173,7 +175,8 @@ def sparse_attention(m_vec, vec_length, n, row_indices, row_offsets, col_indices
     st = _lib.lib().vs_sparse_attention_f16(heads, m_vec, vec_length, n, d_qk, d_v, _ptr(row_indices),
                                             _ptr(row_offsets), _ptr(col_indices), _ptr(q), _stride(q, heads),
                                             _ptr(k), _stride(k, heads), _ptr(v), _stride(v, heads), _ptr(out),
-                                            _stride(out, heads), float(scale), _stream(stream))
+                                            _stride(out, heads), float(scale), int(rows_per_workgroup),
+                                            _stream(stream))
     _lib.check(st, "vs_sparse_attention_f16")
     return out
 
@@ -268,9 +271,9 @@ class SparseAttention:
         if fused is None:
             fused = "layer" if kernel == "wmma" else False
         if fused == "layer":
-            _lib.set_option("attention_rows", self.union_rows)
             return sparse_attention(p.m_vec, p.vec_length, p.n, p.row_indices, p.row_offsets, p.column_indices,
-                                    q, k, v, out=out, scale=scale, stream=stream)
+                                    q, k, v, out=out, scale=scale, stream=stream,
+                                    rows_per_workgroup=self.union_rows)
         sddmm_batched(p.m_vec, d, p.n, p.nnz_vec, p.row_indices, p.row_offsets, p.column_indices, q, k, scores,
                       p.vec_length, kernel=kernel, stream=stream)
         if fused:
