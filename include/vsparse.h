@@ -212,16 +212,45 @@ int vs_wmma_spmm_softmax_f16_batched(int batch, int m_vec, int vec_length, int k
  * external sparse-transformer repository, README.md:76); same result as vs_wmma_sddmm_f16_batched ->
  * vs_sparse_softmax_f16 -> vs_wmma_spmm_f16_batched up to the fp16 rounding of the intermediates.
  * rows_per_workgroup: 0 or 1 = one vector row per workgroup, K / V rows gathered from memory per row
- * (any mask); 2..8 = that many consecutive vector rows per workgroup with the K / V rows they share
- * gathered once into LDS - faster when neighbouring rows share most of their columns (banded, blocky,
- * strided masks), slower on random masks, same results up to summation order; row_indices is then only
- * validated, rows are taken in their natural order.
+ * (any mask); 2..128 = about that many consecutive vector rows per workgroup (rounded up to whole waves
+ * of 16 scalar rows, at most 8 waves) computed as a dense tile against the union of their columns, whose
+ * K / V rows are gathered once into LDS - faster when neighbouring rows share most of their columns
+ * (banded, blocky, strided masks), slower on random masks, same results up to rounding; row_indices is
+ * then only validated, rows are taken in their natural order.  Workgroups whose union exceeds
+ * vs_sparse_attention_union_capacity() columns fall back to per-row gathers inside the same launch.
+ * plan: null, or (rows_per_workgroup >= 2 only) a buffer filled by vs_sparse_attention_plan for this mask,
+ * these head widths and this rows_per_workgroup: the kernel then reads every workgroup's union and row
+ * masks from it instead of rebuilding them at every launch (same results).  A plan made for another shape
+ * is detected and ignored (every workgroup then takes the per-row path: correct, slower).
  */
 int vs_sparse_attention_f16(int batch, int m_vec, int vec_length, int n, int d_qk, int d_v,
                             const int *row_indices, const int *row_offsets, const int *col_indices,
                             const void *q, long long stride_q, const void *k, long long stride_k,
                             const void *v, long long stride_v, void *out, long long stride_out,
-                            float scale, int rows_per_workgroup, void *stream);
+                            float scale, int rows_per_workgroup, const void *plan, void *stream);
+
+/*
+ * Analysis step for rows_per_workgroup >= 2 of vs_sparse_attention_f16: writes into `plan` (device memory,
+ * 16-byte aligned, at least vs_sparse_attention_plan_bytes() bytes, owned by the caller) the distinct
+ * columns and the row masks of every workgroup.  The mask of an attention layer is fixed, so one plan
+ * serves every head, layer and step; asynchronous on `stream`, nothing is kept by the library.
+ * vs_sparse_attention_plan_bytes returns 0 for shapes the union kernel does not support.
+ * No counterpart in the reference.
+ */
+long long vs_sparse_attention_plan_bytes(int m_vec, int vec_length, int n, int d_qk, int d_v,
+                                         int rows_per_workgroup);
+int vs_sparse_attention_plan(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows_per_workgroup,
+                             const int *row_offsets, const int *col_indices, void *plan,
+                             long long plan_bytes, void *stream);
+
+/*
+ * Planning helper for rows_per_workgroup >= 2 of vs_sparse_attention_f16: the number of distinct columns
+ * a workgroup can hold in LDS for this shape (0: shape not supported by the union kernel), and in
+ * *rows_used (may be null) the vector rows per workgroup the request is rounded to.  Host only, no
+ * launch.  No counterpart in the reference.
+ */
+int vs_sparse_attention_union_capacity(int vec_length, int n, int d_qk, int d_v, int rows_per_workgroup,
+                                       int *rows_used);
 
 /*
  * Host helpers (HOST pointers).  Replace IdentityRowSwizzle / SortedRowSwizzle —

@@ -216,7 +216,7 @@ def test_single_launch_attention(gpu, V, dims):
     try:
         # (chunk, waves, rows per workgroup): one chunk / several chunks per long row; rows = 1 is the
         # one-row-per-workgroup kernel, anything else the union-gather kernel (LDS copy or global fallback)
-        for chunk, waves, rows in ((0, 0, 1), (64, 3, 1), (32, 8, 1), (96, 1, 0), (0, 0, 8), (64, 0, 3), (32, 0, 5)):
+        for chunk, waves, rows in ((0, 0, 1), (64, 3, 1), (32, 8, 1), (96, 1, 0), (0, 0, 8), (64, 0, 3), (32, 0, 5), (0, 0, 16), (0, 0, 128)):
             _lib_set("attention_chunk", chunk)
             _lib_set("attention_waves", waves)
             pad = torch.full((heads, mask.m + 16, d_v), 3.0, dtype=torch.float16, device="cuda")
@@ -248,16 +248,50 @@ def test_union_gather_on_structured_and_random_masks(gpu, V):
     for name, mask in masks.items():
         prob = ops.DeviceProblem(mask)
         ref = _dense_attention(mask, q, k, v, 0.125)
-        outs = {}
-        for rows in (1, 2, 4, 8):
+        for rows in (1, 2, 4, 8, 16, 64, 128):
             out = ops.sparse_attention(mask.m_vec, V, seq, prob.row_indices, prob.row_offsets,
                                        prob.column_indices, qd, kd, vd, scale=0.125, rows_per_workgroup=rows)
+            again = ops.sparse_attention(mask.m_vec, V, seq, prob.row_indices, prob.row_offsets,
+                                         prob.column_indices, qd, kd, vd, scale=0.125, rows_per_workgroup=rows)
             torch.cuda.synchronize()
-            outs[rows] = out.cpu().numpy()
-            _check_layer(outs[rows], ref, "%s mask V%d rows%d" % (name, V, rows))
-        # same arithmetic in the same order whatever the source of the gathered rows
-        assert np.array_equal(outs[2], outs[4]) and np.array_equal(outs[4], outs[8])
-        assert ops.SparseAttention(mask).union_rows == (8 if name == "band" else 1)
+            _check_layer(out.cpu().numpy(), ref, "%s mask V%d rows%d" % (name, V, rows))
+            assert torch.equal(out, again)      # deterministic
+        planned = ops.SparseAttention(mask).union_rows(d, d)
+        assert (planned > 1) if name == "band" else (planned == 1)
+
+
+@pytest.mark.parametrize("V", [1, 8])
+def test_planned_launch_equals_unplanned(gpu, V):
+    """The plan holds exactly what the kernel would rebuild: same bits out.  A plan made for another launch
+    shape is ignored safely (per-row path), so the result still meets the layer bound."""
+    heads, seq, d = 2, 1024, 64
+    rng = np.random.default_rng(40 + V)
+    q, k, v = (rng.standard_normal((heads, seq, d)).astype(np.float16) for _ in range(3))
+    qd, kd, vd = (torch.from_numpy(x).cuda() for x in (q, k, v))
+    masks = {
+        "band": cv.band_strided_pattern(seq, V, band_half_width=64, stride=128),
+        "random": cv.uniform_pattern(seq // V, seq, 0.7, seed=3, vec_length=V),   # every union too large
+        "ragged": cv.binomial_pattern(seq // V, seq, 0.97, seed=4, vec_length=V),  # some fit, some do not
+    }
+    for name, mask in masks.items():
+        prob = ops.DeviceProblem(mask)
+        ref = _dense_attention(mask, q, k, v, 0.125)
+        for rows in (16 // V, 4 * (16 // V), 128 // V):
+            args = (mask.m_vec, V, seq, prob.row_indices, prob.row_offsets, prob.column_indices, qd, kd, vd)
+            plain = ops.sparse_attention(*args, scale=0.125, rows_per_workgroup=rows)
+            plan = ops.sparse_attention_plan(mask.m_vec, V, seq, d, d, rows, prob.row_offsets, prob.column_indices)
+            planned = ops.sparse_attention(*args, scale=0.125, rows_per_workgroup=rows, plan=plan)
+            torch.cuda.synchronize()
+            _check_layer(planned.cpu().numpy(), ref, "%s V%d rows%d planned" % (name, V, rows))
+            assert torch.equal(plain, planned), "%s V%d rows%d" % (name, V, rows)
+        # a negative scale (sign handled inside the kernel) through the same paths
+        neg = ops.sparse_attention(*args, scale=-0.125, rows_per_workgroup=128 // V, plan=plan)
+        torch.cuda.synchronize()
+        _check_layer(neg.cpu().numpy(), _dense_attention(mask, q, k, v, -0.125), "%s V%d negative scale" % (name, V))
+        other = ops.sparse_attention_plan(mask.m_vec, V, seq, d, d, 16 // V, prob.row_offsets, prob.column_indices)
+        out = ops.sparse_attention(*args, scale=0.125, rows_per_workgroup=128 // V, plan=other)
+        torch.cuda.synchronize()
+        _check_layer(out.cpu().numpy(), ref, "%s V%d foreign plan" % (name, V))
 
 
 def _lib_set(name, value):

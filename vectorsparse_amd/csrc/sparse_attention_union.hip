@@ -1,39 +1,44 @@
-// Fixed-mask sparse attention for a block of R consecutive vector rows per workgroup, with the K and V
-// rows those R rows need gathered ONCE into LDS ("union gather"), and one wave per vector row.
+// Fixed-mask sparse attention for a block of R consecutive vector rows per workgroup: the K and V rows
+// those rows need are gathered ONCE into LDS ("union gather") and the block is then computed as a dense
+// tile against that union, with a per-row bit mask deciding which scores exist.
 //
 // Structured masks (local band, block-diagonal, strided columns) make neighbouring rows share almost all
-// of their columns: with a band of 257 columns, 8 consecutive vector rows touch ~345 distinct columns,
-// not 8 x 283.  Gathering each row's K / V rows separately (sparse_attention.hip) makes the L2 -> CU
-// gather the bound; gathering the union once and serving every row of the block from LDS removes most
-// of that traffic.  Random masks have no overlap: when the union does not fit the LDS budget the
-// workgroup falls back to gathers from global memory, with the same arithmetic.
+// of their columns: with a band of 257 columns, 16 consecutive vector rows of length 8 touch ~410 distinct
+// columns, not 16 x 283.  Computing every row against the whole union wastes a little arithmetic on
+// masked-out pairs, but it fills all 16 rows of the MFMA tile (one vector row alone fills V of them),
+// needs no per-nonzero address arithmetic (the union's rows sit in LDS in rank order, every address is
+// lane base + immediate) and reads every K / V row from memory once per block.  Random masks have no
+// overlap: when the union does not fit the LDS budget the workgroup falls back to per-row gathers from
+// global memory (the caller should pick the one-row-per-workgroup kernel for such masks).
 //
-// Workgroup steps (R <= 8 rows, one wave per row, K and V share ONE LDS buffer so that two workgroups
-// fit a CU and one's memory phases overlap the other's arithmetic):
+// Workgroup steps (W waves, 16 scalar rows = 16 / V vector rows per wave, K and V share ONE LDS buffer so
+// that two workgroups fit a CU):
 //   1  bitmap of the block's columns in LDS (atomic or), exclusive prefix of its word popcounts:
 //      rank(col) = prefix[col / 32] + popcount(bitmap[col / 32] below bit col % 32) is the position of a
 //      column in the sorted union; U = total popcount.
-//   2  list the union's columns, store the rank of every nonzero of the block (16 bits), copy the K rows
-//      of the union to LDS (row-major 128-bit loads, rows padded by 16 bytes against bank conflicts).
-//   A  per wave: S^T = K_gathered Q^T on v_mfma_f32_16x16x32_f16 with the gathered K rows as the A
-//      operand and the row's Q slices as the B operand: lane (v, g) receives the scores of scalar row v
-//      for nonzeros 4g..4g+3 of every 16-vector group.  Run twice: the first pass keeps only the row
-//      maximum, the second recomputes the scores (LDS reads and MFMA are cheap, registers are not) and
-//      keeps p = exp2(s - max) as packed fp16 plus the row sum.  Statistics of scalar row v combine the
-//      four lanes that hold the same v (ds_swizzle xor 16, ds_bpermute xor 32).
+//   2  list the union's columns; per vector row a bit mask over ranks (bit r set: the row holds the
+//      column of rank r); copy the K rows of the union to LDS (128-bit loads, rows padded by 16 bytes
+//      against bank conflicts, rows U.. of the last 32-rank step zero-filled).
+//   A  per wave and 32-rank step: S^T = K_union Q^T on v_mfma_f32_16x16x32_f16 with the K rows as the A
+//      operand and the wave's 16 Q rows as the B operand: lane (c, g) receives the scores of scalar row
+//      c for ranks 4g..4g+3 of both 16-rank halves.  Steps in which none of the wave's rows holds a
+//      column are skipped.  Run twice: the first pass keeps only the row maximum, the second recomputes
+//      the scores (LDS reads and MFMA are cheap, registers are not) and keeps p = exp2(s - max) as packed
+//      fp16, masked-out pairs as exact zeros.  The maximum of scalar row c combines the four lanes (c, *).
 //   3  barrier, copy the V rows of the union over the K rows, barrier.
-//   C  per wave: P V on the same MFMA with P as the A operand.  The contraction index of an MFMA can be numbered
-//      freely as long as both operands agree, so k-slot (g, e) is DEFINED as the nonzero the lane
-//      already holds: e < 4 -> nonzero 4g + e of the step's first group, e >= 4 -> nonzero 4g + e - 4 of
-//      its second group.  P therefore goes from the score registers into the A operand with no data
-//      movement, and the gathered V rows (transposed in registers with v_perm_b32, as in the SpMM
-//      kernel) are fetched in that same order.
-// Blocks whose union, nonzero count or longest row exceed the LDS / register budget take the fallback.
+//   C  per wave and step: P V on the same MFMA with P as the A operand.  The contraction index of an MFMA
+//      can be numbered freely as long as both operands agree, so k-slot (g, e) is DEFINED as the rank the
+//      lane already holds: e < 4 -> rank 4g + e of the step's first half, e >= 4 -> 4g + e - 4 of its
+//      second half.  P therefore goes from the score registers into the A operand with no data movement,
+//      and the V rows (transposed in registers with v_perm_b32, as in the SpMM kernel) are read in that
+//      same order.  One more MFMA per step with an all-ones B operand yields the row sums of the rounded
+//      p in exactly the accumulator layout, so normalising needs no cross-lane traffic.
 #include "vs_common.hpp"
 
 namespace vs {
 
-constexpr int kMaxSteps = 10;  // 32-vector steps of a row whose scores are held in registers at once
+constexpr int kMaxSteps = 10;   // fallback: 32-vector steps of a row whose scores are held in registers at once
+constexpr int kUnionSteps = 14; // 32-rank steps of the union whose probabilities are held in registers at once
 
 // Value of `x` held by lane `src_lane` (all lanes active).
 __device__ __forceinline__ float from_lane(float x, int src_lane)
@@ -198,68 +203,91 @@ __device__ __forceinline__ void load_q(half8_t (&qb)[KS], const half_t *q, int r
     for (int kk = 0; kk < KS; ++kk) qb[kk] = __builtin_bit_cast(half8_t, load_slice16(q_row, kk, g, d_qk, ok));
 }
 
-// V: vector length; KS: d_qk <= 32*KS; CPL: d_v <= 16*CPL.
-template <int V, int KS, int CPL>
-// four waves per SIMD: two eight-wave workgroups per CU
-__global__ void __launch_bounds__(512, 4)
-sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int rows_per_block, int u_max, int rk_cap,
-                              const int *__restrict__ row_offsets, const int *__restrict__ col_indices,
-                              const half_t *__restrict__ q, const half_t *__restrict__ k,
-                              const half_t *__restrict__ v, half_t *__restrict__ out, long long stride_q,
-                              long long stride_k, long long stride_v, long long stride_out, float scale)
+// 16 consecutive scalar rows of Q as the MFMA B operand: lane (c, g) holds Q[first + c][32kk + 8g .. +8),
+// zeros for rows at or past `limit`.
+template <int KS>
+__device__ __forceinline__ void load_q16(half8_t (&qb)[KS], const half_t *q, long long first, long long limit,
+                                         int d_qk, int c, int g)
 {
-    q += blockIdx.y * stride_q;
-    k += blockIdx.y * stride_k;
-    v += blockIdx.y * stride_v;
-    out += blockIdx.y * stride_out;
-    const int n_words = (n + 31) >> 5;
-    const int n_words_al = (n_words + 3) & ~3;  // keeps the arrays behind the bitmap 16-byte aligned
-    const int pitch = (d_qk > d_v ? d_qk : d_v) + 8;  // halves; +16 bytes: consecutive ranks start 4 banks apart
+    const bool ok = first + c < limit;
+    const half_t *q_row = q + (size_t)(ok ? first + c : 0) * d_qk;
+#pragma unroll
+    for (int kk = 0; kk < KS; ++kk) qb[kk] = __builtin_bit_cast(half8_t, load_slice16(q_row, kk, g, d_qk, ok));
+}
 
-    extern __shared__ __align__(16) unsigned char smem[];
-    unsigned *bitmap = reinterpret_cast<unsigned *>(smem);
-    unsigned *prefix = bitmap + n_words_al;                                // [n_words] exclusive popcount prefix
-    int *wave_tot = reinterpret_cast<int *>(prefix + n_words_al);          // [16]: scan scratch, [14] longest row, [15] U
-    half_t *buf = reinterpret_cast<half_t *>(wave_tot + 16);               // [u_max][pitch]: K rows, later V rows
-    int *ucols = reinterpret_cast<int *>(buf + (size_t)u_max * pitch);     // [u_max] columns of the union
-    unsigned short *rkb = reinterpret_cast<unsigned short *>(ucols + u_max);  // [rk_cap] rank of each nonzero
+// `x` where bit `bit` of `word` is set, `other` elsewhere (v_bfe_i32 + v_bfi_b32).
+__device__ __forceinline__ float select_bit(unsigned word, int bit, float x, float other)
+{
+    const unsigned m = (unsigned)__builtin_amdgcn_sbfe((int)word, bit, 1);  // 0 or ~0
+    return __builtin_bit_cast(float, (__builtin_bit_cast(unsigned, x) & m) | (__builtin_bit_cast(unsigned, other) & ~m));
+}
 
+// Halves between consecutive rows of the LDS copy: room for every slice either phase reads, plus
+// 16 bytes so that consecutive ranks start 4 banks apart.
+constexpr int union_pitch(int ks, int cpl)
+{
+    return (32 * ks > 16 * cpl ? 32 * ks : 16 * cpl) + 8;
+}
+
+// The K rows of one 32-rank step as MFMA A operands: a[u][kk] = row 32t + 16u + c, halves 32kk + 8g .. +8.
+template <int KS, int PITCH>
+__device__ __forceinline__ void load_k_step(half8_t (&a)[2][KS], const half_t *k_lane, int t)
+{
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk)
+            a[u][kk] = *reinterpret_cast<const half8_t *>(k_lane + (32 * t + 16 * u) * PITCH + 32 * kk);
+}
+
+// S^T of one 32-rank step: sacc[u][e] = score of the lane's scalar row against rank 32t + 16u + 4g + e.
+template <int KS>
+__device__ __forceinline__ void scores_step(float4_t (&sacc)[2], const half8_t (&a)[2][KS], const half8_t (&qb)[KS])
+{
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        sacc[u] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) sacc[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u][kk], qb[kk], sacc[u], 0, 0, 0);
+    }
+}
+
+// LDS arrays that describe the union of a block of rows.
+struct UnionLds {
+    unsigned *bitmap;   // [n_words] columns present in the block
+    unsigned *prefix;   // [n_words] exclusive prefix of the bitmap's word popcounts
+    int *wave_tot;      // [16] scan scratch, [15] = number of distinct columns
+    unsigned *rowmask;  // [rows][kUnionSteps] ranks each row holds
+    int *ucols;         // [u_max] columns of the union in ascending order
+};
+
+// Steps 1 and 2 of the header comment for rows [row_first, row_last), by the whole workgroup: returns the
+// number U of distinct columns; rowmask and ucols are complete (and visible to every thread) on return
+// when U <= u_max, otherwise only U is meaningful.
+__device__ __forceinline__ int build_union(const UnionLds &l, int n_words, int mask_words, int u_max, int row_first,
+                                           int row_last, const int *__restrict__ row_offsets,
+                                           const int *__restrict__ col_indices)
+{
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: row bounds stay in scalar registers
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n_waves = blockDim.x >> 6;
     const int n_threads = blockDim.x;
-    const int row_first = blockIdx.x * rows_per_block;
-    const int row_last = (row_first + rows_per_block) < m_vec ? (row_first + rows_per_block) : m_vec;
-    const int c = lane & 15;
-    const int g = lane >> 4;
-    const float s2 = scale * kLog2e;
-    const int col0 = c * CPL;
-    const bool col_ok = col0 < d_v;
-    const int col_off = col_ok ? col0 : 0;
-
-    // ---- 1. bitmap and rank prefix of the block's columns, longest row of the block
-    for (int w = tid; w < n_words; w += n_threads) bitmap[w] = 0u;
-    if (tid == 0) wave_tot[14] = 0;
+    for (int w = tid; w < n_words; w += n_threads) l.bitmap[w] = 0u;
+    for (int w = tid; w < mask_words; w += n_threads) l.rowmask[w] = 0u;
     __syncthreads();
     const int nz_first = row_offsets[row_first];
     const int nz_last = row_offsets[row_last];
-    if (row_first + tid < row_last) atomicMax(&wave_tot[14], row_offsets[row_first + tid + 1] - row_offsets[row_first + tid]);
-    // Every thread keeps up to kOwn of the block's column indices in registers (all loads in flight at
-    // once, reused for the ranks below); blocks with more nonzeros than that take the fallback.
-    constexpr int kOwn = 8;
-    int own_col[kOwn];
+    for (int j0 = nz_first + tid; j0 < nz_last; j0 += 4 * n_threads) {
+        int col[4];
 #pragma unroll
-    for (int i = 0; i < kOwn; ++i) {
-        const int j = nz_first + tid + i * n_threads;
-        own_col[i] = j < nz_last ? col_indices[j] : -1;
-    }
+        for (int i = 0; i < 4; ++i) {
+            const int j = j0 + i * n_threads;
+            col[i] = j < nz_last ? col_indices[j] : -1;
+        }
 #pragma unroll
-    for (int i = 0; i < kOwn; ++i)
-        if (own_col[i] >= 0) atomicOr(&bitmap[own_col[i] >> 5], 1u << (own_col[i] & 31));
-    for (int j = nz_first + tid + kOwn * n_threads; j < nz_last; j += n_threads) {
-        const int col = col_indices[j];
-        atomicOr(&bitmap[col >> 5], 1u << (col & 31));
+        for (int i = 0; i < 4; ++i)
+            if (col[i] >= 0) atomicOr(&l.bitmap[col[i] >> 5], 1u << (col[i] & 31));
     }
     __syncthreads();
     {
@@ -268,32 +296,180 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int rows_per_
         const int per = (n_words + n_threads - 1) / n_threads;
         const int w0 = tid * per;
         int local = 0;
-        for (int w = w0; w < w0 + per && w < n_words; ++w) local += __builtin_popcount(bitmap[w]);
+        for (int w = w0; w < w0 + per && w < n_words; ++w) local += __builtin_popcount(l.bitmap[w]);
         int incl = local;
 #pragma unroll
         for (int d = 1; d < 64; d <<= 1) {
             const int up = __builtin_amdgcn_ds_bpermute(((lane - d) & 63) << 2, incl);
             if (lane >= d) incl += up;
         }
-        if (lane == 63) wave_tot[wave] = incl;
+        if (lane == 63) l.wave_tot[wave] = incl;
         __syncthreads();
         int base = 0;
-        for (int w = 0; w < wave; ++w) base += wave_tot[w];
+        for (int w = 0; w < wave; ++w) base += l.wave_tot[w];
         int run = base + incl - local;
         for (int w = w0; w < w0 + per && w < n_words; ++w) {
-            prefix[w] = (unsigned)run;
-            run += __builtin_popcount(bitmap[w]);
+            l.prefix[w] = (unsigned)run;
+            run += __builtin_popcount(l.bitmap[w]);
         }
-        if (tid == n_threads - 1) wave_tot[15] = run;
+        if (tid == n_threads - 1) l.wave_tot[15] = run;
         __syncthreads();
     }
-    const int n_union = wave_tot[15];
-    const int nz_block = nz_last - nz_first;
-    const bool use_lds = n_union <= u_max && n_union < 65536 && nz_block <= rk_cap && nz_block <= kOwn * n_threads &&
-                         wave_tot[14] <= 32 * kMaxSteps && (row_last - row_first) <= n_waves && (d_v % 8 == 0);
+    const int n_union = l.wave_tot[15];
+    if (n_union > u_max) return n_union;
+    for (int w = tid; w < n_words; w += n_threads) {
+        unsigned bits = l.bitmap[w];
+        int pos = (int)l.prefix[w];
+        while (bits) {
+            const int b = __builtin_ctz(bits);
+            l.ucols[pos++] = (w << 5) + b;
+            bits &= bits - 1;
+        }
+    }
+    for (int r = wave; r < row_last - row_first; r += n_waves) {
+        const int beg = row_offsets[row_first + r];
+        const int end = row_offsets[row_first + r + 1];
+        for (int j0 = beg + lane; j0 < end; j0 += 128) {
+            const int j1 = j0 + 64;
+            const int col_a = col_indices[j0];
+            const int col_b = col_indices[j1 < end ? j1 : j0];
+            const int rank_a = (int)l.prefix[col_a >> 5] + __builtin_popcount(l.bitmap[col_a >> 5] & ((1u << (col_a & 31)) - 1u));
+            const int rank_b = (int)l.prefix[col_b >> 5] + __builtin_popcount(l.bitmap[col_b >> 5] & ((1u << (col_b & 31)) - 1u));
+            atomicOr(&l.rowmask[r * kUnionSteps + (rank_a >> 5)], 1u << (rank_a & 31));
+            atomicOr(&l.rowmask[r * kUnionSteps + (rank_b >> 5)], 1u << (rank_b & 31));
+        }
+    }
+    __syncthreads();
+    return n_union;
+}
+
+// A plan holds what build_union computes for every workgroup of a launch shape, so that launches on the
+// same mask (every head, layer and step) read it instead of rebuilding it.  Layout, in 32-bit words:
+// header [magic, m_vec, V, n, rows per workgroup, u_max, record stride, workgroups, 0...] (16 words), then
+// one record per workgroup: [U, 0, 0, 0], rowmask [mask_words], ucols [u_max].
+constexpr int kPlanMagic = 0x56535041;
+constexpr int kPlanHeader = 16;
+
+__global__ void __launch_bounds__(256)
+sparse_attention_plan_kernel(int m_vec, int vec_length, int n, int rows_per_block, int u_max,
+                             const int *__restrict__ row_offsets, const int *__restrict__ col_indices,
+                             int *__restrict__ plan)
+{
+    const int n_words = (n + 31) >> 5;
+    const int n_words_al = (n_words + 3) & ~3;
+    const int mask_words = (rows_per_block * kUnionSteps + 3) & ~3;
+    extern __shared__ __align__(16) unsigned char smem[];
+    UnionLds l;
+    l.bitmap = reinterpret_cast<unsigned *>(smem);
+    l.prefix = l.bitmap + n_words_al;
+    l.wave_tot = reinterpret_cast<int *>(l.prefix + n_words_al);
+    l.rowmask = reinterpret_cast<unsigned *>(l.wave_tot + 16);
+    l.ucols = reinterpret_cast<int *>(l.rowmask + mask_words);
+    const int stride = 4 + mask_words + u_max;
+    const int tid = threadIdx.x;
+    if (blockIdx.x == 0 && tid < kPlanHeader) {
+        const int header[kPlanHeader] = {kPlanMagic, m_vec, vec_length, n, rows_per_block, u_max, stride,
+                                         (int)gridDim.x, 0, 0, 0, 0, 0, 0, 0, 0};
+        int value = 0;
+#pragma unroll
+        for (int i = 0; i < kPlanHeader; ++i) value = (i == tid) ? header[i] : value;
+        plan[tid] = value;
+    }
+    const int row_first = blockIdx.x * rows_per_block;
+    const int row_last = (row_first + rows_per_block) < m_vec ? (row_first + rows_per_block) : m_vec;
+    const int n_union = build_union(l, n_words, mask_words, u_max, row_first, row_last, row_offsets, col_indices);
+    int *rec = plan + kPlanHeader + (size_t)blockIdx.x * stride;
+    if (tid < 4) rec[tid] = tid == 0 ? n_union : 0;
+    if (n_union > u_max) return;  // this workgroup's rows take the per-row path at every launch
+    for (int w = tid; w < mask_words; w += blockDim.x) rec[4 + w] = (int)l.rowmask[w];
+    for (int u = tid; u < u_max; u += blockDim.x) rec[4 + mask_words + u] = u < n_union ? l.ucols[u] : 0;
+}
+
+// V: vector length; KS: d_qk <= 32*KS; CPL: d_v <= 16*CPL.
+// PLANNED: the union and the row masks come from a plan (sparse_attention_plan_kernel) instead of being
+// rebuilt; a plan made for another mask shape or launch shape sends every workgroup to the per-row path.
+template <int V, int KS, int CPL, bool PLANNED>
+// four waves per SIMD: two eight-wave workgroups per CU
+__global__ void __launch_bounds__(512, 4)
+sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max,
+                              const int *__restrict__ row_offsets, const int *__restrict__ col_indices,
+                              const int *__restrict__ plan,
+                              const half_t *__restrict__ q, const half_t *__restrict__ k,
+                              const half_t *__restrict__ v, half_t *__restrict__ out, long long stride_q,
+                              long long stride_k, long long stride_v, long long stride_out, float scale)
+{
+    q += blockIdx.y * stride_q;
+    k += blockIdx.y * stride_k;
+    v += blockIdx.y * stride_v;
+    out += blockIdx.y * stride_out;
+    constexpr int RPW = 16 / V;  // vector rows per wave: 16 scalar rows fill the MFMA tile
+    constexpr int PITCH = union_pitch(KS, CPL);
+    const int n_words = (n + 31) >> 5;
+    const int n_words_al = (n_words + 3) & ~3;  // keeps the arrays behind the bitmap 16-byte aligned
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: row bounds stay in scalar registers
+    const int n_waves = blockDim.x >> 6;
+    const int n_threads = blockDim.x;
+    const int rows_per_block = n_waves * RPW;
+    const int mask_words = (rows_per_block * kUnionSteps + 3) & ~3;
+
+    extern __shared__ __align__(16) unsigned char smem[];
+    UnionLds l;
+    half_t *buf;  // [u_max][PITCH]: K rows, later V rows
+    if constexpr (PLANNED) {
+        l.bitmap = l.prefix = nullptr;
+        l.wave_tot = nullptr;
+        l.rowmask = reinterpret_cast<unsigned *>(smem);
+        buf = reinterpret_cast<half_t *>(l.rowmask + mask_words);
+        l.ucols = nullptr;
+    } else {
+        l.bitmap = reinterpret_cast<unsigned *>(smem);
+        l.prefix = l.bitmap + n_words_al;
+        l.wave_tot = reinterpret_cast<int *>(l.prefix + n_words_al);
+        l.rowmask = reinterpret_cast<unsigned *>(l.wave_tot + 16);
+        buf = reinterpret_cast<half_t *>(l.rowmask + mask_words);
+        l.ucols = reinterpret_cast<int *>(buf + (size_t)u_max * PITCH);
+    }
+    const unsigned *rowmask = l.rowmask;
+
+    // Consecutive workgroups go to different XCDs (each with its own L2); neighbouring row blocks share
+    // most of their K / V rows, so every XCD takes a contiguous run of row blocks instead.
+    int bx = blockIdx.x;
+    if ((gridDim.x & 7) == 0) bx = (bx & 7) * (gridDim.x >> 3) + (bx >> 3);
+    const int row_first = bx * rows_per_block;
+    const int row_last = (row_first + rows_per_block) < m_vec ? (row_first + rows_per_block) : m_vec;
+    const int c = lane & 15;
+    const int g = lane >> 4;
+    const float s2 = scale * kLog2e;
+    const int col0 = c * CPL;
+    const bool col_ok = col0 < d_v;
+    const int col_off = col_ok ? col0 : 0;
+
+    // ---- 1, 2. the union's columns and every row's mask over ranks: built here or read from the plan
+    const int nz_first = row_offsets[row_first];
+    int n_union;
+    const int *cols;  // columns of the union: LDS (built) or the plan's record (global)
+    if constexpr (PLANNED) {
+        const int stride = 4 + mask_words + u_max;
+        const bool plan_ok = plan[0] == kPlanMagic && plan[1] == m_vec && plan[2] == V && plan[3] == n &&
+                             plan[4] == rows_per_block && plan[5] == u_max && plan[6] == stride &&
+                             plan[7] == (int)gridDim.x;
+        const int *rec = plan + kPlanHeader + (size_t)(plan_ok ? bx : 0) * stride;
+        n_union = plan_ok ? rec[0] : 0x7fffffff;
+        cols = rec + 4 + mask_words;
+        if (n_union <= u_max)
+            for (int w = tid; w < mask_words; w += n_threads) l.rowmask[w] = (unsigned)rec[4 + w];
+        // visible to the other waves after the barrier that follows the K gather
+    } else {
+        n_union = build_union(l, n_words, mask_words, u_max, row_first, row_last, row_offsets, col_indices);
+        cols = l.ucols;
+    }
+    const bool use_lds = n_union <= u_max && (d_v % 8 == 0);
     if (!use_lds) {
-        // Fallback: same arithmetic with the K / V rows read from global memory by column; no barrier, so
-        // every wave walks its rows on its own, long rows in chunks with a running maximum and sum.
+        // Fallback: one vector row per wave at a time with the K / V rows read from global memory by
+        // column; no barrier, long rows in chunks with a running maximum and sum.
         const RowSource<false> ksrc = {k, d_qk, nullptr, col_indices, nz_first};
         const RowSource<false> vsrc = {v, d_v, nullptr, col_indices, nz_first};
         for (int row = row_first + wave; row < row_last; row += n_waves) {
@@ -326,31 +502,15 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int rows_per_
         return;
     }
 
-    // ---- 2. the union's columns, the rank of every nonzero, the K rows of the union
-    for (int w = tid; w < n_words; w += n_threads) {
-        unsigned bits = bitmap[w];
-        int pos = (int)prefix[w];
-        while (bits) {
-            const int b = __builtin_ctz(bits);
-            ucols[pos++] = (w << 5) + b;
-            bits &= bits - 1;
-        }
-    }
-#pragma unroll
-    for (int i = 0; i < kOwn; ++i) {
-        if (own_col[i] >= 0) {
-            const int col = own_col[i];
-            const unsigned word = bitmap[col >> 5];
-            rkb[tid + i * n_threads] =
-                (unsigned short)(prefix[col >> 5] + __builtin_popcount(word & ((1u << (col & 31)) - 1u)));
-        }
-    }
-    __syncthreads();
-    // copy one operand's rows of the union into buf: 16 bytes per thread and slice, kBatch slices in flight
-    auto gather = [&](const half_t *src, int d) {
+    // ---- 2b. the K rows of the union
+    const int n_steps = (n_union + 31) >> 5;  // <= kUnionSteps because u_max <= 32 * kUnionSteps
+    // Copy one operand's rows of the union into buf: 16 bytes per thread and slice, kBatch slices in
+    // flight; rows past the union (the last step's padding) and slices past `d` are written as zeros, so
+    // the arithmetic below never meets stale bits.
+    auto gather = [&](const half_t *src, int d, int slice_shift) {
         constexpr int kBatch = 8;
         const int slices = d >> 3;
-        const int total = n_union * slices;
+        const int total = (32 * n_steps) << slice_shift;
         for (int s0 = tid; s0 < total; s0 += kBatch * n_threads) {
             uint4_t data[kBatch];
             int dst[kBatch];
@@ -359,9 +519,13 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int rows_per_
                 const int sidx = s0 + i * n_threads;
                 dst[i] = -1;
                 if (sidx < total) {
-                    const int u = sidx / slices, sl = sidx - u * slices;
-                    data[i] = *reinterpret_cast<const uint4_t *>(src + (size_t)ucols[u] * d + 8 * sl);
-                    dst[i] = u * pitch + 8 * sl;
+                    const int u = sidx >> slice_shift, sl = sidx & ((1 << slice_shift) - 1);
+                    const bool real = u < n_union && sl < slices;
+                    const int col = PLANNED ? cols[real ? u : 0] : l.ucols[real ? u : 0];  // two address spaces
+                    const uint4_t x = *reinterpret_cast<const uint4_t *>(src + (size_t)col * d + (real ? 8 * sl : 0));
+                    const uint4_t zero = {0u, 0u, 0u, 0u};
+                    data[i] = real ? x : zero;
+                    dst[i] = u * PITCH + 8 * sl;
                 }
             }
 #pragma unroll
@@ -369,75 +533,209 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int rows_per_
                 if (dst[i] >= 0) *reinterpret_cast<uint4_t *>(buf + dst[i]) = data[i];
         }
     };
-    gather(k, d_qk);
+    constexpr int kShiftK = KS == 1 ? 2 : (KS == 2 ? 3 : 4);  // 4 * KS slices of 8 halves per K row
+    constexpr int kShiftV = CPL == 4 ? 3 : 4;                 // 2 * CPL slices per V row
+    const int q_first = 16 * wave;                                 // first scalar row of the wave inside the block
+    const long long q_global = (long long)row_first * V + q_first;  // the same in the whole operand
+    const long long q_limit = (long long)row_last * V;
+    half8_t qb[KS];  // requested before the K rows so that the first MFMA does not wait for it
+    load_q16<KS>(qb, q, q_global, q_limit, d_qk, c, g);
+    gather(k, d_qk, kShiftK);
     __syncthreads();
 
-    // ---- A. one wave per vector row: maximum, then exponentials (packed fp16) and their sum
-    const int row = row_first + wave;
-    const bool has_row = row < row_last;
-    const int beg = has_row ? row_offsets[row] : 0;
-    const int end = has_row ? row_offsets[row + 1] : 0;
-    const RowSource<true> src = {buf, pitch, rkb, nullptr, nz_first};  // K rows now, V rows after step 3
-    half8_t p[kMaxSteps];
-    float l_sum = 0.f;
-    if (end > beg) {
-        half8_t qb[KS];
-        load_q<V, KS>(qb, q, row, d_qk, c, g);
-        float mx;
-        softmax_chunk<KS, true>(p, mx, l_sum, -__builtin_inff(), src, beg, end, d_qk, qb, s2, c, g);
+    // ---- A. per wave: 16 scalar rows against the whole union; maximum, then masked exponentials
+    const unsigned *mrow = rowmask + ((q_first + c) / V) * kUnionSteps;  // mask of the lane's vector row
+    const half_t *k_lane = buf + c * PITCH + 8 * g;
+    // The maximum is tracked on the raw dot products, so the scale must be non-negative: a negative one
+    // moves its sign into Q.
+    const float s2a = __builtin_fabsf(s2);
+    if (s2 < 0.f) {
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) {
+            uint4_t bits = __builtin_bit_cast(uint4_t, qb[kk]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) bits[i] ^= 0x80008000u;
+            qb[kk] = __builtin_bit_cast(half8_t, bits);
+        }
+    }
+    const float neg_inf = -__builtin_inff();
+    constexpr unsigned kLaneBits = 0x000F000Fu;  // after the shift by 4g: the lane's 4 + 4 ranks of a step
+    unsigned act = 0;   // steps in which at least one row of the wave holds a column (uniform)
+    unsigned full = 0;  // steps in which every lane's rows hold all of the lane's ranks: no masking needed
+    float mx_raw = neg_inf;
+#pragma unroll
+    for (int t = 0; t < kUnionSteps; ++t) {
+        if (t < n_steps) {
+            const unsigned word = mrow[t];
+            if (__builtin_amdgcn_ballot_w64(word != 0u) != 0ull) {
+                act |= 1u << t;
+                const unsigned wg = word >> (4 * g);
+                half8_t a[2][KS];
+                load_k_step<KS, PITCH>(a, k_lane, t);
+                float4_t sacc[2];
+                scores_step<KS>(sacc, a, qb);
+                if (__builtin_amdgcn_ballot_w64((wg & kLaneBits) != kLaneBits) == 0ull) {
+                    full |= 1u << t;
+#pragma unroll
+                    for (int u = 0; u < 2; ++u)
+                        mx_raw = fmaxf(fmaxf(mx_raw, fmaxf(sacc[u][0], sacc[u][1])), fmaxf(sacc[u][2], sacc[u][3]));
+                } else {
+#pragma unroll
+                    for (int u = 0; u < 2; ++u)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) mx_raw = fmaxf(mx_raw, select_bit(wg, 16 * u + e, sacc[u][e], neg_inf));
+                }
+            }
+        }
+    }
+    act = __builtin_amdgcn_readfirstlane(act);
+    full = __builtin_amdgcn_readfirstlane(full);
+    mx_raw = fmaxf(mx_raw, partner<16>(mx_raw));  // scalar row c lives in the four lanes (c, g = 0..3)
+    mx_raw = fmaxf(mx_raw, partner<32>(mx_raw));
+    const float neg_mx = mx_raw == neg_inf ? 0.f : -(mx_raw * s2a);  // a row with no column: every exponent stays -inf
+    half8_t p[kUnionSteps];
+#pragma unroll
+    for (int t = 0; t < kUnionSteps; ++t) {
+        p[t] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        if ((act >> t) & 1u) {
+            half8_t a[2][KS];
+            load_k_step<KS, PITCH>(a, k_lane, t);
+            float4_t sacc[2];
+            scores_step<KS>(sacc, a, qb);
+            // k-slot (g, e) of step t: e < 4 -> rank 4g + e of the first half, e >= 4 -> 4g + e - 4 of the second
+            if ((full >> t) & 1u) {
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        p[t][4 * u + e] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf(sacc[u][e], s2a, neg_mx));
+            } else {
+                const unsigned wg = mrow[t] >> (4 * g);
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float bias = select_bit(wg, 16 * u + e, neg_mx, neg_inf);
+                        p[t][4 * u + e] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf(sacc[u][e], s2a, bias));
+                    }
+            }
+        }
     }
 
     // ---- 3. V rows of the union over the K rows
     __syncthreads();
-    gather(v, d_v);
+    gather(v, d_v, kShiftV);
     __syncthreads();
 
-    // ---- C. P V, normalise, store (one wave owns the whole row: nothing to reduce)
-    if (!has_row) return;
+    // ---- C. P V and the row sums, normalise, store (one wave owns its rows: nothing to reduce)
     float4_t acc[CPL];
 #pragma unroll
     for (int cc = 0; cc < CPL; ++cc) acc[cc] = float4_t{0.f, 0.f, 0.f, 0.f};
-    if (end > beg) accumulate_chunk<CPL, true>(acc, p, src, beg, end, col_off, g);
-    store_row<V, CPL>(out, row, d_v, acc, l_sum, end == beg, c, g);
+    float4_t lacc = {0.f, 0.f, 0.f, 0.f};
+    const half8_t ones = {1, 1, 1, 1, 1, 1, 1, 1};
+    const half_t *v_lane = buf + 4 * g * PITCH + col_off;
+#pragma unroll
+    for (int t = 0; t < kUnionSteps; ++t) {
+        if ((act >> t) & 1u) {
+            RowChunk<CPL> rows[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) rows[e].load(v_lane + (32 * t + (e < 4 ? e : 12 + e)) * PITCH);
+#pragma unroll
+            for (int pp = 0; pp < CPL / 2; ++pp) {
+                uint4_t even, odd;
+#pragma unroll
+                for (int qq = 0; qq < 4; ++qq) {
+                    even[qq] = pack_lo(rows[2 * qq].dword(pp), rows[2 * qq + 1].dword(pp));
+                    odd[qq] = pack_hi(rows[2 * qq].dword(pp), rows[2 * qq + 1].dword(pp));
+                }
+                acc[2 * pp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(p[t], __builtin_bit_cast(half8_t, even), acc[2 * pp], 0, 0, 0);
+                acc[2 * pp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(p[t], __builtin_bit_cast(half8_t, odd), acc[2 * pp + 1], 0, 0, 0);
+            }
+            lacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(p[t], ones, lacc, 0, 0, 0);  // row sums, in accumulator layout
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const long long row = q_global + 4 * g + e;  // accumulator register e of lane (c, g) is scalar row 4g + e
+        if (row < q_limit && col_ok) {
+            const float norm = lacc[e] > 0.f ? 1.f / lacc[e] : 0.f;  // a row with no column attends to nothing: zeros
+            float tmp[CPL];
+#pragma unroll
+            for (int cc = 0; cc < CPL; ++cc) tmp[cc] = acc[cc][e] * norm;
+            store_converted<half_t, CPL>(out + (size_t)row * d_v + col0, tmp);
+        }
+    }
 }
 
-template <int V, int KS, int CPL>
-static int launch_one(int m_vec, int n, int d_qk, int d_v, int rows, const int *row_offsets, const int *col_indices,
-                      const half_t *q, const half_t *k, const half_t *v, half_t *out, float scale,
-                      hipStream_t stream, const Batch &batch, long long stride_v)
+// 32-bit words of the row masks of a workgroup of `rows` vector rows, padded to 16 bytes.
+static int union_mask_words(int rows) { return (rows * kUnionSteps + 3) & ~3; }
+
+// Launch shape of the union kernel for a request of `rows` vector rows per workgroup.
+struct UnionShape {
+    int waves;   // 16 scalar rows each
+    int rows;    // vector rows per workgroup actually used
+    int u_max;   // distinct columns a workgroup can hold in LDS
+    size_t lds;
+};
+
+static bool union_shape(UnionShape &s, int vec_length, int n, int d_qk, int d_v, int rows)
 {
     // Half of a CU's LDS per workgroup, so that two workgroups overlap each other's memory phases.
     constexpr size_t kLdsBudget = 72 * 1024;
-    const int waves = 8;
-    if (rows > waves) rows = waves;  // one wave per row
-    if (rows < 1) rows = 1;
+    const int rpw = 16 / vec_length;
+    s.waves = ceil_div(rows < 1 ? 1 : rows, rpw);
+    if (s.waves > 8) s.waves = 8;
+    s.rows = s.waves * rpw;
+    const int ks = d_qk <= 32 ? 1 : (d_qk <= 64 ? 2 : 4);
+    const int cpl = d_v <= 64 ? 4 : 8;
     const int n_words = (((n + 31) / 32) + 3) & ~3;
-    const size_t fixed = 2 * (size_t)n_words * sizeof(unsigned) + 16 * sizeof(int);
-    const int rk_cap = rows * 32 * kMaxSteps;  // ranks of the block's nonzeros, 16 bits each
-    if (fixed + (size_t)rk_cap * 2 + 16 * 1024 > kLdsBudget) return hipErrorNotSupported;
-    const int pitch = (d_qk > d_v ? d_qk : d_v) + 8;
-    const size_t per_union_row = (size_t)pitch * sizeof(half_t) + sizeof(int);
-    int u_max = (int)((kLdsBudget - fixed - (size_t)rk_cap * 2 - 64) / per_union_row);
-    u_max &= ~7;
-    const size_t lds = fixed + (size_t)rk_cap * 2 + (size_t)u_max * per_union_row;
-    auto kernel = sparse_attention_union_kernel<V, KS, CPL>;
+    const size_t fixed = 2 * (size_t)n_words * sizeof(unsigned) + 16 * sizeof(int) +
+                         (size_t)union_mask_words(s.rows) * sizeof(unsigned);
+    const size_t per_union_row = (size_t)union_pitch(ks, cpl) * sizeof(half_t) + sizeof(int);
+    if (fixed + 32 * per_union_row > kLdsBudget) return false;  // the column bitmap alone fills the budget
+    s.u_max = (int)((kLdsBudget - fixed) / per_union_row) & ~31;
+    if (s.u_max > 32 * kUnionSteps) s.u_max = 32 * kUnionSteps;
+    s.lds = fixed + (size_t)s.u_max * per_union_row;
+    return true;
+}
+
+static bool union_dims_ok(int d_qk, int d_v)
+{
+    if (d_qk <= 0 || d_qk % 8 != 0 || d_qk > 128) return false;
+    if (d_v <= 0 || d_v % 4 != 0 || d_v > 128 || (d_v > 64 && d_v % 8 != 0)) return false;
+    return true;
+}
+
+template <int V, int KS, int CPL, bool PLANNED>
+static int launch_one(int m_vec, int n, int d_qk, int d_v, int rows, const int *row_offsets, const int *col_indices,
+                      const int *plan, const half_t *q, const half_t *k, const half_t *v, half_t *out, float scale,
+                      hipStream_t stream, const Batch &batch, long long stride_v)
+{
+    UnionShape s;
+    if (!union_shape(s, V, n, d_qk, d_v, rows)) return hipErrorNotSupported;
+    auto kernel = sparse_attention_union_kernel<V, KS, CPL, PLANNED>;
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr != hipSuccess) return (int)attr;
-    const int blocks = ceil_div(m_vec, rows);
-    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)batch.count), dim3(64 * waves), lds, stream, m_vec, n,
-                       d_qk, d_v, rows, u_max, rk_cap, row_offsets, col_indices, q, k, v, out, batch.stride_a,
+    const int blocks = ceil_div(m_vec, s.rows);
+    // with a plan only the row masks and the K / V rows live in LDS
+    const size_t lds = PLANNED ? (size_t)union_mask_words(s.rows) * sizeof(unsigned) +
+                                     (size_t)s.u_max * union_pitch(KS, CPL) * sizeof(half_t)
+                               : s.lds;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)batch.count), dim3(64 * s.waves), lds, stream, m_vec,
+                       n, d_qk, d_v, s.u_max, row_offsets, col_indices, plan, q, k, v, out, batch.stride_a,
                        batch.stride_b, stride_v, batch.stride_out, scale);
     return (int)hipGetLastError();
 }
 
-template <int V>
+template <int V, bool PLANNED>
 static int launch_shape(int m_vec, int n, int d_qk, int d_v, int rows, const int *row_offsets, const int *col_indices,
-                        const half_t *q, const half_t *k, const half_t *v, half_t *out, float scale,
+                        const int *plan, const half_t *q, const half_t *k, const half_t *v, half_t *out, float scale,
                         hipStream_t stream, const Batch &batch, long long stride_v)
 {
-#define VS_ATT(KS, CPL) \
-    return launch_one<V, KS, CPL>(m_vec, n, d_qk, d_v, rows, row_offsets, col_indices, q, k, v, out, scale, stream, batch, stride_v)
+#define VS_ATT(KS, CPL)                                                                                             \
+    return launch_one<V, KS, CPL, PLANNED>(m_vec, n, d_qk, d_v, rows, row_offsets, col_indices, plan, q, k, v, out, \
+                                           scale, stream, batch, stride_v)
     if (d_v <= 64) {
         if (d_qk <= 32) VS_ATT(1, 4);
         if (d_qk <= 64) VS_ATT(2, 4);
@@ -449,23 +747,77 @@ static int launch_shape(int m_vec, int n, int d_qk, int d_v, int rows, const int
 #undef VS_ATT
 }
 
+template <bool PLANNED>
+static int launch_v(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, const int *row_offsets,
+                    const int *col_indices, const int *plan, const half_t *q, const half_t *k, const half_t *v,
+                    half_t *out, float scale, hipStream_t stream, const Batch &batch, long long stride_v)
+{
+    switch (vec_length) {
+    case 1: return launch_shape<1, PLANNED>(m_vec, n, d_qk, d_v, rows, row_offsets, col_indices, plan, q, k, v, out, scale, stream, batch, stride_v);
+    case 2: return launch_shape<2, PLANNED>(m_vec, n, d_qk, d_v, rows, row_offsets, col_indices, plan, q, k, v, out, scale, stream, batch, stride_v);
+    case 4: return launch_shape<4, PLANNED>(m_vec, n, d_qk, d_v, rows, row_offsets, col_indices, plan, q, k, v, out, scale, stream, batch, stride_v);
+    case 8: return launch_shape<8, PLANNED>(m_vec, n, d_qk, d_v, rows, row_offsets, col_indices, plan, q, k, v, out, scale, stream, batch, stride_v);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+static bool union_supported(int vec_length, int n, int d_qk, int d_v)
+{
+    if (vec_length != 1 && vec_length != 2 && vec_length != 4 && vec_length != 8) return false;
+    return n >= 0 && n <= 1024 * 1024 && union_dims_ok(d_qk, d_v);  // the column bitmap lives in LDS
+}
+
+int sparse_attention_union_capacity(int vec_length, int n, int d_qk, int d_v, int rows, int *rows_used)
+{
+    UnionShape s;
+    if (!union_supported(vec_length, n, d_qk, d_v) || d_v % 8 != 0) return 0;
+    if (!union_shape(s, vec_length, n, d_qk, d_v, rows)) return 0;
+    if (rows_used) *rows_used = s.rows;
+    return s.u_max;
+}
+
+long long sparse_attention_plan_bytes(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows)
+{
+    UnionShape s;
+    if (m_vec < 0 || !union_supported(vec_length, n, d_qk, d_v)) return 0;
+    if (!union_shape(s, vec_length, n, d_qk, d_v, rows)) return 0;
+    const long long stride = 4 + union_mask_words(s.rows) + s.u_max;
+    return (long long)sizeof(int) * (kPlanHeader + stride * ceil_div(m_vec, s.rows));
+}
+
+int launch_sparse_attention_plan(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, const int *row_offsets,
+                                 const int *col_indices, int *plan, long long plan_bytes, hipStream_t stream)
+{
+    UnionShape s;
+    if (!union_supported(vec_length, n, d_qk, d_v)) return hipErrorNotSupported;
+    if (!union_shape(s, vec_length, n, d_qk, d_v, rows)) return hipErrorNotSupported;
+    const long long need = sparse_attention_plan_bytes(m_vec, vec_length, n, d_qk, d_v, rows);
+    if (plan_bytes < need) return hipErrorInvalidValue;
+    if (m_vec == 0) return hipSuccess;
+    const int n_words = (((n + 31) / 32) + 3) & ~3;
+    const size_t lds = 2 * (size_t)n_words * sizeof(unsigned) + 16 * sizeof(int) +
+                       (size_t)union_mask_words(s.rows) * sizeof(unsigned) + (size_t)s.u_max * sizeof(int);
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(sparse_attention_plan_kernel),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (attr != hipSuccess) return (int)attr;
+    hipLaunchKernelGGL(sparse_attention_plan_kernel, dim3((unsigned)ceil_div(m_vec, s.rows)), dim3(256), lds, stream,
+                       m_vec, vec_length, n, s.rows, s.u_max, row_offsets, col_indices, plan);
+    return (int)hipGetLastError();
+}
+
 int launch_sparse_attention_union(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, const int *row_offsets,
-                                  const int *col_indices, const half_t *q, const half_t *k, const half_t *v,
-                                  half_t *out, float scale, hipStream_t stream, const Batch &batch,
+                                  const int *col_indices, const int *plan, const half_t *q, const half_t *k,
+                                  const half_t *v, half_t *out, float scale, hipStream_t stream, const Batch &batch,
                                   long long stride_v)
 {
     if (m_vec == 0 || batch.count == 0 || d_v == 0) return hipSuccess;
     if (batch.count > 65535) return hipErrorNotSupported;
-    if (d_qk <= 0 || d_qk % 8 != 0 || d_qk > 128) return hipErrorNotSupported;
-    if (d_v % 4 != 0 || d_v > 128 || (d_v > 64 && d_v % 8 != 0)) return hipErrorNotSupported;
-    if (n > 1024 * 1024) return hipErrorNotSupported;  // the column bitmap lives in LDS
-    switch (vec_length) {
-    case 1: return launch_shape<1>(m_vec, n, d_qk, d_v, rows, row_offsets, col_indices, q, k, v, out, scale, stream, batch, stride_v);
-    case 2: return launch_shape<2>(m_vec, n, d_qk, d_v, rows, row_offsets, col_indices, q, k, v, out, scale, stream, batch, stride_v);
-    case 4: return launch_shape<4>(m_vec, n, d_qk, d_v, rows, row_offsets, col_indices, q, k, v, out, scale, stream, batch, stride_v);
-    case 8: return launch_shape<8>(m_vec, n, d_qk, d_v, rows, row_offsets, col_indices, q, k, v, out, scale, stream, batch, stride_v);
-    default: return hipErrorInvalidValue;
-    }
+    if (!union_supported(vec_length, n, d_qk, d_v)) return hipErrorNotSupported;
+    if (plan)
+        return launch_v<true>(m_vec, vec_length, n, d_qk, d_v, rows, row_offsets, col_indices, plan, q, k, v, out, scale,
+                              stream, batch, stride_v);
+    return launch_v<false>(m_vec, vec_length, n, d_qk, d_v, rows, row_offsets, col_indices, nullptr, q, k, v, out, scale,
+                           stream, batch, stride_v);
 }
 
 }  // namespace vs

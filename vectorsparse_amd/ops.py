@@ -8,6 +8,8 @@ addresses; the output dtype of ``output_matrix`` / ``output_values`` (fp16 or
 fp32) picks the overload, as C++ overload resolution does in the reference.
 Every call is asynchronous on ``stream`` (default: torch's current stream).
 """
+import ctypes
+
 import numpy as np
 import torch
 
@@ -153,12 +155,12 @@ def spmm_softmax_batched(m_vec, vec_length, k, n, row_indices, row_offsets, colu
 
 
 def sparse_attention(m_vec, vec_length, n, row_indices, row_offsets, col_indices, q, k, v, out=None, scale=None,
-                     stream=None, rows_per_workgroup=0):
+                     stream=None, rows_per_workgroup=0, plan=None):
     """Single-launch fixed-mask attention: out = softmax(scale * mask(q k^T)) v.
 
     q: [heads, m, d_qk], k: [heads, n, d_qk], v: [heads, n, d_v] (or 2-D for one head), fp16.
-    rows_per_workgroup: 0 / 1 = one vector row per workgroup; 2..8 = union-gather kernel for masks whose
-    neighbouring rows share columns.
+    rows_per_workgroup: 0 / 1 = one vector row per workgroup; >= 2 = union-gather kernel for masks whose
+    neighbouring rows share columns, optionally with a plan from `sparse_attention_plan`.
     """
     if q.dim() == 2:
         q, k, v = q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0)
@@ -176,7 +178,7 @@ def sparse_attention(m_vec, vec_length, n, row_indices, row_offsets, col_indices
                                             _ptr(row_offsets), _ptr(col_indices), _ptr(q), _stride(q, heads),
                                             _ptr(k), _stride(k, heads), _ptr(v), _stride(v, heads), _ptr(out),
                                             _stride(out, heads), float(scale), int(rows_per_workgroup),
-                                            _stream(stream))
+                                            _ptr(plan), _stream(stream))
     _lib.check(st, "vs_sparse_attention_f16")
     return out
 
@@ -227,6 +229,19 @@ def _expect_batched(t, dtype, name):
         raise ValueError("%s must be contiguous in its trailing dimensions" % name)
 
 
+def sparse_attention_plan(m_vec, vec_length, n, d_qk, d_v, rows_per_workgroup, row_offsets, col_indices, stream=None):
+    """Analyse a fixed mask once for the union-gather kernel: returns the plan (a device byte tensor) that
+    `sparse_attention(..., rows_per_workgroup=..., plan=...)` reads instead of rebuilding it per launch."""
+    size = _lib.lib().vs_sparse_attention_plan_bytes(m_vec, vec_length, n, d_qk, d_v, rows_per_workgroup)
+    if size <= 0:
+        raise _lib.VSparseError("vs_sparse_attention_plan_bytes: shape not supported by the union kernel")
+    plan = torch.empty(size, dtype=torch.uint8, device=row_offsets.device)
+    st = _lib.lib().vs_sparse_attention_plan(m_vec, vec_length, n, d_qk, d_v, rows_per_workgroup, _ptr(row_offsets),
+                                             _ptr(col_indices), _ptr(plan), size, _stream(stream))
+    _lib.check(st, "vs_sparse_attention_plan")
+    return plan
+
+
 class SparseAttention:
     """One fixed-mask sparse attention layer: SDDMM (QK^T on the mask) -> row softmax -> SpMM (P V).
 
@@ -237,21 +252,57 @@ class SparseAttention:
 
     def __init__(self, mask, device="cuda", sort=True):
         self.prob = DeviceProblem(mask, sort=sort, device=device)
-        self.union_rows = self._union_rows(mask)
+        self.mask = mask
+        self._plans = {}
+        self._rows = {}
+
+    def union_rows(self, d_qk, d_v):
+        """Rows per workgroup for the single-launch kernel with these head widths (cached per shape)."""
+        key = (int(d_qk), int(d_v))
+        if key not in self._rows:
+            self._rows[key] = self._union_rows(self.mask, *key)
+        return self._rows[key]
+
+    def plan(self, d_qk, d_v):
+        """Device plan of the union kernel for these head widths (built on first use), or None."""
+        key = (int(d_qk), int(d_v))
+        rows = self.union_rows(*key)
+        if rows < 2:
+            return None
+        if key not in self._plans:
+            p = self.prob
+            self._plans[key] = sparse_attention_plan(p.m_vec, p.vec_length, p.n, key[0], key[1], rows,
+                                                     p.row_offsets, p.column_indices)
+        return self._plans[key]
 
     @staticmethod
-    def _union_rows(mask, rows=8, budget_rows=400, max_len=320):
-        """Rows per workgroup for the single-launch kernel: 8 when every block of 8 consecutive vector
-        rows touches few enough distinct columns for their K / V rows to sit in LDS (banded, blocky or
-        strided masks) and no row is too long for the register-resident scores, else 1."""
+    def _union_rows(mask, d_qk, d_v, min_fill=0.4):
+        """Vector rows per workgroup for the single-launch kernel: the largest block of consecutive rows
+        whose distinct columns fit the library's LDS capacity for this shape in every block and whose
+        dense tile (rows x union) is at least `min_fill` full (banded, blocky or strided masks), else 1
+        (one row per workgroup, any mask)."""
         ro, ci = mask.row_offsets, mask.column_indices
-        if mask.m_vec == 0 or int(np.max(np.diff(ro))) > max_len:
+        if mask.m_vec == 0 or mask.nnz_vec == 0:
             return 1
-        for first in range(0, mask.m_vec, rows):
-            last = min(first + rows, mask.m_vec)
-            if np.unique(ci[ro[first]:ro[last]]).size > budget_rows:
-                return 1
-        return rows
+        per_wave = 16 // mask.vec_length
+        for waves in (8, 4, 2):
+            used = ctypes.c_int(0)
+            cap = _lib.lib().vs_sparse_attention_union_capacity(mask.vec_length, mask.n, d_qk, d_v, waves * per_wave,
+                                                                ctypes.addressof(used))
+            rows = used.value
+            if cap <= 0 or rows != waves * per_wave:
+                continue
+            fits, tile = True, 0
+            for first in range(0, mask.m_vec, rows):
+                last = min(first + rows, mask.m_vec)
+                union = np.unique(ci[ro[first]:ro[last]]).size
+                if union > cap:
+                    fits = False
+                    break
+                tile += union * (last - first)
+            if fits and mask.nnz_vec >= min_fill * tile:
+                return rows
+        return 1
 
     def forward(self, q, k, v, scale=None, kernel="wmma", stream=None, scores=None, out=None, fused=None):
         """q, k, v: fp16 [heads, seq, d] on the device.  Returns fp16 [heads, seq, d].
@@ -273,7 +324,8 @@ class SparseAttention:
         if fused == "layer":
             return sparse_attention(p.m_vec, p.vec_length, p.n, p.row_indices, p.row_offsets, p.column_indices,
                                     q, k, v, out=out, scale=scale, stream=stream,
-                                    rows_per_workgroup=self.union_rows)
+                                    rows_per_workgroup=self.union_rows(q.shape[2], v.shape[2]),
+                                    plan=self.plan(q.shape[2], v.shape[2]))
         sddmm_batched(p.m_vec, d, p.n, p.nnz_vec, p.row_indices, p.row_offsets, p.column_indices, q, k, scores,
                       p.vec_length, kernel=kernel, stream=stream)
         if fused:
