@@ -260,6 +260,16 @@ def test_union_gather_on_structured_and_random_masks(gpu, V):
         assert (planned > 1) if name == "band" else (planned == 1)
 
 
+def _with_empty_rows(mask, first, last):
+    """The same pattern with vector rows [first, last) emptied: whole workgroups without a single column."""
+    lengths = np.diff(mask.row_offsets).copy()
+    keep = np.ones(mask.nnz_vec, dtype=bool)
+    keep[mask.row_offsets[first]:mask.row_offsets[last]] = False
+    lengths[first:last] = 0
+    offsets = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    return cv.ColVecCSR(mask.m_vec, mask.n, mask.vec_length, offsets, mask.column_indices[keep].copy())
+
+
 @pytest.mark.parametrize("V", [1, 8])
 def test_planned_launch_equals_unplanned(gpu, V):
     """The plan holds exactly what the kernel would rebuild: same bits out.  A plan made for another launch
@@ -272,6 +282,7 @@ def test_planned_launch_equals_unplanned(gpu, V):
         "band": cv.band_strided_pattern(seq, V, band_half_width=64, stride=128),
         "random": cv.uniform_pattern(seq // V, seq, 0.7, seed=3, vec_length=V),   # every union too large
         "ragged": cv.binomial_pattern(seq // V, seq, 0.97, seed=4, vec_length=V),  # some fit, some do not
+        "hollow": _with_empty_rows(cv.band_strided_pattern(seq, V, band_half_width=32, stride=256), 16 // V, 9 * (16 // V)),
     }
     for name, mask in masks.items():
         prob = ops.DeviceProblem(mask)
