@@ -35,6 +35,23 @@ def build(verbose=False):
     return LIB_PATH
 
 
+def build_cxx_caller(verbose=False):
+    """Compile tests/cxx/reference_call_sites.cpp (a C++ program that calls the operators the way the
+    reference's benchmarks do, through include/vsparse_shim.hpp) and link it with libvsparse.so."""
+    root = os.path.dirname(_HERE)
+    src = os.path.join(root, "tests", "cxx", "reference_call_sites.cpp")
+    exe = os.path.join(root, "tests", "cxx", "reference_call_sites")
+    cmd = [HIPCC, "-O2", "--offload-arch=gfx950", "-std=c++17", "-I", os.path.join(root, "include"), src,
+           "-L", _HERE, "-lvsparse", "-Wl,-rpath,$ORIGIN/../../vectorsparse_amd", "-o", exe]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + proc.stdout)
+    return exe
+
+
 if __name__ == "__main__":
     print(build(verbose=True))
+    print(build_cxx_caller(verbose=True))
     sys.exit(0)
