@@ -141,14 +141,19 @@ int vs_cuda_sddmm_f16_f32out(int m_vec, int k, int n, int nonzeros_vec,
  * problem per process; they exist because sparse attention runs one mask over
  * many heads (the reference only links an external sparse-transformer repository,
  * README.md:76).
+ * nonzeros_vec of the SpMM forms: the number of nonzero vectors of the pattern
+ * (row_offsets[m_vec]) when the caller knows it, negative otherwise.  It only
+ * sizes the workgroups (the unbatched SpMM entry points keep the reference's
+ * argument list, which does not carry it, and size them by n instead); results do
+ * not depend on it.
  */
-int vs_wmma_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n,
+int vs_wmma_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
                              const int *row_indices, const int *row_offsets,
                              const int *column_indices,
                              const void *values, long long stride_values,
                              const void *rhs_matrix, long long stride_rhs,
                              void *output_matrix, long long stride_output, void *stream);
-int vs_cuda_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n,
+int vs_cuda_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
                              const int *row_indices, const int *row_offsets,
                              const int *column_indices,
                              const void *values, long long stride_values,
@@ -192,7 +197,7 @@ int vs_sparse_softmax_f16(int batch, int m_vec, int vec_length,
  * accumulated tile by the row sum.  Same requirements as vs_wmma_spmm_f16_batched.  No counterpart in
  * the reference (see vs_sparse_softmax_f16).
  */
-int vs_wmma_spmm_softmax_f16_batched(int batch, int m_vec, int vec_length, int k, int n,
+int vs_wmma_spmm_softmax_f16_batched(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
                                      const int *row_indices, const int *row_offsets,
                                      const int *column_indices,
                                      const void *scores, long long stride_scores,

@@ -180,3 +180,24 @@ def test_wrong_dtype_and_host_tensor_are_rejected(gpu):
         prob.spmm(B)
     with pytest.raises(ValueError):
         prob.spmm(torch.ones((32, 64), dtype=torch.float16))
+
+
+@pytest.mark.parametrize("kernel", ["wmma", "cuda"])
+def test_row_length_hint_changes_the_launch_shape_not_the_result(gpu, kernel):
+    # the batched entry point takes the pattern's nonzero count: any value (right, wrong, absent) must give
+    # parity, and the right one the same bits as the reference-shaped entry point up to summation order
+    for (m_vec, n, s, V) in ((64, 4608, 0.9, 8), (256, 1152, 0.98, 8), (96, 2304, 0.5, 2), (40, 640, 0.95, 1)):
+        pat = cv.random_values(cv.binomial_pattern(m_vec, n, s, seed=m_vec, vec_length=V), seed=9)
+        B = cv.dense_uniform(n, 128, seed=10)
+        ref = _oracle(pat, B)
+        prob = ops.DeviceProblem(pat, sort=True)
+        Bd = torch.from_numpy(B).cuda()
+        for hint in (pat.nnz_vec, -1, 0, 1, 50 * pat.nnz_vec):
+            out = torch.empty((1, pat.m, 128), dtype=torch.float16, device="cuda")
+            ops.spmm_batched(pat.m_vec, V, 128, n, prob.row_indices, prob.row_offsets, prob.column_indices,
+                             prob.values, Bd, out, kernel=kernel, nonzeros_vec=hint)
+            torch.cuda.synchronize()
+            assert_parity(out[0].cpu().numpy(), ref, "hint %d on %s" % (hint, (m_vec, n, s, V)))
+        hinted = prob.spmm(Bd, kernel=kernel, row_length_hint=True)
+        torch.cuda.synchronize()
+        assert_parity(hinted.cpu().numpy(), ref, "DeviceProblem hinted")

@@ -20,9 +20,10 @@ def load_pattern(bm, vec_length):
     return cv.read_smtx(bm, vec_length)
 
 
-def time_launches(torch, fn, iters=50, warmup=5):
-    """Average device time of one call (HIP events on the launch stream around `iters` calls
-    replayed from a HIP graph, so host launch cost is not part of it)."""
+def time_launches(torch, fn, iters=50, warmup=5, replays=5):
+    """Device time of one call in microseconds: HIP events on the launch stream around `iters` calls
+    replayed from a HIP graph (host launch cost is not part of it); the median of `replays` replays, because
+    a single replay now and then runs at twice its usual time (clock ramp after an idle gap)."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -38,13 +39,17 @@ def time_launches(torch, fn, iters=50, warmup=5):
             fn()
     graph.replay()
     torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    e0.record()
-    graph.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e3 / iters   # microseconds
+    times = []
+    for _ in range(max(1, replays)):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        times.append(e0.elapsed_time(e1) * 1e3 / iters)
+    times.sort()
+    return times[len(times) // 2]
 
 
 def verdict(name, got, ref):

@@ -348,10 +348,19 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
     int waves = options().spmm_waves;
     if (waves <= 0) {
         waves = next_pow2((int)((kTargetWaves + blocks - 1) / blocks));
-        const int max_useful = next_pow2(ceil_div(n > 0 ? n : 1, kStep));  // a row holds at most n vectors
-        if (waves > max_useful) waves = max_useful;
-        // two waves per row even on a full chip: measured 30 % faster than one on 8192 rows of ~280 vectors
-        if (waves < 2 && n >= 4 * kStep) waves = 2;
+        if (batch.nonzeros_vec >= 0) {
+            // Row lengths known: a wave is worth launching for about three 32-vector steps (measured over
+            // the ResNet-shaped grid: within 0.4 % of the best power of two, 7 % better than sizing by n).
+            const int steps = ceil_div(ceil_div(batch.nonzeros_vec, m_vec), kStep);
+            const int by_rows = next_pow2(ceil_div(steps > 0 ? steps : 1, 3));
+            if (waves > by_rows) waves = by_rows;
+            if (waves < 2 && steps >= 4) waves = 2;
+        } else {
+            const int max_useful = next_pow2(ceil_div(n > 0 ? n : 1, kStep));  // a row holds at most n vectors
+            if (waves > max_useful) waves = max_useful;
+            // two waves per row even on a full chip: measured 30 % faster than one on 8192 rows of ~280 vectors
+            if (waves < 2 && n >= 4 * kStep) waves = 2;
+        }
     }
     if (waves < 1) waves = 1;
     if (waves > 16) waves = 16;

@@ -204,6 +204,7 @@ struct Batch {
     long long stride_a = 0;    // SpMM: values        SDDMM: lhs_matrix
     long long stride_b = 0;    // SpMM: rhs_matrix    SDDMM: rhs_matrix
     long long stride_out = 0;  // SpMM: output_matrix SDDMM: output_values
+    int nonzeros_vec = -1;     // SpMM: nonzero vectors of the pattern when the caller knows them (launch-shape hint)
 };
 
 // Launchers (one per kernel family); return a hipError_t-valued int.

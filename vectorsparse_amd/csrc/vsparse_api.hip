@@ -171,20 +171,22 @@ int vs_cuda_sddmm_f16_f32out(int m_vec, int k, int n, int nonzeros_vec, const in
                                         static_cast<hipStream_t>(stream));
 }
 
-static vs::Batch make_batch(int batch, long long a, long long b, long long out)
+static vs::Batch make_batch(int batch, long long a, long long b, long long out, int nonzeros_vec = -1)
 {
     vs::Batch x;
     x.count = batch;
     x.stride_a = a;
     x.stride_b = b;
     x.stride_out = out;
+    x.nonzeros_vec = nonzeros_vec;
     return x;
 }
 
 // Strides keep every problem's operand as aligned as the first one.
 static bool stride_ok(long long stride, long long multiple) { return stride >= 0 && stride % multiple == 0; }
 
-int vs_wmma_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n, const int *row_indices,
+int vs_wmma_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
+    const int *row_indices,
                              const int *row_offsets, const int *column_indices, const void *values,
                              long long stride_values, const void *rhs_matrix, long long stride_rhs,
                              void *output_matrix, long long stride_output, void *stream)
@@ -198,10 +200,11 @@ int vs_wmma_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n,
     return vs::launch_spmm_mfma<half_t>(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices,
                                         static_cast<const half_t *>(values), static_cast<const half_t *>(rhs_matrix),
                                         static_cast<half_t *>(output_matrix), static_cast<hipStream_t>(stream),
-                                        make_batch(batch, stride_values, stride_rhs, stride_output));
+                                        make_batch(batch, stride_values, stride_rhs, stride_output, nonzeros_vec));
 }
 
-int vs_cuda_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n, const int *row_indices,
+int vs_cuda_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
+    const int *row_indices,
                              const int *row_offsets, const int *column_indices, const void *values,
                              long long stride_values, const void *rhs_matrix, long long stride_rhs,
                              void *output_matrix, long long stride_output, void *stream)
@@ -215,7 +218,7 @@ int vs_cuda_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n,
     return vs::launch_spmm_valu<half_t>(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices,
                                         static_cast<const half_t *>(values), static_cast<const half_t *>(rhs_matrix),
                                         static_cast<half_t *>(output_matrix), static_cast<hipStream_t>(stream),
-                                        make_batch(batch, stride_values, stride_rhs, stride_output));
+                                        make_batch(batch, stride_values, stride_rhs, stride_output, nonzeros_vec));
 }
 
 int vs_wmma_sddmm_f16_batched(int batch, int m_vec, int k, int n, int nonzeros_vec, const int *row_indices,
@@ -258,7 +261,8 @@ int vs_cuda_sddmm_f16_batched(int batch, int m_vec, int k, int n, int nonzeros_v
                                          make_batch(batch, stride_lhs, stride_rhs, stride_output));
 }
 
-int vs_wmma_spmm_softmax_f16_batched(int batch, int m_vec, int vec_length, int k, int n, const int *row_indices,
+int vs_wmma_spmm_softmax_f16_batched(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
+    const int *row_indices,
                                      const int *row_offsets, const int *column_indices, const void *scores,
                                      long long stride_scores, const void *rhs_matrix, long long stride_rhs,
                                      void *output_matrix, long long stride_output, float scale, void *stream)
@@ -273,7 +277,7 @@ int vs_wmma_spmm_softmax_f16_batched(int batch, int m_vec, int vec_length, int k
                                         static_cast<const half_t *>(scores), static_cast<const half_t *>(rhs_matrix),
                                         static_cast<half_t *>(output_matrix), scale,
                                         static_cast<hipStream_t>(stream),
-                                        make_batch(batch, stride_scores, stride_rhs, stride_output));
+                                        make_batch(batch, stride_scores, stride_rhs, stride_output, nonzeros_vec));
 }
 
 int vs_sparse_attention_f16(int batch, int m_vec, int vec_length, int n, int d_qk, int d_v, const int *row_indices,

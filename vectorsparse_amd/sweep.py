@@ -42,7 +42,10 @@ def main(argv=None):
     ap.add_argument("--out", default="spmm_sweep.csv")
     ap.add_argument("--quick", action="store_true", help="a 3 x 3 x 3 corner of the grid")
     ap.add_argument("--smtx-dir", default=None, help="sweep every .smtx under this directory instead")
-    ap.add_argument("--iters", type=int, default=20)
+    ap.add_argument("--hint", action="store_true",
+                    help="call through the batched entry point with the pattern's nonzero count (workgroups sized "
+                         "by the real row lengths) instead of the reference-shaped entry points")
+    ap.add_argument("--iters", type=int, default=100, help="launches per timed HIP-graph replay")
     args = ap.parse_args(argv)
 
     import torch
@@ -86,7 +89,7 @@ def main(argv=None):
         flops = 2.0 * pat.nnz * N_DENSE
         nbytes = spmm_bytes(pat, N_DENSE)
         for kernel in ("wmma", "cuda"):
-            us = time_launches(torch, lambda: prob.spmm(B, kernel=kernel, out=out), args.iters)
+            us = time_launches(torch, lambda: prob.spmm(B, kernel=kernel, out=out, row_length_hint=args.hint), args.iters)
             rows.append({"bm": label, "M": M, "K": K, "N": N_DENSE, "sparsity": round(s, 4), "V": V,
                          "kernel": kernel, "nnz_vec": pat.nnz_vec, "us": round(us, 3),
                          "dense_us": round(dense_us[(M, K)], 3), "speedup": round(dense_us[(M, K)] / us, 4),
