@@ -204,6 +204,10 @@ def main():
 
     wall_ms, ev_ms = time_graph(torch, step, args.steps, args.warmup)
     eager_wall_ms, _ = time_eager(torch, step, args.steps, args.warmup)
+    # the same problem through the batched entry point, which also takes the pattern's nonzero count
+    _, hinted_ms = time_graph(torch, lambda: prob.spmm(Bd, kernel="wmma", out=out, row_length_hint=True),
+                              args.steps, args.warmup)
+    step()
 
     # correctness of what was just timed (reference criterion and 1e-2 relative)
     from oracle import c_oracle as co
@@ -273,6 +277,7 @@ def main():
         "parity": {"max_rel_err": max_rel, "errors_gt_0.5": errors},
         "extra": {
             "eager_ms_per_step": eager_wall_ms,
+            "batched_entry_with_nonzero_count_ms": hinted_ms,
             "dense_gemm_ms": dense_ms,
             "speedup_vs_dense_gemm": dense_ms / ev_ms,
             "cold_cache_launch_us": cold_ms * 1e3,
