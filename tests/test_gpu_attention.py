@@ -333,3 +333,46 @@ def test_single_launch_attention_rejects_unsupported_shapes(gpu):
     v = torch.zeros((1, 64, 64), dtype=torch.float16, device="cuda")
     with pytest.raises(_lib.VSparseError):     # d_qk > 128: use the three-operator chain
         ops.sparse_attention(4, 8, 64, prob.row_indices, prob.row_offsets, prob.column_indices, q, k, v)
+
+
+def test_union_kernel_on_awkward_shapes(gpu):
+    """Seeded random shapes around the kernel's granularities: n not a multiple of 32 (bitmap words), fewer
+    rows than a workgroup takes, head widths that leave MFMA slices partly empty, a column in the last
+    position, with and without a plan."""
+    rng = np.random.default_rng(2024)
+    for case in range(40):
+        V = int(rng.choice([1, 2, 4, 8]))
+        n = int(rng.choice([1, 7, 31, 32, 33, 100, 257, 500]))
+        m_vec = int(rng.choice([1, 3, 16 // V, 16 // V + 1, 37]))
+        d_qk = int(rng.choice([8, 24, 40, 64, 104, 128]))
+        d_v = int(rng.choice([8, 16, 48, 64, 72, 128]))
+        rows = int(rng.choice([2, 3, 16 // V, 5 * (16 // V), 128]))
+        heads = int(rng.choice([1, 3]))
+        lengths = rng.integers(0, min(n, 60) + 1, m_vec)
+        ro, ci = cv._pattern_from_lengths(rng, m_vec, n, lengths)
+        if ro[m_vec] > ro[m_vec - 1]:
+            ci[-1] = n - 1        # columns of a row ascend, so its last one can be moved to the mask's last column
+        mask = cv.ColVecCSR(m_vec, n, V, ro, ci)
+        mask.validate()
+        q = rng.standard_normal((heads, mask.m, d_qk)).astype(np.float16)
+        k = rng.standard_normal((heads, n, d_qk)).astype(np.float16)
+        v = rng.standard_normal((heads, n, d_v)).astype(np.float16)
+        scale = 1.0 / np.sqrt(d_qk)
+        ref = _dense_attention(mask, q, k, v, scale)
+        prob = ops.DeviceProblem(mask)
+        qd, kd, vd = (torch.from_numpy(x).cuda() for x in (q, k, v))
+        what = "case %d: V%d n%d m_vec%d dqk%d dv%d rows%d heads%d" % (case, V, n, m_vec, d_qk, d_v, rows, heads)
+        print(what, flush=True)
+        args = (mask.m_vec, V, n, prob.row_indices, prob.row_offsets, prob.column_indices, qd, kd, vd)
+        pad = torch.full((heads, mask.m + 16, d_v), 5.0, dtype=torch.float16, device="cuda")
+        ops.sparse_attention(*args, out=pad[:, 8:8 + mask.m], scale=scale, rows_per_workgroup=rows)
+        plan = ops.sparse_attention_plan(mask.m_vec, V, n, d_qk, d_v, rows, prob.row_offsets, prob.column_indices)
+        planned = ops.sparse_attention(*args, scale=scale, rows_per_workgroup=rows, plan=plan)
+        torch.cuda.synchronize()
+        host = pad.cpu().numpy()
+        assert np.all(host[:, :8] == 5.0) and np.all(host[:, 8 + mask.m:] == 5.0), what + ": wrote outside the output"
+        if np.sqrt(np.mean(ref * ref)) > 0:
+            _check_layer(host[:, 8:8 + mask.m], ref, what)
+            _check_layer(planned.cpu().numpy(), ref, what + " planned")
+        else:
+            assert not host[:, 8:8 + mask.m].any() and not planned.cpu().numpy().any(), what
