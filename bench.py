@@ -156,9 +156,10 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--pmc", action="store_true",
+    ap.add_argument("--pmc", nargs="?", const="spmm", default=None, choices=["spmm", "attention"],
                     help="counter-collection mode for `rocprofv3 --pmc`: a 64 MiB device copy of known size "
-                         "(calibration), then a few eager launches of the headline kernel, nothing else")
+                         "(calibration), then a few eager launches of one kernel (the headline SpMM, or the "
+                         "config-5 attention layer with its plan), nothing else")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the SpMM/SDDMM path has no multi-GPU leg (rows shard with no "
@@ -195,11 +196,24 @@ def main():
         for _ in range(3):
             dst.copy_(src)
         torch.cuda.synchronize()
-        for _ in range(10):
-            step()
+        info = {"pmc_mode": args.pmc, "copy_bytes_each_way": src.numel() * 2}
+        if args.pmc == "spmm":
+            for _ in range(10):
+                step()
+            info["algorithmic_bytes"] = alg_bytes
+        else:
+            heads, seq, dim = 16, 4096, 64
+            amask = cv.band_strided_pattern(seq, 8, band_half_width=128, stride=128)
+            layer = ops.SparseAttention(amask)
+            gen = torch.Generator(device="cuda").manual_seed(5)
+            q, kk_, vv = (torch.randn((heads, seq, dim), device="cuda", generator=gen).half() for _ in range(3))
+            ctx = torch.empty((heads, seq, dim), dtype=torch.float16, device="cuda")
+            for _ in range(10):
+                layer.forward(q, kk_, vv, out=ctx)
+            info["algorithmic_bytes"] = 4 * heads * seq * dim * 2      # q, k, v read once, out written once
+            info["rows_per_workgroup"] = layer.union_rows(dim, dim)
         torch.cuda.synchronize()
-        print(json.dumps({"pmc_mode": True, "copy_bytes_each_way": src.numel() * 2,
-                          "algorithmic_bytes": alg_bytes}))
+        print(json.dumps(info))
         return
 
     wall_ms, ev_ms = time_graph(torch, step, args.steps, args.warmup)
