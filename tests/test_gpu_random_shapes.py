@@ -67,3 +67,32 @@ def test_sddmm_random(gpu, seed):
         ref2 = co.sddmm_host_ref_f32(pat.m_vec, K2, V, pat.row_offsets, pat.column_indices, A2, B2)
         got = prob.sddmm(torch.from_numpy(A2).cuda(), torch.from_numpy(B2).cuda(), kernel="cuda")
         assert_parity(got.cpu().numpy().reshape(-1), ref2, "cuda K%d " % K2 + what)
+
+
+def test_concurrent_streams_do_not_interfere(gpu):
+    """The library keeps no per-call state: different problems launched back to back on two streams (no
+    synchronisation between them) give the same bits as when each runs alone."""
+    import torch
+    from vectorsparse_amd import ops
+    rng = np.random.default_rng(99)
+    probs = []
+    for i, (m_vec, n, V, k) in enumerate(((64, 4608, 8, 256), (300, 512, 2, 64), (128, 1024, 4, 128))):
+        pat = cv.random_values(cv.binomial_pattern(m_vec, n, 0.9, seed=i, vec_length=V), seed=50 + i)
+        B = torch.from_numpy(cv.dense_uniform(n, k, seed=60 + i)).cuda()
+        A = torch.from_numpy(cv.dense_normal(pat.m, k, seed=70 + i)).cuda()
+        R = torch.from_numpy(cv.dense_normal(n, k, seed=80 + i)).cuda()
+        probs.append((ops.DeviceProblem(pat, sort=True), B, A, R))
+    alone = []
+    for prob, B, A, R in probs:
+        alone.append((prob.spmm(B).clone(), prob.sddmm(A, R).clone()))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = []
+    for rep in range(20):
+        for i, (prob, B, A, R) in enumerate(probs):
+            s = streams[(i + rep) % 2]
+            with torch.cuda.stream(s):
+                outs.append((i, prob.spmm(B, stream=s), prob.sddmm(A, R, stream=s)))
+    torch.cuda.synchronize()
+    for i, c, d in outs:
+        assert torch.equal(c, alone[i][0]) and torch.equal(d, alone[i][1])
