@@ -96,3 +96,49 @@ def test_concurrent_streams_do_not_interfere(gpu):
     torch.cuda.synchronize()
     for i, c, d in outs:
         assert torch.equal(c, alone[i][0]) and torch.equal(d, alone[i][1])
+
+
+def test_hip_graph_replays_equal_eager(gpu):
+    """Every entry point is capturable (no allocation, no memset, no synchronisation inside): a captured
+    SDDMM -> softmax -> SpMM chain plus the single-launch layer, replayed several times with eager work and
+    synchronisations in between and fresh inputs each time, equals the eager result every time."""
+    import torch
+    from vectorsparse_amd import ops
+    V, heads, seq, d = 8, 4, 512, 64
+    mask = cv.band_strided_pattern(seq, V, band_half_width=48, stride=64)
+    layer = ops.SparseAttention(mask)
+    layer.plan(d, d)                     # built outside the capture
+    g = torch.Generator(device="cuda").manual_seed(3)
+    q, k, v = (torch.randn((heads, seq, d), device="cuda", generator=g).half() for _ in range(3))
+    scores = torch.empty((heads, mask.nnz_vec, V), dtype=torch.float16, device="cuda")
+    out_chain = torch.empty((heads, seq, d), dtype=torch.float16, device="cuda")
+    out_layer = torch.empty((heads, seq, d), dtype=torch.float16, device="cuda")
+
+    def work():
+        layer.forward(q, k, v, scores=scores, out=out_chain, fused=False)
+        layer.forward(q, k, v, out=out_layer, fused="layer")
+
+    work()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        work()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        work()
+    for rep in range(4):
+        for t in (q, k, v):
+            t.copy_(torch.randn(t.shape, device="cuda", generator=g).half())   # new inputs, same buffers
+        work()
+        torch.cuda.synchronize()
+        want_chain, want_layer = out_chain.clone(), out_layer.clone()
+        out_chain.zero_()
+        out_layer.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_chain, want_chain), "replay %d: chain" % rep
+        assert torch.equal(out_layer, want_layer), "replay %d: layer" % rep
