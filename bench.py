@@ -156,10 +156,10 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--pmc", nargs="?", const="spmm", default=None, choices=["spmm", "attention"],
+    ap.add_argument("--pmc", nargs="?", const="spmm", default=None, choices=["spmm", "sddmm", "attention"],
                     help="counter-collection mode for `rocprofv3 --pmc`: a 64 MiB device copy of known size "
-                         "(calibration), then a few eager launches of one kernel (the headline SpMM, or the "
-                         "config-5 attention layer with its plan), nothing else")
+                         "(calibration), then a few eager launches of one kernel (the headline SpMM, the "
+                         "config-4 SDDMM, or the config-5 attention layer with its plan), nothing else")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the SpMM/SDDMM path has no multi-GPU leg (rows shard with no "
@@ -201,6 +201,15 @@ def main():
             for _ in range(10):
                 step()
             info["algorithmic_bytes"] = alg_bytes
+        elif args.pmc == "sddmm":
+            mask = cv.uniform_pattern(2048 // 8, 2048, 0.9, seed=4, vec_length=8)
+            lhs = torch.from_numpy(cv.dense_normal(2048, 64, seed=14)).cuda()
+            rhs = torch.from_numpy(cv.dense_normal(2048, 64, seed=24)).cuda()
+            sprob = ops.DeviceProblem(mask)
+            sout = torch.empty((mask.nnz_vec, 8), dtype=torch.float16, device="cuda")
+            for _ in range(10):
+                sprob.sddmm(lhs, rhs, kernel="wmma", out=sout)
+            info["algorithmic_bytes"] = sddmm_algorithmic_bytes(mask, 64)
         else:
             heads, seq, dim = 16, 4096, 64
             amask = cv.band_strided_pattern(seq, 8, band_half_width=128, stride=128)
