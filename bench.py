@@ -274,6 +274,7 @@ def main():
     attn_flops = 2.0 * amask.nnz * heads * dim * 2
 
     cold_ms = time_cold(torch, step)
+    cold_dense_ms = time_cold(torch, lambda: torch.matmul(Ad, Bd, out=dense_out))
 
     achieved = alg_bytes / (ev_ms * 1e-3) * 1e-9
     traffic = measured_traffic(os.path.join(ROOT, "profiles", "spmm_mfma_config2_pmc.txt"))
@@ -304,6 +305,7 @@ def main():
             "dense_gemm_ms": dense_ms,
             "speedup_vs_dense_gemm": dense_ms / ev_ms,
             "cold_cache_launch_us": cold_ms * 1e3,
+            "cold_cache_dense_gemm_us": cold_dense_ms * 1e3,
             "attention_config5": {"layer_ms": attn_ms, "density": 1.0 - amask.sparsity,
                                   "tflops": attn_flops / (attn_ms * 1e-3) * 1e-12,
                                   "dense_masked_attention_ms": dense_attn_ms,
