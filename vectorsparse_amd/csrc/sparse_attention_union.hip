@@ -290,9 +290,31 @@ __device__ __forceinline__ int build_union(const UnionLds &l, int n_words, int m
             if (col[i] >= 0) atomicOr(&l.bitmap[col[i] >> 5], 1u << (col[i] & 31));
     }
     __syncthreads();
-    {
-        // exclusive prefix of popcounts: every thread takes a contiguous run of words, the per-thread
-        // totals are scanned inside each wave and the wave totals added up
+    if (n_words <= 1024) {
+        // exclusive prefix of the word popcounts by one wave: a contiguous run of words per lane (one
+        // barrier and no cross-wave step; the other waves only wait)
+        if (wave == 0) {
+            const int per = (n_words + 63) >> 6;
+            const int w0 = lane * per;
+            int local = 0;
+            for (int w = w0; w < w0 + per && w < n_words; ++w) local += __builtin_popcount(l.bitmap[w]);
+            int incl = local;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const int up = __builtin_amdgcn_ds_bpermute(((lane - d) & 63) << 2, incl);
+                if (lane >= d) incl += up;
+            }
+            int run = incl - local;
+            for (int w = w0; w < w0 + per && w < n_words; ++w) {
+                l.prefix[w] = (unsigned)run;
+                run += __builtin_popcount(l.bitmap[w]);
+            }
+            if (lane == 63) l.wave_tot[15] = incl;
+        }
+        __syncthreads();
+    } else {
+        // the same with every thread taking a run of words: per-thread totals scanned inside each wave,
+        // then the wave totals added up
         const int per = (n_words + n_threads - 1) / n_threads;
         const int w0 = tid * per;
         int local = 0;
@@ -317,15 +339,8 @@ __device__ __forceinline__ int build_union(const UnionLds &l, int n_words, int m
     }
     const int n_union = l.wave_tot[15];
     if (n_union > u_max) return n_union;
-    for (int w = tid; w < n_words; w += n_threads) {
-        unsigned bits = l.bitmap[w];
-        int pos = (int)l.prefix[w];
-        while (bits) {
-            const int b = __builtin_ctz(bits);
-            l.ucols[pos++] = (w << 5) + b;
-            bits &= bits - 1;
-        }
-    }
+    // every nonzero sets its bit in its row's mask and writes its column at the column's rank (all writers
+    // of one rank write the same value), which lists the union without a pass over the bitmap
     for (int r = wave; r < row_last - row_first; r += n_waves) {
         const int beg = row_offsets[row_first + r];
         const int end = row_offsets[row_first + r + 1];
@@ -337,6 +352,8 @@ __device__ __forceinline__ int build_union(const UnionLds &l, int n_words, int m
             const int rank_b = (int)l.prefix[col_b >> 5] + __builtin_popcount(l.bitmap[col_b >> 5] & ((1u << (col_b & 31)) - 1u));
             atomicOr(&l.rowmask[r * kUnionSteps + (rank_a >> 5)], 1u << (rank_a & 31));
             atomicOr(&l.rowmask[r * kUnionSteps + (rank_b >> 5)], 1u << (rank_b & 31));
+            l.ucols[rank_a] = col_a;
+            l.ucols[rank_b] = col_b;
         }
     }
     __syncthreads();
