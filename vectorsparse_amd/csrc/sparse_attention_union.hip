@@ -46,27 +46,22 @@ __device__ __forceinline__ float from_lane(float x, int src_lane)
     return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src_lane << 2, __builtin_bit_cast(int, x)));
 }
 
-// Where the K / V rows of a block come from.  LDS = true: the workgroup's LDS copy, indexed by the rank
-// of a nonzero's column in the union; LDS = false: global memory, indexed by the column itself.
-template <bool LDS>
+// The K or V rows of a vector row's nonzeros, read from global memory by column (per-row path).
 struct RowSource {
-    const half_t *base;            // LDS copy (K rows, later V rows) or the global operand
-    int pitch;                     // halves between consecutive rows of `base`
-    const unsigned short *rkb;     // LDS: rank of nonzero j at rkb[j - nz_first]
-    const int *col_indices;        // global: column of nonzero j
-    int nz_first;
+    const half_t *base;      // the global operand
+    int pitch;               // halves between consecutive rows of `base`
+    const int *col_indices;  // column of nonzero j
     __device__ __forceinline__ const half_t *row_of(int j, int end) const
     {
         const int jc = j < end ? j : end - 1;  // slots past the row's end repeat its last vector
-        if constexpr (LDS) return base + (size_t)rkb[jc - nz_first] * pitch;
-        else return base + (size_t)col_indices[jc] * pitch;
+        return base + (size_t)col_indices[jc] * pitch;
     }
 };
 
 // Scores of the 64 nonzeros [j0, j0 + 64) of a row against the row's Q slices.
 // out[u][e]: group u (16 vectors), register e -> nonzero j0 + 16u + 4g + e, base-2 units, -inf past `end`.
-template <int KS, bool LDS>
-__device__ __forceinline__ void scores64(float (&out)[4][4], const RowSource<LDS> &ksrc, int j0, int end, int d_qk,
+template <int KS>
+__device__ __forceinline__ void scores64(float (&out)[4][4], const RowSource &ksrc, int j0, int end, int d_qk,
                                          const half8_t (&qb)[KS], float s2, int c, int g)
 {
     half8_t a[4][KS];
@@ -93,9 +88,9 @@ __device__ __forceinline__ void scores64(float (&out)[4][4], const RowSource<LDS
 // base-2 scores joined with `m_floor`, then p = exp2(s - mx) as packed fp16 in MFMA k-slot order and
 // the sum of the p.  Two passes over K: the first keeps only the maximum, the second recomputes the
 // scores (LDS / cache reads and MFMA are cheap, registers are not).
-template <int KS, bool LDS>
+template <int KS>
 __device__ __forceinline__ void softmax_chunk(half8_t (&p)[kMaxSteps], float &mx, float &sum, float m_floor,
-                                              const RowSource<LDS> &ksrc, int c0, int cend, int d_qk,
+                                              const RowSource &ksrc, int c0, int cend, int d_qk,
                                               const half8_t (&qb)[KS], float s2, int c, int g)
 {
     const int n_steps = (cend - c0 + 31) >> 5;
@@ -104,7 +99,7 @@ __device__ __forceinline__ void softmax_chunk(half8_t (&p)[kMaxSteps], float &mx
     for (int ss = 0; ss < kMaxSteps / 2; ++ss) {
         if (2 * ss < n_steps) {
             float sc[4][4];
-            scores64<KS, LDS>(sc, ksrc, c0 + 64 * ss, cend, d_qk, qb, s2, c, g);
+            scores64<KS>(sc, ksrc, c0 + 64 * ss, cend, d_qk, qb, s2, c, g);
 #pragma unroll
             for (int u = 0; u < 4; ++u)
 #pragma unroll
@@ -120,7 +115,7 @@ __device__ __forceinline__ void softmax_chunk(half8_t (&p)[kMaxSteps], float &mx
         p[2 * ss + 1] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
         if (2 * ss < n_steps) {
             float sc[4][4];
-            scores64<KS, LDS>(sc, ksrc, c0 + 64 * ss, cend, d_qk, qb, s2, c, g);
+            scores64<KS>(sc, ksrc, c0 + 64 * ss, cend, d_qk, qb, s2, c, g);
             // k-slot (g, e) of step t: e < 4 -> nonzero 4g + e of group 2t, e >= 4 -> 4g + e - 4 of group 2t + 1
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
@@ -138,9 +133,9 @@ __device__ __forceinline__ void softmax_chunk(half8_t (&p)[kMaxSteps], float &mx
 }
 
 // Phase C for the same nonzeros: acc += P V with the gathered V rows transposed in registers.
-template <int CPL, bool LDS>
+template <int CPL>
 __device__ __forceinline__ void accumulate_chunk(float4_t (&acc)[CPL], const half8_t (&p)[kMaxSteps],
-                                                 const RowSource<LDS> &vsrc, int c0, int cend, int col_off, int g)
+                                                 const RowSource &vsrc, int c0, int cend, int col_off, int g)
 {
     const int n_steps = (cend - c0 + 31) >> 5;
 #pragma unroll
@@ -465,7 +460,6 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max,
     const int col_off = col_ok ? col0 : 0;
 
     // ---- 1, 2. the union's columns and every row's mask over ranks: built here or read from the plan
-    const int nz_first = row_offsets[row_first];
     int n_union;
     const int *cols;  // columns of the union: LDS (built) or the plan's record (global)
     if constexpr (PLANNED) {
@@ -487,8 +481,8 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max,
     if (!use_lds) {
         // Fallback: one vector row per wave at a time with the K / V rows read from global memory by
         // column; no barrier, long rows in chunks with a running maximum and sum.
-        const RowSource<false> ksrc = {k, d_qk, nullptr, col_indices, nz_first};
-        const RowSource<false> vsrc = {v, d_v, nullptr, col_indices, nz_first};
+        const RowSource ksrc = {k, d_qk, col_indices};
+        const RowSource vsrc = {v, d_v, col_indices};
         for (int row = row_first + wave; row < row_last; row += n_waves) {
             const int beg = row_offsets[row];
             const int end = row_offsets[row + 1];
@@ -502,7 +496,7 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max,
                 const int cend = (c0 + 32 * kMaxSteps) < end ? (c0 + 32 * kMaxSteps) : end;
                 half8_t p[kMaxSteps];
                 float m_new, sum;
-                softmax_chunk<KS, false>(p, m_new, sum, m_run, ksrc, c0, cend, d_qk, qb, s2, c, g);
+                softmax_chunk<KS>(p, m_new, sum, m_run, ksrc, c0, cend, d_qk, qb, s2, c, g);
                 const float f = __builtin_amdgcn_exp2f(m_run - m_new);  // 0 on the first chunk (m_run = -inf)
                 l_run = l_run * f + sum;
                 m_run = m_new;
@@ -512,7 +506,7 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max,
 #pragma unroll
                     for (int cc = 0; cc < CPL; ++cc) acc[cc][e] *= fe;
                 }
-                accumulate_chunk<CPL, false>(acc, p, vsrc, c0, cend, col_off, g);
+                accumulate_chunk<CPL>(acc, p, vsrc, c0, cend, col_off, g);
             }
             store_row<V, CPL>(out, row, d_v, acc, l_run, end == beg, c, g);
         }
