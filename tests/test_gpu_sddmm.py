@@ -156,3 +156,43 @@ def test_sddmm_output_chains_into_spmm(gpu):
     assert_parity(vals.reshape(-1), _oracle(pat, Q, Kmat), "chain sddmm")
     ref = co.spmm_host_ref_f32(pat.m_vec, V, N, 512, pat.row_offsets, pat.column_indices, vals, W)
     assert_parity(out.cpu().numpy(), ref, "chain spmm")
+
+
+@pytest.mark.parametrize("V", [1, 2, 4, 8])
+def test_algorithm_2_splits_the_nonzero_range_same_bits(gpu, V):
+    """algorithm = 2 of wmmaSddmm (waves own ranges of nonzeros, not rows) gives the same bits as the row-slot
+    schedule on uniform, ragged, heavily skewed and mostly empty patterns, for every contraction length class."""
+    rng = np.random.default_rng(70 + V)
+    n = 700
+    patterns = {
+        "uniform": cv.uniform_pattern(96, n, 0.9, seed=1, vec_length=V),
+        "short rows": cv.uniform_pattern(300, n, 0.995, seed=2, vec_length=V),
+    }
+    lengths = np.minimum((rng.pareto(1.2, 150) + 0.05) * 40, n).astype(np.int64)
+    lengths[::7] = 0
+    lengths[3] = n
+    ro, ci = cv._pattern_from_lengths(rng, 150, n, lengths)
+    patterns["skewed with empty rows"] = cv.ColVecCSR(150, n, V, ro, ci)
+    lengths = np.zeros(130, dtype=np.int64)
+    lengths[[0, 64, 65, 129]] = [5, 1, 300, 17]
+    ro, ci = cv._pattern_from_lengths(rng, 130, n, lengths)
+    patterns["long runs of empty rows"] = cv.ColVecCSR(130, n, V, ro, ci)
+    for name, mask in patterns.items():
+        prob = ops.DeviceProblem(mask, sort=True)
+        for K in (8, 40, 64, 104, 128, 200, 256):
+            A = torch.from_numpy(cv.dense_normal(mask.m, K, seed=K)).cuda()
+            B = torch.from_numpy(cv.dense_normal(n, K, seed=K + 1)).cuda()
+            for dtype in (torch.float16, torch.float32):
+                slot = prob.sddmm(A, B, kernel="wmma", out_dtype=dtype, algorithm=1)
+                pad = torch.full((mask.nnz_vec + 32, V), 7.0, dtype=dtype, device="cuda")
+                flat = pad[16:16 + mask.nnz_vec]
+                prob.sddmm(A, B, kernel="wmma", out=flat, algorithm=2)
+                torch.cuda.synchronize()
+                assert torch.equal(slot, flat), "%s V%d K%d %s" % (name, V, K, dtype)
+                assert bool((pad[:16] == 7.0).all()) and bool((pad[16 + mask.nnz_vec:] == 7.0).all())
+        ref = co.sddmm_host_ref_f32(mask.m_vec, 64, V, mask.row_offsets, mask.column_indices,
+                                    cv.dense_normal(mask.m, 64, seed=64), cv.dense_normal(n, 64, seed=65))
+        got = prob.sddmm(torch.from_numpy(cv.dense_normal(mask.m, 64, seed=64)).cuda(),
+                         torch.from_numpy(cv.dense_normal(n, 64, seed=65)).cuda(), kernel="wmma", algorithm=2)
+        torch.cuda.synchronize()
+        assert_parity(got.cpu().numpy().reshape(-1), ref, name)

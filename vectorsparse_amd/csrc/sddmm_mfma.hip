@@ -127,12 +127,145 @@ sddmm_mfma_kernel(int m_vec, int K, int slots, const int *__restrict__ row_indic
     }
 }
 
+// Flat variant (K <= 256): the waves split the NONZERO range instead of the rows.  Wave w owns `supers`
+// consecutive super-groups of 16*GRP nonzero vectors of the CSR arrays, whatever rows they belong to, so
+// every wave has the same amount of work however skewed the row lengths are, none is launched idle, and
+// the row swizzle is not needed.  The wave requests the column indices and rhs rows of its first
+// super-group at once (they do not depend on the rows), finds the row of its first nonzero meanwhile with a
+// 64-ary search over row_offsets (one probe per lane and round: two dependent loads for up to 4095 vector
+// rows), then walks the row segments inside each super-group: the lhs slices are fetched when the row
+// changes and stay in registers while it lasts, one MFMA pass over the touched 16-vector groups per
+// segment.  The arithmetic of an output is the same as in the row-slot kernel (same operands, same MFMA
+// order): same bits.
+template <int V, int KS, int GRP, typename OutT>
+__global__ void __launch_bounds__(512)
+sddmm_mfma_flat_kernel(int m_vec, int K, int nonzeros_vec, int supers, const int *__restrict__ row_offsets,
+                       const int *__restrict__ col_indices, const half_t *__restrict__ lhs,
+                       const half_t *__restrict__ rhs, OutT *__restrict__ out, long long stride_lhs,
+                       long long stride_rhs, long long stride_out)
+{
+    lhs += blockIdx.y * stride_lhs;
+    rhs += blockIdx.y * stride_rhs;
+    out += blockIdx.y * stride_out;
+    constexpr int SUPER = 16 * GRP;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const long long first = ((long long)blockIdx.x * (blockDim.x >> 6) + wave) * supers * SUPER;
+    if (first >= nonzeros_vec) return;
+    const int range_begin = (int)first;
+    const int range_end = first + (long long)supers * SUPER < nonzeros_vec ? range_begin + supers * SUPER : nonzeros_vec;
+    const int c = lane & 15;        // MFMA order: column (nonzero vector) index
+    const int g = lane >> 4;        //             k group
+    const int r = lane >> 2;        // load order: row within the group of 16
+    const int q = lane & 3;         //             16-byte slice within a 64-byte k step
+    const int src = (4 * c + g) << 2;
+    const bool a_row_ok = r < V;
+
+    // column indices of a super-group, one group of 16 per register; slots past the range's end repeat its
+    // last vector (in bounds), their results are dropped
+    int col[GRP];
+    auto fetch_cols = [&](int j0) {
+#pragma unroll
+        for (int u = 0; u < GRP; ++u) {
+            const int jl = j0 + 16 * u + r;
+            col[u] = col_indices[jl < range_end ? jl : range_end - 1];
+        }
+    };
+    fetch_cols(range_begin);
+
+    // the last row index i in [0, m_vec] with row_offsets[i] <= range_begin (skips empty rows that start there)
+    int lo = 0, span = m_vec + 1;
+    while (span > 1) {
+        const int step = (span + 63) >> 6;
+        const int idx = lo + lane * step;
+        const int val = idx < lo + span ? row_offsets[idx] : 0x7fffffff;
+        const int below = __builtin_popcountll(__builtin_amdgcn_ballot_w64(val <= range_begin));  // a prefix of the lanes
+        const int k = below > 0 ? below - 1 : 0;
+        lo += k * step;
+        span = span - k * step < step ? span - k * step : step;
+    }
+    int base_row = lo;
+    if (base_row >= m_vec) return;  // nonzeros_vec exceeds row_offsets[m_vec]: nothing of the pattern is here
+    int ends = row_offsets[base_row + 1 + lane <= m_vec ? base_row + 1 + lane : m_vec];  // lane l: end of row base_row + l
+    int ri = 0;        // row base_row + ri is the candidate for the next nonzero
+    int cur_row = -1;  // row whose lhs slices are in `a`
+    half8_t a[KS];
+#pragma unroll
+    for (int kk = 0; kk < KS; ++kk) a[kk] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+
+    for (int j0 = range_begin; j0 < range_end; j0 += SUPER) {
+        const int jend = j0 + SUPER < range_end ? j0 + SUPER : range_end;
+        uint4_t raw[GRP][KS];
+#pragma unroll
+        for (int u = 0; u < GRP; ++u) {
+            const half_t *rhs_row = rhs + (size_t)col[u] * K;
+#pragma unroll
+            for (int kk = 0; kk < KS; ++kk) raw[u][kk] = load_slice16(rhs_row, kk, q, K, true);
+        }
+        if (j0 + SUPER < range_end) fetch_cols(j0 + SUPER);  // under the rhs rows in flight
+        int j = j0;
+        while (j < jend) {
+            if (ri == 64) {
+                base_row += 64;
+                ri = 0;
+                if (base_row >= m_vec) return;
+                ends = row_offsets[base_row + 1 + lane <= m_vec ? base_row + 1 + lane : m_vec];
+            }
+            const int row = base_row + ri;
+            if (row >= m_vec) return;
+            const int row_end = __builtin_amdgcn_readlane(ends, ri);
+            if (row_end <= j) {  // the row ended (or is empty): next one
+                ++ri;
+                continue;
+            }
+            const int seg_end = row_end < jend ? row_end : jend;
+            if (row != cur_row) {
+                const half_t *lhs_row = lhs + ((size_t)row * V + (a_row_ok ? r : 0)) * K;
+#pragma unroll
+                for (int kk = 0; kk < KS; ++kk) a[kk] = to_mfma_order(load_slice16(lhs_row, kk, q, K, a_row_ok), src);
+                cur_row = row;
+            }
+#pragma unroll
+            for (int u = 0; u < GRP; ++u) {
+                const int g0 = j0 + 16 * u;
+                if (g0 < seg_end && g0 + 16 > j) {  // the group holds nonzeros of this row segment
+                    float4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int kk = 0; kk < KS; ++kk)
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[kk], to_mfma_order(raw[u][kk], src), acc, 0, 0, 0);
+                    const int jj = g0 + c;
+                    if (jj >= j && jj < seg_end) store_group<V, OutT>(out, jj, g, acc);
+                }
+            }
+            j = seg_end;
+        }
+    }
+}
+
 template <int V, int KS, int GRP, typename OutT>
 static int launch_one(int m_vec, int k, int nonzeros_vec, const int *row_indices, const int *row_offsets,
                       const int *col_indices, const half_t *lhs, const half_t *rhs, OutT *out, hipStream_t stream,
                       const Batch &batch)
 {
     const int kWavesPerBlock = options().sddmm_block_waves > 0 ? options().sddmm_block_waves : 8;
+    if constexpr (KS > 0) {
+        if (batch.algorithm == 2) {
+            // super-groups per wave: enough waves to fill the chip (~8192), at least `min_supers` of them per
+            // wave so that the lhs slices and the row search are amortised, at most 16
+            const long long n_supers = ((long long)nonzeros_vec + 16 * GRP - 1) / (16 * GRP);
+            long long supers = (n_supers * batch.count + 8191) / 8192;
+            const int min_supers = options().sddmm_flat_supers > 0 ? options().sddmm_flat_supers : (KS >= 8 ? 4 : (KS >= 4 ? 2 : 1));
+            if (supers < min_supers) supers = min_supers;
+            if (supers > 16) supers = 16;
+            const long long flat_waves = (n_supers + supers - 1) / supers;
+            const long long flat_blocks = (flat_waves + 7) / 8;
+            if (flat_blocks > 0x7fffffffLL) return hipErrorNotSupported;
+            hipLaunchKernelGGL((sddmm_mfma_flat_kernel<V, KS, GRP, OutT>), dim3((unsigned)flat_blocks, (unsigned)batch.count),
+                               dim3(512), 0, stream, m_vec, k, nonzeros_vec, (int)supers, row_offsets, col_indices, lhs, rhs,
+                               out, batch.stride_a, batch.stride_b, batch.stride_out);
+            return (int)hipGetLastError();
+        }
+    }
     const int slots = sddmm_auto_slots(m_vec * batch.count, nonzeros_vec * batch.count, 16 * GRP);
     const long long waves = (long long)m_vec * slots;
     const long long blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;

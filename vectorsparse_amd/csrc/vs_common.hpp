@@ -187,6 +187,7 @@ struct Options {
     int spmm_cols_per_lane = 0;
     int sddmm_slots = 0;
     int sddmm_block_waves = 0;
+    int sddmm_flat_supers = 0;  // flat MFMA SDDMM (algorithm 2): super-groups per wave, 0 = automatic
     int attention_waves = 0;
     int attention_chunk = 0;
 };
@@ -205,6 +206,7 @@ struct Batch {
     long long stride_b = 0;    // SpMM: rhs_matrix    SDDMM: rhs_matrix
     long long stride_out = 0;  // SpMM: output_matrix SDDMM: output_values
     int nonzeros_vec = -1;     // SpMM: nonzero vectors of the pattern when the caller knows them (launch-shape hint)
+    int algorithm = 0;         // SDDMM on MFMA: 2 = waves split the nonzero range, else (row, slot) per wave
 };
 
 // Launchers (one per kernel family); return a hipError_t-valued int.

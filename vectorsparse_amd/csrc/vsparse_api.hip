@@ -122,11 +122,13 @@ int vs_wmma_sddmm_f16(int m_vec, int k, int n, int nonzeros_vec, const int *row_
     int st = check_sddmm(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices, lhs_matrix, rhs_matrix,
                          output_values, vec_length, sizeof(half_t));
     if (st != VS_SUCCESS) return st;
+    vs::Batch one;
+    one.algorithm = algorithm;
     return vs::launch_sddmm_mfma<half_t>(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices,
                                          static_cast<const half_t *>(lhs_matrix),
                                          static_cast<const half_t *>(rhs_matrix),
                                          static_cast<half_t *>(output_values), vec_length,
-                                         static_cast<hipStream_t>(stream));
+                                         static_cast<hipStream_t>(stream), one);
 }
 
 int vs_wmma_sddmm_f16_f32out(int m_vec, int k, int n, int nonzeros_vec, const int *row_indices,
@@ -138,10 +140,12 @@ int vs_wmma_sddmm_f16_f32out(int m_vec, int k, int n, int nonzeros_vec, const in
     int st = check_sddmm(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices, lhs_matrix, rhs_matrix,
                          output_values, vec_length, sizeof(float));
     if (st != VS_SUCCESS) return st;
+    vs::Batch one;
+    one.algorithm = algorithm;
     return vs::launch_sddmm_mfma<float>(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices,
                                         static_cast<const half_t *>(lhs_matrix),
                                         static_cast<const half_t *>(rhs_matrix), output_values, vec_length,
-                                        static_cast<hipStream_t>(stream));
+                                        static_cast<hipStream_t>(stream), one);
 }
 
 int vs_cuda_sddmm_f16(int m_vec, int k, int n, int nonzeros_vec, const int *row_indices, const int *row_offsets,
@@ -233,12 +237,13 @@ int vs_wmma_sddmm_f16_batched(int batch, int m_vec, int k, int n, int nonzeros_v
     if (st != VS_SUCCESS) return st;
     if (!stride_ok(stride_lhs, 8) || !stride_ok(stride_rhs, 8) || !stride_ok(stride_output, vec_length))
         return VS_ERROR_INVALID_VALUE;
+    vs::Batch many = make_batch(batch, stride_lhs, stride_rhs, stride_output);
+    many.algorithm = algorithm;
     return vs::launch_sddmm_mfma<half_t>(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices,
                                          static_cast<const half_t *>(lhs_matrix),
                                          static_cast<const half_t *>(rhs_matrix),
                                          static_cast<half_t *>(output_values), vec_length,
-                                         static_cast<hipStream_t>(stream),
-                                         make_batch(batch, stride_lhs, stride_rhs, stride_output));
+                                         static_cast<hipStream_t>(stream), many);
 }
 
 int vs_cuda_sddmm_f16_batched(int batch, int m_vec, int k, int n, int nonzeros_vec, const int *row_indices,
@@ -376,6 +381,9 @@ int vs_set_option(const char *name, int value)
         o.spmm_cols_per_lane = value;
     } else if (std::strcmp(name, "sddmm_slots") == 0) {
         o.sddmm_slots = value;
+    } else if (std::strcmp(name, "sddmm_flat_supers") == 0) {
+        if (value > 16) return VS_ERROR_INVALID_VALUE;
+        o.sddmm_flat_supers = value;
     } else if (std::strcmp(name, "sddmm_block_waves") == 0) {
         if (value > 16) return VS_ERROR_INVALID_VALUE;
         o.sddmm_block_waves = value;

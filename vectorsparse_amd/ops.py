@@ -363,6 +363,9 @@ class DeviceProblem:
         self.vec_length = pattern.vec_length
         self.n = pattern.n
         self.nnz_vec = pattern.nnz_vec
+        lengths = np.diff(pattern.row_offsets)
+        # a few rows far longer than the rest: schedules that give every row the same number of waves stall on them
+        self.skewed = bool(pattern.nnz_vec >= 65536 and lengths.max() >= 8 * max(1.0, lengths.mean()))
         swz = SortedRowSwizzle(pattern.m_vec, pattern.row_offsets) if sort else IdentityRowSwizzle(pattern.m_vec)
         self.row_indices = torch.from_numpy(swz).to(device)
         self.row_offsets = torch.from_numpy(np.ascontiguousarray(pattern.row_offsets)).to(device)
@@ -388,10 +391,14 @@ class DeviceProblem:
                   self.column_indices, self.values, rhs_matrix, out, stream)
 
     def sddmm(self, lhs_matrix, rhs_matrix, kernel="wmma", out_dtype=torch.float16, out=None, stream=None,
-              algorithm=1):
+              algorithm=None):
+        """SDDMM on the mask.  algorithm (MFMA path): 1 = a wave per (row, slot), 2 = waves split the nonzero
+        range (robust to skewed row lengths); None picks 2 for large, heavily skewed masks, else 1."""
         k = lhs_matrix.shape[1]
         if out is None:
             out = torch.empty((self.nnz_vec, self.vec_length), dtype=out_dtype, device=lhs_matrix.device)
+        if algorithm is None:
+            algorithm = 2 if (self.skewed and k <= 256) else 1
         if kernel == "wmma":
             return sddmm.wmmaSddmm(self.m_vec, k, self.n, self.nnz_vec, self.row_indices, self.row_offsets,
                                    self.column_indices, lhs_matrix, rhs_matrix, out, self.vec_length, stream,
