@@ -173,20 +173,31 @@ sddmm_mfma_flat_kernel(int m_vec, int K, int nonzeros_vec, int supers, const int
     };
     fetch_cols(range_begin);
 
-    // the last row index i in [0, m_vec] with row_offsets[i] <= range_begin (skips empty rows that start there)
+    // The last row index i in [0, m_vec] with row_offsets[i] <= range_begin (skips empty rows that start
+    // there).  The final round probes consecutive offsets, which are also the row ends the walk below needs:
+    // they are shifted into place (lane l: end of row base_row + l) instead of being loaded again.
     int lo = 0, span = m_vec + 1;
-    while (span > 1) {
-        const int step = (span + 63) >> 6;
+    int probe = 0, k = 0, step = 1;
+    do {
+        step = (span + 63) >> 6;
         const int idx = lo + lane * step;
-        const int val = idx < lo + span ? row_offsets[idx] : 0x7fffffff;
-        const int below = __builtin_popcountll(__builtin_amdgcn_ballot_w64(val <= range_begin));  // a prefix of the lanes
-        const int k = below > 0 ? below - 1 : 0;
+        probe = idx < lo + span ? row_offsets[idx] : 0x7fffffff;
+        const int below = __builtin_popcountll(__builtin_amdgcn_ballot_w64(probe <= range_begin));  // a prefix of the lanes
+        k = below > 0 ? below - 1 : 0;
         lo += k * step;
         span = span - k * step < step ? span - k * step : step;
-    }
+    } while (span > 1);
     int base_row = lo;
     if (base_row >= m_vec) return;  // nonzeros_vec exceeds row_offsets[m_vec]: nothing of the pattern is here
-    int ends = row_offsets[base_row + 1 + lane <= m_vec ? base_row + 1 + lane : m_vec];  // lane l: end of row base_row + l
+    int ends;  // lane l: end of row base_row + l (row_offsets[base_row + 1 + l], clamped to the last offset)
+    if (step == 1) {
+        // probe of lane l is row_offsets[base_row - k + l] (0x7fffffff past the array): take lane l + k + 1
+        const int shifted = __builtin_amdgcn_ds_bpermute(((lane + k + 1) & 63) << 2, probe);
+        const bool have = lane + k + 1 < 64 && shifted != 0x7fffffff;
+        ends = have ? shifted : row_offsets[base_row + 1 + lane <= m_vec ? base_row + 1 + lane : m_vec];
+    } else {
+        ends = row_offsets[base_row + 1 + lane <= m_vec ? base_row + 1 + lane : m_vec];
+    }
     int ri = 0;        // row base_row + ri is the candidate for the next nonzero
     int cur_row = -1;  // row whose lhs slices are in `a`
     half8_t a[KS];
