@@ -1,6 +1,6 @@
-"""ResNet-50-shaped SpMM sweep against dense fp16 GEMM.
+"""ResNet-50-shaped SpMM sweep (and a square-mask SDDMM sweep) against dense fp16 GEMM.
 
-    python -m vectorsparse_amd.sweep --out results.csv [--quick]
+    python -m vectorsparse_amd.sweep --out results.csv [--quick] [--op spmm|sddmm]
 
 The counterpart of the reference's experiment driver (launch.py:11-36 -> job_launcher.py:38-63 ->
 ncu_profile.py:80-96, then plot_spmm.py:43-58): for every (M, K, sparsity, V) of the grid it times
@@ -37,11 +37,67 @@ def geomean(xs):
     return math.exp(sum(math.log(x) for x in xs) / len(xs)) if xs else float("nan")
 
 
+def sddmm_bytes(pat, k):
+    n_ref = int(np.unique(pat.column_indices[:pat.nnz_vec]).size)
+    return 2 * pat.m * k + 2 * n_ref * k + 4 * pat.nnz_vec + 4 * (pat.m_vec + 1) + 4 * pat.m_vec + 2 * pat.nnz
+
+
+def sddmm_sweep(args, torch, cv, ops, time_launches):
+    sizes, ks, ss = ((512, 1024, 2048, 4096), (64, 128, 256), SPARSITIES) if not args.quick else \
+        ((512, 2048), (64, 256), (0.7, 0.9, 0.98))
+    rows, dense_us = [], {}
+    for M in sizes:
+        for K in ks:
+            A = torch.randn((M, K), dtype=torch.float16, device="cuda")
+            B = torch.randn((M, K), dtype=torch.float16, device="cuda")
+            full = torch.empty((M, M), dtype=torch.float16, device="cuda")
+            dense_us[(M, K)] = time_launches(torch, lambda: torch.matmul(A, B.t(), out=full), args.iters)
+            for s in ss:
+                for V in VS:
+                    seed = (M * 1000003 + K * 10007 + int(round(s * 100)) * 101 + V) % (2 ** 31)
+                    pat = cv.uniform_pattern(M // V, M, s, seed, V)
+                    prob = ops.DeviceProblem(pat, sort=True)
+                    out = torch.empty((pat.nnz_vec, V), dtype=torch.float16, device="cuda")
+                    flops = 2.0 * pat.nnz * K
+                    for kernel in ("wmma", "cuda"):
+                        us = time_launches(torch, lambda: prob.sddmm(A, B, kernel=kernel, out=out), args.iters)
+                        rows.append({"bm": "synthetic", "M": M, "K": K, "N": M, "sparsity": round(s, 4), "V": V,
+                                     "kernel": kernel, "nnz_vec": pat.nnz_vec, "us": round(us, 3),
+                                     "dense_us": round(dense_us[(M, K)], 3),
+                                     "speedup": round(dense_us[(M, K)] / us, 4),
+                                     "tflops": round(flops / us * 1e-6, 3),
+                                     "gbs": round(sddmm_bytes(pat, K) / us * 1e-3, 1)})
+                    print("M=N=%d K=%d s=%.2f V=%d  wmma %.2f us  cuda %.2f us  dense %.2f us" % (
+                        M, K, s, V, rows[-2]["us"], rows[-1]["us"], dense_us[(M, K)]), flush=True)
+    report(args.out, rows, "SDDMM: geometric-mean speed-up over the dense fp16 product A B^T (hipBLASLt)")
+    return 0
+
+
+def report(path, rows, title):
+    with open(path, "w", newline="") as f:
+        w = csv.DictWriter(f, fieldnames=list(rows[0].keys()))
+        w.writeheader()
+        w.writerows(rows)
+    print("\n" + title + ", by vector length and sparsity")
+    buckets = sorted({r["sparsity"] for r in rows})
+    print("%-12s" % "kernel/V" + "".join("%9s" % ("s=%.2f" % b) for b in buckets))
+    for kernel in ("wmma", "cuda"):
+        for V in VS:
+            line = "%-12s" % ("%s V=%d" % (kernel, V))
+            for b in buckets:
+                xs = [r["speedup"] for r in rows if r["kernel"] == kernel and r["V"] == V and r["sparsity"] == b]
+                line += "%9.2f" % geomean(xs)
+            print(line)
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--out", default="spmm_sweep.csv")
     ap.add_argument("--quick", action="store_true", help="a 3 x 3 x 3 corner of the grid")
     ap.add_argument("--smtx-dir", default=None, help="sweep every .smtx under this directory instead")
+    ap.add_argument("--op", choices=["spmm", "sddmm"], default="spmm",
+                    help="sddmm: masks of M = N in {512, 1024, 2048, 4096} x contraction K in {64, 128, 256} "
+                         "(the counterpart of the reference's SDDMM figure), dense baseline = the full A B^T")
     ap.add_argument("--hint", action="store_true",
                     help="call through the batched entry point with the pattern's nonzero count (workgroups sized "
                          "by the real row lengths) instead of the reference-shaped entry points")
@@ -54,6 +110,8 @@ def main(argv=None):
     from . import ops
     from .benchmark_common import time_launches
 
+    if args.op == "sddmm":
+        return sddmm_sweep(args, torch, cv, ops, time_launches)
     ms, ks, ss = (MS, KS, SPARSITIES) if not args.quick else ((64, 512, 2048), (256, 1152, 4608), (0.7, 0.9, 0.98))
     cases = []
     if args.smtx_dir:
@@ -97,21 +155,7 @@ def main(argv=None):
         print("M=%d K=%d s=%.2f V=%d  wmma %.2f us  cuda %.2f us  dense %.2f us" % (
             M, K, s, V, rows[-2]["us"], rows[-1]["us"], dense_us[(M, K)]), flush=True)
 
-    with open(args.out, "w", newline="") as f:
-        w = csv.DictWriter(f, fieldnames=list(rows[0].keys()))
-        w.writeheader()
-        w.writerows(rows)
-
-    print("\ngeometric-mean speed-up over dense fp16 GEMM (hipBLASLt), by vector length and sparsity")
-    buckets = sorted({r["sparsity"] for r in rows})
-    print("%-12s" % "kernel/V" + "".join("%9s" % ("s=%.2f" % b) for b in buckets))
-    for kernel in ("wmma", "cuda"):
-        for V in VS:
-            line = "%-12s" % ("%s V=%d" % (kernel, V))
-            for b in buckets:
-                xs = [r["speedup"] for r in rows if r["kernel"] == kernel and r["V"] == V and r["sparsity"] == b]
-                line += "%9.2f" % geomean(xs)
-            print(line)
+    report(args.out, rows, "SpMM: geometric-mean speed-up over dense fp16 GEMM (hipBLASLt)")
     return 0
 
 
