@@ -274,8 +274,11 @@ void vs_sorted_row_swizzle(int rows, const int *row_offsets, int *row_indices);
  * Launch-shape tuning knob (process-wide, not thread-safe against concurrent
  * launches).  Names: "spmm_waves" (waves per workgroup, 0 = automatic),
  * "spmm_cols_per_lane" (4, 8, 0 = automatic), "sddmm_slots" (waves per
- * vector row, 0 = automatic), "sddmm_block_waves" (1..16, 0 = automatic), "attention_waves" (1..8, 0 = automatic),
- * "attention_chunk" (nonzero vectors per LDS chunk, 0 = automatic).  Returns 0, or 1 for an unknown name / bad value.
+ * vector row, 0 = automatic), "sddmm_block_waves" (1..16, 0 = automatic),
+ * "sddmm_flat_supers" (super-groups per wave of algorithm 2, 1..16, 0 = automatic),
+ * "attention_waves" (1..8, 0 = automatic), "attention_chunk" (nonzero vectors per
+ * LDS chunk of the one-row-per-workgroup attention kernel, 0 = automatic).
+ * Returns 0, or 1 for an unknown name / bad value.
  * No counterpart in the reference, whose tile sizes are compile-time constants
  * (src/wmma_spmm.cu:396).
  */
