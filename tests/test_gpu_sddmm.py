@@ -196,3 +196,23 @@ def test_algorithm_2_splits_the_nonzero_range_same_bits(gpu, V):
                          torch.from_numpy(cv.dense_normal(n, 64, seed=65)).cuda(), kernel="wmma", algorithm=2)
         torch.cuda.synchronize()
         assert_parity(got.cpu().numpy().reshape(-1), ref, name)
+
+
+def test_algorithm_2_batched_equals_unbatched(gpu):
+    V, heads, n, K = 8, 3, 640, 64
+    rng = np.random.default_rng(5)
+    lengths = np.minimum((rng.pareto(1.3, 90) + 0.1) * 30, n).astype(np.int64)
+    ro, ci = cv._pattern_from_lengths(rng, 90, n, lengths)
+    mask = cv.ColVecCSR(90, n, V, ro, ci)
+    prob = ops.DeviceProblem(mask)
+    g = torch.Generator(device="cuda").manual_seed(1)
+    A = torch.randn((heads, mask.m, K), device="cuda", generator=g).half()
+    B = torch.randn((heads, n, K), device="cuda", generator=g).half()
+    out = torch.empty((heads, mask.nnz_vec, V), dtype=torch.float16, device="cuda")
+    ops.sddmm_batched(mask.m_vec, K, n, mask.nnz_vec, prob.row_indices, prob.row_offsets, prob.column_indices, A, B, out,
+                      V, algorithm=2)
+    torch.cuda.synchronize()
+    for h in range(heads):
+        one = prob.sddmm(A[h], B[h], algorithm=1)
+        torch.cuda.synchronize()
+        assert torch.equal(out[h], one), "head %d" % h
