@@ -179,6 +179,16 @@ int launch_spmm_valu(int m_vec, int vec_length, int k, int n, const int *row_ind
         const long long blocks = (long long)m_vec * ceil_div(k, 512) * batch.count;
         waves = 2;
         while (waves < 8 && blocks * waves < 8192) waves <<= 1;
+        if (batch.nonzeros_vec >= 0) {
+            // Row lengths known (batched entry points): a wave consumes 4 nonzeros per group and turn, and a
+            // turn is one memory round trip, so a wave per turn of an average row is as wide as it pays.
+            const int groups = k <= 64 ? 8 : (k <= 128 ? 4 : (k <= 256 ? 2 : 1));
+            // (V = 8 does eight times the arithmetic per nonzero: twice the waves measured better)
+            const int turns = ceil_div(ceil_div(batch.nonzeros_vec, m_vec), 4 * groups) * (vec_length == 8 ? 2 : 1);
+            int by_rows = 1;
+            while (by_rows < turns) by_rows <<= 1;
+            if (waves > by_rows) waves = by_rows;
+        }
     }
     if (waves > 16) waves = 16;
     switch (vec_length) {
