@@ -256,11 +256,13 @@ int vs_sparse_attention_plan(int m_vec, int vec_length, int n, int d_qk, int d_v
 /*
  * Planning helper for rows_per_workgroup >= 2 of vs_sparse_attention_f16: the number of distinct columns
  * a workgroup can hold in LDS for this shape (0: shape not supported by the union kernel), and in
- * *rows_used (may be null) the vector rows per workgroup the request is rounded to.  Host only, no
- * launch.  No counterpart in the reference.
+ * *rows_used (may be null) the vector rows per workgroup the request is rounded to.  with_plan: nonzero
+ * for launches that pass a plan - they keep only the K / V rows and the row masks in LDS, so they hold
+ * more columns (up to 512) and accept a larger n than launches that rebuild the union (up to 480).
+ * Host only, no launch.  No counterpart in the reference.
  */
 int vs_sparse_attention_union_capacity(int vec_length, int n, int d_qk, int d_v, int rows_per_workgroup,
-                                       int *rows_used);
+                                       int with_plan, int *rows_used);
 
 /*
  * Host helpers (HOST pointers).  Replace IdentityRowSwizzle / SortedRowSwizzle —

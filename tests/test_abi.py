@@ -87,21 +87,26 @@ def test_attention_planning_helpers_are_consistent():
     for V in (1, 2, 4, 8):
         per_wave = 16 // V
         for request in (2, per_wave, 3 * per_wave + 1, 8 * per_wave, 128):
-            cap = L.vs_sparse_attention_union_capacity(V, 4096, 64, 64, request, ctypes.addressof(used))
-            assert cap > 0 and cap % 32 == 0
+            built = L.vs_sparse_attention_union_capacity(V, 4096, 64, 64, request, 0, None)
+            cap = L.vs_sparse_attention_union_capacity(V, 4096, 64, 64, request, 1, ctypes.addressof(used))
+            assert cap > 0 and cap % 32 == 0 and 0 < built <= cap <= 512    # a plan frees LDS for more columns
             assert used.value % per_wave == 0 and used.value <= 8 * per_wave      # whole waves, at most 8
             assert used.value >= min(request, 8 * per_wave)
             blocks = -(-512 // used.value)
             size = L.vs_sparse_attention_plan_bytes(512, V, 4096, 64, 64, request)
-            mask_words = (used.value * 14 + 3) // 4 * 4
+            mask_words = (used.value * 16 + 3) // 4 * 4
             assert size == 4 * (16 + blocks * (4 + mask_words + cap))
-    wide = L.vs_sparse_attention_union_capacity(8, 4096, 128, 128, 16, None)
-    narrow = L.vs_sparse_attention_union_capacity(8, 4096, 32, 32, 16, None)
+    wide = L.vs_sparse_attention_union_capacity(8, 4096, 128, 128, 16, 0, None)
+    narrow = L.vs_sparse_attention_union_capacity(8, 4096, 32, 32, 16, 0, None)
     assert 0 < wide < narrow                                   # wider rows: fewer of them fit in LDS
-    assert L.vs_sparse_attention_union_capacity(8, 4096, 64, 36, 16, None) == 0    # d_v % 8 != 0: per-row path only
-    assert L.vs_sparse_attention_union_capacity(8, 4096, 256, 64, 16, None) == 0   # d_qk > 128
-    assert L.vs_sparse_attention_union_capacity(8, 1 << 22, 64, 64, 16, None) == 0  # column bitmap too large for LDS
-    assert L.vs_sparse_attention_union_capacity(3, 4096, 64, 64, 16, None) == 0
+    assert L.vs_sparse_attention_union_capacity(8, 4096, 64, 36, 16, 0, None) == 0    # d_v % 8 != 0: per-row path only
+    assert L.vs_sparse_attention_union_capacity(8, 4096, 256, 64, 16, 0, None) == 0   # d_qk > 128
+    for with_plan in (0, 1):
+        assert L.vs_sparse_attention_union_capacity(8, 1 << 22, 64, 64, 16, with_plan, None) == 0  # column bitmap too large for LDS
+    # the bitmap of 400k columns fits the plan kernel's LDS but not beside the K / V rows
+    assert L.vs_sparse_attention_union_capacity(8, 400000, 64, 64, 16, 0, None) == 0
+    assert L.vs_sparse_attention_union_capacity(8, 400000, 64, 64, 16, 1, None) > 0
+    assert L.vs_sparse_attention_union_capacity(3, 4096, 64, 64, 16, 0, None) == 0
     assert L.vs_sparse_attention_plan_bytes(512, 8, 4096, 64, 64, 1) == 0
     # a plan buffer that is too small, null or misaligned is rejected before any launch
     assert L.vs_sparse_attention_plan(512, 8, 4096, 64, 64, 16, 64, 64, 256, 16, None) == 1

@@ -273,6 +273,45 @@ def _with_empty_rows(mask, first, last):
     return cv.ColVecCSR(mask.m_vec, mask.n, mask.vec_length, offsets, mask.column_indices[keep].copy())
 
 
+def _capacity(V, n, d_qk, d_v, rows, with_plan):
+    from vectorsparse_amd import _lib
+    return _lib.lib().vs_sparse_attention_union_capacity(V, n, d_qk, d_v, rows, with_plan, None)
+
+
+def _unions(mask, rows):
+    """Distinct columns of every block of `rows` consecutive vector rows."""
+    ro, ci = mask.row_offsets, mask.column_indices
+    return [int(np.unique(ci[ro[f]:ro[min(f + rows, mask.m_vec)]]).size) for f in range(0, mask.m_vec, rows)]
+
+
+@pytest.mark.parametrize("V,seq,half_width,stride,rows", [(4, 4096, 176, 32, 8), (1, 2048, 128, 16, 128)])
+def test_plan_raises_the_union_capacity(gpu, V, seq, half_width, stride, rows):
+    """Blocks whose distinct columns fit a workgroup's LDS only when the column bitmap and the column list
+    stay out of it: dense tile with a plan, per-row path without, both equal to dense masked attention."""
+    d = 64
+    mask = cv.band_strided_pattern(seq, V, band_half_width=half_width, stride=stride)
+    built, held = _capacity(V, seq, d, d, rows, 0), _capacity(V, seq, d, d, rows, 1)
+    unions = _unions(mask, rows)
+    assert built < max(unions) <= held and min(unions) <= built, (built, held, min(unions), max(unions))
+    rng = np.random.default_rng(70 + V)
+    q, k, v = (rng.standard_normal((1, seq, d)).astype(np.float16) for _ in range(3))
+    qd, kd, vd = (torch.from_numpy(x).cuda() for x in (q, k, v))
+    ref = _dense_attention(mask, q, k, v, 0.125)
+    layer = ops.SparseAttention(mask)
+    assert layer.union_rows(d, d) == rows                 # the host-side choice counts on the plan
+    prob = layer.prob
+    args = (mask.m_vec, V, seq, prob.row_indices, prob.row_offsets, prob.column_indices, qd, kd, vd)
+    plan = ops.sparse_attention_plan(mask.m_vec, V, seq, d, d, rows, prob.row_offsets, prob.column_indices)
+    planned = ops.sparse_attention(*args, scale=0.125, rows_per_workgroup=rows, plan=plan)
+    rebuilt = ops.sparse_attention(*args, scale=0.125, rows_per_workgroup=rows)
+    out = layer.forward(qd, kd, vd, scale=0.125)
+    torch.cuda.synchronize()
+    _check_layer(planned.cpu().numpy(), ref, "V%d planned" % V)
+    _check_layer(rebuilt.cpu().numpy(), ref, "V%d rebuilt" % V)
+    _check_layer(out.cpu().numpy(), ref, "V%d layer" % V)
+    assert not torch.equal(planned, rebuilt)              # different summation orders: the paths did differ
+
+
 @pytest.mark.parametrize("V", [1, 8])
 def test_planned_launch_equals_unplanned(gpu, V):
     """The plan holds exactly what the kernel would rebuild: same bits out.  A plan made for another launch
@@ -297,7 +336,12 @@ def test_planned_launch_equals_unplanned(gpu, V):
             planned = ops.sparse_attention(*args, scale=0.125, rows_per_workgroup=rows, plan=plan)
             torch.cuda.synchronize()
             _check_layer(planned.cpu().numpy(), ref, "%s V%d rows%d planned" % (name, V, rows))
-            assert torch.equal(plain, planned), "%s V%d rows%d" % (name, V, rows)
+            # a planned launch holds more columns per workgroup: same bits unless some union fits only then
+            built, held = _capacity(V, seq, d, d, rows, 0), _capacity(V, seq, d, d, rows, 1)
+            if not any(built < u <= held for u in _unions(mask, rows)):
+                assert torch.equal(plain, planned), "%s V%d rows%d" % (name, V, rows)
+            else:
+                _check_layer(plain.cpu().numpy(), ref, "%s V%d rows%d rebuilt" % (name, V, rows))
         # a negative scale (sign handled inside the kernel) through the same paths
         neg = ops.sparse_attention(*args, scale=-0.125, rows_per_workgroup=128 // V, plan=plan)
         torch.cuda.synchronize()

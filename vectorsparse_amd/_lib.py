@@ -30,7 +30,7 @@ SIGNATURES = {
     "vs_sparse_attention_f16": ([_int] * 6 + [_vp] * 3 + [_vp, _ll, _vp, _ll, _vp, _ll, _vp, _ll, ctypes.c_float, _int,
                                  _vp, _vp],
                                 _int),
-    "vs_sparse_attention_union_capacity": ([_int] * 5 + [_vp], _int),
+    "vs_sparse_attention_union_capacity": ([_int] * 6 + [_vp], _int),
     "vs_sparse_attention_plan_bytes": ([_int] * 6, _ll),
     "vs_sparse_attention_plan": ([_int] * 6 + [_vp] * 3 + [_ll, _vp], _int),
     "vs_sparse_softmax_f16": ([_int] * 3 + [_vp] * 2 + [_vp, _ll, _vp, _ll, ctypes.c_float, _vp], _int),

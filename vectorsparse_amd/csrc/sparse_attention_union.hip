@@ -38,7 +38,7 @@
 namespace vs {
 
 constexpr int kMaxSteps = 10;   // fallback: 32-vector steps of a row whose scores are held in registers at once
-constexpr int kUnionSteps = 14; // 32-rank steps of the union whose probabilities are held in registers at once
+constexpr int kUnionSteps = 16; // 32-rank steps of the union whose probabilities are held in registers at once
 
 // Value of `x` held by lane `src_lane` (all lanes active).
 __device__ __forceinline__ float from_lane(float x, int src_lane)
@@ -689,10 +689,11 @@ struct UnionShape {
     size_t lds;
 };
 
-static bool union_shape(UnionShape &s, int vec_length, int n, int d_qk, int d_v, int rows)
+static bool union_shape(UnionShape &s, int vec_length, int n, int d_qk, int d_v, int rows, bool planned)
 {
-    // Half of a CU's LDS per workgroup, so that two workgroups overlap each other's memory phases.
-    constexpr size_t kLdsBudget = 72 * 1024;
+    // Half of a CU's LDS per workgroup, so that two workgroups overlap each other's memory phases.  With a
+    // plan the column bitmap, its prefix sums and the column list stay out of the attention kernel's LDS.
+    const size_t budget = (planned ? 80 : 72) * 1024;
     const int rpw = 16 / vec_length;
     s.waves = ceil_div(rows < 1 ? 1 : rows, rpw);
     if (s.waves > 8) s.waves = 8;
@@ -700,12 +701,15 @@ static bool union_shape(UnionShape &s, int vec_length, int n, int d_qk, int d_v,
     const int ks = d_qk <= 32 ? 1 : (d_qk <= 64 ? 2 : 4);
     const int cpl = d_v <= 64 ? 4 : 8;
     const int n_words = (((n + 31) / 32) + 3) & ~3;
-    const size_t fixed = 2 * (size_t)n_words * sizeof(unsigned) + 16 * sizeof(int) +
-                         (size_t)union_mask_words(s.rows) * sizeof(unsigned);
-    const size_t per_union_row = (size_t)union_pitch(ks, cpl) * sizeof(half_t) + sizeof(int);
-    if (fixed + 32 * per_union_row > kLdsBudget) return false;  // the column bitmap alone fills the budget
-    s.u_max = (int)((kLdsBudget - fixed) / per_union_row) & ~31;
+    const size_t mask = (size_t)union_mask_words(s.rows) * sizeof(unsigned);
+    const size_t build = 2 * (size_t)n_words * sizeof(unsigned) + 16 * sizeof(int) + mask;  // + one int per column
+    const size_t fixed = planned ? mask : build;
+    const size_t per_union_row = (size_t)union_pitch(ks, cpl) * sizeof(half_t) + (planned ? 0 : sizeof(int));
+    if (fixed + 32 * per_union_row > budget) return false;  // the column bitmap alone fills the budget
+    s.u_max = (int)((budget - fixed) / per_union_row) & ~31;
     if (s.u_max > 32 * kUnionSteps) s.u_max = 32 * kUnionSteps;
+    // the plan kernel holds the bitmap and the column list of one workgroup in LDS
+    if (planned && build + (size_t)s.u_max * sizeof(int) > 160 * 1024) return false;
     s.lds = fixed + (size_t)s.u_max * per_union_row;
     return true;
 }
@@ -723,17 +727,13 @@ static int launch_one(int m_vec, int n, int d_qk, int d_v, int rows, const int *
                       hipStream_t stream, const Batch &batch, long long stride_v)
 {
     UnionShape s;
-    if (!union_shape(s, V, n, d_qk, d_v, rows)) return hipErrorNotSupported;
+    if (!union_shape(s, V, n, d_qk, d_v, rows, PLANNED)) return hipErrorNotSupported;
     auto kernel = sparse_attention_union_kernel<V, KS, CPL, PLANNED>;
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr != hipSuccess) return (int)attr;
     const int blocks = ceil_div(m_vec, s.rows);
-    // with a plan only the row masks and the K / V rows live in LDS
-    const size_t lds = PLANNED ? (size_t)union_mask_words(s.rows) * sizeof(unsigned) +
-                                     (size_t)s.u_max * union_pitch(KS, CPL) * sizeof(half_t)
-                               : s.lds;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)batch.count), dim3(64 * s.waves), lds, stream, m_vec,
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)batch.count), dim3(64 * s.waves), s.lds, stream, m_vec,
                        n, d_qk, d_v, s.u_max, row_offsets, col_indices, plan, q, k, v, out, batch.stride_a,
                        batch.stride_b, stride_v, batch.stride_out, scale);
     return (int)hipGetLastError();
@@ -778,11 +778,11 @@ static bool union_supported(int vec_length, int n, int d_qk, int d_v)
     return n >= 0 && n <= 1024 * 1024 && union_dims_ok(d_qk, d_v);  // the column bitmap lives in LDS
 }
 
-int sparse_attention_union_capacity(int vec_length, int n, int d_qk, int d_v, int rows, int *rows_used)
+int sparse_attention_union_capacity(int vec_length, int n, int d_qk, int d_v, int rows, bool with_plan, int *rows_used)
 {
     UnionShape s;
     if (!union_supported(vec_length, n, d_qk, d_v) || d_v % 8 != 0) return 0;
-    if (!union_shape(s, vec_length, n, d_qk, d_v, rows)) return 0;
+    if (!union_shape(s, vec_length, n, d_qk, d_v, rows, with_plan)) return 0;
     if (rows_used) *rows_used = s.rows;
     return s.u_max;
 }
@@ -791,7 +791,7 @@ long long sparse_attention_plan_bytes(int m_vec, int vec_length, int n, int d_qk
 {
     UnionShape s;
     if (m_vec < 0 || !union_supported(vec_length, n, d_qk, d_v)) return 0;
-    if (!union_shape(s, vec_length, n, d_qk, d_v, rows)) return 0;
+    if (!union_shape(s, vec_length, n, d_qk, d_v, rows, true)) return 0;
     const long long stride = 4 + union_mask_words(s.rows) + s.u_max;
     return (long long)sizeof(int) * (kPlanHeader + stride * ceil_div(m_vec, s.rows));
 }
@@ -801,7 +801,7 @@ int launch_sparse_attention_plan(int m_vec, int vec_length, int n, int d_qk, int
 {
     UnionShape s;
     if (!union_supported(vec_length, n, d_qk, d_v)) return hipErrorNotSupported;
-    if (!union_shape(s, vec_length, n, d_qk, d_v, rows)) return hipErrorNotSupported;
+    if (!union_shape(s, vec_length, n, d_qk, d_v, rows, true)) return hipErrorNotSupported;
     const long long need = sparse_attention_plan_bytes(m_vec, vec_length, n, d_qk, d_v, rows);
     if (plan_bytes < need) return hipErrorInvalidValue;
     if (m_vec == 0) return hipSuccess;

@@ -244,7 +244,7 @@ int launch_sparse_attention_union(int m_vec, int vec_length, int n, int d_qk, in
 long long sparse_attention_plan_bytes(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows);
 int launch_sparse_attention_plan(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, const int *row_offsets,
                                  const int *col_indices, int *plan, long long plan_bytes, hipStream_t stream);
-int sparse_attention_union_capacity(int vec_length, int n, int d_qk, int d_v, int rows, int *rows_used);
+int sparse_attention_union_capacity(int vec_length, int n, int d_qk, int d_v, int rows, bool with_plan, int *rows_used);
 int launch_sparse_softmax(int m_vec, int vec_length, const int *row_indices, const int *row_offsets,
                           const half_t *values_in, half_t *values_out, float scale, hipStream_t stream,
                           const Batch &batch = Batch());

@@ -330,10 +330,11 @@ int vs_sparse_attention_plan(int m_vec, int vec_length, int n, int d_qk, int d_v
                                             static_cast<hipStream_t>(stream));
 }
 
-int vs_sparse_attention_union_capacity(int vec_length, int n, int d_qk, int d_v, int rows_per_workgroup, int *rows_used)
+int vs_sparse_attention_union_capacity(int vec_length, int n, int d_qk, int d_v, int rows_per_workgroup, int with_plan,
+                                       int *rows_used)
 {
     if (!vec_ok(vec_length) || n < 0 || rows_per_workgroup < 2 || rows_per_workgroup > 128) return 0;
-    return vs::sparse_attention_union_capacity(vec_length, n, d_qk, d_v, rows_per_workgroup, rows_used);
+    return vs::sparse_attention_union_capacity(vec_length, n, d_qk, d_v, rows_per_workgroup, with_plan != 0, rows_used);
 }
 
 int vs_sparse_softmax_f16(int batch, int m_vec, int vec_length, const int *row_indices, const int *row_offsets,

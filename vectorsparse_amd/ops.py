@@ -279,17 +279,25 @@ class SparseAttention:
     @staticmethod
     def _union_rows(mask, d_qk, d_v, min_fill=0.4):
         """Vector rows per workgroup for the single-launch kernel: the largest block of consecutive rows
-        whose distinct columns fit the library's LDS capacity for this shape in every block and whose
-        dense tile (rows x union) is at least `min_fill` full (banded, blocky or strided masks), else 1
-        (one row per workgroup, any mask)."""
+        whose distinct columns fit the library's LDS capacity for this shape (with a plan) in every block
+        and whose dense tile (rows x union) is at least `min_fill` full (banded, blocky or strided masks),
+        else 1 (one row per workgroup, any mask).
+
+        Every workgroup gathers its whole union, so small workgroups pay the gather for few rows: measured
+        on MI355X (16 heads, 4096 x 4096 band + strided masks with unions near the capacity) two waves
+        beat the per-row kernel only for V <= 4 (132 us against 165 us at V = 4, 133 us against 99 us at
+        V = 8) and a single wave only for V = 1 (385 us against 481 us)."""
         ro, ci = mask.row_offsets, mask.column_indices
         if mask.m_vec == 0 or mask.nnz_vec == 0:
             return 1
         per_wave = 16 // mask.vec_length
-        for waves in (8, 4, 2):
+        min_waves = {1: 1, 2: 2, 4: 2, 8: 4}[mask.vec_length]
+        for waves in (8, 4, 2, 1):
+            if waves < min_waves:
+                break
             used = ctypes.c_int(0)
             cap = _lib.lib().vs_sparse_attention_union_capacity(mask.vec_length, mask.n, d_qk, d_v, waves * per_wave,
-                                                                ctypes.addressof(used))
+                                                                1, ctypes.addressof(used))
             rows = used.value
             if cap <= 0 or rows != waves * per_wave:
                 continue
