@@ -81,3 +81,34 @@ def test_host_swizzle_mirror():
     ro = np.array([0, 3, 3, 10, 12, 19], np.int32)
     assert cv.identity_row_swizzle(5).tolist() == [0, 1, 2, 3, 4]
     assert cv.sorted_row_swizzle(ro).tolist() == [2, 4, 0, 3, 1]
+
+
+def test_duration_files_follow_the_plot_scripts_layout(tmp_path):
+    """Names as file_name_server.py:6-45 builds them; records as its reader (:57-81) sums them: for every row
+    whose fourth field from the end contains "Duration", the next-to-last field in the unit before it."""
+    import csv
+    from vectorsparse_amd import benchmark_common as bc
+
+    root = str(tmp_path)
+    bm = "dlmc/rn50/random_pruning/0.8/bottleneck_1_block_group1_1_1.smtx"
+    stem = "dlmc/rn50/random_pruning/0.8/bottleneck_1_block_group1_1_1"
+    assert bc.duration_csv_path(root, bm, 256, 8, "wmma", "spmm") == \
+        "%s/spmm/%s_wmma_half_sort_k256_v8.csv" % (root, stem)
+    assert bc.duration_csv_path(root, bm, 64, 4, "dense", "spmm", sort=False) == \
+        "%s/spmm/%s_dense_half_k64_v4.csv" % (root, stem)
+    assert bc.duration_csv_path(root, bm, 128, 2, "wmma", "sddmm", sddmm_alg=2) == \
+        "%s/sddmm/%s_wmma_half_sort_mma_shfl_k128_v2.csv" % (root, stem)
+    assert bc.duration_csv_path(root, bm, 128, 2, "cuda", "sddmm", precision="single") == \
+        "%s/sddmm/%s_cuda_single_sort_k128_v2.csv" % (root, stem)
+    with pytest.raises(ValueError):
+        bc.duration_csv_path(root, bm, 128, 2, "sputnik", "spmm")
+
+    path = bc.duration_csv_path(root, bm, 256, 8, "wmma", "spmm")
+    bc.write_duration_csv(path, "spmm_mfma_kernel", 3.84)
+    total_ms = 0.0
+    with open(path) as f:
+        for row in csv.reader(f):
+            if len(row) >= 4 and "Duration" in row[-4]:
+                assert row[-3] == "nsecond"
+                total_ms += float(row[-2]) / 1e6
+    assert total_ms == pytest.approx(3.84e-3)

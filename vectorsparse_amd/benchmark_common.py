@@ -66,3 +66,39 @@ def verdict(name, got, ref):
         print("Results verified: they agree.")
     print("max relative error %.3e (%s 1e-2)" % (rel, "<=" if rel <= 1e-2 else ">"))
     return errors == 0 and rel <= 1e-2
+
+
+_SDDMM_ALGORITHMS = {0: "wmma", 1: "mma_reg", 2: "mma_shfl", 3: "mma_arch"}
+
+
+def duration_csv_path(root, bm, dim_k, dim_v, kernel, job, sort=True, precision="half", sddmm_alg=1):
+    """Path of the per-run duration file for one (benchmark, k, v, kernel) point, laid out the way the
+    reference's plot scripts look it up (file_name_server.py:6-45): `<root>/<job>/<bm>_<kernel>_<precision>
+    [_sort][_<sddmm algorithm>]_k<k>_v<v>.csv`, where `bm` is the benchmark's name below the data set root
+    without its extension and `kernel` is "wmma", "cuda" or "dense"."""
+    if kernel not in ("wmma", "cuda", "dense"):
+        raise ValueError("kernel must be wmma, cuda or dense")
+    if job not in ("spmm", "sddmm"):
+        raise ValueError("job must be spmm or sddmm")
+    name = bm[:-len(".smtx")] if bm.endswith(".smtx") else bm
+    name += "_%s_%s" % (kernel, "half" if precision == "half" else "single")
+    if sort:
+        name += "_sort"
+    if job == "sddmm" and kernel == "wmma":
+        name += "_" + _SDDMM_ALGORITHMS.get(sddmm_alg, "mma_reg")
+    return os.path.join(root, job, "%s_k%d_v%d.csv" % (name, dim_k, dim_v))
+
+
+def write_duration_csv(path, kernel_name, duration_us, process="vectorsparse_amd"):
+    """One profiler-style record per kernel launch of the run: the reference's reader
+    (file_name_server.py:57-81) sums, over the rows of the file, the value in the next-to-last field of every
+    row whose fourth field from the end contains "Duration", with the unit ("nsecond") in between."""
+    os.makedirs(os.path.dirname(path), exist_ok=True)
+    header = ["ID", "Process ID", "Process Name", "Host Name", "Kernel Name", "Kernel Time", "Context", "Stream",
+              "Section Name", "Metric Name", "Metric Unit", "Metric Value", "Rule Name"]
+    stamp = time.strftime("%Y-%b-%d %H:%M:%S")
+    with open(path, "w") as f:
+        f.write(",".join('"%s"' % h for h in header) + "\n")
+        row = ["0", str(os.getpid()), process, "127.0.0.1", kernel_name, stamp, "1", "0", "GPU Speed Of Light",
+               "Duration", "nsecond", "%.0f" % (duration_us * 1e3), ""]
+        f.write(",".join('"%s"' % x for x in row[:-1]) + ",\n")

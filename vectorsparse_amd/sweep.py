@@ -9,6 +9,8 @@ reports speed-up = dense duration / kernel duration with the geometric mean per 
 bucket.  Patterns are synthetic (uniform vector placement, exactly round((1-s)K) vectors per row)
 because the DLMC files are not available offline; any directory of .smtx files can be swept instead
 with --smtx-dir.  Durations are device time per launch (HIP events around a HIP-graph replay).
+--csv-dir also writes one duration file per (benchmark, k, v, kernel) point under the names and in the
+record layout the reference's plot scripts read (file_name_server.py:6-45, :57-81), dense baseline included.
 """
 import argparse
 import csv
@@ -59,8 +61,12 @@ def sddmm_sweep(args, torch, cv, ops, time_launches):
                     prob = ops.DeviceProblem(pat, sort=True)
                     out = torch.empty((pat.nnz_vec, V), dtype=torch.float16, device="cuda")
                     flops = 2.0 * pat.nnz * K
+                    bm = "synthetic/uniform/%g/m%d_n%d" % (s, M, M)
+                    args.per_point(bm, K, V, "dense", "sddmm", "hipblaslt_gemm_f16", dense_us[(M, K)])
                     for kernel in ("wmma", "cuda"):
                         us = time_launches(torch, lambda: prob.sddmm(A, B, kernel=kernel, out=out), args.iters)
+                        args.per_point(bm, K, V, kernel, "sddmm",
+                                       "sddmm_mfma_kernel" if kernel == "wmma" else "sddmm_valu_kernel", us)
                         rows.append({"bm": "synthetic", "M": M, "K": K, "N": M, "sparsity": round(s, 4), "V": V,
                                      "kernel": kernel, "nnz_vec": pat.nnz_vec, "us": round(us, 3),
                                      "dense_us": round(dense_us[(M, K)], 3),
@@ -102,13 +108,21 @@ def main(argv=None):
                     help="call through the batched entry point with the pattern's nonzero count (workgroups sized "
                          "by the real row lengths) instead of the reference-shaped entry points")
     ap.add_argument("--iters", type=int, default=100, help="launches per timed HIP-graph replay")
+    ap.add_argument("--csv-dir", default=None,
+                    help="also write <csv-dir>/<spmm|sddmm>/<benchmark>_<kernel>_half_sort[_<alg>]_k<k>_v<v>.csv, one "
+                         "profiler-style Duration record each, as the reference's plot scripts expect them")
     args = ap.parse_args(argv)
 
     import torch
 
     from . import colvec_csr as cv
     from . import ops
-    from .benchmark_common import time_launches
+    from .benchmark_common import duration_csv_path, time_launches, write_duration_csv
+
+    def per_point(bm, dim_k, V, kernel, job, name, us):
+        if args.csv_dir:
+            write_duration_csv(duration_csv_path(args.csv_dir, bm, dim_k, V, kernel, job), name, us)
+    args.per_point = per_point
 
     if args.op == "sddmm":
         return sddmm_sweep(args, torch, cv, ops, time_launches)
@@ -132,22 +146,26 @@ def main(argv=None):
             pat = cv.read_smtx(spec, V)
             M, K, s = pat.m, pat.n, pat.sparsity
             label = os.path.basename(spec)
+            bm = os.path.relpath(spec, args.smtx_dir)
         else:
             M, K, s = spec
             seed = (M * 1000003 + K * 10007 + int(round(s * 100)) * 101 + V) % (2 ** 31)
             pat = cv.uniform_pattern(M // V, K, s, seed, V)
             label = "synthetic"
+            bm = "synthetic/uniform/%g/m%d_k%d" % (s, M, K)
         pat = cv.random_values(pat, seed=V + 7)
         B = torch.from_numpy(cv.dense_uniform(K, N_DENSE, seed=11)).cuda()
         out = torch.empty((M, N_DENSE), dtype=torch.float16, device="cuda")
         if (M, K) not in dense_us:
             A = torch.randn((M, K), dtype=torch.float16, device="cuda")
             dense_us[(M, K)] = time_launches(torch, lambda: torch.matmul(A, B, out=out), args.iters)
+        args.per_point(bm, N_DENSE, V, "dense", "spmm", "hipblaslt_gemm_f16", dense_us[(M, K)])
         prob = ops.DeviceProblem(pat, sort=True)
         flops = 2.0 * pat.nnz * N_DENSE
         nbytes = spmm_bytes(pat, N_DENSE)
         for kernel in ("wmma", "cuda"):
             us = time_launches(torch, lambda: prob.spmm(B, kernel=kernel, out=out, row_length_hint=args.hint), args.iters)
+            args.per_point(bm, N_DENSE, V, kernel, "spmm", "spmm_mfma_kernel" if kernel == "wmma" else "spmm_valu_kernel", us)
             rows.append({"bm": label, "M": M, "K": K, "N": N_DENSE, "sparsity": round(s, 4), "V": V,
                          "kernel": kernel, "nnz_vec": pat.nnz_vec, "us": round(us, 3),
                          "dense_us": round(dense_us[(M, K)], 3), "speedup": round(dense_us[(M, K)] / us, 4),
