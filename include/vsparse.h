@@ -146,20 +146,23 @@ int vs_cuda_sddmm_f16_f32out(int m_vec, int k, int n, int nonzeros_vec,
  * problem per process; they exist because sparse attention runs one mask over
  * many heads (the reference only links an external sparse-transformer repository,
  * README.md:76).
- * nonzeros_vec of the SpMM forms: the number of nonzero vectors of the pattern
- * (row_offsets[m_vec]) when the caller knows it, negative otherwise.  It only
- * sizes the workgroups (the unbatched SpMM entry points keep the reference's
- * argument list, which does not carry it, and size them by n instead); results do
- * not depend on it.
+ * nonzeros_vec, longest_row_vec of the SpMM forms: the number of nonzero vectors
+ * of the pattern (row_offsets[m_vec]) and of its longest vector row when the caller
+ * knows them, negative otherwise.  They only size the workgroups (the unbatched SpMM
+ * entry points keep the reference's argument list, which does not carry them, and
+ * size them by n instead): by the mean row length, and - when the longest row is
+ * more than four times the mean - with enough waves per row that the longest one
+ * does not outlast the rest of the launch.  Results do not depend on them beyond the
+ * order of the fp32 summation.
  */
 int vs_wmma_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
-                             const int *row_indices, const int *row_offsets,
+                             int longest_row_vec, const int *row_indices, const int *row_offsets,
                              const int *column_indices,
                              const void *values, long long stride_values,
                              const void *rhs_matrix, long long stride_rhs,
                              void *output_matrix, long long stride_output, void *stream);
 int vs_cuda_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
-                             const int *row_indices, const int *row_offsets,
+                             int longest_row_vec, const int *row_indices, const int *row_offsets,
                              const int *column_indices,
                              const void *values, long long stride_values,
                              const void *rhs_matrix, long long stride_rhs,
@@ -203,7 +206,7 @@ int vs_sparse_softmax_f16(int batch, int m_vec, int vec_length,
  * the reference (see vs_sparse_softmax_f16).
  */
 int vs_wmma_spmm_softmax_f16_batched(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
-                                     const int *row_indices, const int *row_offsets,
+                                     int longest_row_vec, const int *row_indices, const int *row_offsets,
                                      const int *column_indices,
                                      const void *scores, long long stride_scores,
                                      const void *rhs_matrix, long long stride_rhs,

@@ -198,6 +198,35 @@ def test_row_length_hint_changes_the_launch_shape_not_the_result(gpu, kernel):
                              prob.values, Bd, out, kernel=kernel, nonzeros_vec=hint)
             torch.cuda.synchronize()
             assert_parity(out[0].cpu().numpy(), ref, "hint %d on %s" % (hint, (m_vec, n, s, V)))
+            for longest in (int(np.diff(pat.row_offsets).max()), 0, 1 << 30):
+                ops.spmm_batched(pat.m_vec, V, 128, n, prob.row_indices, prob.row_offsets, prob.column_indices,
+                                 prob.values, Bd, out, kernel=kernel, nonzeros_vec=hint, longest_row_vec=longest)
+                torch.cuda.synchronize()
+                assert_parity(out[0].cpu().numpy(), ref, "hints %d, %d on %s" % (hint, longest, (m_vec, n, s, V)))
         hinted = prob.spmm(Bd, kernel=kernel, row_length_hint=True)
         torch.cuda.synchronize()
         assert_parity(hinted.cpu().numpy(), ref, "DeviceProblem hinted")
+
+
+def test_longest_row_hint_on_heavy_tailed_rows(gpu):
+    """A few rows far longer than the mean (one of them dense): the hinted launch gives the long rows more
+    waves; parity with the oracle either way and with every wave count forced by hand."""
+    rng = np.random.default_rng(5)
+    m_vec, n, V, N = 192, 2048, 8, 128
+    lengths = np.minimum((rng.pareto(1.5, m_vec) + 0.3) * 40, n).astype(np.int64)
+    lengths[7] = n
+    lengths[100] = 0
+    ro, ci = cv._pattern_from_lengths(rng, m_vec, n, lengths)
+    pat = cv.random_values(cv.ColVecCSR(m_vec, n, V, ro, ci), seed=6)
+    assert lengths.max() > 4 * lengths.mean()
+    B = cv.dense_uniform(n, N, seed=7)
+    ref = _oracle(pat, B)
+    Bd = torch.from_numpy(B).cuda()
+    for sort in (False, True):
+        prob = ops.DeviceProblem(pat, sort=sort)
+        assert prob.longest_row_vec == n
+        plain = prob.spmm(Bd)
+        hinted = prob.spmm(Bd, row_length_hint=True)
+        torch.cuda.synchronize()
+        assert_parity(plain.cpu().numpy(), ref, "heavy tail, reference-shaped entry")
+        assert_parity(hinted.cpu().numpy(), ref, "heavy tail, hinted")

@@ -206,6 +206,7 @@ struct Batch {
     long long stride_b = 0;    // SpMM: rhs_matrix    SDDMM: rhs_matrix
     long long stride_out = 0;  // SpMM: output_matrix SDDMM: output_values
     int nonzeros_vec = -1;     // SpMM: nonzero vectors of the pattern when the caller knows them (launch-shape hint)
+    int longest_row_vec = -1;  // SpMM: nonzero vectors of the longest row when the caller knows them (same)
     int algorithm = 0;         // SDDMM on MFMA: 2 = waves split the nonzero range, else (row, slot) per wave
 };
 

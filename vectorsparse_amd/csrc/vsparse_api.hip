@@ -175,7 +175,8 @@ int vs_cuda_sddmm_f16_f32out(int m_vec, int k, int n, int nonzeros_vec, const in
                                         static_cast<hipStream_t>(stream));
 }
 
-static vs::Batch make_batch(int batch, long long a, long long b, long long out, int nonzeros_vec = -1)
+static vs::Batch make_batch(int batch, long long a, long long b, long long out, int nonzeros_vec = -1,
+                            int longest_row_vec = -1)
 {
     vs::Batch x;
     x.count = batch;
@@ -183,6 +184,7 @@ static vs::Batch make_batch(int batch, long long a, long long b, long long out, 
     x.stride_b = b;
     x.stride_out = out;
     x.nonzeros_vec = nonzeros_vec;
+    x.longest_row_vec = longest_row_vec;
     return x;
 }
 
@@ -190,7 +192,7 @@ static vs::Batch make_batch(int batch, long long a, long long b, long long out, 
 static bool stride_ok(long long stride, long long multiple) { return stride >= 0 && stride % multiple == 0; }
 
 int vs_wmma_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
-    const int *row_indices,
+                             int longest_row_vec, const int *row_indices,
                              const int *row_offsets, const int *column_indices, const void *values,
                              long long stride_values, const void *rhs_matrix, long long stride_rhs,
                              void *output_matrix, long long stride_output, void *stream)
@@ -204,11 +206,11 @@ int vs_wmma_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n,
     return vs::launch_spmm_mfma<half_t>(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices,
                                         static_cast<const half_t *>(values), static_cast<const half_t *>(rhs_matrix),
                                         static_cast<half_t *>(output_matrix), static_cast<hipStream_t>(stream),
-                                        make_batch(batch, stride_values, stride_rhs, stride_output, nonzeros_vec));
+                                        make_batch(batch, stride_values, stride_rhs, stride_output, nonzeros_vec, longest_row_vec));
 }
 
 int vs_cuda_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
-    const int *row_indices,
+                             int longest_row_vec, const int *row_indices,
                              const int *row_offsets, const int *column_indices, const void *values,
                              long long stride_values, const void *rhs_matrix, long long stride_rhs,
                              void *output_matrix, long long stride_output, void *stream)
@@ -222,7 +224,7 @@ int vs_cuda_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n,
     return vs::launch_spmm_valu<half_t>(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices,
                                         static_cast<const half_t *>(values), static_cast<const half_t *>(rhs_matrix),
                                         static_cast<half_t *>(output_matrix), static_cast<hipStream_t>(stream),
-                                        make_batch(batch, stride_values, stride_rhs, stride_output, nonzeros_vec));
+                                        make_batch(batch, stride_values, stride_rhs, stride_output, nonzeros_vec, longest_row_vec));
 }
 
 int vs_wmma_sddmm_f16_batched(int batch, int m_vec, int k, int n, int nonzeros_vec, const int *row_indices,
@@ -267,7 +269,7 @@ int vs_cuda_sddmm_f16_batched(int batch, int m_vec, int k, int n, int nonzeros_v
 }
 
 int vs_wmma_spmm_softmax_f16_batched(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
-    const int *row_indices,
+                             int longest_row_vec, const int *row_indices,
                                      const int *row_offsets, const int *column_indices, const void *scores,
                                      long long stride_scores, const void *rhs_matrix, long long stride_rhs,
                                      void *output_matrix, long long stride_output, float scale, void *stream)
@@ -282,7 +284,7 @@ int vs_wmma_spmm_softmax_f16_batched(int batch, int m_vec, int vec_length, int k
                                         static_cast<const half_t *>(scores), static_cast<const half_t *>(rhs_matrix),
                                         static_cast<half_t *>(output_matrix), scale,
                                         static_cast<hipStream_t>(stream),
-                                        make_batch(batch, stride_scores, stride_rhs, stride_output, nonzeros_vec));
+                                        make_batch(batch, stride_scores, stride_rhs, stride_output, nonzeros_vec, longest_row_vec));
 }
 
 int vs_sparse_attention_f16(int batch, int m_vec, int vec_length, int n, int d_qk, int d_v, const int *row_indices,

@@ -120,7 +120,7 @@ def _stride(t, batch):
 
 
 def spmm_batched(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices, values, rhs_matrix,
-                 output_matrix, kernel="wmma", stream=None, nonzeros_vec=-1):
+                 output_matrix, kernel="wmma", stream=None, nonzeros_vec=-1, longest_row_vec=-1):
     """`batch` SpMMs sharing one pattern in one launch.
 
     values: [batch, nnz_vec, V] (or [nnz_vec, V] shared), rhs_matrix: [batch, n, k] (or [n, k] shared),
@@ -130,8 +130,8 @@ def spmm_batched(m_vec, vec_length, k, n, row_indices, row_offsets, column_indic
     for t, nm in ((values, "values"), (rhs_matrix, "rhs_matrix"), (output_matrix, "output_matrix")):
         _expect_batched(t, torch.float16, nm)
     entry = "vs_wmma_spmm_f16_batched" if kernel == "wmma" else "vs_cuda_spmm_f16_batched"
-    st = getattr(_lib.lib(), entry)(batch, m_vec, vec_length, k, n, int(nonzeros_vec), _ptr(row_indices), _ptr(row_offsets),
-                                    _ptr(column_indices), _ptr(values), _stride(values, batch), _ptr(rhs_matrix),
+    st = getattr(_lib.lib(), entry)(batch, m_vec, vec_length, k, n, int(nonzeros_vec), int(longest_row_vec),
+                                    _ptr(row_indices), _ptr(row_offsets), _ptr(column_indices), _ptr(values), _stride(values, batch), _ptr(rhs_matrix),
                                     _stride(rhs_matrix, batch), _ptr(output_matrix), _stride(output_matrix, batch),
                                     _stream(stream))
     _lib.check(st, entry)
@@ -139,7 +139,7 @@ def spmm_batched(m_vec, vec_length, k, n, row_indices, row_offsets, column_indic
 
 
 def spmm_softmax_batched(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices, scores, rhs_matrix,
-                         output_matrix, scale=1.0, stream=None, nonzeros_vec=-1):
+                         output_matrix, scale=1.0, stream=None, nonzeros_vec=-1, longest_row_vec=-1):
     """out[b] = softmax_row(scale * scores[b]) @ rhs_matrix[b] in one launch (softmax fused into SpMM)."""
     if output_matrix.dim() == 2:
         output_matrix = output_matrix.unsqueeze(0)
@@ -147,8 +147,8 @@ def spmm_softmax_batched(m_vec, vec_length, k, n, row_indices, row_offsets, colu
     for t, nm in ((scores, "scores"), (rhs_matrix, "rhs_matrix"), (output_matrix, "output_matrix")):
         _expect_batched(t, torch.float16, nm)
     st = _lib.lib().vs_wmma_spmm_softmax_f16_batched(
-        batch, m_vec, vec_length, k, n, int(nonzeros_vec), _ptr(row_indices), _ptr(row_offsets), _ptr(column_indices),
-        _ptr(scores),
+        batch, m_vec, vec_length, k, n, int(nonzeros_vec), int(longest_row_vec), _ptr(row_indices), _ptr(row_offsets),
+        _ptr(column_indices), _ptr(scores),
         _stride(scores, batch), _ptr(rhs_matrix), _stride(rhs_matrix, batch), _ptr(output_matrix),
         _stride(output_matrix, batch), float(scale), _stream(stream))
     _lib.check(st, "vs_wmma_spmm_softmax_f16_batched")
@@ -340,10 +340,11 @@ class SparseAttention:
         if fused:
             return spmm_softmax_batched(p.m_vec, p.vec_length, v.shape[2], p.n, p.row_indices, p.row_offsets,
                                         p.column_indices, scores, v, out, scale, stream=stream,
-                                        nonzeros_vec=p.nnz_vec)
+                                        nonzeros_vec=p.nnz_vec, longest_row_vec=p.longest_row_vec)
         sparse_softmax(p.m_vec, p.vec_length, p.row_indices, p.row_offsets, scores, scores, scale, stream=stream)
         spmm_batched(p.m_vec, p.vec_length, v.shape[2], p.n, p.row_indices, p.row_offsets, p.column_indices,
-                     scores, v, out, kernel=kernel, stream=stream, nonzeros_vec=p.nnz_vec)
+                     scores, v, out, kernel=kernel, stream=stream, nonzeros_vec=p.nnz_vec,
+                     longest_row_vec=p.longest_row_vec)
         return out
 
 
@@ -372,6 +373,7 @@ class DeviceProblem:
         self.n = pattern.n
         self.nnz_vec = pattern.nnz_vec
         lengths = np.diff(pattern.row_offsets)
+        self.longest_row_vec = int(lengths.max()) if lengths.size else 0
         # a few rows far longer than the rest: schedules that give every row the same number of waves stall on them
         self.skewed = bool(pattern.nnz_vec >= 65536 and lengths.max() >= 8 * max(1.0, lengths.mean()))
         swz = SortedRowSwizzle(pattern.m_vec, pattern.row_offsets) if sort else IdentityRowSwizzle(pattern.m_vec)
@@ -384,15 +386,15 @@ class DeviceProblem:
 
     def spmm(self, rhs_matrix, kernel="wmma", out_dtype=torch.float16, out=None, stream=None, row_length_hint=False):
         """SpMM through the reference-shaped entry points; with row_length_hint (fp16 output only) through the
-        batched entry point with batch = 1, which also takes the pattern's nonzero count and sizes its
-        workgroups by the real row lengths instead of by n."""
+        batched entry point with batch = 1, which also takes the pattern's nonzero count and longest row and
+        sizes its workgroups by the real row lengths instead of by n."""
         k = rhs_matrix.shape[1]
         if out is None:
             out = torch.empty((self.m_vec * self.vec_length, k), dtype=out_dtype, device=rhs_matrix.device)
         if row_length_hint and out.dtype == torch.float16:
             spmm_batched(self.m_vec, self.vec_length, k, self.n, self.row_indices, self.row_offsets,
                          self.column_indices, self.values, rhs_matrix, out.unsqueeze(0), kernel=kernel, stream=stream,
-                         nonzeros_vec=self.nnz_vec)
+                         nonzeros_vec=self.nnz_vec, longest_row_vec=self.longest_row_vec)
             return out
         fn = spmm.wmmaSpmm if kernel == "wmma" else spmm.cudaSpmm
         return fn(self.m_vec, self.vec_length, k, self.n, self.row_indices, self.row_offsets,
