@@ -93,9 +93,14 @@ def test_attention_planning_helpers_are_consistent():
             assert used.value % per_wave == 0 and used.value <= 8 * per_wave      # whole waves, at most 8
             assert used.value >= min(request, 8 * per_wave)
             blocks = -(-512 // used.value)
-            size = L.vs_sparse_attention_plan_bytes(512, V, 4096, 64, 64, request)
             mask_words = (used.value * 16 + 3) // 4 * 4
-            assert size == 4 * (16 + blocks * (4 + mask_words + cap))
+            for rounds in (1, 2, 3, 4):                                     # larger unions, taken in rounds
+                assert L.vs_sparse_attention_union_capacity(V, 4096, 64, 64, request, rounds, None) == rounds * cap
+                size = L.vs_sparse_attention_plan_bytes(512, V, 4096, 64, 64, request, rounds)
+                assert size == 4 * (16 + blocks * (4 + rounds * (mask_words + cap)))
+            assert L.vs_sparse_attention_plan_bytes(512, V, 4096, 64, 64, request, 0) == 0
+            assert L.vs_sparse_attention_plan_bytes(512, V, 4096, 64, 64, request, 5) == 0
+            assert L.vs_sparse_attention_union_capacity(V, 4096, 64, 64, request, 5, None) == 0
     wide = L.vs_sparse_attention_union_capacity(8, 4096, 128, 128, 16, 0, None)
     narrow = L.vs_sparse_attention_union_capacity(8, 4096, 32, 32, 16, 0, None)
     assert 0 < wide < narrow                                   # wider rows: fewer of them fit in LDS
@@ -107,11 +112,12 @@ def test_attention_planning_helpers_are_consistent():
     assert L.vs_sparse_attention_union_capacity(8, 400000, 64, 64, 16, 0, None) == 0
     assert L.vs_sparse_attention_union_capacity(8, 400000, 64, 64, 16, 1, None) > 0
     assert L.vs_sparse_attention_union_capacity(3, 4096, 64, 64, 16, 0, None) == 0
-    assert L.vs_sparse_attention_plan_bytes(512, 8, 4096, 64, 64, 1) == 0
+    assert L.vs_sparse_attention_plan_bytes(512, 8, 4096, 64, 64, 1, 1) == 0
     # a plan buffer that is too small, null or misaligned is rejected before any launch
-    assert L.vs_sparse_attention_plan(512, 8, 4096, 64, 64, 16, 64, 64, 256, 16, None) == 1
-    assert L.vs_sparse_attention_plan(512, 8, 4096, 64, 64, 16, 64, 64, None, 1 << 20, None) == 1
-    assert L.vs_sparse_attention_plan(512, 8, 4096, 64, 64, 16, 64, 64, 264, 1 << 20, None) == 1
+    assert L.vs_sparse_attention_plan(512, 8, 4096, 64, 64, 16, 1, 64, 64, 256, 16, None) == 1
+    assert L.vs_sparse_attention_plan(512, 8, 4096, 64, 64, 16, 1, 64, 64, None, 1 << 20, None) == 1
+    assert L.vs_sparse_attention_plan(512, 8, 4096, 64, 64, 16, 1, 64, 64, 264, 1 << 20, None) == 1
+    assert L.vs_sparse_attention_plan(512, 8, 4096, 64, 64, 16, 0, 64, 64, 256, 1 << 20, None) == 1
 
 
 def test_options():

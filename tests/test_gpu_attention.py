@@ -273,9 +273,10 @@ def _with_empty_rows(mask, first, last):
     return cv.ColVecCSR(mask.m_vec, mask.n, mask.vec_length, offsets, mask.column_indices[keep].copy())
 
 
-def _capacity(V, n, d_qk, d_v, rows, with_plan):
+def _capacity(V, n, d_qk, d_v, rows, plan_rounds):
+    """Distinct columns a workgroup takes: without a plan (0) or with a plan of that many rounds."""
     from vectorsparse_amd import _lib
-    return _lib.lib().vs_sparse_attention_union_capacity(V, n, d_qk, d_v, rows, with_plan, None)
+    return _lib.lib().vs_sparse_attention_union_capacity(V, n, d_qk, d_v, rows, plan_rounds, None)
 
 
 def _unions(mask, rows):
@@ -298,7 +299,7 @@ def test_plan_raises_the_union_capacity(gpu, V, seq, half_width, stride, rows):
     qd, kd, vd = (torch.from_numpy(x).cuda() for x in (q, k, v))
     ref = _dense_attention(mask, q, k, v, 0.125)
     layer = ops.SparseAttention(mask)
-    assert layer.union_rows(d, d) == rows                 # the host-side choice counts on the plan
+    assert layer.union_rows(d, d) >= rows                 # the host-side choice counts on the plan
     prob = layer.prob
     args = (mask.m_vec, V, seq, prob.row_indices, prob.row_offsets, prob.column_indices, qd, kd, vd)
     plan = ops.sparse_attention_plan(mask.m_vec, V, seq, d, d, rows, prob.row_offsets, prob.column_indices)
@@ -310,6 +311,56 @@ def test_plan_raises_the_union_capacity(gpu, V, seq, half_width, stride, rows):
     _check_layer(rebuilt.cpu().numpy(), ref, "V%d rebuilt" % V)
     _check_layer(out.cpu().numpy(), ref, "V%d layer" % V)
     assert not torch.equal(planned, rebuilt)              # different summation orders: the paths did differ
+
+
+@pytest.mark.parametrize("V,seq,half_width,stride,dims,want_rounds", [
+    (8, 4096, 300, 64, (64, 64), 2),      # two rounds of 512 ranks
+    (8, 4096, 900, 128, (64, 64), 4),     # four rounds
+    (2, 2048, 400, 0, (32, 128), 4),      # plain band, four rounds of 256 ranks with the wide V rows
+    (1, 2048, 400, 256, (64, 64), 2),     # 128 vector rows per workgroup, masks restaged every round
+])
+def test_planned_launch_takes_large_unions_in_rounds(gpu, V, seq, half_width, stride, dims, want_rounds):
+    """Unions of more columns than fit in LDS at once: with a plan the workgroup walks them in rounds with a
+    running maximum and sum; rows whose columns all fall into a later round, rows empty in some round, and a
+    negative scale go through the same rescaling."""
+    d_qk, d_v = dims
+    mask = cv.band_strided_pattern(seq, V, band_half_width=half_width, stride=stride or seq)
+    mask = _with_empty_rows(mask, 3, 5)
+    rows = 128 // V
+    unions = _unions(mask, rows)
+    rounds = next(r for r in (1, 2, 3, 4) if max(unions) <= _capacity(V, seq, d_qk, d_v, rows, r))
+    assert rounds == want_rounds, (rounds, max(unions), _capacity(V, seq, d_qk, d_v, rows, 1))
+    rng = np.random.default_rng(90 + V)
+    q = rng.standard_normal((2, seq, d_qk)).astype(np.float16)
+    k = rng.standard_normal((2, seq, d_qk)).astype(np.float16)
+    v = rng.standard_normal((2, seq, d_v)).astype(np.float16)
+    # make the maximum of many rows sit in a late round: large keys at the top end of the sequence
+    k[:, seq - seq // 8:, :] *= 3.0
+    qd, kd, vd = (torch.from_numpy(x).cuda() for x in (q, k, v))
+    prob = ops.DeviceProblem(mask)
+    args = (mask.m_vec, V, seq, prob.row_indices, prob.row_offsets, prob.column_indices, qd, kd, vd)
+    plan = ops.sparse_attention_plan(mask.m_vec, V, seq, d_qk, d_v, rows, prob.row_offsets, prob.column_indices,
+                                     plan_rounds=rounds)
+    for scale in (0.125, -0.125, 0.0):
+        ref = _dense_attention(mask, q, k, v, scale)
+        planned = ops.sparse_attention(*args, scale=scale, rows_per_workgroup=rows, plan=plan)
+        again = ops.sparse_attention(*args, scale=scale, rows_per_workgroup=rows, plan=plan)
+        torch.cuda.synchronize()
+        _check_layer(planned.cpu().numpy(), ref, "V%d scale %g in rounds" % (V, scale))
+        assert torch.equal(planned, again)
+    # a plan of more rounds than needed, and the one-round kernel given a plan of several (ignored: per-row path)
+    spare = ops.sparse_attention_plan(mask.m_vec, V, seq, d_qk, d_v, rows, prob.row_offsets, prob.column_indices,
+                                      plan_rounds=4)
+    ref = _dense_attention(mask, q, k, v, 0.125)
+    for given, told in ((spare, 4), (spare, 1), (plan, 1)):
+        out = ops.sparse_attention(*args, scale=0.125, rows_per_workgroup=rows, plan=given, plan_rounds=told)
+        torch.cuda.synchronize()
+        _check_layer(out.cpu().numpy(), ref, "V%d plan of %d rounds read as %d" % (V, given.plan_rounds, told))
+    layer = ops.SparseAttention(mask)
+    assert layer.union_shape(d_qk, d_v)[0] > 1 and layer.union_shape(d_qk, d_v)[1] > 1   # the host-side choice counts on the rounds
+    out = layer.forward(qd, kd, vd, scale=0.125)
+    torch.cuda.synchronize()
+    _check_layer(out.cpu().numpy(), _dense_attention(mask, q, k, v, 0.125), "V%d layer in rounds" % V)
 
 
 @pytest.mark.parametrize("V", [1, 8])

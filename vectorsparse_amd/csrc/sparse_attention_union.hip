@@ -16,8 +16,10 @@
 //   1  bitmap of the block's columns in LDS (atomic or), exclusive prefix of its word popcounts:
 //      rank(col) = prefix[col / 32] + popcount(bitmap[col / 32] below bit col % 32) is the position of a
 //      column in the sorted union; U = total popcount.
-//   2  list the union's columns; per vector row a bit mask over ranks (bit r set: the row holds the
-//      column of rank r); copy the K rows of the union to LDS (128-bit loads, rows padded by 16 bytes
+//   2  every nonzero writes its column at the column's rank (the list of the union) and sets its bit in
+//      its vector row's mask over ranks (bit r set: the row holds the column of rank r).  Steps 1 and 2
+//      depend only on the mask: a plan (sparse_attention_plan_kernel) holds their result for every
+//      workgroup, and launches that are given one read it instead.  Copy the K rows of the union to LDS (128-bit loads, rows padded by 16 bytes
 //      against bank conflicts, rows U.. of the last 32-rank step zero-filled).
 //   A  per wave and 32-rank step: S^T = K_union Q^T on v_mfma_f32_16x16x32_f16 with the K rows as the A
 //      operand and the wave's 16 Q rows as the B operand: lane (c, g) receives the scores of scalar row
@@ -33,6 +35,8 @@
 //      and the V rows (transposed in registers with v_perm_b32, as in the SpMM kernel) are read in that
 //      same order.  One more MFMA per step with an all-ones B operand yields the row sums of the rounded
 //      p in exactly the accumulator layout, so normalising needs no cross-lane traffic.
+// A plan of several rounds lets a workgroup take a union that does not fit LDS at once: steps 2 (the copy)
+// to C run once per round of u_max ranks, with the maximum and the sums carried across the rounds.
 #include "vs_common.hpp"
 
 namespace vs {
@@ -252,15 +256,15 @@ struct UnionLds {
     unsigned *bitmap;   // [n_words] columns present in the block
     unsigned *prefix;   // [n_words] exclusive prefix of the bitmap's word popcounts
     int *wave_tot;      // [16] scan scratch, [15] = number of distinct columns
-    unsigned *rowmask;  // [rows][kUnionSteps] ranks each row holds
-    int *ucols;         // [u_max] columns of the union in ascending order
+    unsigned *rowmask;  // [rounds][rows][kUnionSteps] ranks each row holds, u_max ranks per round
+    int *ucols;         // [rounds * u_max] columns of the union in ascending order
 };
 
 // Steps 1 and 2 of the header comment for rows [row_first, row_last), by the whole workgroup: returns the
-// number U of distinct columns; rowmask and ucols are complete (and visible to every thread) on return
-// when U <= u_max, otherwise only U is meaningful.
-__device__ __forceinline__ int build_union(const UnionLds &l, int n_words, int mask_words, int u_max, int row_first,
-                                           int row_last, const int *__restrict__ row_offsets,
+// number U of distinct columns; rowmask ([rounds][mask_words]) and ucols are complete (and visible to every
+// thread) on return when U <= rounds * u_max, otherwise only U is meaningful.
+__device__ __forceinline__ int build_union(const UnionLds &l, int n_words, int mask_words, int u_max, int rounds,
+                                           int row_first, int row_last, const int *__restrict__ row_offsets,
                                            const int *__restrict__ col_indices)
 {
     const int tid = threadIdx.x;
@@ -269,7 +273,7 @@ __device__ __forceinline__ int build_union(const UnionLds &l, int n_words, int m
     const int n_waves = blockDim.x >> 6;
     const int n_threads = blockDim.x;
     for (int w = tid; w < n_words; w += n_threads) l.bitmap[w] = 0u;
-    for (int w = tid; w < mask_words; w += n_threads) l.rowmask[w] = 0u;
+    for (int w = tid; w < rounds * mask_words; w += n_threads) l.rowmask[w] = 0u;
     __syncthreads();
     const int nz_first = row_offsets[row_first];
     const int nz_last = row_offsets[row_last];
@@ -333,9 +337,19 @@ __device__ __forceinline__ int build_union(const UnionLds &l, int n_words, int m
         __syncthreads();
     }
     const int n_union = l.wave_tot[15];
-    if (n_union > u_max) return n_union;
+    if (n_union > rounds * u_max) return n_union;
     // every nonzero sets its bit in its row's mask and writes its column at the column's rank (all writers
-    // of one rank write the same value), which lists the union without a pass over the bitmap
+    // of one rank write the same value), which lists the union without a pass over the bitmap; ranks
+    // [i * u_max, (i + 1) * u_max) belong to round i, whose masks follow those of round i - 1
+    auto mask_bit = [&](int r, int rank) {
+        int word = r * kUnionSteps;
+        if (rounds > 1) {
+            const int round = rank / u_max;
+            rank -= round * u_max;
+            word += round * mask_words;
+        }
+        atomicOr(&l.rowmask[word + (rank >> 5)], 1u << (rank & 31));
+    };
     for (int r = wave; r < row_last - row_first; r += n_waves) {
         const int beg = row_offsets[row_first + r];
         const int end = row_offsets[row_first + r + 1];
@@ -345,8 +359,8 @@ __device__ __forceinline__ int build_union(const UnionLds &l, int n_words, int m
             const int col_b = col_indices[j1 < end ? j1 : j0];
             const int rank_a = (int)l.prefix[col_a >> 5] + __builtin_popcount(l.bitmap[col_a >> 5] & ((1u << (col_a & 31)) - 1u));
             const int rank_b = (int)l.prefix[col_b >> 5] + __builtin_popcount(l.bitmap[col_b >> 5] & ((1u << (col_b & 31)) - 1u));
-            atomicOr(&l.rowmask[r * kUnionSteps + (rank_a >> 5)], 1u << (rank_a & 31));
-            atomicOr(&l.rowmask[r * kUnionSteps + (rank_b >> 5)], 1u << (rank_b & 31));
+            mask_bit(r, rank_a);
+            mask_bit(r, rank_b);
             l.ucols[rank_a] = col_a;
             l.ucols[rank_b] = col_b;
         }
@@ -357,13 +371,17 @@ __device__ __forceinline__ int build_union(const UnionLds &l, int n_words, int m
 
 // A plan holds what build_union computes for every workgroup of a launch shape, so that launches on the
 // same mask (every head, layer and step) read it instead of rebuilding it.  Layout, in 32-bit words:
-// header [magic, m_vec, V, n, rows per workgroup, u_max, record stride, workgroups, 0...] (16 words), then
-// one record per workgroup: [U, 0, 0, 0], rowmask [mask_words], ucols [u_max].
+// header [magic, m_vec, V, n, rows per workgroup, u_max, record stride, workgroups, rounds, 0...] (16 words),
+// then one record per workgroup: [U, 0, 0, 0], rowmask [rounds][mask_words], ucols [rounds * u_max].
+// A plan of one round serves launches that hold a workgroup's whole union in LDS; a plan of up to
+// kMaxPlanRounds rounds serves launches that take a larger union in rounds of u_max ranks (the K / V rows of
+// one round in LDS at a time, running maximum and sums across the rounds).
 constexpr int kPlanMagic = 0x56535041;
 constexpr int kPlanHeader = 16;
+constexpr int kMaxPlanRounds = 4;
 
 __global__ void __launch_bounds__(256)
-sparse_attention_plan_kernel(int m_vec, int vec_length, int n, int rows_per_block, int u_max,
+sparse_attention_plan_kernel(int m_vec, int vec_length, int n, int rows_per_block, int u_max, int rounds,
                              const int *__restrict__ row_offsets, const int *__restrict__ col_indices,
                              int *__restrict__ plan)
 {
@@ -376,12 +394,13 @@ sparse_attention_plan_kernel(int m_vec, int vec_length, int n, int rows_per_bloc
     l.prefix = l.bitmap + n_words_al;
     l.wave_tot = reinterpret_cast<int *>(l.prefix + n_words_al);
     l.rowmask = reinterpret_cast<unsigned *>(l.wave_tot + 16);
-    l.ucols = reinterpret_cast<int *>(l.rowmask + mask_words);
-    const int stride = 4 + mask_words + u_max;
+    l.ucols = reinterpret_cast<int *>(l.rowmask + rounds * mask_words);
+    const int cap = rounds * u_max;
+    const int stride = 4 + rounds * mask_words + cap;
     const int tid = threadIdx.x;
     if (blockIdx.x == 0 && tid < kPlanHeader) {
         const int header[kPlanHeader] = {kPlanMagic, m_vec, vec_length, n, rows_per_block, u_max, stride,
-                                         (int)gridDim.x, 0, 0, 0, 0, 0, 0, 0, 0};
+                                         (int)gridDim.x, rounds, 0, 0, 0, 0, 0, 0, 0};
         int value = 0;
 #pragma unroll
         for (int i = 0; i < kPlanHeader; ++i) value = (i == tid) ? header[i] : value;
@@ -389,21 +408,24 @@ sparse_attention_plan_kernel(int m_vec, int vec_length, int n, int rows_per_bloc
     }
     const int row_first = blockIdx.x * rows_per_block;
     const int row_last = (row_first + rows_per_block) < m_vec ? (row_first + rows_per_block) : m_vec;
-    const int n_union = build_union(l, n_words, mask_words, u_max, row_first, row_last, row_offsets, col_indices);
+    const int n_union = build_union(l, n_words, mask_words, u_max, rounds, row_first, row_last, row_offsets,
+                                    col_indices);
     int *rec = plan + kPlanHeader + (size_t)blockIdx.x * stride;
     if (tid < 4) rec[tid] = tid == 0 ? n_union : 0;
-    if (n_union > u_max) return;  // this workgroup's rows take the per-row path at every launch
-    for (int w = tid; w < mask_words; w += blockDim.x) rec[4 + w] = (int)l.rowmask[w];
-    for (int u = tid; u < u_max; u += blockDim.x) rec[4 + mask_words + u] = u < n_union ? l.ucols[u] : 0;
+    if (n_union > cap) return;  // this workgroup's rows take the per-row path at every launch
+    for (int w = tid; w < rounds * mask_words; w += blockDim.x) rec[4 + w] = (int)l.rowmask[w];
+    for (int u = tid; u < cap; u += blockDim.x) rec[4 + rounds * mask_words + u] = u < n_union ? l.ucols[u] : 0;
 }
 
 // V: vector length; KS: d_qk <= 32*KS; CPL: d_v <= 16*CPL.
-// PLANNED: the union and the row masks come from a plan (sparse_attention_plan_kernel) instead of being
-// rebuilt; a plan made for another mask shape or launch shape sends every workgroup to the per-row path.
-template <int V, int KS, int CPL, bool PLANNED>
+// MODE 0: the workgroup builds its union.  MODE 1, 2 (PLANNED): the union and the row masks come from a plan
+// (sparse_attention_plan_kernel) of plan_rounds rounds instead of being rebuilt; 1: one round, the whole
+// union in LDS at once as in mode 0; 2 (ROUNDS): a union of up to plan_rounds * u_max columns, u_max at a
+// time.  A plan made for another mask shape or launch shape sends every workgroup to the per-row path.
+template <int V, int KS, int CPL, int MODE>
 // four waves per SIMD: two eight-wave workgroups per CU
 __global__ void __launch_bounds__(512, 4)
-sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max,
+sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max, int plan_rounds,
                               const int *__restrict__ row_offsets, const int *__restrict__ col_indices,
                               const int *__restrict__ plan,
                               const half_t *__restrict__ q, const half_t *__restrict__ k,
@@ -414,6 +436,8 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max,
     k += blockIdx.y * stride_k;
     v += blockIdx.y * stride_v;
     out += blockIdx.y * stride_out;
+    constexpr bool PLANNED = MODE != 0;
+    constexpr bool ROUNDS = MODE == 2;
     constexpr int RPW = 16 / V;  // vector rows per wave: 16 scalar rows fill the MFMA tile
     constexpr int PITCH = union_pitch(KS, CPL);
     const int n_words = (n + 31) >> 5;
@@ -461,23 +485,27 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max,
 
     // ---- 1, 2. the union's columns and every row's mask over ranks: built here or read from the plan
     int n_union;
-    const int *cols;  // columns of the union: LDS (built) or the plan's record (global)
+    const int *cols;            // columns of the union: LDS (built) or the plan's record (global)
+    const int *masks = nullptr;  // the plan's row masks, one set per round
+    int u_cap = u_max;          // columns the workgroup can take: in LDS at once, or in the plan's rounds
     if constexpr (PLANNED) {
-        const int stride = 4 + mask_words + u_max;
+        u_cap = plan_rounds * u_max;
+        const int stride = 4 + plan_rounds * mask_words + u_cap;
         const bool plan_ok = plan[0] == kPlanMagic && plan[1] == m_vec && plan[2] == V && plan[3] == n &&
                              plan[4] == rows_per_block && plan[5] == u_max && plan[6] == stride &&
-                             plan[7] == (int)gridDim.x;
+                             plan[7] == (int)gridDim.x && plan[8] == plan_rounds;
         const int *rec = plan + kPlanHeader + (size_t)(plan_ok ? bx : 0) * stride;
         n_union = plan_ok ? rec[0] : 0x7fffffff;
-        cols = rec + 4 + mask_words;
-        if (n_union <= u_max)
-            for (int w = tid; w < mask_words; w += n_threads) l.rowmask[w] = (unsigned)rec[4 + w];
+        masks = rec + 4;
+        cols = rec + 4 + plan_rounds * mask_words;
+        if (n_union <= u_cap)
+            for (int w = tid; w < mask_words; w += n_threads) l.rowmask[w] = (unsigned)masks[w];
         // visible to the other waves after the barrier that follows the K gather
     } else {
-        n_union = build_union(l, n_words, mask_words, u_max, row_first, row_last, row_offsets, col_indices);
+        n_union = build_union(l, n_words, mask_words, u_max, 1, row_first, row_last, row_offsets, col_indices);
         cols = l.ucols;
     }
-    const bool use_lds = n_union <= u_max && (d_v % 8 == 0);
+    const bool use_lds = n_union <= u_cap && (d_v % 8 == 0);
     if (!use_lds) {
         // Fallback: one vector row per wave at a time with the K / V rows read from global memory by
         // column; no barrier, long rows in chunks with a running maximum and sum.
@@ -513,12 +541,12 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max,
         return;
     }
 
-    // ---- 2b. the K rows of the union
-    const int n_steps = (n_union + 31) >> 5;  // <= kUnionSteps because u_max <= 32 * kUnionSteps
-    // Copy one operand's rows of the union into buf: 16 bytes per thread and slice, kBatch slices in
-    // flight; rows past the union (the last step's padding) and slices past `d` are written as zeros, so
-    // the arithmetic below never meets stale bits.
-    auto gather = [&](const half_t *src, int d, int slice_shift) {
+    // ---- 2b .. C, once per round of at most u_max ranks of the union (one round unless a plan lists more
+    // columns than fit in LDS at once; then the maximum and the sums run across the rounds)
+    // Copy one operand's rows of ranks [u_first, u_first + n_here) into buf: 16 bytes per thread and slice,
+    // kBatch slices in flight; rows past the round's ranks (the last step's padding) and slices past `d` are
+    // written as zeros, so the arithmetic below never meets stale bits.
+    auto gather = [&](const half_t *src, int d, int slice_shift, int u_first, int n_here, int n_steps) {
         constexpr int kBatch = 8;
         const int slices = d >> 3;
         const int total = (32 * n_steps) << slice_shift;
@@ -531,8 +559,9 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max,
                 dst[i] = -1;
                 if (sidx < total) {
                     const int u = sidx >> slice_shift, sl = sidx & ((1 << slice_shift) - 1);
-                    const bool real = u < n_union && sl < slices;
-                    const int col = PLANNED ? cols[real ? u : 0] : l.ucols[real ? u : 0];  // two address spaces
+                    const bool real = u < n_here && sl < slices;
+                    const int at = real ? u_first + u : 0;
+                    const int col = PLANNED ? cols[at] : l.ucols[at];  // two address spaces
                     const uint4_t x = *reinterpret_cast<const uint4_t *>(src + (size_t)col * d + (real ? 8 * sl : 0));
                     const uint4_t zero = {0u, 0u, 0u, 0u};
                     data[i] = real ? x : zero;
@@ -551,12 +580,6 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max,
     const long long q_limit = (long long)row_last * V;
     half8_t qb[KS];  // requested before the K rows so that the first MFMA does not wait for it
     load_q16<KS>(qb, q, q_global, q_limit, d_qk, c, g);
-    gather(k, d_qk, kShiftK);
-    __syncthreads();
-
-    // ---- A. per wave: 16 scalar rows against the whole union; maximum, then masked exponentials
-    const unsigned *mrow = rowmask + ((q_first + c) / V) * kUnionSteps;  // mask of the lane's vector row
-    const half_t *k_lane = buf + c * PITCH + 8 * g;
     // The maximum is tracked on the raw dot products, so the scale must be non-negative: a negative one
     // moves its sign into Q.
     const float s2a = __builtin_fabsf(s2);
@@ -569,102 +592,165 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max,
             qb[kk] = __builtin_bit_cast(half8_t, bits);
         }
     }
+    const unsigned *mrow = rowmask + ((q_first + c) / V) * kUnionSteps;  // mask of the lane's vector row
+    const half_t *k_lane = buf + c * PITCH + 8 * g;
+    const half_t *v_lane = buf + 4 * g * PITCH + col_off;
     const float neg_inf = -__builtin_inff();
-    constexpr unsigned kLaneBits = 0x000F000Fu;  // after the shift by 4g: the lane's 4 + 4 ranks of a step
-    unsigned act = 0;   // steps in which at least one row of the wave holds a column (uniform)
-    unsigned full = 0;  // steps in which every lane's rows hold all of the lane's ranks: no masking needed
-    float mx_raw = neg_inf;
+
+    // ---- A. per wave: 16 scalar rows against the n_steps steps of ranks in buf; maximum (joined with mx_run,
+    // the maximum of earlier rounds), then masked exponentials.  Returns the new maximum of the lane's scalar
+    // row c (raw dot products); act = steps in which at least one row of the wave holds a column (uniform).
+    auto scores = [&](int n_steps, float mx_run, half8_t (&p)[kUnionSteps], unsigned &act) {
+        constexpr unsigned kLaneBits = 0x000F000Fu;  // after the shift by 4g: the lane's 4 + 4 ranks of a step
+        unsigned full = 0;  // steps in which every lane's rows hold all of the lane's ranks: no masking needed
+        float mx_raw = neg_inf;
+        act = 0;
 #pragma unroll
-    for (int t = 0; t < kUnionSteps; ++t) {
-        if (t < n_steps) {
-            const unsigned word = mrow[t];
-            if (__builtin_amdgcn_ballot_w64(word != 0u) != 0ull) {
-                act |= 1u << t;
-                const unsigned wg = word >> (4 * g);
+        for (int t = 0; t < kUnionSteps; ++t) {
+            if (t < n_steps) {
+                const unsigned word = mrow[t];
+                if (__builtin_amdgcn_ballot_w64(word != 0u) != 0ull) {
+                    act |= 1u << t;
+                    const unsigned wg = word >> (4 * g);
+                    half8_t a[2][KS];
+                    load_k_step<KS, PITCH>(a, k_lane, t);
+                    float4_t sacc[2];
+                    scores_step<KS>(sacc, a, qb);
+                    if (__builtin_amdgcn_ballot_w64((wg & kLaneBits) != kLaneBits) == 0ull) {
+                        full |= 1u << t;
+#pragma unroll
+                        for (int u = 0; u < 2; ++u)
+                            mx_raw = fmaxf(fmaxf(mx_raw, fmaxf(sacc[u][0], sacc[u][1])), fmaxf(sacc[u][2], sacc[u][3]));
+                    } else {
+#pragma unroll
+                        for (int u = 0; u < 2; ++u)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                mx_raw = fmaxf(mx_raw, select_bit(wg, 16 * u + e, sacc[u][e], neg_inf));
+                    }
+                }
+            }
+        }
+        act = __builtin_amdgcn_readfirstlane(act);
+        full = __builtin_amdgcn_readfirstlane(full);
+        mx_raw = fmaxf(mx_raw, partner<16>(mx_raw));  // scalar row c lives in the four lanes (c, g = 0..3)
+        mx_raw = fmaxf(mx_raw, partner<32>(mx_raw));
+        const float mx_new = fmaxf(mx_run, mx_raw);
+        const float neg_mx = mx_new == neg_inf ? 0.f : -(mx_new * s2a);  // a row with no column: every exponent stays -inf
+#pragma unroll
+        for (int t = 0; t < kUnionSteps; ++t) {
+            p[t] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+            if ((act >> t) & 1u) {
                 half8_t a[2][KS];
                 load_k_step<KS, PITCH>(a, k_lane, t);
                 float4_t sacc[2];
                 scores_step<KS>(sacc, a, qb);
-                if (__builtin_amdgcn_ballot_w64((wg & kLaneBits) != kLaneBits) == 0ull) {
-                    full |= 1u << t;
+                // k-slot (g, e) of step t: e < 4 -> rank 4g + e of the first half, e >= 4 -> 4g + e - 4 of the second
+                if ((full >> t) & 1u) {
 #pragma unroll
                     for (int u = 0; u < 2; ++u)
-                        mx_raw = fmaxf(fmaxf(mx_raw, fmaxf(sacc[u][0], sacc[u][1])), fmaxf(sacc[u][2], sacc[u][3]));
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            p[t][4 * u + e] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf(sacc[u][e], s2a, neg_mx));
                 } else {
+                    const unsigned wg = mrow[t] >> (4 * g);
 #pragma unroll
                     for (int u = 0; u < 2; ++u)
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) mx_raw = fmaxf(mx_raw, select_bit(wg, 16 * u + e, sacc[u][e], neg_inf));
+                        for (int e = 0; e < 4; ++e) {
+                            const float bias = select_bit(wg, 16 * u + e, neg_mx, neg_inf);
+                            p[t][4 * u + e] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf(sacc[u][e], s2a, bias));
+                        }
                 }
             }
         }
-    }
-    act = __builtin_amdgcn_readfirstlane(act);
-    full = __builtin_amdgcn_readfirstlane(full);
-    mx_raw = fmaxf(mx_raw, partner<16>(mx_raw));  // scalar row c lives in the four lanes (c, g = 0..3)
-    mx_raw = fmaxf(mx_raw, partner<32>(mx_raw));
-    const float neg_mx = mx_raw == neg_inf ? 0.f : -(mx_raw * s2a);  // a row with no column: every exponent stays -inf
-    half8_t p[kUnionSteps];
-#pragma unroll
-    for (int t = 0; t < kUnionSteps; ++t) {
-        p[t] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-        if ((act >> t) & 1u) {
-            half8_t a[2][KS];
-            load_k_step<KS, PITCH>(a, k_lane, t);
-            float4_t sacc[2];
-            scores_step<KS>(sacc, a, qb);
-            // k-slot (g, e) of step t: e < 4 -> rank 4g + e of the first half, e >= 4 -> 4g + e - 4 of the second
-            if ((full >> t) & 1u) {
-#pragma unroll
-                for (int u = 0; u < 2; ++u)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        p[t][4 * u + e] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf(sacc[u][e], s2a, neg_mx));
-            } else {
-                const unsigned wg = mrow[t] >> (4 * g);
-#pragma unroll
-                for (int u = 0; u < 2; ++u)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const float bias = select_bit(wg, 16 * u + e, neg_mx, neg_inf);
-                        p[t][4 * u + e] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf(sacc[u][e], s2a, bias));
-                    }
-            }
-        }
-    }
+        return mx_new;
+    };
 
-    // ---- 3. V rows of the union over the K rows
-    __syncthreads();
-    gather(v, d_v, kShiftV);
-    __syncthreads();
-
-    // ---- C. P V and the row sums, normalise, store (one wave owns its rows: nothing to reduce)
+    // ---- C. P V and the row sums against the V rows in buf (one wave owns its rows: nothing to reduce)
     float4_t acc[CPL];
+    float4_t lacc;
+    auto weighted_sum = [&](const half8_t (&p)[kUnionSteps], unsigned act) {
+        const half8_t ones = {1, 1, 1, 1, 1, 1, 1, 1};
 #pragma unroll
-    for (int cc = 0; cc < CPL; ++cc) acc[cc] = float4_t{0.f, 0.f, 0.f, 0.f};
-    float4_t lacc = {0.f, 0.f, 0.f, 0.f};
-    const half8_t ones = {1, 1, 1, 1, 1, 1, 1, 1};
-    const half_t *v_lane = buf + 4 * g * PITCH + col_off;
+        for (int t = 0; t < kUnionSteps; ++t) {
+            if ((act >> t) & 1u) {
+                RowChunk<CPL> rows[8];
 #pragma unroll
-    for (int t = 0; t < kUnionSteps; ++t) {
-        if ((act >> t) & 1u) {
-            RowChunk<CPL> rows[8];
+                for (int e = 0; e < 8; ++e) rows[e].load(v_lane + (32 * t + (e < 4 ? e : 12 + e)) * PITCH);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) rows[e].load(v_lane + (32 * t + (e < 4 ? e : 12 + e)) * PITCH);
+                for (int pp = 0; pp < CPL / 2; ++pp) {
+                    uint4_t even, odd;
 #pragma unroll
-            for (int pp = 0; pp < CPL / 2; ++pp) {
-                uint4_t even, odd;
-#pragma unroll
-                for (int qq = 0; qq < 4; ++qq) {
-                    even[qq] = pack_lo(rows[2 * qq].dword(pp), rows[2 * qq + 1].dword(pp));
-                    odd[qq] = pack_hi(rows[2 * qq].dword(pp), rows[2 * qq + 1].dword(pp));
+                    for (int qq = 0; qq < 4; ++qq) {
+                        even[qq] = pack_lo(rows[2 * qq].dword(pp), rows[2 * qq + 1].dword(pp));
+                        odd[qq] = pack_hi(rows[2 * qq].dword(pp), rows[2 * qq + 1].dword(pp));
+                    }
+                    acc[2 * pp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(p[t], __builtin_bit_cast(half8_t, even), acc[2 * pp], 0, 0, 0);
+                    acc[2 * pp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(p[t], __builtin_bit_cast(half8_t, odd), acc[2 * pp + 1], 0, 0, 0);
                 }
-                acc[2 * pp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(p[t], __builtin_bit_cast(half8_t, even), acc[2 * pp], 0, 0, 0);
-                acc[2 * pp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(p[t], __builtin_bit_cast(half8_t, odd), acc[2 * pp + 1], 0, 0, 0);
+                lacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(p[t], ones, lacc, 0, 0, 0);  // row sums, in accumulator layout
             }
-            lacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(p[t], ones, lacc, 0, 0, 0);  // row sums, in accumulator layout
+        }
+    };
+    auto clear_sums = [&]() {
+#pragma unroll
+        for (int cc = 0; cc < CPL; ++cc) acc[cc] = float4_t{0.f, 0.f, 0.f, 0.f};
+        lacc = float4_t{0.f, 0.f, 0.f, 0.f};
+    };
+
+    if constexpr (!ROUNDS) {
+        // the whole union at once: the accumulators come to life only after the exponentials are packed
+        const int n_steps = (n_union + 31) >> 5;  // <= kUnionSteps because u_max <= 32 * kUnionSteps
+        gather(k, d_qk, kShiftK, 0, n_union, n_steps);
+        __syncthreads();
+        half8_t p[kUnionSteps];
+        unsigned act;
+        scores(n_steps, neg_inf, p, act);
+        __syncthreads();
+        gather(v, d_v, kShiftV, 0, n_union, n_steps);  // V rows over the K rows
+        __syncthreads();
+        clear_sums();
+        weighted_sum(p, act);
+    } else {
+        // rounds of u_max ranks: K rows, scores, V rows, sums - the maximum and the sums run across the rounds
+        clear_sums();
+        float mx_run = neg_inf;
+        const int n_rounds = (n_union + u_max - 1) / u_max;
+        for (int round = 0; round < n_rounds; ++round) {
+            const int u_first = round * u_max;
+            const int n_here = (n_union - u_first) < u_max ? (n_union - u_first) : u_max;
+            const int n_steps = (n_here + 31) >> 5;
+            if (round > 0) {
+                __syncthreads();  // every wave is done with the previous round's V rows and row masks
+                for (int w = tid; w < mask_words; w += n_threads) l.rowmask[w] = (unsigned)masks[round * mask_words + w];
+            }
+            gather(k, d_qk, kShiftK, u_first, n_here, n_steps);
+            __syncthreads();
+            half8_t p[kUnionSteps];
+            unsigned act;
+            const float mx_new = scores(n_steps, mx_run, p, act);
+            if (round > 0) {
+                // what the earlier rounds accumulated was taken against their maximum: bring it to the new one
+                // (0 where the row had no column yet, 1 where it still has none)
+                const float f = mx_new == neg_inf ? 1.f
+                                : (mx_run == neg_inf ? 0.f : __builtin_amdgcn_exp2f((mx_run - mx_new) * s2a));
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float fe = from_lane(f, (4 * g + e) & 15);  // accumulator register e of lane (c, g) is scalar row 4g + e
+                    lacc[e] *= fe;
+#pragma unroll
+                    for (int cc = 0; cc < CPL; ++cc) acc[cc][e] *= fe;
+                }
+            }
+            mx_run = mx_new;
+            __syncthreads();
+            gather(v, d_v, kShiftV, u_first, n_here, n_steps);
+            __syncthreads();
+            weighted_sum(p, act);
         }
     }
+    // normalise and store
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         const long long row = q_global + 4 * g + e;  // accumulator register e of lane (c, g) is scalar row 4g + e
@@ -687,12 +773,16 @@ struct UnionShape {
     int rows;    // vector rows per workgroup actually used
     int u_max;   // distinct columns a workgroup can hold in LDS
     size_t lds;
+    size_t plan_lds;  // LDS of the plan kernel for this shape
 };
 
-static bool union_shape(UnionShape &s, int vec_length, int n, int d_qk, int d_v, int rows, bool planned)
+// plan_rounds: 0 for launches that rebuild the union, else the rounds of the plan (1..kMaxPlanRounds).
+static bool union_shape(UnionShape &s, int vec_length, int n, int d_qk, int d_v, int rows, int plan_rounds)
 {
+    if (plan_rounds < 0 || plan_rounds > kMaxPlanRounds) return false;
     // Half of a CU's LDS per workgroup, so that two workgroups overlap each other's memory phases.  With a
     // plan the column bitmap, its prefix sums and the column list stay out of the attention kernel's LDS.
+    const bool planned = plan_rounds > 0;
     const size_t budget = (planned ? 80 : 72) * 1024;
     const int rpw = 16 / vec_length;
     s.waves = ceil_div(rows < 1 ? 1 : rows, rpw);
@@ -708,8 +798,9 @@ static bool union_shape(UnionShape &s, int vec_length, int n, int d_qk, int d_v,
     if (fixed + 32 * per_union_row > budget) return false;  // the column bitmap alone fills the budget
     s.u_max = (int)((budget - fixed) / per_union_row) & ~31;
     if (s.u_max > 32 * kUnionSteps) s.u_max = 32 * kUnionSteps;
-    // the plan kernel holds the bitmap and the column list of one workgroup in LDS
-    if (planned && build + (size_t)s.u_max * sizeof(int) > 160 * 1024) return false;
+    // the plan kernel holds the bitmap, the masks of every round and the column list of one workgroup in LDS
+    s.plan_lds = planned ? build + (plan_rounds - 1) * mask + (size_t)plan_rounds * s.u_max * sizeof(int) : 0;
+    if (s.plan_lds > 160 * 1024) return false;
     s.lds = fixed + (size_t)s.u_max * per_union_row;
     return true;
 }
@@ -721,53 +812,54 @@ static bool union_dims_ok(int d_qk, int d_v)
     return true;
 }
 
-template <int V, int KS, int CPL, bool PLANNED>
-static int launch_one(int m_vec, int n, int d_qk, int d_v, int rows, const int *row_offsets, const int *col_indices,
-                      const int *plan, const half_t *q, const half_t *k, const half_t *v, half_t *out, float scale,
-                      hipStream_t stream, const Batch &batch, long long stride_v)
+struct UnionLaunch {
+    int m_vec, n, d_qk, d_v, rows, plan_rounds;
+    const int *row_offsets, *col_indices, *plan;
+    const half_t *q, *k, *v;
+    half_t *out;
+    float scale;
+    hipStream_t stream;
+    const Batch *batch;
+    long long stride_v;
+};
+
+template <int V, int KS, int CPL, int MODE>
+static int launch_one(const UnionLaunch &a)
 {
     UnionShape s;
-    if (!union_shape(s, V, n, d_qk, d_v, rows, PLANNED)) return hipErrorNotSupported;
-    auto kernel = sparse_attention_union_kernel<V, KS, CPL, PLANNED>;
+    if (!union_shape(s, V, a.n, a.d_qk, a.d_v, a.rows, a.plan_rounds)) return hipErrorNotSupported;
+    auto kernel = sparse_attention_union_kernel<V, KS, CPL, MODE>;
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr != hipSuccess) return (int)attr;
-    const int blocks = ceil_div(m_vec, s.rows);
-    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)batch.count), dim3(64 * s.waves), s.lds, stream, m_vec,
-                       n, d_qk, d_v, s.u_max, row_offsets, col_indices, plan, q, k, v, out, batch.stride_a,
-                       batch.stride_b, stride_v, batch.stride_out, scale);
+    const int blocks = ceil_div(a.m_vec, s.rows);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)a.batch->count), dim3(64 * s.waves), s.lds, a.stream,
+                       a.m_vec, a.n, a.d_qk, a.d_v, s.u_max, a.plan_rounds, a.row_offsets, a.col_indices, a.plan, a.q,
+                       a.k, a.v, a.out, a.batch->stride_a, a.batch->stride_b, a.stride_v, a.batch->stride_out, a.scale);
     return (int)hipGetLastError();
 }
 
-template <int V, bool PLANNED>
-static int launch_shape(int m_vec, int n, int d_qk, int d_v, int rows, const int *row_offsets, const int *col_indices,
-                        const int *plan, const half_t *q, const half_t *k, const half_t *v, half_t *out, float scale,
-                        hipStream_t stream, const Batch &batch, long long stride_v)
+template <int V, int MODE>
+static int launch_shape(const UnionLaunch &a)
 {
-#define VS_ATT(KS, CPL)                                                                                             \
-    return launch_one<V, KS, CPL, PLANNED>(m_vec, n, d_qk, d_v, rows, row_offsets, col_indices, plan, q, k, v, out, \
-                                           scale, stream, batch, stride_v)
-    if (d_v <= 64) {
-        if (d_qk <= 32) VS_ATT(1, 4);
-        if (d_qk <= 64) VS_ATT(2, 4);
-        VS_ATT(4, 4);
+    if (a.d_v <= 64) {
+        if (a.d_qk <= 32) return launch_one<V, 1, 4, MODE>(a);
+        if (a.d_qk <= 64) return launch_one<V, 2, 4, MODE>(a);
+        return launch_one<V, 4, 4, MODE>(a);
     }
-    if (d_qk <= 32) VS_ATT(1, 8);
-    if (d_qk <= 64) VS_ATT(2, 8);
-    VS_ATT(4, 8);
-#undef VS_ATT
+    if (a.d_qk <= 32) return launch_one<V, 1, 8, MODE>(a);
+    if (a.d_qk <= 64) return launch_one<V, 2, 8, MODE>(a);
+    return launch_one<V, 4, 8, MODE>(a);
 }
 
-template <bool PLANNED>
-static int launch_v(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, const int *row_offsets,
-                    const int *col_indices, const int *plan, const half_t *q, const half_t *k, const half_t *v,
-                    half_t *out, float scale, hipStream_t stream, const Batch &batch, long long stride_v)
+template <int MODE>
+static int launch_v(int vec_length, const UnionLaunch &a)
 {
     switch (vec_length) {
-    case 1: return launch_shape<1, PLANNED>(m_vec, n, d_qk, d_v, rows, row_offsets, col_indices, plan, q, k, v, out, scale, stream, batch, stride_v);
-    case 2: return launch_shape<2, PLANNED>(m_vec, n, d_qk, d_v, rows, row_offsets, col_indices, plan, q, k, v, out, scale, stream, batch, stride_v);
-    case 4: return launch_shape<4, PLANNED>(m_vec, n, d_qk, d_v, rows, row_offsets, col_indices, plan, q, k, v, out, scale, stream, batch, stride_v);
-    case 8: return launch_shape<8, PLANNED>(m_vec, n, d_qk, d_v, rows, row_offsets, col_indices, plan, q, k, v, out, scale, stream, batch, stride_v);
+    case 1: return launch_shape<1, MODE>(a);
+    case 2: return launch_shape<2, MODE>(a);
+    case 4: return launch_shape<4, MODE>(a);
+    case 8: return launch_shape<8, MODE>(a);
     default: return hipErrorInvalidValue;
     }
 }
@@ -778,57 +870,56 @@ static bool union_supported(int vec_length, int n, int d_qk, int d_v)
     return n >= 0 && n <= 1024 * 1024 && union_dims_ok(d_qk, d_v);  // the column bitmap lives in LDS
 }
 
-int sparse_attention_union_capacity(int vec_length, int n, int d_qk, int d_v, int rows, bool with_plan, int *rows_used)
+int sparse_attention_union_capacity(int vec_length, int n, int d_qk, int d_v, int rows, int plan_rounds, int *rows_used)
 {
     UnionShape s;
     if (!union_supported(vec_length, n, d_qk, d_v) || d_v % 8 != 0) return 0;
-    if (!union_shape(s, vec_length, n, d_qk, d_v, rows, with_plan)) return 0;
+    if (!union_shape(s, vec_length, n, d_qk, d_v, rows, plan_rounds)) return 0;
     if (rows_used) *rows_used = s.rows;
-    return s.u_max;
+    return plan_rounds > 1 ? plan_rounds * s.u_max : s.u_max;
 }
 
-long long sparse_attention_plan_bytes(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows)
+long long sparse_attention_plan_bytes(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, int plan_rounds)
 {
     UnionShape s;
-    if (m_vec < 0 || !union_supported(vec_length, n, d_qk, d_v)) return 0;
-    if (!union_shape(s, vec_length, n, d_qk, d_v, rows, true)) return 0;
-    const long long stride = 4 + union_mask_words(s.rows) + s.u_max;
+    if (m_vec < 0 || plan_rounds < 1 || !union_supported(vec_length, n, d_qk, d_v)) return 0;
+    if (!union_shape(s, vec_length, n, d_qk, d_v, rows, plan_rounds)) return 0;
+    const long long stride = 4 + plan_rounds * ((long long)union_mask_words(s.rows) + s.u_max);
     return (long long)sizeof(int) * (kPlanHeader + stride * ceil_div(m_vec, s.rows));
 }
 
-int launch_sparse_attention_plan(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, const int *row_offsets,
-                                 const int *col_indices, int *plan, long long plan_bytes, hipStream_t stream)
+int launch_sparse_attention_plan(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, int plan_rounds,
+                                 const int *row_offsets, const int *col_indices, int *plan, long long plan_bytes,
+                                 hipStream_t stream)
 {
     UnionShape s;
-    if (!union_supported(vec_length, n, d_qk, d_v)) return hipErrorNotSupported;
-    if (!union_shape(s, vec_length, n, d_qk, d_v, rows, true)) return hipErrorNotSupported;
-    const long long need = sparse_attention_plan_bytes(m_vec, vec_length, n, d_qk, d_v, rows);
+    if (plan_rounds < 1 || !union_supported(vec_length, n, d_qk, d_v)) return hipErrorNotSupported;
+    if (!union_shape(s, vec_length, n, d_qk, d_v, rows, plan_rounds)) return hipErrorNotSupported;
+    const long long need = sparse_attention_plan_bytes(m_vec, vec_length, n, d_qk, d_v, rows, plan_rounds);
     if (plan_bytes < need) return hipErrorInvalidValue;
     if (m_vec == 0) return hipSuccess;
-    const int n_words = (((n + 31) / 32) + 3) & ~3;
-    const size_t lds = 2 * (size_t)n_words * sizeof(unsigned) + 16 * sizeof(int) +
-                       (size_t)union_mask_words(s.rows) * sizeof(unsigned) + (size_t)s.u_max * sizeof(int);
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(sparse_attention_plan_kernel),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (attr != hipSuccess) return (int)attr;
-    hipLaunchKernelGGL(sparse_attention_plan_kernel, dim3((unsigned)ceil_div(m_vec, s.rows)), dim3(256), lds, stream,
-                       m_vec, vec_length, n, s.rows, s.u_max, row_offsets, col_indices, plan);
+    hipLaunchKernelGGL(sparse_attention_plan_kernel, dim3((unsigned)ceil_div(m_vec, s.rows)), dim3(256), s.plan_lds,
+                       stream, m_vec, vec_length, n, s.rows, s.u_max, plan_rounds, row_offsets, col_indices, plan);
     return (int)hipGetLastError();
 }
 
-int launch_sparse_attention_union(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, const int *row_offsets,
-                                  const int *col_indices, const int *plan, const half_t *q, const half_t *k,
-                                  const half_t *v, half_t *out, float scale, hipStream_t stream, const Batch &batch,
-                                  long long stride_v)
+int launch_sparse_attention_union(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, int plan_rounds,
+                                  const int *row_offsets, const int *col_indices, const int *plan, const half_t *q,
+                                  const half_t *k, const half_t *v, half_t *out, float scale, hipStream_t stream,
+                                  const Batch &batch, long long stride_v)
 {
     if (m_vec == 0 || batch.count == 0 || d_v == 0) return hipSuccess;
     if (batch.count > 65535) return hipErrorNotSupported;
     if (!union_supported(vec_length, n, d_qk, d_v)) return hipErrorNotSupported;
-    if (plan)
-        return launch_v<true>(m_vec, vec_length, n, d_qk, d_v, rows, row_offsets, col_indices, plan, q, k, v, out, scale,
-                              stream, batch, stride_v);
-    return launch_v<false>(m_vec, vec_length, n, d_qk, d_v, rows, row_offsets, col_indices, nullptr, q, k, v, out, scale,
-                           stream, batch, stride_v);
+    if (!plan) plan_rounds = 0;
+    const UnionLaunch a = {m_vec, n, d_qk, d_v, rows, plan_rounds, row_offsets, col_indices, plan, q, k, v, out,
+                           scale, stream, &batch, stride_v};
+    if (plan_rounds > 1) return launch_v<2>(vec_length, a);
+    if (plan_rounds == 1) return launch_v<1>(vec_length, a);
+    return launch_v<0>(vec_length, a);
 }
 
 }  // namespace vs
