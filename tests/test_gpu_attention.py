@@ -316,7 +316,7 @@ def test_plan_raises_the_union_capacity(gpu, V, seq, half_width, stride, rows):
 @pytest.mark.parametrize("V,seq,half_width,stride,dims,want_rounds", [
     (8, 4096, 300, 64, (64, 64), 2),      # two rounds of 512 ranks
     (8, 4096, 900, 128, (64, 64), 4),     # four rounds
-    (2, 2048, 400, 0, (32, 128), 4),      # plain band, four rounds of 256 ranks with the wide V rows
+    (2, 2048, 400, 0, (32, 128), 2),      # plain band, wide V rows: one workgroup per CU, two rounds
     (1, 2048, 400, 256, (64, 64), 2),     # 128 vector rows per workgroup, masks restaged every round
 ])
 def test_planned_launch_takes_large_unions_in_rounds(gpu, V, seq, half_width, stride, dims, want_rounds):

@@ -228,6 +228,9 @@ constexpr int union_pitch(int ks, int cpl)
     return (32 * ks > 16 * cpl ? 32 * ks : 16 * cpl) + 8;
 }
 
+// Head widths above 64 on either side (128 halves per K or V row).
+constexpr bool union_wide(int ks, int cpl) { return ks == 4 || cpl == 8; }
+
 // The K rows of one 32-rank step as MFMA A operands: a[u][kk] = row 32t + 16u + c, halves 32kk + 8g .. +8.
 template <int KS, int PITCH>
 __device__ __forceinline__ void load_k_step(half8_t (&a)[2][KS], const half_t *k_lane, int t)
@@ -423,8 +426,10 @@ sparse_attention_plan_kernel(int m_vec, int vec_length, int n, int rows_per_bloc
 // union in LDS at once as in mode 0; 2 (ROUNDS): a union of up to plan_rounds * u_max columns, u_max at a
 // time.  A plan made for another mask shape or launch shape sends every workgroup to the per-row path.
 template <int V, int KS, int CPL, int MODE>
-// four waves per SIMD: two eight-wave workgroups per CU
-__global__ void __launch_bounds__(512, 4)
+// Heads up to 64 wide: four waves per SIMD (128 registers), two eight-wave workgroups per CU.  Wider heads
+// hold twice the Q / K / V slices per lane and 272-byte rows in LDS: two waves per SIMD (256 registers), one
+// workgroup per CU with all of its LDS.
+__global__ void __launch_bounds__(512, union_wide(KS, CPL) ? 2 : 4)
 sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max, int plan_rounds,
                               const int *__restrict__ row_offsets, const int *__restrict__ col_indices,
                               const int *__restrict__ plan,
@@ -780,16 +785,17 @@ struct UnionShape {
 static bool union_shape(UnionShape &s, int vec_length, int n, int d_qk, int d_v, int rows, int plan_rounds)
 {
     if (plan_rounds < 0 || plan_rounds > kMaxPlanRounds) return false;
-    // Half of a CU's LDS per workgroup, so that two workgroups overlap each other's memory phases.  With a
-    // plan the column bitmap, its prefix sums and the column list stay out of the attention kernel's LDS.
+    // Half of a CU's LDS per workgroup, so that two workgroups overlap each other's memory phases (wide heads:
+    // one workgroup per CU, all of it).  With a plan the column bitmap, its prefix sums and the column list
+    // stay out of the attention kernel's LDS.
     const bool planned = plan_rounds > 0;
-    const size_t budget = (planned ? 80 : 72) * 1024;
+    const int ks = d_qk <= 32 ? 1 : (d_qk <= 64 ? 2 : 4);
+    const int cpl = d_v <= 64 ? 4 : 8;
+    const size_t budget = (union_wide(ks, cpl) ? 152 : (planned ? 80 : 72)) * 1024;
     const int rpw = 16 / vec_length;
     s.waves = ceil_div(rows < 1 ? 1 : rows, rpw);
     if (s.waves > 8) s.waves = 8;
     s.rows = s.waves * rpw;
-    const int ks = d_qk <= 32 ? 1 : (d_qk <= 64 ? 2 : 4);
-    const int cpl = d_v <= 64 ? 4 : 8;
     const int n_words = (((n + 31) / 32) + 3) & ~3;
     const size_t mask = (size_t)union_mask_words(s.rows) * sizeof(unsigned);
     const size_t build = 2 * (size_t)n_words * sizeof(unsigned) + 16 * sizeof(int) + mask;  // + one int per column
