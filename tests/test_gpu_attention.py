@@ -143,6 +143,12 @@ def test_fused_and_unfused_layers_agree(gpu):
     b = layer.forward(q, k, v, fused=False).float().cpu().numpy()
     rms = float(np.sqrt(np.mean(b * b)))
     assert float(np.max(np.abs(a - b))) <= 1e-2 * rms
+    # the default: one launch where blocks of rows share their columns, two launches where they do not
+    assert layer.union_rows(d, d) >= 2
+    assert torch.equal(layer.forward(q, k, v), layer.forward(q, k, v, fused="layer"))
+    scattered = ops.SparseAttention(cv.uniform_pattern(seq // V, seq, 0.9, seed=2, vec_length=V))
+    assert scattered.union_rows(d, d) == 1
+    assert torch.equal(scattered.forward(q, k, v), scattered.forward(q, k, v, fused=True))
 
 
 def test_attention_steps_match_the_oracle_chain(gpu):

@@ -32,6 +32,7 @@ int check_spmm(int m_vec, int vec_length, int k, int n, const int *row_indices, 
     if (!row_indices || !row_offsets || !out) return VS_ERROR_INVALID_VALUE;
     // column_indices / values may be null when the pattern has no nonzero at all (an empty device
     // allocation); the host cannot see the pattern, so only the dense operand is required here.
+    (void)column_indices;
     if (n > 0 && !rhs) return VS_ERROR_INVALID_VALUE;
     if (!aligned(values, 2 * (size_t)vec_length) || !aligned(rhs, 16) || !aligned(out, 8 * out_elem))
         return VS_ERROR_INVALID_VALUE;
