@@ -150,10 +150,11 @@ int vs_cuda_sddmm_f16_f32out(int m_vec, int k, int n, int nonzeros_vec,
  * of the pattern (row_offsets[m_vec]) and of its longest vector row when the caller
  * knows them, negative otherwise.  They only size the workgroups (the unbatched SpMM
  * entry points keep the reference's argument list, which does not carry them, and
- * size them by n instead): by the mean row length, and - when the longest row is
- * more than four times the mean - with enough waves per row that the longest one
- * does not outlast the rest of the launch.  Results do not depend on them beyond the
- * order of the fp32 summation.
+ * size them by n instead): by the longest row while the launch leaves room on the
+ * chip, by the mean row length once it fills it, and - when the longest row is more
+ * than four times the mean - with enough waves per row that the longest one does not
+ * outlast the rest of the launch.  Results do not depend on them beyond the order of
+ * the fp32 summation.
  */
 int vs_wmma_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
                              int longest_row_vec, const int *row_indices, const int *row_offsets,

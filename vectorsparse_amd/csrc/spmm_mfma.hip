@@ -351,8 +351,12 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
         if (batch.nonzeros_vec >= 0) {
             // Row lengths known: a wave is worth launching for about three 32-vector steps (measured over
             // the ResNet-shaped grid: within 0.4 % of the best power of two, 7 % better than sizing by n).
+            // While the chip has room (`waves` so far is the room per workgroup) the workgroup of the longest
+            // row ends last, so that row sets the size; idle waves of the shorter rows cost nothing then.
             const int steps = ceil_div(ceil_div(batch.nonzeros_vec, m_vec), kStep);
-            const int by_rows = next_pow2(ceil_div(steps > 0 ? steps : 1, 3));
+            const int longest_known = ceil_div(batch.longest_row_vec > 0 ? batch.longest_row_vec : 0, kStep);
+            const int sizing = longest_known > steps ? longest_known : steps;
+            const int by_rows = next_pow2(ceil_div(sizing > 0 ? sizing : 1, 3));
             if (waves > by_rows) waves = by_rows;
             if (waves < 2 && steps >= 4) waves = 2;
             // A few rows far longer than the mean: a wave takes about half a microsecond per step of a lone
