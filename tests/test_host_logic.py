@@ -1,0 +1,57 @@
+"""Host-side choices of the Python layer that need no GPU: they only read the mask and ask the library's
+host-only capacity query."""
+import numpy as np
+
+from vectorsparse_amd import colvec_csr as cv
+from vectorsparse_amd import ops
+
+
+def _largest_union(mask, rows):
+    ro, ci = mask.row_offsets, mask.column_indices
+    return max(int(np.unique(ci[ro[f]:ro[min(f + rows, mask.m_vec)]]).size) for f in range(0, mask.m_vec, rows))
+
+
+def test_attention_launch_shape_follows_the_mask():
+    shape = ops.SparseAttention._union_shape
+    # band + strided columns: eight waves per workgroup, the whole union in LDS at once
+    band = cv.band_strided_pattern(4096, 8, band_half_width=128, stride=128)
+    assert shape(band, 64, 64) == (16, 1)
+    assert _largest_union(band, 16) <= 512
+    # a 513-wide window: the same workgroups, unions of more than 512 columns in two rounds
+    window = cv.band_strided_pattern(4096, 8, band_half_width=256, stride=4096)
+    assert 512 < _largest_union(window, 16) <= 1024
+    assert shape(window, 64, 64) == (16, 2)
+    # wide heads get the whole LDS of a CU: still one round for the band
+    assert shape(band, 128, 128) == (16, 1)
+    # every vector length fills its waves with 16 scalar rows
+    for V in (1, 2, 4):
+        assert shape(cv.band_strided_pattern(2048, V, band_half_width=128, stride=128), 64, 64) == (128 // V, 1)
+    # scattered columns: a dense tile over the union would be mostly masked out -> one row per workgroup
+    scattered = cv.uniform_pattern(512, 4096, 0.9, seed=3, vec_length=8)
+    assert shape(scattered, 64, 64) == (1, 1)
+    # head widths the union kernel does not take
+    assert shape(band, 64, 36) == (1, 1)
+    # empty masks
+    empty = cv.ColVecCSR(4, 64, 8, np.zeros(5, np.int32), np.zeros(0, np.int32))
+    assert shape(empty, 64, 64) == (1, 1)
+
+
+def _moving_blocks(m_vec, n, V, rows_per_block, width=600, step=700):
+    """Every vector row holds `width` consecutive columns; the window jumps by `step` every rows_per_block rows."""
+    lengths = np.full(m_vec, width, dtype=np.int64)
+    offsets = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    cols = np.concatenate([np.arange(width) + step * ((r // rows_per_block) % 11) for r in range(m_vec)])
+    return cv.ColVecCSR(m_vec, n, V, offsets, cols.astype(np.int32)).validate()
+
+
+def test_small_workgroups_only_where_they_beat_the_per_row_kernel():
+    """Unions that fit only small blocks of rows: two waves are taken for V <= 4, never for V = 8."""
+    shape = ops.SparseAttention._union_shape
+    # V = 4: 16 rows (four waves) span four windows, more than four rounds hold; 8 rows (two waves) span two
+    mask = _moving_blocks(256, 8192, 4, rows_per_block=4)
+    assert _largest_union(mask, 16) > 2048 >= _largest_union(mask, 8)
+    assert shape(mask, 64, 64)[0] == 8
+    # V = 8: 8 rows (four waves) do not fit, 4 rows (two waves) would - but lose to the per-row kernel
+    mask = _moving_blocks(256, 8192, 8, rows_per_block=2)
+    assert _largest_union(mask, 8) > 2048 >= _largest_union(mask, 4)
+    assert shape(mask, 64, 64) == (1, 1)
