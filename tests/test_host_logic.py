@@ -55,3 +55,21 @@ def test_small_workgroups_only_where_they_beat_the_per_row_kernel():
     mask = _moving_blocks(256, 8192, 8, rows_per_block=2)
     assert _largest_union(mask, 8) > 2048 >= _largest_union(mask, 4)
     assert shape(mask, 64, 64) == (1, 1)
+
+
+def test_device_problem_reads_the_row_statistics():
+    """Row statistics that steer the schedules (no launch: operands stay in host memory here)."""
+    rng = np.random.default_rng(0)
+    lengths = np.minimum((rng.pareto(1.5, 1024) + 0.3) * 150, 4608).astype(np.int64)
+    lengths[5] = 4608
+    ro, ci = cv._pattern_from_lengths(rng, 1024, 4608, lengths)
+    heavy = ops.DeviceProblem(cv.ColVecCSR(1024, 4608, 8, ro, ci), sort=True, device="cpu")
+    assert heavy.longest_row_vec == 4608 and heavy.nnz_vec == int(lengths.sum())
+    assert heavy.skewed                                    # SDDMM takes the nonzero-range schedule by default
+    swz = heavy.row_indices.numpy()
+    assert sorted(swz.tolist()) == list(range(1024)) and np.all(np.diff(lengths[swz]) <= 0)
+    even = ops.DeviceProblem(cv.uniform_pattern(1024, 4608, 0.9, seed=1, vec_length=8), device="cpu")
+    assert not even.skewed and even.longest_row_vec == 461
+    assert even.row_indices.numpy().tolist() == list(range(1024))
+    tiny = ops.DeviceProblem(cv.ColVecCSR(2, 8, 2, np.array([0, 0, 0], np.int32), np.zeros(0, np.int32)), device="cpu")
+    assert tiny.longest_row_vec == 0 and not tiny.skewed
