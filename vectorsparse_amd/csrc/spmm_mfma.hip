@@ -358,7 +358,9 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
             const int sizing = longest_known > steps ? longest_known : steps;
             const int by_rows = next_pow2(ceil_div(sizing > 0 ? sizing : 1, 3));
             if (waves > by_rows) waves = by_rows;
-            if (waves < 2 && steps >= 4) waves = 2;
+            // a second wave per row pays on a full chip from about ten steps per row (256 to 2048 vector rows,
+            // N = 256 to 1024: one wave 3-8 % ahead at 4 to 8 steps, two waves 3-10 % ahead at 12 and more)
+            if (waves < 2 && steps >= 10) waves = 2;
             // A few rows far longer than the mean: a wave takes about half a microsecond per step of a lone
             // long row, so that row gets at most sixteen steps per wave - as far as the idle waves this hands
             // to every short row stay cheap (about half a nanosecond each: 16384 waves per launch, or four
