@@ -377,8 +377,9 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
         } else {
             const int max_useful = next_pow2(ceil_div(n > 0 ? n : 1, kStep));  // a row holds at most n vectors
             if (waves > max_useful) waves = max_useful;
-            // two waves per row even on a full chip: measured 30 % faster than one on 8192 rows of ~280 vectors
-            if (waves < 2 && n >= 4 * kStep) waves = 2;
+            // On a full chip a second wave per row pays from about ten steps per row (see above); the row
+            // lengths are unknown here, so they are taken to be a tenth of n (90 % sparsity).
+            if (waves < 2 && n >= 100 * kStep) waves = 2;
         }
     }
     if (waves < 1) waves = 1;
