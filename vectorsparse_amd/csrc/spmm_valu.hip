@@ -105,16 +105,21 @@ spmm_valu_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
         return;
     }
 
-    float *mine = partial + (size_t)(wave * G + g) * V * TN;
+    // Group p starts at nonzero beg + p * U: on a short row only the first few groups had any, and only
+    // their partial tiles are written and summed (the others hold zeros).
+    int n_partials = (end - beg + U - 1) / U;
+    n_partials = n_partials < 1 ? 1 : (n_partials > n_waves * G ? n_waves * G : n_partials);
+    if (wave * G + g < n_partials) {
+        float *mine = partial + (size_t)(wave * G + g) * V * TN;
 #pragma unroll
-    for (int v = 0; v < V; ++v) {
-        float4_t lo = {acc[v][0], acc[v][1], acc[v][2], acc[v][3]};
-        float4_t hi = {acc[v][4], acc[v][5], acc[v][6], acc[v][7]};
-        *reinterpret_cast<float4_t *>(mine + v * TN + cl * 8) = lo;
-        *reinterpret_cast<float4_t *>(mine + v * TN + cl * 8 + 4) = hi;
+        for (int v = 0; v < V; ++v) {
+            float4_t lo = {acc[v][0], acc[v][1], acc[v][2], acc[v][3]};
+            float4_t hi = {acc[v][4], acc[v][5], acc[v][6], acc[v][7]};
+            *reinterpret_cast<float4_t *>(mine + v * TN + cl * 8) = lo;
+            *reinterpret_cast<float4_t *>(mine + v * TN + cl * 8 + 4) = hi;
+        }
     }
     __syncthreads();
-    const int n_partials = n_waves * G;
     for (int item = threadIdx.x; item < V * LR; item += blockDim.x) {
         const int v = item / LR;
         const int cl2 = item % LR;
@@ -155,14 +160,24 @@ static int launch_one(int m_vec, int k, int waves, const int *row_indices, const
     return (int)hipGetLastError();
 }
 
+// Lanes per column tile: as wide as the dense matrix allows (one group covers a whole row of it), narrower
+// while that leaves the chip without a workgroup per CU - narrow tiles put more groups on every nonzero range.
+static int valu_tile_lanes(int m_vec, int k, int batch)
+{
+    int lr = k <= 64 ? 8 : (k <= 128 ? 16 : (k <= 256 ? 32 : 64));
+    while (lr > 8 && (long long)m_vec * ceil_div(k, 8 * lr) * batch < 256) lr >>= 1;
+    return lr;
+}
+
 template <int V, typename OutT>
 static int launch_lr(int m_vec, int k, int waves, const int *row_indices, const int *row_offsets,
                      const int *column_indices, const half_t *values, const half_t *rhs, OutT *out,
                      hipStream_t stream, const Batch &batch)
 {
-    if (k <= 64) return launch_one<V, 8, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
-    if (k <= 128) return launch_one<V, 16, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
-    if (k <= 256) return launch_one<V, 32, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
+    const int lr = valu_tile_lanes(m_vec, k, batch.count);
+    if (lr == 8) return launch_one<V, 8, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
+    if (lr == 16) return launch_one<V, 16, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
+    if (lr == 32) return launch_one<V, 32, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
     return launch_one<V, 64, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
 }
 
@@ -176,13 +191,14 @@ int launch_spmm_valu(int m_vec, int vec_length, int k, int n, const int *row_ind
     if (k % 8 != 0 || batch.count > 65535) return hipErrorNotSupported;
     int waves = options().spmm_waves;
     if (waves <= 0) {
-        const long long blocks = (long long)m_vec * ceil_div(k, 512) * batch.count;
+        const int lr = valu_tile_lanes(m_vec, k, batch.count);
+        const long long blocks = (long long)m_vec * ceil_div(k, 8 * lr) * batch.count;
         waves = 2;
         while (waves < 8 && blocks * waves < 8192) waves <<= 1;
         if (batch.nonzeros_vec >= 0) {
             // Row lengths known (batched entry points): a wave consumes 4 nonzeros per group and turn, and a
             // turn is one memory round trip, so a wave per turn of an average row is as wide as it pays.
-            const int groups = k <= 64 ? 8 : (k <= 128 ? 4 : (k <= 256 ? 2 : 1));
+            const int groups = 64 / lr;
             // (V = 8 does eight times the arithmetic per nonzero: twice the waves measured better)
             const int turns = ceil_div(ceil_div(batch.nonzeros_vec, m_vec), 4 * groups) * (vec_length == 8 ? 2 : 1);
             int by_rows = 1;
