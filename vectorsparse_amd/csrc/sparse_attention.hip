@@ -218,8 +218,8 @@ static int launch_one(int m_vec, int d_qk, int d_v, const int *row_indices, cons
     const size_t lds = (size_t)chunk * (V * (sizeof(float) + sizeof(half_t)) + sizeof(int)) + 3 * V * sizeof(float);
     if (lds > 150 * 1024) return hipErrorNotSupported;
     auto kernel = sparse_attention_kernel<V, KS, CPL>;
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+    static std::atomic<unsigned long long> lds_allowed{0};
+    const hipError_t attr = allow_large_lds(reinterpret_cast<const void *>(kernel), 150 * 1024, lds_allowed);
     if (attr != hipSuccess) return (int)attr;
     hipLaunchKernelGGL(kernel, dim3((unsigned)m_vec, (unsigned)batch.count), dim3(64 * waves), lds, stream, d_qk, d_v,
                        chunk, row_indices, row_offsets, col_indices, q, k, v, out, batch.stride_a, batch.stride_b,

@@ -835,8 +835,8 @@ static int launch_one(const UnionLaunch &a)
     UnionShape s;
     if (!union_shape(s, V, a.n, a.d_qk, a.d_v, a.rows, a.plan_rounds)) return hipErrorNotSupported;
     auto kernel = sparse_attention_union_kernel<V, KS, CPL, MODE>;
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    static std::atomic<unsigned long long> lds_allowed{0};
+    const hipError_t attr = allow_large_lds(reinterpret_cast<const void *>(kernel), 160 * 1024, lds_allowed);
     if (attr != hipSuccess) return (int)attr;
     const int blocks = ceil_div(a.m_vec, s.rows);
     hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)a.batch->count), dim3(64 * s.waves), s.lds, a.stream,
@@ -904,8 +904,8 @@ int launch_sparse_attention_plan(int m_vec, int vec_length, int n, int d_qk, int
     const long long need = sparse_attention_plan_bytes(m_vec, vec_length, n, d_qk, d_v, rows, plan_rounds);
     if (plan_bytes < need) return hipErrorInvalidValue;
     if (m_vec == 0) return hipSuccess;
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(sparse_attention_plan_kernel),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    static std::atomic<unsigned long long> lds_allowed{0};
+    const hipError_t attr = allow_large_lds(reinterpret_cast<const void *>(sparse_attention_plan_kernel), 160 * 1024, lds_allowed);
     if (attr != hipSuccess) return (int)attr;
     hipLaunchKernelGGL(sparse_attention_plan_kernel, dim3((unsigned)ceil_div(m_vec, s.rows)), dim3(256), s.plan_lds,
                        stream, m_vec, vec_length, n, s.rows, s.u_max, plan_rounds, row_offsets, col_indices, plan);

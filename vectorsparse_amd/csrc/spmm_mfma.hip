@@ -293,8 +293,8 @@ static int launch_idx(int m_vec, int k, int n, int waves, const int *row_indices
     const size_t lds = (size_t)waves * stage_bytes<V>() +
                        (waves > 1 ? (size_t)waves * V * (TN + 1) * sizeof(float) : 0);
     auto kernel = spmm_mfma_kernel<V, CPL, SOFTMAX, IDX32, OutT>;
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+    static std::atomic<unsigned long long> lds_allowed{0};
+    const hipError_t attr = allow_large_lds(reinterpret_cast<const void *>(kernel), 96 * 1024, lds_allowed);
     if (attr != hipSuccess) return (int)attr;
     hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)batch.count), dim3(64 * waves), lds, stream,
                        k, n_tiles, row_indices, row_offsets, column_indices, values, rhs, out,

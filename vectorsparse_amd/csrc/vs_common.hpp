@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace vs {
 
 typedef _Float16 half_t;
@@ -194,6 +196,20 @@ struct Options {
 Options &options();
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// Raise a kernel's dynamic LDS limit above the 64 KB default.  The attribute belongs to the current device, so
+// it is set once per (kernel, device): `done` is the call site's own mask of the devices already served.
+inline hipError_t allow_large_lds(const void *kernel, int bytes, std::atomic<unsigned long long> &done)
+{
+    int device = 0;
+    hipError_t status = hipGetDevice(&device);
+    if (status != hipSuccess) return status;
+    const unsigned long long bit = 1ull << (device & 63);
+    if (device < 64 && (done.load(std::memory_order_acquire) & bit)) return hipSuccess;
+    status = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (status == hipSuccess && device < 64) done.fetch_or(bit, std::memory_order_release);
+    return status;
+}
 
 // Waves per vector row for the SDDMM kernels; `group` = nonzero vectors a wave covers per step.
 int sddmm_auto_slots(int m_vec, int nonzeros_vec, int group);
