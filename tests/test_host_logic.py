@@ -73,3 +73,37 @@ def test_device_problem_reads_the_row_statistics():
     assert even.row_indices.numpy().tolist() == list(range(1024))
     tiny = ops.DeviceProblem(cv.ColVecCSR(2, 8, 2, np.array([0, 0, 0], np.int32), np.zeros(0, np.int32)), device="cpu")
     assert tiny.longest_row_vec == 0 and not tiny.skewed
+
+
+def test_sweep_benchmark_selection(tmp_path):
+    """The sweep driver's file handling (job_launcher.py:25-50): list files, ranges, layer widths, buckets."""
+    from vectorsparse_amd import sweep
+
+    root = tmp_path / "dlmc"
+    names = ["rn50/random_pruning/0.8/layer_a", "rn50/random_pruning/0.95/layer_b", "rn50/magnitude_pruning/0.9/layer_c"]
+    for i, name in enumerate(names):
+        path = root / (name + ".smtx")
+        path.parent.mkdir(parents=True, exist_ok=True)
+        pat = cv.uniform_pattern(8, 64, 0.5, seed=i, vec_length=1)
+        cv.write_smtx(str(path), pat.m_vec, pat.n, pat.row_offsets, pat.column_indices)
+    listing = tmp_path / "rn50_matrices.txt"
+    listing.write_text("".join(n + ".smtx\n" for n in names))
+    widths = tmp_path / "rn50_batchsizes.txt"
+    widths.write_text("layer_a,196\nlayer_b,49\nlayer_c,3136\n")
+
+    everything = sweep.file_benchmarks(str(root))
+    assert sorted(n for n, _ in everything) == sorted(names)
+    picked = sweep.file_benchmarks(str(root), str(listing), 1, 3)
+    assert [n for n, _ in picked] == names[1:3]
+    assert all(p.endswith(".smtx") and cv.read_smtx(p, 2).m_vec == 8 for _, p in picked)
+
+    table = sweep.layer_widths(str(widths))
+    assert table == {"layer_a": 196, "layer_b": 49, "layer_c": 3136}
+    assert sweep.widths_for(names[0], (64, 256), 1, table) == [64, 256]
+    assert sweep.widths_for(names[1], (-1,), 2, table) == [98]          # the layer's own width, scaled
+    assert sweep.int_list("1,2, 8") == (1, 2, 8)
+
+    assert sweep.sparsity_bucket(names[0], 0.79) == 0.8
+    assert sweep.sparsity_bucket(names[1], 0.5) == 0.95                 # the directory decides, not the file
+    assert sweep.sparsity_bucket(names[2], 0.5) == 0.9
+    assert sweep.sparsity_bucket("synthetic/m64", 0.8765) == 0.88

@@ -1,16 +1,24 @@
-"""ResNet-50-shaped SpMM sweep (and a square-mask SDDMM sweep) against dense fp16 GEMM.
+"""SpMM and SDDMM sweeps against dense fp16 GEMM: a synthetic ResNet-50-shaped grid, or a tree of .smtx files.
 
-    python -m vectorsparse_amd.sweep --out results.csv [--quick] [--op spmm|sddmm]
+    python -m vectorsparse_amd.sweep --out results.csv [--quick] [--op spmm|sddmm] [--hint]
+    python -m vectorsparse_amd.sweep --smtx-dir /data/dlmc --matrix-list /data/dlmc/rn50_matrices.txt \\
+           --start 0 --end 323 --dimK 64,128,256 --dimV 1,2,4,8 --csv-dir csv --out rn50.csv
 
 The counterpart of the reference's experiment driver (launch.py:11-36 -> job_launcher.py:38-63 ->
-ncu_profile.py:80-96, then plot_spmm.py:43-58): for every (M, K, sparsity, V) of the grid it times
-the MFMA path and the fine-grained path, times hipBLASLt's dense fp16 GEMM once per (M, K), and
-reports speed-up = dense duration / kernel duration with the geometric mean per (V, sparsity)
-bucket.  Patterns are synthetic (uniform vector placement, exactly round((1-s)K) vectors per row)
-because the DLMC files are not available offline; any directory of .smtx files can be swept instead
-with --smtx-dir.  Durations are device time per launch (HIP events around a HIP-graph replay).
---csv-dir also writes one duration file per (benchmark, k, v, kernel) point under the names and in the
-record layout the reference's plot scripts read (file_name_server.py:6-45, :57-81), dense baseline included.
+ncu_profile.py:80-96, then plot_spmm.py:43-58 / plot_sddmm.py): for every (benchmark, k, V) it times the MFMA
+path and the fine-grained path, times hipBLASLt's dense fp16 product of the same shape once, and reports
+speed-up = dense duration / kernel duration with the geometric mean per (V, sparsity) bucket.
+
+Benchmarks: without --smtx-dir a synthetic grid (uniform vector placement, exactly round((1-s) n) vectors per
+row; the DLMC files are not available offline) - SpMM: M x K of the ResNet-50 layer shapes with N = 256,
+SDDMM: square masks M = N in {512..4096} with K in {64, 128, 256}.  With --smtx-dir every .smtx below it, or
+the entries [--start, --end) of --matrix-list (one path per line, relative to --smtx-dir, as in the
+reference's rn50_matrices.txt); the file's pattern is the sparse operand (SpMM) or the mask (SDDMM), --dimK
+the dense width / contraction length (job_launcher.py:41-50: a value <= 0 looks the layer up in --batchsizes,
+lines `layer,k`; --dimK-mul scales it), --dimV the vector lengths.
+Durations are device time per launch (HIP events around a HIP-graph replay).  --csv-dir also writes one
+duration file per (benchmark, k, v, kernel) point under the names and in the record layout the reference's
+plot scripts read (file_name_server.py:6-45, :57-81), dense baseline included.
 """
 import argparse
 import csv
@@ -34,49 +42,67 @@ def spmm_bytes(pat, n_dense):
             + 2 * k_ref * n_dense + 2 * pat.m * n_dense)
 
 
-def geomean(xs):
-    xs = [x for x in xs if x > 0]
-    return math.exp(sum(math.log(x) for x in xs) / len(xs)) if xs else float("nan")
-
-
 def sddmm_bytes(pat, k):
     n_ref = int(np.unique(pat.column_indices[:pat.nnz_vec]).size)
     return 2 * pat.m * k + 2 * n_ref * k + 4 * pat.nnz_vec + 4 * (pat.m_vec + 1) + 4 * pat.m_vec + 2 * pat.nnz
 
 
-def sddmm_sweep(args, torch, cv, ops, time_launches):
-    sizes, ks, ss = ((512, 1024, 2048, 4096), (64, 128, 256), SPARSITIES) if not args.quick else \
-        ((512, 2048), (64, 256), (0.7, 0.9, 0.98))
-    rows, dense_us = [], {}
-    for M in sizes:
-        for K in ks:
-            A = torch.randn((M, K), dtype=torch.float16, device="cuda")
-            B = torch.randn((M, K), dtype=torch.float16, device="cuda")
-            full = torch.empty((M, M), dtype=torch.float16, device="cuda")
-            dense_us[(M, K)] = time_launches(torch, lambda: torch.matmul(A, B.t(), out=full), args.iters)
-            for s in ss:
-                for V in VS:
-                    seed = (M * 1000003 + K * 10007 + int(round(s * 100)) * 101 + V) % (2 ** 31)
-                    pat = cv.uniform_pattern(M // V, M, s, seed, V)
-                    prob = ops.DeviceProblem(pat, sort=True)
-                    out = torch.empty((pat.nnz_vec, V), dtype=torch.float16, device="cuda")
-                    flops = 2.0 * pat.nnz * K
-                    bm = "synthetic/uniform/%g/m%d_n%d" % (s, M, M)
-                    args.per_point(bm, K, V, "dense", "sddmm", "hipblaslt_gemm_f16", dense_us[(M, K)])
-                    for kernel in ("wmma", "cuda"):
-                        us = time_launches(torch, lambda: prob.sddmm(A, B, kernel=kernel, out=out), args.iters)
-                        args.per_point(bm, K, V, kernel, "sddmm",
-                                       "sddmm_mfma_kernel" if kernel == "wmma" else "sddmm_valu_kernel", us)
-                        rows.append({"bm": "synthetic", "M": M, "K": K, "N": M, "sparsity": round(s, 4), "V": V,
-                                     "kernel": kernel, "nnz_vec": pat.nnz_vec, "us": round(us, 3),
-                                     "dense_us": round(dense_us[(M, K)], 3),
-                                     "speedup": round(dense_us[(M, K)] / us, 4),
-                                     "tflops": round(flops / us * 1e-6, 3),
-                                     "gbs": round(sddmm_bytes(pat, K) / us * 1e-3, 1)})
-                    print("M=N=%d K=%d s=%.2f V=%d  wmma %.2f us  cuda %.2f us  dense %.2f us" % (
-                        M, K, s, V, rows[-2]["us"], rows[-1]["us"], dense_us[(M, K)]), flush=True)
-    report(args.out, rows, "SDDMM: geometric-mean speed-up over the dense fp16 product A B^T (hipBLASLt)")
-    return 0
+def geomean(xs):
+    xs = [x for x in xs if x > 0]
+    return math.exp(sum(math.log(x) for x in xs) / len(xs)) if xs else float("nan")
+
+
+def int_list(text):
+    return tuple(int(x) for x in str(text).split(",") if x.strip())
+
+
+def sparsity_bucket(name, sparsity):
+    """The reference's plot scripts bucket a DLMC file by the sparsity directory in its path
+    (plot_spmm.py:45-58, '0.95' and '0.98' looked for before '0.9'); other names fall back to the
+    pattern's own sparsity."""
+    parts = name.replace("\\", "/").split("/")
+    for tag in ("0.95", "0.98", "0.9", "0.8", "0.7", "0.5"):
+        if tag in parts:
+            return float(tag)
+    return round(float(sparsity), 2)
+
+
+def file_benchmarks(smtx_dir, matrix_list=None, start=0, end=None):
+    """[(name below smtx_dir without extension, path)] - every .smtx below smtx_dir, or the entries
+    [start, end) of a list file (job_launcher.py:34-40: one benchmark per line, '.smtx' optional)."""
+    if matrix_list:
+        with open(matrix_list) as f:
+            names = [line.strip() for line in f if line.strip()]
+        names = names[start:end]
+        names = [n[:-len(".smtx")] if n.endswith(".smtx") else n for n in names]
+        return [(n, os.path.join(smtx_dir, n + ".smtx")) for n in names]
+    paths = sorted(glob.glob(os.path.join(smtx_dir, "**", "*.smtx"), recursive=True))
+    return [(os.path.relpath(p, smtx_dir)[:-len(".smtx")], p) for p in paths][start:end]
+
+
+def layer_widths(path):
+    """`layer,k` lines (the reference's rn50_batchsizes.txt, job_launcher.py:25-31) -> {layer: k}."""
+    table = {}
+    if path:
+        with open(path) as f:
+            for line in f:
+                if "," in line:
+                    layer, k = line.strip().split(",")[:2]
+                    table[layer] = int(k)
+    return table
+
+
+def widths_for(name, dim_ks, dim_k_mul, table):
+    """The k values to run for one benchmark: the requested ones, a value <= 0 replaced by the layer's own."""
+    out = []
+    for k in dim_ks:
+        if k <= 0:
+            layer = name.split("/")[-1]
+            if layer not in table:
+                raise SystemExit("--dimK <= 0 needs a --batchsizes entry for layer %s" % layer)
+            k = table[layer]
+        out.append(k * dim_k_mul)
+    return out
 
 
 def report(path, rows, title):
@@ -88,7 +114,7 @@ def report(path, rows, title):
     buckets = sorted({r["sparsity"] for r in rows})
     print("%-12s" % "kernel/V" + "".join("%9s" % ("s=%.2f" % b) for b in buckets))
     for kernel in ("wmma", "cuda"):
-        for V in VS:
+        for V in sorted({r["V"] for r in rows}):
             line = "%-12s" % ("%s V=%d" % (kernel, V))
             for b in buckets:
                 xs = [r["speedup"] for r in rows if r["kernel"] == kernel and r["V"] == V and r["sparsity"] == b]
@@ -99,19 +125,28 @@ def report(path, rows, title):
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--out", default="spmm_sweep.csv")
-    ap.add_argument("--quick", action="store_true", help="a 3 x 3 x 3 corner of the grid")
-    ap.add_argument("--smtx-dir", default=None, help="sweep every .smtx under this directory instead")
-    ap.add_argument("--op", choices=["spmm", "sddmm"], default="spmm",
-                    help="sddmm: masks of M = N in {512, 1024, 2048, 4096} x contraction K in {64, 128, 256} "
-                         "(the counterpart of the reference's SDDMM figure), dense baseline = the full A B^T")
+    ap.add_argument("--op", choices=["spmm", "sddmm"], default="spmm")
+    ap.add_argument("--quick", action="store_true", help="a 3 x 3 x 3 corner of the synthetic grid")
+    ap.add_argument("--smtx-dir", default=None, help="sweep .smtx files below this directory instead of the grid")
+    ap.add_argument("--matrix-list", default=None, help="file with one benchmark per line, relative to --smtx-dir")
+    ap.add_argument("--start", type=int, default=0, help="first entry of the list (or of the sorted directory) to run")
+    ap.add_argument("--end", type=int, default=None, help="one past the last entry to run")
+    ap.add_argument("--dimK", default=None,
+                    help="comma list: dense width (SpMM) / contraction length (SDDMM) for file benchmarks, default 256 "
+                         "(SpMM) or 64,128,256 (SDDMM); <= 0: the layer's own width from --batchsizes")
+    ap.add_argument("--dimK-mul", type=int, default=1, help="scale every k by this factor")
+    ap.add_argument("--batchsizes", default=None, help="file of `layer,k` lines for --dimK <= 0")
+    ap.add_argument("--dimV", default="1,2,4,8", help="comma list of vector lengths")
     ap.add_argument("--hint", action="store_true",
-                    help="call through the batched entry point with the pattern's nonzero count (workgroups sized "
-                         "by the real row lengths) instead of the reference-shaped entry points")
+                    help="SpMM through the batched entry point with the pattern's nonzero count and longest row "
+                         "(workgroups sized by the real row lengths) instead of the reference-shaped entry points")
     ap.add_argument("--iters", type=int, default=100, help="launches per timed HIP-graph replay")
     ap.add_argument("--csv-dir", default=None,
                     help="also write <csv-dir>/<spmm|sddmm>/<benchmark>_<kernel>_half_sort[_<alg>]_k<k>_v<v>.csv, one "
                          "profiler-style Duration record each, as the reference's plot scripts expect them")
     args = ap.parse_args(argv)
+    if args.matrix_list and not args.smtx_dir:
+        raise SystemExit("--matrix-list needs --smtx-dir")
 
     import torch
 
@@ -119,61 +154,90 @@ def main(argv=None):
     from . import ops
     from .benchmark_common import duration_csv_path, time_launches, write_duration_csv
 
-    def per_point(bm, dim_k, V, kernel, job, name, us):
-        if args.csv_dir:
-            write_duration_csv(duration_csv_path(args.csv_dir, bm, dim_k, V, kernel, job), name, us)
-    args.per_point = per_point
+    vs = int_list(args.dimV)
+    spmm = args.op == "spmm"
 
-    if args.op == "sddmm":
-        return sddmm_sweep(args, torch, cv, ops, time_launches)
-    ms, ks, ss = (MS, KS, SPARSITIES) if not args.quick else ((64, 512, 2048), (256, 1152, 4608), (0.7, 0.9, 0.98))
+    # (benchmark name, sparsity bucket or None, V -> pattern, the k values to run)
     cases = []
     if args.smtx_dir:
-        for path in sorted(glob.glob(os.path.join(args.smtx_dir, "**", "*.smtx"), recursive=True)):
-            for V in VS:
-                cases.append((path, V))
-    else:
+        table = layer_widths(args.batchsizes)
+        dim_ks = int_list(args.dimK) if args.dimK else ((N_DENSE,) if spmm else (64, 128, 256))
+        for name, path in file_benchmarks(args.smtx_dir, args.matrix_list, args.start, args.end):
+            cases.append((name, None, (lambda V, path=path: cv.read_smtx(path, V)),
+                          widths_for(name, dim_ks, args.dimK_mul, table)))
+    elif spmm:
+        ms, ks, ss = (MS, KS, SPARSITIES) if not args.quick else ((64, 512, 2048), (256, 1152, 4608), (0.7, 0.9, 0.98))
+        widths = [k * args.dimK_mul for k in (int_list(args.dimK) if args.dimK else (N_DENSE,))]
         for M in ms:
             for K in ks:
                 for s in ss:
-                    for V in VS:
-                        cases.append(((M, K, s), V))
+                    def make(V, M=M, K=K, s=s):
+                        seed = (M * 1000003 + K * 10007 + int(round(s * 100)) * 101 + V) % (2 ** 31)
+                        return cv.uniform_pattern(M // V, K, s, seed, V)
+                    cases.append(("synthetic/uniform/%g/m%d_k%d" % (s, M, K), s, make, widths))
+    else:
+        sizes, ks, ss = ((512, 1024, 2048, 4096), (64, 128, 256), SPARSITIES) if not args.quick else \
+            ((512, 2048), (64, 256), (0.7, 0.9, 0.98))
+        widths = [k * args.dimK_mul for k in (int_list(args.dimK) if args.dimK else ks)]
+        for M in sizes:
+            for s in ss:
+                def make(V, M=M, s=s):
+                    seed = (M * 1000003 + int(round(s * 100)) * 101 + V) % (2 ** 31)
+                    return cv.uniform_pattern(M // V, M, s, seed, V)
+                cases.append(("synthetic/uniform/%g/m%d_n%d" % (s, M, M), s, make, widths))
 
-    dense_us = {}
-    rows = []
-    for spec, V in cases:
-        if isinstance(spec, str):
-            pat = cv.read_smtx(spec, V)
-            M, K, s = pat.m, pat.n, pat.sparsity
-            label = os.path.basename(spec)
-            bm = os.path.relpath(spec, args.smtx_dir)
-        else:
-            M, K, s = spec
-            seed = (M * 1000003 + K * 10007 + int(round(s * 100)) * 101 + V) % (2 ** 31)
-            pat = cv.uniform_pattern(M // V, K, s, seed, V)
-            label = "synthetic"
-            bm = "synthetic/uniform/%g/m%d_k%d" % (s, M, K)
-        pat = cv.random_values(pat, seed=V + 7)
-        B = torch.from_numpy(cv.dense_uniform(K, N_DENSE, seed=11)).cuda()
-        out = torch.empty((M, N_DENSE), dtype=torch.float16, device="cuda")
-        if (M, K) not in dense_us:
-            A = torch.randn((M, K), dtype=torch.float16, device="cuda")
-            dense_us[(M, K)] = time_launches(torch, lambda: torch.matmul(A, B, out=out), args.iters)
-        args.per_point(bm, N_DENSE, V, "dense", "spmm", "hipblaslt_gemm_f16", dense_us[(M, K)])
-        prob = ops.DeviceProblem(pat, sort=True)
-        flops = 2.0 * pat.nnz * N_DENSE
-        nbytes = spmm_bytes(pat, N_DENSE)
-        for kernel in ("wmma", "cuda"):
-            us = time_launches(torch, lambda: prob.spmm(B, kernel=kernel, out=out, row_length_hint=args.hint), args.iters)
-            args.per_point(bm, N_DENSE, V, kernel, "spmm", "spmm_mfma_kernel" if kernel == "wmma" else "spmm_valu_kernel", us)
-            rows.append({"bm": label, "M": M, "K": K, "N": N_DENSE, "sparsity": round(s, 4), "V": V,
-                         "kernel": kernel, "nnz_vec": pat.nnz_vec, "us": round(us, 3),
-                         "dense_us": round(dense_us[(M, K)], 3), "speedup": round(dense_us[(M, K)] / us, 4),
-                         "tflops": round(flops / us * 1e-6, 3), "gbs": round(nbytes / us * 1e-3, 1)})
-        print("M=%d K=%d s=%.2f V=%d  wmma %.2f us  cuda %.2f us  dense %.2f us" % (
-            M, K, s, V, rows[-2]["us"], rows[-1]["us"], dense_us[(M, K)]), flush=True)
+    def per_point(bm, dim_k, V, kernel, name, us):
+        if args.csv_dir:
+            write_duration_csv(duration_csv_path(args.csv_dir, bm, dim_k, V, kernel, args.op), name, us)
 
-    report(args.out, rows, "SpMM: geometric-mean speed-up over dense fp16 GEMM (hipBLASLt)")
+    rows, dense_us = [], {}
+    for name, bucket, make, widths in cases:
+        for V in vs:
+            pat = cv.random_values(make(V), seed=V + 7)
+            if pat.nnz_vec == 0:
+                continue
+            M, n = pat.m, pat.n
+            s = bucket if bucket is not None else sparsity_bucket(name, pat.sparsity)
+            prob = ops.DeviceProblem(pat, sort=True)
+            for k in widths:
+                if spmm:
+                    # C[M, k] = A_sparse[M, n] B[n, k]
+                    B = torch.from_numpy(cv.dense_uniform(n, k, seed=11)).cuda()
+                    out = torch.empty((M, k), dtype=torch.float16, device="cuda")
+                    if (M, n, k) not in dense_us:
+                        A = torch.randn((M, n), dtype=torch.float16, device="cuda")
+                        dense_us[(M, n, k)] = time_launches(torch, lambda: torch.matmul(A, B, out=out), args.iters)
+                    run = {kern: (lambda kern=kern: prob.spmm(B, kernel=kern, out=out, row_length_hint=args.hint))
+                           for kern in ("wmma", "cuda")}
+                    flops, nbytes = 2.0 * pat.nnz * k, spmm_bytes(pat, k)
+                    names = {"wmma": "spmm_mfma_kernel", "cuda": "spmm_valu_kernel"}
+                else:
+                    # out[nnz] = (A[M, k] B[n, k]^T) sampled on the mask
+                    A = torch.randn((M, k), dtype=torch.float16, device="cuda")
+                    B = torch.randn((n, k), dtype=torch.float16, device="cuda")
+                    out = torch.empty((pat.nnz_vec, V), dtype=torch.float16, device="cuda")
+                    if (M, n, k) not in dense_us:
+                        full = torch.empty((M, n), dtype=torch.float16, device="cuda")
+                        dense_us[(M, n, k)] = time_launches(torch, lambda: torch.matmul(A, B.t(), out=full), args.iters)
+                        del full
+                    run = {kern: (lambda kern=kern: prob.sddmm(A, B, kernel=kern, out=out)) for kern in ("wmma", "cuda")}
+                    flops, nbytes = 2.0 * pat.nnz * k, sddmm_bytes(pat, k)
+                    names = {"wmma": "sddmm_mfma_kernel", "cuda": "sddmm_valu_kernel"}
+                dense = dense_us[(M, n, k)]
+                per_point(name, k, V, "dense", "hipblaslt_gemm_f16", dense)
+                for kern in ("wmma", "cuda"):
+                    us = time_launches(torch, run[kern], args.iters)
+                    per_point(name, k, V, kern, names[kern], us)
+                    rows.append({"bm": name, "M": M, "K": n if spmm else k, "N": k if spmm else n,
+                                 "sparsity": round(s, 4), "V": V, "kernel": kern, "nnz_vec": pat.nnz_vec,
+                                 "us": round(us, 3), "dense_us": round(dense, 3), "speedup": round(dense / us, 4),
+                                 "tflops": round(flops / us * 1e-6, 3), "gbs": round(nbytes / us * 1e-3, 1)})
+                print("%s M=%d n=%d k=%d s=%.2f V=%d  wmma %.2f us  cuda %.2f us  dense %.2f us" % (
+                    name, M, n, k, s, V, rows[-2]["us"], rows[-1]["us"], dense), flush=True)
+    if not rows:
+        raise SystemExit("nothing to run")
+    report(args.out, rows, "SpMM: geometric-mean speed-up over dense fp16 GEMM (hipBLASLt)" if spmm else
+           "SDDMM: geometric-mean speed-up over the dense fp16 product A B^T (hipBLASLt)")
     return 0
 
 
