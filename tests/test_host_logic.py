@@ -1,6 +1,7 @@
 """Host-side choices of the Python layer that need no GPU: they only read the mask and ask the library's
 host-only capacity query."""
 import numpy as np
+import pytest
 
 from vectorsparse_amd import colvec_csr as cv
 from vectorsparse_amd import ops
@@ -107,3 +108,34 @@ def test_sweep_benchmark_selection(tmp_path):
     assert sweep.sparsity_bucket(names[1], 0.5) == 0.95                 # the directory decides, not the file
     assert sweep.sparsity_bucket(names[2], 0.5) == 0.9
     assert sweep.sparsity_bucket("synthetic/m64", 0.8765) == 0.88
+
+
+def test_plot_reads_the_sweep_result_file(tmp_path):
+    """Geometric means per (path, V, k, sparsity bucket) and a figure from the rows the sweep writes."""
+    import csv
+    from vectorsparse_amd import plot
+
+    rows = []
+    for V in (2, 8):
+        for k in (64, 256):
+            for s, ups in ((0.7, (1.0, 4.0)), (0.9, (2.0, 8.0))):
+                for kernel, scale in (("wmma", 1.0), ("cuda", 0.5)):
+                    for up in ups:
+                        rows.append({"op": "spmm", "bm": "x", "k": k, "M": 64, "K": 128, "N": k, "sparsity": s, "V": V,
+                                     "kernel": kernel, "nnz_vec": 1, "us": 1.0, "dense_us": up, "speedup": up * scale,
+                                     "tflops": 1.0, "gbs": 1.0})
+    result = tmp_path / "result.csv"
+    with open(result, "w", newline="") as f:
+        w = csv.DictWriter(f, fieldnames=list(rows[0].keys()))
+        w.writeheader()
+        w.writerows(rows)
+    figure, geo = tmp_path / "speedup.png", tmp_path / "geo.csv"
+    assert plot.main(["--csv", str(result), "--out", str(figure), "--geo", str(geo)]) == 0
+    assert figure.stat().st_size > 1000
+    with open(geo) as f:
+        table = list(csv.reader(f))
+    assert table[0] == ["path", "V", "k", "0.7", "0.9"]
+    means = {(r[0], int(r[1]), int(r[2])): (float(r[3]), float(r[4])) for r in table[1:]}
+    assert len(means) == 8
+    assert means[("mma", 8, 256)] == pytest.approx((2.0, 4.0))      # sqrt(1 * 4), sqrt(2 * 8)
+    assert means[("fpu", 2, 64)] == pytest.approx((1.0, 2.0))

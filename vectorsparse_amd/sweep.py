@@ -228,7 +228,7 @@ def main(argv=None):
                 for kern in ("wmma", "cuda"):
                     us = time_launches(torch, run[kern], args.iters)
                     per_point(name, k, V, kern, names[kern], us)
-                    rows.append({"bm": name, "M": M, "K": n if spmm else k, "N": k if spmm else n,
+                    rows.append({"op": args.op, "bm": name, "k": k, "M": M, "K": n if spmm else k, "N": k if spmm else n,
                                  "sparsity": round(s, 4), "V": V, "kernel": kern, "nnz_vec": pat.nnz_vec,
                                  "us": round(us, 3), "dense_us": round(dense, 3), "speedup": round(dense / us, 4),
                                  "tflops": round(flops / us * 1e-6, 3), "gbs": round(nbytes / us * 1e-3, 1)})
