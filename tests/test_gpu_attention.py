@@ -511,3 +511,64 @@ def test_config5_full_size(gpu):
     _check_layer(out.cpu().numpy(), ref, "config 5, union kernel with plan")
     _check_layer(per_row.cpu().numpy(), ref, "config 5, per-row kernel")
     _check_layer(chain.cpu().numpy(), ref, "config 5, three operators")
+
+
+def _random_mask(rng, seq, V, kind):
+    m_vec = seq // V
+    if kind == "band":
+        return cv.band_strided_pattern(seq, V, band_half_width=int(rng.integers(8, 200)),
+                                       stride=int(rng.choice([16, 64, 128, seq])))
+    if kind == "blocks":
+        block = int(rng.choice([32, 64, 256]))
+        shared = np.sort(rng.choice(seq, int(rng.integers(0, 64)), replace=False))
+        rows = [np.union1d(np.arange((r * V) // block * block, min(seq, ((r * V) // block + 1) * block)), shared)
+                for r in range(m_vec)]
+    else:  # ragged: anything from empty rows to nearly full ones
+        rows = [np.sort(rng.choice(seq, int(rng.integers(0, seq if r % 7 == 0 else 40)), replace=False))
+                for r in range(m_vec)]
+    offsets = np.concatenate([[0], np.cumsum([len(r) for r in rows])]).astype(np.int32)
+    return cv.ColVecCSR(m_vec, seq, V, offsets, np.concatenate(rows).astype(np.int32)).validate()
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_attention_random_cases(gpu, seed):
+    """Seeded mixes of vector length, sequence length, head widths, mask family, workgroup size and plan
+    rounds through every attention path, against dense masked attention."""
+    rng = np.random.default_rng(1000 + seed)
+    V = int(rng.choice([1, 2, 4, 8]))
+    seq = int(rng.choice([128, 200, 512, 1000])) // V * V
+    d_qk = int(rng.choice([8, 32, 64, 72, 128]))
+    d_v = int(rng.choice([8, 40, 64, 128]))
+    heads = int(rng.integers(1, 4))
+    mask = _random_mask(rng, seq, V, ["band", "blocks", "ragged"][seed % 3])
+    q = rng.standard_normal((heads, seq, d_qk)).astype(np.float16)
+    k = rng.standard_normal((heads, seq, d_qk)).astype(np.float16)
+    v = rng.standard_normal((heads, seq, d_v)).astype(np.float16)
+    scale = float(rng.choice([0.05, 0.125, -0.1]))
+    ref = _dense_attention(mask, q, k, v, scale)
+    qd, kd, vd = (torch.from_numpy(x).cuda() for x in (q, k, v))
+    prob = ops.DeviceProblem(mask, sort=bool(seed % 2))
+    args = (mask.m_vec, V, seq, prob.row_indices, prob.row_offsets, prob.column_indices, qd, kd, vd)
+    what = "seed %d V%d seq %d d %d/%d" % (seed, V, seq, d_qk, d_v)
+    out = ops.sparse_attention(*args, scale=scale)
+    torch.cuda.synchronize()
+    _check_layer(out.cpu().numpy(), ref, what + " per row")
+    for rows in (16 // V, 128 // V):
+        if rows < 2:
+            continue
+        out = ops.sparse_attention(*args, scale=scale, rows_per_workgroup=rows)
+        torch.cuda.synchronize()
+        _check_layer(out.cpu().numpy(), ref, what + " rows %d rebuilt" % rows)
+        for rounds in (1, 3):
+            if _capacity(V, seq, d_qk, d_v, rows, rounds) <= 0:
+                continue
+            plan = ops.sparse_attention_plan(mask.m_vec, V, seq, d_qk, d_v, rows, prob.row_offsets,
+                                             prob.column_indices, plan_rounds=rounds)
+            out = ops.sparse_attention(*args, scale=scale, rows_per_workgroup=rows, plan=plan)
+            torch.cuda.synchronize()
+            _check_layer(out.cpu().numpy(), ref, what + " rows %d plan of %d rounds" % (rows, rounds))
+    layer = ops.SparseAttention(mask)
+    for fused in (None, True, False):
+        out = layer.forward(qd, kd, vd, scale=scale, fused=fused)
+        torch.cuda.synchronize()
+        _check_layer(out.cpu().numpy(), ref, what + " layer fused=%s" % fused)
