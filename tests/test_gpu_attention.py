@@ -483,7 +483,7 @@ def test_union_kernel_on_awkward_shapes(gpu):
 
 
 def test_config5_full_size(gpu):
-    """BASELINE config 5 at its real size (16 heads x 4096 x 64, V = 8, band 257 + every 128th column) through
+    """The benchmark set's attention layer at its real size (16 heads x 4096 x 64, V = 8, band 257 + every 128th column) through
     the path the benchmark takes (plan + union kernel) and through the per-row kernel, against a float64
     dense masked attention computed head by head."""
     V, heads, seq, d = 8, 16, 4096, 64
