@@ -156,10 +156,11 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--pmc", nargs="?", const="spmm", default=None, choices=["spmm", "sddmm", "attention"],
+    ap.add_argument("--pmc", nargs="?", const="spmm", default=None, choices=["spmm", "sddmm", "attention", "attention_window"],
                     help="counter-collection mode for `rocprofv3 --pmc`: a 64 MiB device copy of known size "
                          "(calibration), then a few eager launches of one kernel (the headline SpMM, the "
-                         "config-4 SDDMM, or the config-5 attention layer with its plan), nothing else")
+                         "config-4 SDDMM, the config-5 attention layer with its plan, or the same layer with a "
+                         "plain 513-wide window mask, whose unions of up to 634 columns are streamed through LDS), nothing else")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the SpMM/SDDMM path has no multi-GPU leg (rows shard with no "
@@ -212,7 +213,10 @@ def main():
             info["algorithmic_bytes"] = sddmm_algorithmic_bytes(mask, 64)
         else:
             heads, seq, dim = 16, 4096, 64
-            amask = cv.band_strided_pattern(seq, 8, band_half_width=128, stride=128)
+            if args.pmc == "attention_window":
+                amask = cv.band_strided_pattern(seq, 8, band_half_width=256, stride=seq)
+            else:
+                amask = cv.band_strided_pattern(seq, 8, band_half_width=128, stride=128)
             layer = ops.SparseAttention(amask)
             gen = torch.Generator(device="cuda").manual_seed(5)
             q, kk_, vv = (torch.randn((heads, seq, dim), device="cuda", generator=gen).half() for _ in range(3))
@@ -221,6 +225,7 @@ def main():
                 layer.forward(q, kk_, vv, out=ctx)
             info["algorithmic_bytes"] = 4 * heads * seq * dim * 2      # q, k, v read once, out written once
             info["rows_per_workgroup"] = layer.union_rows(dim, dim)
+            info["nonzero_vectors"] = int(amask.nnz_vec)
         torch.cuda.synchronize()
         print(json.dumps(info))
         return

@@ -233,45 +233,45 @@ int vs_wmma_spmm_softmax_f16_batched(int batch, int m_vec, int vec_length, int k
  * then only validated, rows are taken in their natural order.  Workgroups whose union exceeds
  * vs_sparse_attention_union_capacity() columns fall back to per-row gathers inside the same launch.
  * plan: null, or (rows_per_workgroup >= 2 only) a buffer filled by vs_sparse_attention_plan for this mask,
- * these head widths, this rows_per_workgroup and this plan_rounds: the kernel then reads every workgroup's
- * union and row masks from it instead of rebuilding them at every launch (same results).  A plan made for
- * another shape is detected and ignored (every workgroup then takes the per-row path: correct, slower).
- * plan_rounds (1..4, ignored without a plan): 1 = a workgroup's whole union must fit in LDS (the fastest
- * kernel); 2..4 = unions of up to plan_rounds times that many columns are taken in rounds, with the running
- * maximum and sums of flash attention between them (about 15 % slower on unions that would have fit one
- * round, several times faster than the per-row path on those that do not).
+ * these head widths and this rows_per_workgroup: the kernel then reads every workgroup's union and row
+ * masks from it instead of rebuilding them at every launch (same results up to the order of summation).
+ * With a plan, workgroups of eight waves (rows_per_workgroup >= 128 / vec_length) stream their union
+ * through LDS 128 columns at a time with the next columns' K / V rows already on their way, keeping the
+ * running maximum and sums of flash attention: the fastest path, and one that takes unions of up to 2048
+ * columns.  A plan made for another shape is detected and ignored (every workgroup then takes the per-row
+ * path: correct, slower).
  */
 int vs_sparse_attention_f16(int batch, int m_vec, int vec_length, int n, int d_qk, int d_v,
                             const int *row_indices, const int *row_offsets, const int *col_indices,
                             const void *q, long long stride_q, const void *k, long long stride_k,
                             const void *v, long long stride_v, void *out, long long stride_out,
-                            float scale, int rows_per_workgroup, const void *plan, int plan_rounds,
-                            void *stream);
+                            float scale, int rows_per_workgroup, const void *plan, void *stream);
 
 /*
  * Analysis step for rows_per_workgroup >= 2 of vs_sparse_attention_f16: writes into `plan` (device memory,
  * 16-byte aligned, at least vs_sparse_attention_plan_bytes() bytes, owned by the caller) the distinct
- * columns and the row masks of every workgroup, laid out for launches with the same plan_rounds (1..4).
- * The mask of an attention layer is fixed, so one plan serves every head, layer and step; asynchronous
- * on `stream`, nothing is kept by the library.  vs_sparse_attention_plan_bytes returns 0 for shapes the
- * union kernel does not support.  No counterpart in the reference.
+ * columns and the row masks of every workgroup.  The mask of an attention layer is fixed, so one plan
+ * serves every head, layer and step; asynchronous on `stream`, nothing is kept by the library.
+ * vs_sparse_attention_plan_bytes returns 0 for shapes the union kernel does not support.
+ * No counterpart in the reference.
  */
 long long vs_sparse_attention_plan_bytes(int m_vec, int vec_length, int n, int d_qk, int d_v,
-                                         int rows_per_workgroup, int plan_rounds);
+                                         int rows_per_workgroup);
 int vs_sparse_attention_plan(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows_per_workgroup,
-                             int plan_rounds, const int *row_offsets, const int *col_indices, void *plan,
+                             const int *row_offsets, const int *col_indices, void *plan,
                              long long plan_bytes, void *stream);
 
 /*
  * Planning helper for rows_per_workgroup >= 2 of vs_sparse_attention_f16: the number of distinct columns
- * a workgroup can hold in LDS for this shape (0: shape not supported by the union kernel), and in
- * *rows_used (may be null) the vector rows per workgroup the request is rounded to.  plan_rounds: 0 for
- * launches without a plan (up to 480 columns); 1..4 for launches with a plan of that many rounds - they
- * keep only the K / V rows and the row masks in LDS, so they hold more columns per round (up to 512, times
- * plan_rounds) and accept a larger n.  Host only, no launch.  No counterpart in the reference.
+ * a workgroup can take for this shape (0: shape not supported by the union kernel), and in
+ * *rows_used (may be null) the vector rows per workgroup the request is rounded to.  with_plan: nonzero
+ * for launches that pass a plan: up to 2048 columns for workgroups of eight waves (streamed), up to 512 for
+ * smaller ones (only the K / V rows and the row masks in LDS), against up to 480 without a plan (the column
+ * bitmap and the column list share the LDS); a plan also accepts a larger n.  Host only, no launch.
+ * No counterpart in the reference.
  */
 int vs_sparse_attention_union_capacity(int vec_length, int n, int d_qk, int d_v, int rows_per_workgroup,
-                                       int plan_rounds, int *rows_used);
+                                       int with_plan, int *rows_used);
 
 /*
  * Host helpers (HOST pointers).  Replace IdentityRowSwizzle / SortedRowSwizzle —

@@ -89,18 +89,19 @@ def test_attention_planning_helpers_are_consistent():
         for request in (2, per_wave, 3 * per_wave + 1, 8 * per_wave, 128):
             built = L.vs_sparse_attention_union_capacity(V, 4096, 64, 64, request, 0, None)
             cap = L.vs_sparse_attention_union_capacity(V, 4096, 64, 64, request, 1, ctypes.addressof(used))
-            assert cap > 0 and cap % 32 == 0 and 0 < built <= cap <= 512    # a plan frees LDS for more columns
             assert used.value % per_wave == 0 and used.value <= 8 * per_wave      # whole waves, at most 8
             assert used.value >= min(request, 8 * per_wave)
             blocks = -(-512 // used.value)
-            mask_words = (used.value * 16 + 3) // 4 * 4
-            for rounds in (1, 2, 3, 4):                                     # larger unions, taken in rounds
-                assert L.vs_sparse_attention_union_capacity(V, 4096, 64, 64, request, rounds, None) == rounds * cap
-                size = L.vs_sparse_attention_plan_bytes(512, V, 4096, 64, 64, request, rounds)
-                assert size == 4 * (16 + blocks * (4 + rounds * (mask_words + cap)))
-            assert L.vs_sparse_attention_plan_bytes(512, V, 4096, 64, 64, request, 0) == 0
-            assert L.vs_sparse_attention_plan_bytes(512, V, 4096, 64, 64, request, 5) == 0
-            assert L.vs_sparse_attention_union_capacity(V, 4096, 64, 64, request, 5, None) == 0
+            size = L.vs_sparse_attention_plan_bytes(512, V, 4096, 64, 64, request)
+            if used.value == 8 * per_wave:
+                # eight waves stream the union: 16 rounds of 128 ranks, 4 mask words per row and round
+                assert 0 < built <= 512 and cap == 2048
+                assert size == 4 * (16 + blocks * (4 + 16 * (used.value * 4 + 128)))
+            else:
+                # smaller workgroups hold it at once; a plan frees LDS for more columns
+                assert cap % 32 == 0 and 0 < built <= cap <= 512
+                mask_words = (used.value * 16 + 3) // 4 * 4
+                assert size == 4 * (16 + blocks * (4 + mask_words + cap))
     wide = L.vs_sparse_attention_union_capacity(8, 4096, 128, 128, 16, 0, None)
     narrow = L.vs_sparse_attention_union_capacity(8, 4096, 32, 32, 16, 0, None)
     assert 0 < narrow <= 512 and 0 < wide <= 512               # wide heads: one workgroup per CU with all of its LDS
@@ -112,12 +113,11 @@ def test_attention_planning_helpers_are_consistent():
     assert L.vs_sparse_attention_union_capacity(8, 400000, 64, 64, 16, 0, None) == 0
     assert L.vs_sparse_attention_union_capacity(8, 400000, 64, 64, 16, 1, None) > 0
     assert L.vs_sparse_attention_union_capacity(3, 4096, 64, 64, 16, 0, None) == 0
-    assert L.vs_sparse_attention_plan_bytes(512, 8, 4096, 64, 64, 1, 1) == 0
+    assert L.vs_sparse_attention_plan_bytes(512, 8, 4096, 64, 64, 1) == 0
     # a plan buffer that is too small, null or misaligned is rejected before any launch
-    assert L.vs_sparse_attention_plan(512, 8, 4096, 64, 64, 16, 1, 64, 64, 256, 16, None) == 1
-    assert L.vs_sparse_attention_plan(512, 8, 4096, 64, 64, 16, 1, 64, 64, None, 1 << 20, None) == 1
-    assert L.vs_sparse_attention_plan(512, 8, 4096, 64, 64, 16, 1, 64, 64, 264, 1 << 20, None) == 1
-    assert L.vs_sparse_attention_plan(512, 8, 4096, 64, 64, 16, 0, 64, 64, 256, 1 << 20, None) == 1
+    assert L.vs_sparse_attention_plan(512, 8, 4096, 64, 64, 16, 64, 64, 256, 16, None) == 1
+    assert L.vs_sparse_attention_plan(512, 8, 4096, 64, 64, 16, 64, 64, None, 1 << 20, None) == 1
+    assert L.vs_sparse_attention_plan(512, 8, 4096, 64, 64, 16, 64, 64, 264, 1 << 20, None) == 1
 
 
 def test_options():

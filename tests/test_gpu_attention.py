@@ -279,10 +279,10 @@ def _with_empty_rows(mask, first, last):
     return cv.ColVecCSR(mask.m_vec, mask.n, mask.vec_length, offsets, mask.column_indices[keep].copy())
 
 
-def _capacity(V, n, d_qk, d_v, rows, plan_rounds):
-    """Distinct columns a workgroup takes: without a plan (0) or with a plan of that many rounds."""
+def _capacity(V, n, d_qk, d_v, rows, with_plan):
+    """Distinct columns a workgroup takes without (0) or with (1) a plan."""
     from vectorsparse_amd import _lib
-    return _lib.lib().vs_sparse_attention_union_capacity(V, n, d_qk, d_v, rows, plan_rounds, None)
+    return _lib.lib().vs_sparse_attention_union_capacity(V, n, d_qk, d_v, rows, with_plan, None)
 
 
 def _unions(mask, rows):
@@ -319,60 +319,51 @@ def test_plan_raises_the_union_capacity(gpu, V, seq, half_width, stride, rows):
     assert not torch.equal(planned, rebuilt)              # different summation orders: the paths did differ
 
 
-@pytest.mark.parametrize("V,seq,half_width,stride,dims,want_rounds", [
-    (8, 4096, 300, 64, (64, 64), 2),      # two rounds of 512 ranks
-    (8, 4096, 900, 128, (64, 64), 4),     # four rounds
-    (2, 2048, 400, 0, (32, 128), 2),      # plain band, wide V rows: one workgroup per CU, two rounds
-    (1, 2048, 400, 256, (64, 64), 2),     # 128 vector rows per workgroup, masks restaged every round
+@pytest.mark.parametrize("V,seq,half_width,stride,dims", [
+    (8, 4096, 300, 64, (64, 64)),      # unions of about 700 columns: six sub-rounds of 128
+    (8, 4096, 900, 128, (64, 64)),     # about 1900 columns: fifteen sub-rounds
+    (2, 2048, 400, 0, (32, 128)),      # plain band, wide V rows (one workgroup per CU)
+    (1, 2048, 400, 256, (64, 64)),     # 128 vector rows per workgroup
 ])
-def test_planned_launch_takes_large_unions_in_rounds(gpu, V, seq, half_width, stride, dims, want_rounds):
-    """Unions of more columns than fit in LDS at once: with a plan the workgroup walks them in rounds with a
-    running maximum and sum; rows whose columns all fall into a later round, rows empty in some round, and a
-    negative scale go through the same rescaling."""
+def test_planned_launch_streams_large_unions(gpu, V, seq, half_width, stride, dims):
+    """Unions of more columns than fit in LDS at once: with a plan, eight waves stream them through LDS with
+    a running maximum and sums; rows whose columns all fall into a late sub-round, rows empty in some
+    sub-round, a negative and a zero scale go through the same rescaling."""
     d_qk, d_v = dims
     mask = cv.band_strided_pattern(seq, V, band_half_width=half_width, stride=stride or seq)
     mask = _with_empty_rows(mask, 3, 5)
     rows = 128 // V
     unions = _unions(mask, rows)
-    rounds = next(r for r in (1, 2, 3, 4) if max(unions) <= _capacity(V, seq, d_qk, d_v, rows, r))
-    assert rounds == want_rounds, (rounds, max(unions), _capacity(V, seq, d_qk, d_v, rows, 1))
+    assert 512 < max(unions) <= _capacity(V, seq, d_qk, d_v, rows, 1) == 2048
     rng = np.random.default_rng(90 + V)
     q = rng.standard_normal((2, seq, d_qk)).astype(np.float16)
     k = rng.standard_normal((2, seq, d_qk)).astype(np.float16)
     v = rng.standard_normal((2, seq, d_v)).astype(np.float16)
-    # make the maximum of many rows sit in a late round: large keys at the top end of the sequence
+    # make the maximum of many rows sit in a late sub-round: large keys at the top end of the sequence
     k[:, seq - seq // 8:, :] *= 3.0
     qd, kd, vd = (torch.from_numpy(x).cuda() for x in (q, k, v))
     prob = ops.DeviceProblem(mask)
     args = (mask.m_vec, V, seq, prob.row_indices, prob.row_offsets, prob.column_indices, qd, kd, vd)
-    plan = ops.sparse_attention_plan(mask.m_vec, V, seq, d_qk, d_v, rows, prob.row_offsets, prob.column_indices,
-                                     plan_rounds=rounds)
+    plan = ops.sparse_attention_plan(mask.m_vec, V, seq, d_qk, d_v, rows, prob.row_offsets, prob.column_indices)
     for scale in (0.125, -0.125, 0.0):
         ref = _dense_attention(mask, q, k, v, scale)
         planned = ops.sparse_attention(*args, scale=scale, rows_per_workgroup=rows, plan=plan)
         again = ops.sparse_attention(*args, scale=scale, rows_per_workgroup=rows, plan=plan)
         torch.cuda.synchronize()
-        _check_layer(planned.cpu().numpy(), ref, "V%d scale %g in rounds" % (V, scale))
+        _check_layer(planned.cpu().numpy(), ref, "V%d scale %g streamed" % (V, scale))
         assert torch.equal(planned, again)
-    # a plan of more rounds than needed, and the one-round kernel given a plan of several (ignored: per-row path)
-    spare = ops.sparse_attention_plan(mask.m_vec, V, seq, d_qk, d_v, rows, prob.row_offsets, prob.column_indices,
-                                      plan_rounds=4)
-    ref = _dense_attention(mask, q, k, v, 0.125)
-    for given, told in ((spare, 4), (spare, 1), (plan, 1)):
-        out = ops.sparse_attention(*args, scale=0.125, rows_per_workgroup=rows, plan=given, plan_rounds=told)
-        torch.cuda.synchronize()
-        _check_layer(out.cpu().numpy(), ref, "V%d plan of %d rounds read as %d" % (V, given.plan_rounds, told))
     layer = ops.SparseAttention(mask)
-    assert layer.union_shape(d_qk, d_v)[0] > 1 and layer.union_shape(d_qk, d_v)[1] > 1   # the host-side choice counts on the rounds
+    assert layer.union_rows(d_qk, d_v) == rows            # the host-side choice counts on the streamed kernel
     out = layer.forward(qd, kd, vd, scale=0.125)
     torch.cuda.synchronize()
-    _check_layer(out.cpu().numpy(), _dense_attention(mask, q, k, v, 0.125), "V%d layer in rounds" % V)
+    _check_layer(out.cpu().numpy(), _dense_attention(mask, q, k, v, 0.125), "V%d layer streamed" % V)
 
 
 @pytest.mark.parametrize("V", [1, 8])
 def test_planned_launch_equals_unplanned(gpu, V):
-    """The plan holds exactly what the kernel would rebuild: same bits out.  A plan made for another launch
-    shape is ignored safely (per-row path), so the result still meets the layer bound."""
+    """Workgroups of fewer than eight waves: the plan holds exactly what the kernel would rebuild, same bits
+    out.  Eight waves stream the union when they have a plan (another order of summation): both meet the
+    layer bound.  A plan made for another launch shape is ignored safely (per-row path)."""
     heads, seq, d = 2, 1024, 64
     rng = np.random.default_rng(40 + V)
     q, k, v = (rng.standard_normal((heads, seq, d)).astype(np.float16) for _ in range(3))
@@ -395,7 +386,8 @@ def test_planned_launch_equals_unplanned(gpu, V):
             _check_layer(planned.cpu().numpy(), ref, "%s V%d rows%d planned" % (name, V, rows))
             # a planned launch holds more columns per workgroup: same bits unless some union fits only then
             built, held = _capacity(V, seq, d, d, rows, 0), _capacity(V, seq, d, d, rows, 1)
-            if not any(built < u <= held for u in _unions(mask, rows)):
+            streamed = rows == 128 // V
+            if not streamed and not any(built < u <= held for u in _unions(mask, rows)):
                 assert torch.equal(plain, planned), "%s V%d rows%d" % (name, V, rows)
             else:
                 _check_layer(plain.cpu().numpy(), ref, "%s V%d rows%d rebuilt" % (name, V, rows))
@@ -532,8 +524,8 @@ def _random_mask(rng, seq, V, kind):
 
 @pytest.mark.parametrize("seed", range(12))
 def test_attention_random_cases(gpu, seed):
-    """Seeded mixes of vector length, sequence length, head widths, mask family, workgroup size and plan
-    rounds through every attention path, against dense masked attention."""
+    """Seeded mixes of vector length, sequence length, head widths, mask family and workgroup size through
+    every attention path, against dense masked attention."""
     rng = np.random.default_rng(1000 + seed)
     V = int(rng.choice([1, 2, 4, 8]))
     seq = int(rng.choice([128, 200, 512, 1000])) // V * V
@@ -559,14 +551,12 @@ def test_attention_random_cases(gpu, seed):
         out = ops.sparse_attention(*args, scale=scale, rows_per_workgroup=rows)
         torch.cuda.synchronize()
         _check_layer(out.cpu().numpy(), ref, what + " rows %d rebuilt" % rows)
-        for rounds in (1, 3):
-            if _capacity(V, seq, d_qk, d_v, rows, rounds) <= 0:
-                continue
+        if _capacity(V, seq, d_qk, d_v, rows, 1) > 0:
             plan = ops.sparse_attention_plan(mask.m_vec, V, seq, d_qk, d_v, rows, prob.row_offsets,
-                                             prob.column_indices, plan_rounds=rounds)
+                                             prob.column_indices)
             out = ops.sparse_attention(*args, scale=scale, rows_per_workgroup=rows, plan=plan)
             torch.cuda.synchronize()
-            _check_layer(out.cpu().numpy(), ref, what + " rows %d plan of %d rounds" % (rows, rounds))
+            _check_layer(out.cpu().numpy(), ref, what + " rows %d planned" % rows)
     layer = ops.SparseAttention(mask)
     for fused in (None, True, False):
         out = layer.forward(qd, kd, vd, scale=scale, fused=fused)

@@ -13,28 +13,26 @@ def _largest_union(mask, rows):
 
 
 def test_attention_launch_shape_follows_the_mask():
-    shape = ops.SparseAttention._union_shape
-    # band + strided columns: eight waves per workgroup, the whole union in LDS at once
+    rows_for = ops.SparseAttention._union_rows
+    # band + strided columns: eight waves per workgroup
     band = cv.band_strided_pattern(4096, 8, band_half_width=128, stride=128)
-    assert shape(band, 64, 64) == (16, 1)
-    assert _largest_union(band, 16) <= 512
-    # a 513-wide window: the same workgroups, unions of more than 512 columns in two rounds
+    assert rows_for(band, 64, 64) == 16
+    # a 513-wide window: unions of more than 512 columns, which eight waves stream through LDS
     window = cv.band_strided_pattern(4096, 8, band_half_width=256, stride=4096)
-    assert 512 < _largest_union(window, 16) <= 1024
-    assert shape(window, 64, 64) == (16, 2)
-    # wide heads get the whole LDS of a CU: still one round for the band
-    assert shape(band, 128, 128) == (16, 1)
+    assert 512 < _largest_union(window, 16) <= 2048
+    assert rows_for(window, 64, 64) == 16
+    assert rows_for(band, 128, 128) == 16
     # every vector length fills its waves with 16 scalar rows
     for V in (1, 2, 4):
-        assert shape(cv.band_strided_pattern(2048, V, band_half_width=128, stride=128), 64, 64) == (128 // V, 1)
+        assert rows_for(cv.band_strided_pattern(2048, V, band_half_width=128, stride=128), 64, 64) == 128 // V
     # scattered columns: a dense tile over the union would be mostly masked out -> one row per workgroup
     scattered = cv.uniform_pattern(512, 4096, 0.9, seed=3, vec_length=8)
-    assert shape(scattered, 64, 64) == (1, 1)
+    assert rows_for(scattered, 64, 64) == 1
     # head widths the union kernel does not take
-    assert shape(band, 64, 36) == (1, 1)
+    assert rows_for(band, 64, 36) == 1
     # empty masks
     empty = cv.ColVecCSR(4, 64, 8, np.zeros(5, np.int32), np.zeros(0, np.int32))
-    assert shape(empty, 64, 64) == (1, 1)
+    assert rows_for(empty, 64, 64) == 1
 
 
 def _moving_blocks(m_vec, n, V, rows_per_block, width=600, step=700):
@@ -46,16 +44,19 @@ def _moving_blocks(m_vec, n, V, rows_per_block, width=600, step=700):
 
 
 def test_small_workgroups_only_where_they_beat_the_per_row_kernel():
-    """Unions that fit only small blocks of rows: two waves are taken for V <= 4, never for V = 8."""
-    shape = ops.SparseAttention._union_shape
-    # V = 4: 16 rows (four waves) span four windows, more than four rounds hold; 8 rows (two waves) span two
-    mask = _moving_blocks(256, 8192, 4, rows_per_block=4)
-    assert _largest_union(mask, 16) > 2048 >= _largest_union(mask, 8)
-    assert shape(mask, 64, 64)[0] == 8
-    # V = 8: 8 rows (four waves) do not fit, 4 rows (two waves) would - but lose to the per-row kernel
-    mask = _moving_blocks(256, 8192, 8, rows_per_block=2)
-    assert _largest_union(mask, 8) > 2048 >= _largest_union(mask, 4)
-    assert shape(mask, 64, 64) == (1, 1)
+    """Masks whose dense tile is full enough only over small blocks of rows: two waves are taken for V <= 4,
+    never for V = 8."""
+    rows_for = ops.SparseAttention._union_rows
+    # V = 4, the window jumps every 4 rows: tiles of 32 and 16 rows are 1/8 and 1/4 full, tiles of 8 rows (two
+    # waves) half full, and their 480 columns fit LDS at once
+    mask = _moving_blocks(256, 8192, 4, rows_per_block=4, width=240, step=300)
+    assert _largest_union(mask, 8) == 480
+    assert rows_for(mask, 64, 64) == 8
+    # V = 8, the window jumps every 2 rows: only tiles of 4 rows (two waves) would be full enough - but two
+    # waves lose to the per-row kernel at V = 8
+    mask = _moving_blocks(256, 8192, 8, rows_per_block=2, width=240, step=300)
+    assert _largest_union(mask, 4) == 480
+    assert rows_for(mask, 64, 64) == 1
 
 
 def test_device_problem_reads_the_row_statistics():

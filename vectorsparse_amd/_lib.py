@@ -28,11 +28,11 @@ SIGNATURES = {
     "vs_wmma_spmm_softmax_f16_batched": ([_int] * 7 + [_vp] * 3 + [_vp, _ll, _vp, _ll, _vp, _ll, ctypes.c_float, _vp],
                                          _int),
     "vs_sparse_attention_f16": ([_int] * 6 + [_vp] * 3 + [_vp, _ll, _vp, _ll, _vp, _ll, _vp, _ll, ctypes.c_float, _int,
-                                 _vp, _int, _vp],
+                                 _vp, _vp],
                                 _int),
     "vs_sparse_attention_union_capacity": ([_int] * 6 + [_vp], _int),
-    "vs_sparse_attention_plan_bytes": ([_int] * 7, _ll),
-    "vs_sparse_attention_plan": ([_int] * 7 + [_vp] * 3 + [_ll, _vp], _int),
+    "vs_sparse_attention_plan_bytes": ([_int] * 6, _ll),
+    "vs_sparse_attention_plan": ([_int] * 6 + [_vp] * 3 + [_ll, _vp], _int),
     "vs_sparse_softmax_f16": ([_int] * 3 + [_vp] * 2 + [_vp, _ll, _vp, _ll, ctypes.c_float, _vp], _int),
     "vs_identity_row_swizzle": ([_int, _vp], None),
     "vs_sorted_row_swizzle": ([_int, _vp, _vp], None),

@@ -254,12 +254,53 @@ __device__ __forceinline__ void scores_step(float4_t (&sacc)[2], const half8_t (
     }
 }
 
+// The per-row path for the vector rows [row_first, row_last) of a workgroup: one vector row per wave at a time
+// with the K / V rows read from global memory by column; no barrier, long rows in chunks with a running
+// maximum and sum.
+template <int V, int KS, int CPL>
+__device__ __forceinline__ void per_row_block(int row_first, int row_last, int wave, int n_waves,
+                                              const int *__restrict__ row_offsets, const int *__restrict__ col_indices,
+                                              const half_t *__restrict__ q, const half_t *__restrict__ k,
+                                              const half_t *__restrict__ v, half_t *__restrict__ out, int d_qk, int d_v,
+                                              float s2, int c, int g, int col_off)
+{
+    const RowSource ksrc = {k, d_qk, col_indices};
+    const RowSource vsrc = {v, d_v, col_indices};
+    for (int row = row_first + wave; row < row_last; row += n_waves) {
+        const int beg = row_offsets[row];
+        const int end = row_offsets[row + 1];
+        half8_t qb[KS];
+        load_q<V, KS>(qb, q, row, d_qk, c, g);
+        float m_run = -__builtin_inff(), l_run = 0.f;
+        float4_t acc[CPL];
+#pragma unroll
+        for (int cc = 0; cc < CPL; ++cc) acc[cc] = float4_t{0.f, 0.f, 0.f, 0.f};
+        for (int c0 = beg; c0 < end; c0 += 32 * kMaxSteps) {
+            const int cend = (c0 + 32 * kMaxSteps) < end ? (c0 + 32 * kMaxSteps) : end;
+            half8_t p[kMaxSteps];
+            float m_new, sum;
+            softmax_chunk<KS>(p, m_new, sum, m_run, ksrc, c0, cend, d_qk, qb, s2, c, g);
+            const float f = __builtin_amdgcn_exp2f(m_run - m_new);  // 0 on the first chunk (m_run = -inf)
+            l_run = l_run * f + sum;
+            m_run = m_new;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float fe = from_lane(f, (4 * g + e) & 15);  // accumulator row 4g + e belongs to scalar row 4g + e
+#pragma unroll
+                for (int cc = 0; cc < CPL; ++cc) acc[cc][e] *= fe;
+            }
+            accumulate_chunk<CPL>(acc, p, vsrc, c0, cend, col_off, g);
+        }
+        store_row<V, CPL>(out, row, d_v, acc, l_run, end == beg, c, g);
+    }
+}
+
 // LDS arrays that describe the union of a block of rows.
 struct UnionLds {
     unsigned *bitmap;   // [n_words] columns present in the block
     unsigned *prefix;   // [n_words] exclusive prefix of the bitmap's word popcounts
     int *wave_tot;      // [16] scan scratch, [15] = number of distinct columns
-    unsigned *rowmask;  // [rounds][rows][kUnionSteps] ranks each row holds, u_max ranks per round
+    unsigned *rowmask;  // [rounds][rows][steps] ranks each row holds, u_max = 32 * steps ranks per round at most
     int *ucols;         // [rounds * u_max] columns of the union in ascending order
 };
 
@@ -267,7 +308,7 @@ struct UnionLds {
 // number U of distinct columns; rowmask ([rounds][mask_words]) and ucols are complete (and visible to every
 // thread) on return when U <= rounds * u_max, otherwise only U is meaningful.
 __device__ __forceinline__ int build_union(const UnionLds &l, int n_words, int mask_words, int u_max, int rounds,
-                                           int row_first, int row_last, const int *__restrict__ row_offsets,
+                                           int steps, int row_first, int row_last, const int *__restrict__ row_offsets,
                                            const int *__restrict__ col_indices)
 {
     const int tid = threadIdx.x;
@@ -345,7 +386,7 @@ __device__ __forceinline__ int build_union(const UnionLds &l, int n_words, int m
     // of one rank write the same value), which lists the union without a pass over the bitmap; ranks
     // [i * u_max, (i + 1) * u_max) belong to round i, whose masks follow those of round i - 1
     auto mask_bit = [&](int r, int rank) {
-        int word = r * kUnionSteps;
+        int word = r * steps;
         if (rounds > 1) {
             const int round = rank / u_max;
             rank -= round * u_max;
@@ -374,23 +415,25 @@ __device__ __forceinline__ int build_union(const UnionLds &l, int n_words, int m
 
 // A plan holds what build_union computes for every workgroup of a launch shape, so that launches on the
 // same mask (every head, layer and step) read it instead of rebuilding it.  Layout, in 32-bit words:
-// header [magic, m_vec, V, n, rows per workgroup, u_max, record stride, workgroups, rounds, 0...] (16 words),
-// then one record per workgroup: [U, 0, 0, 0], rowmask [rounds][mask_words], ucols [rounds * u_max].
-// A plan of one round serves launches that hold a workgroup's whole union in LDS; a plan of up to
-// kMaxPlanRounds rounds serves launches that take a larger union in rounds of u_max ranks (the K / V rows of
-// one round in LDS at a time, running maximum and sums across the rounds).
+// header [magic, m_vec, V, n, rows per workgroup, u_max, record stride, workgroups, rounds, steps, 0...]
+// (16 words), then one record per workgroup: [U, 0, 0, 0], rowmask [rounds][rows][steps] (each round padded
+// to 4 words), ucols [rounds * u_max].  Workgroups of eight waves stream the union through LDS
+// (sparse_attention_stream_kernel): kStreamRounds rounds of kStreamRanks ranks.  Smaller workgroups hold the
+// whole union in LDS at once: one round of up to 32 * kUnionSteps ranks.
 constexpr int kPlanMagic = 0x56535041;
 constexpr int kPlanHeader = 16;
-constexpr int kMaxPlanRounds = 4;
+constexpr int kStreamSteps = 4;
+constexpr int kStreamRanks = 32 * kStreamSteps;
+constexpr int kStreamRounds = 16;
 
 __global__ void __launch_bounds__(256)
-sparse_attention_plan_kernel(int m_vec, int vec_length, int n, int rows_per_block, int u_max, int rounds,
+sparse_attention_plan_kernel(int m_vec, int vec_length, int n, int rows_per_block, int u_max, int rounds, int steps,
                              const int *__restrict__ row_offsets, const int *__restrict__ col_indices,
                              int *__restrict__ plan)
 {
     const int n_words = (n + 31) >> 5;
     const int n_words_al = (n_words + 3) & ~3;
-    const int mask_words = (rows_per_block * kUnionSteps + 3) & ~3;
+    const int mask_words = (rows_per_block * steps + 3) & ~3;
     extern __shared__ __align__(16) unsigned char smem[];
     UnionLds l;
     l.bitmap = reinterpret_cast<unsigned *>(smem);
@@ -403,7 +446,7 @@ sparse_attention_plan_kernel(int m_vec, int vec_length, int n, int rows_per_bloc
     const int tid = threadIdx.x;
     if (blockIdx.x == 0 && tid < kPlanHeader) {
         const int header[kPlanHeader] = {kPlanMagic, m_vec, vec_length, n, rows_per_block, u_max, stride,
-                                         (int)gridDim.x, rounds, 0, 0, 0, 0, 0, 0, 0};
+                                         (int)gridDim.x, rounds, steps, 0, 0, 0, 0, 0, 0};
         int value = 0;
 #pragma unroll
         for (int i = 0; i < kPlanHeader; ++i) value = (i == tid) ? header[i] : value;
@@ -411,8 +454,8 @@ sparse_attention_plan_kernel(int m_vec, int vec_length, int n, int rows_per_bloc
     }
     const int row_first = blockIdx.x * rows_per_block;
     const int row_last = (row_first + rows_per_block) < m_vec ? (row_first + rows_per_block) : m_vec;
-    const int n_union = build_union(l, n_words, mask_words, u_max, rounds, row_first, row_last, row_offsets,
-                                    col_indices);
+    const int n_union = build_union(l, n_words, mask_words, u_max, rounds, steps, row_first, row_last,
+                                    row_offsets, col_indices);
     int *rec = plan + kPlanHeader + (size_t)blockIdx.x * stride;
     if (tid < 4) rec[tid] = tid == 0 ? n_union : 0;
     if (n_union > cap) return;  // this workgroup's rows take the per-row path at every launch
@@ -421,16 +464,15 @@ sparse_attention_plan_kernel(int m_vec, int vec_length, int n, int rows_per_bloc
 }
 
 // V: vector length; KS: d_qk <= 32*KS; CPL: d_v <= 16*CPL.
-// MODE 0: the workgroup builds its union.  MODE 1, 2 (PLANNED): the union and the row masks come from a plan
-// (sparse_attention_plan_kernel) of plan_rounds rounds instead of being rebuilt; 1: one round, the whole
-// union in LDS at once as in mode 0; 2 (ROUNDS): a union of up to plan_rounds * u_max columns, u_max at a
-// time.  A plan made for another mask shape or launch shape sends every workgroup to the per-row path.
-template <int V, int KS, int CPL, int MODE>
+// PLANNED: the union and the row masks come from a plan of one round (sparse_attention_plan_kernel) instead
+// of being rebuilt; a plan made for another mask shape or launch shape sends every workgroup to the per-row
+// path.
+template <int V, int KS, int CPL, bool PLANNED>
 // Heads up to 64 wide: four waves per SIMD (128 registers), two eight-wave workgroups per CU.  Wider heads
 // hold twice the Q / K / V slices per lane and 272-byte rows in LDS: two waves per SIMD (256 registers), one
 // workgroup per CU with all of its LDS.
 __global__ void __launch_bounds__(512, union_wide(KS, CPL) ? 2 : 4)
-sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max, int plan_rounds,
+sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max,
                               const int *__restrict__ row_offsets, const int *__restrict__ col_indices,
                               const int *__restrict__ plan,
                               const half_t *__restrict__ q, const half_t *__restrict__ k,
@@ -441,8 +483,6 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max, in
     k += blockIdx.y * stride_k;
     v += blockIdx.y * stride_v;
     out += blockIdx.y * stride_out;
-    constexpr bool PLANNED = MODE != 0;
-    constexpr bool ROUNDS = MODE == 2;
     constexpr int RPW = 16 / V;  // vector rows per wave: 16 scalar rows fill the MFMA tile
     constexpr int PITCH = union_pitch(KS, CPL);
     const int n_words = (n + 31) >> 5;
@@ -490,64 +530,31 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max, in
 
     // ---- 1, 2. the union's columns and every row's mask over ranks: built here or read from the plan
     int n_union;
-    const int *cols;            // columns of the union: LDS (built) or the plan's record (global)
-    const int *masks = nullptr;  // the plan's row masks, one set per round
-    int u_cap = u_max;          // columns the workgroup can take: in LDS at once, or in the plan's rounds
+    const int *cols;  // columns of the union: LDS (built) or the plan's record (global)
     if constexpr (PLANNED) {
-        u_cap = plan_rounds * u_max;
-        const int stride = 4 + plan_rounds * mask_words + u_cap;
+        const int stride = 4 + mask_words + u_max;
         const bool plan_ok = plan[0] == kPlanMagic && plan[1] == m_vec && plan[2] == V && plan[3] == n &&
                              plan[4] == rows_per_block && plan[5] == u_max && plan[6] == stride &&
-                             plan[7] == (int)gridDim.x && plan[8] == plan_rounds;
+                             plan[7] == (int)gridDim.x && plan[8] == 1 && plan[9] == kUnionSteps;
         const int *rec = plan + kPlanHeader + (size_t)(plan_ok ? bx : 0) * stride;
         n_union = plan_ok ? rec[0] : 0x7fffffff;
-        masks = rec + 4;
-        cols = rec + 4 + plan_rounds * mask_words;
-        if (n_union <= u_cap)
-            for (int w = tid; w < mask_words; w += n_threads) l.rowmask[w] = (unsigned)masks[w];
+        cols = rec + 4 + mask_words;
+        if (n_union <= u_max)
+            for (int w = tid; w < mask_words; w += n_threads) l.rowmask[w] = (unsigned)rec[4 + w];
         // visible to the other waves after the barrier that follows the K gather
     } else {
-        n_union = build_union(l, n_words, mask_words, u_max, 1, row_first, row_last, row_offsets, col_indices);
+        n_union = build_union(l, n_words, mask_words, u_max, 1, kUnionSteps, row_first, row_last, row_offsets,
+                              col_indices);
         cols = l.ucols;
     }
-    const bool use_lds = n_union <= u_cap && (d_v % 8 == 0);
+    const bool use_lds = n_union <= u_max && (d_v % 8 == 0);
     if (!use_lds) {
-        // Fallback: one vector row per wave at a time with the K / V rows read from global memory by
-        // column; no barrier, long rows in chunks with a running maximum and sum.
-        const RowSource ksrc = {k, d_qk, col_indices};
-        const RowSource vsrc = {v, d_v, col_indices};
-        for (int row = row_first + wave; row < row_last; row += n_waves) {
-            const int beg = row_offsets[row];
-            const int end = row_offsets[row + 1];
-            half8_t qb[KS];
-            load_q<V, KS>(qb, q, row, d_qk, c, g);
-            float m_run = -__builtin_inff(), l_run = 0.f;
-            float4_t acc[CPL];
-#pragma unroll
-            for (int cc = 0; cc < CPL; ++cc) acc[cc] = float4_t{0.f, 0.f, 0.f, 0.f};
-            for (int c0 = beg; c0 < end; c0 += 32 * kMaxSteps) {
-                const int cend = (c0 + 32 * kMaxSteps) < end ? (c0 + 32 * kMaxSteps) : end;
-                half8_t p[kMaxSteps];
-                float m_new, sum;
-                softmax_chunk<KS>(p, m_new, sum, m_run, ksrc, c0, cend, d_qk, qb, s2, c, g);
-                const float f = __builtin_amdgcn_exp2f(m_run - m_new);  // 0 on the first chunk (m_run = -inf)
-                l_run = l_run * f + sum;
-                m_run = m_new;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const float fe = from_lane(f, (4 * g + e) & 15);  // accumulator row 4g + e belongs to scalar row 4g + e
-#pragma unroll
-                    for (int cc = 0; cc < CPL; ++cc) acc[cc][e] *= fe;
-                }
-                accumulate_chunk<CPL>(acc, p, vsrc, c0, cend, col_off, g);
-            }
-            store_row<V, CPL>(out, row, d_v, acc, l_run, end == beg, c, g);
-        }
+        per_row_block<V, KS, CPL>(row_first, row_last, wave, n_waves, row_offsets, col_indices, q, k, v, out, d_qk, d_v,
+                                  s2, c, g, col_off);
         return;
     }
 
-    // ---- 2b .. C, once per round of at most u_max ranks of the union (one round unless a plan lists more
-    // columns than fit in LDS at once; then the maximum and the sums run across the rounds)
+    // ---- 2b .. C
     // Copy one operand's rows of ranks [u_first, u_first + n_here) into buf: 16 bytes per thread and slice,
     // kBatch slices in flight; rows past the round's ranks (the last step's padding) and slices past `d` are
     // written as zeros, so the arithmetic below never meets stale bits.
@@ -704,8 +711,8 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max, in
         lacc = float4_t{0.f, 0.f, 0.f, 0.f};
     };
 
-    if constexpr (!ROUNDS) {
-        // the whole union at once: the accumulators come to life only after the exponentials are packed
+    {
+        // the accumulators come to life only after the exponentials are packed
         const int n_steps = (n_union + 31) >> 5;  // <= kUnionSteps because u_max <= 32 * kUnionSteps
         gather(k, d_qk, kShiftK, 0, n_union, n_steps);
         __syncthreads();
@@ -717,43 +724,6 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max, in
         __syncthreads();
         clear_sums();
         weighted_sum(p, act);
-    } else {
-        // rounds of u_max ranks: K rows, scores, V rows, sums - the maximum and the sums run across the rounds
-        clear_sums();
-        float mx_run = neg_inf;
-        const int n_rounds = (n_union + u_max - 1) / u_max;
-        for (int round = 0; round < n_rounds; ++round) {
-            const int u_first = round * u_max;
-            const int n_here = (n_union - u_first) < u_max ? (n_union - u_first) : u_max;
-            const int n_steps = (n_here + 31) >> 5;
-            if (round > 0) {
-                __syncthreads();  // every wave is done with the previous round's V rows and row masks
-                for (int w = tid; w < mask_words; w += n_threads) l.rowmask[w] = (unsigned)masks[round * mask_words + w];
-            }
-            gather(k, d_qk, kShiftK, u_first, n_here, n_steps);
-            __syncthreads();
-            half8_t p[kUnionSteps];
-            unsigned act;
-            const float mx_new = scores(n_steps, mx_run, p, act);
-            if (round > 0) {
-                // what the earlier rounds accumulated was taken against their maximum: bring it to the new one
-                // (0 where the row had no column yet, 1 where it still has none)
-                const float f = mx_new == neg_inf ? 1.f
-                                : (mx_run == neg_inf ? 0.f : __builtin_amdgcn_exp2f((mx_run - mx_new) * s2a));
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const float fe = from_lane(f, (4 * g + e) & 15);  // accumulator register e of lane (c, g) is scalar row 4g + e
-                    lacc[e] *= fe;
-#pragma unroll
-                    for (int cc = 0; cc < CPL; ++cc) acc[cc][e] *= fe;
-                }
-            }
-            mx_run = mx_new;
-            __syncthreads();
-            gather(v, d_v, kShiftV, u_first, n_here, n_steps);
-            __syncthreads();
-            weighted_sum(p, act);
-        }
     }
     // normalise and store
 #pragma unroll
@@ -769,46 +739,316 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max, in
     }
 }
 
-// 32-bit words of the row masks of a workgroup of `rows` vector rows, padded to 16 bytes.
-static int union_mask_words(int rows) { return (rows * kUnionSteps + 3) & ~3; }
+// Planned launches of eight waves stream the union through LDS in sub-rounds of kStreamRanks ranks, K and V
+// rows side by side: the rows, row masks and column numbers of the NEXT sub-round are requested before the
+// current one is computed and parked in registers meanwhile, so after the first sub-round no wave waits for
+// a gather.  A sub-round is short enough to keep its raw scores in registers: the K rows are read and
+// multiplied once, not twice.  Maximum and sums run across the sub-rounds as in flash attention, so a
+// workgroup takes unions of up to kStreamRounds * kStreamRanks columns.
+template <int V, int KS, int CPL>
+__global__ void __launch_bounds__(512, union_wide(KS, CPL) ? 2 : 4)
+sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
+                               const int *__restrict__ row_offsets, const int *__restrict__ col_indices,
+                               const int *__restrict__ plan,
+                               const half_t *__restrict__ q, const half_t *__restrict__ k,
+                               const half_t *__restrict__ v, half_t *__restrict__ out, long long stride_q,
+                               long long stride_k, long long stride_v, long long stride_out, float scale)
+{
+    q += blockIdx.y * stride_q;
+    k += blockIdx.y * stride_k;
+    v += blockIdx.y * stride_v;
+    out += blockIdx.y * stride_out;
+    constexpr int RPW = 16 / V;
+    constexpr int PITCH = union_pitch(KS, CPL);
+    constexpr int SS = kStreamSteps;
+    constexpr int SR = kStreamRanks;
+    constexpr int kThreads = 512;
+    constexpr int kRows = 8 * RPW;                                  // vector rows per workgroup
+    constexpr int kMaskWords = (kRows * SS + 3) & ~3;               // the plan's words per round: [kRows][SS]
+    constexpr int kShiftK = KS == 1 ? 2 : (KS == 2 ? 3 : 4);        // 4 * KS slices of 8 halves per K row
+    constexpr int kShiftV = CPL == 4 ? 3 : 4;                       // 2 * CPL slices per V row
+    constexpr int NK = (SR << kShiftK) / kThreads;                  // 16-byte slices per thread and sub-round
+    constexpr int NV = (SR << kShiftV) / kThreads;
 
-// Launch shape of the union kernel for a request of `rows` vector rows per workgroup.
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    extern __shared__ __align__(16) unsigned char smem[];
+    unsigned *maskbuf = reinterpret_cast<unsigned *>(smem);        // [kRows][SS] masks of the sub-round in LDS
+    half_t *kbuf = reinterpret_cast<half_t *>(maskbuf + kRows * SS);
+    half_t *vbuf = kbuf + SR * PITCH;
+
+    int bx = blockIdx.x;
+    if ((gridDim.x & 7) == 0) bx = (bx & 7) * (gridDim.x >> 3) + (bx >> 3);  // a run of row blocks per XCD
+    const int row_first = bx * kRows;
+    const int row_last = (row_first + kRows) < m_vec ? (row_first + kRows) : m_vec;
+    const int c = lane & 15;
+    const int g = lane >> 4;
+    const float s2 = scale * kLog2e;
+    const int col0 = c * CPL;
+    const bool col_ok = col0 < d_v;
+    const int col_off = col_ok ? col0 : 0;
+
+    constexpr int u_cap = kStreamRounds * SR;
+    constexpr int stride = 4 + kStreamRounds * kMaskWords + u_cap;
+    const bool plan_ok = plan[0] == kPlanMagic && plan[1] == m_vec && plan[2] == V && plan[3] == n &&
+                         plan[4] == kRows && plan[5] == SR && plan[6] == stride && plan[7] == (int)gridDim.x &&
+                         plan[8] == kStreamRounds && plan[9] == SS;
+    const int *rec = plan + kPlanHeader + (size_t)(plan_ok ? bx : 0) * stride;
+    const int n_union = plan_ok ? rec[0] : 0x7fffffff;
+    const int *masks = rec + 4;
+    const int *cols = rec + 4 + kStreamRounds * kMaskWords;
+    if (n_union > u_cap || d_v % 8 != 0) {
+        per_row_block<V, KS, CPL>(row_first, row_last, wave, 8, row_offsets, col_indices, q, k, v, out, d_qk, d_v, s2,
+                                  c, g, col_off);
+        return;
+    }
+    const int n_rounds = (n_union + SR - 1) / SR;
+
+    // What a thread fetches per sub-round: NK slices of K rows, NV slices of V rows (thread t takes slices
+    // t, t + 512, ...: consecutive threads read consecutive 16 bytes of a row) and one mask word.
+    int col_k[NK], col_v[NV];
+    uint4_t stage_k[NK], stage_v[NV];
+    unsigned stage_m = 0;
+    auto fetch_cols = [&](int round) {  // column numbers of sub-round `round` (0 past the union: row 0, unused)
+#pragma unroll
+        for (int i = 0; i < NK; ++i) {
+            const int u = round * SR + ((tid + i * kThreads) >> kShiftK);
+            col_k[i] = cols[u < n_union ? u : 0];
+        }
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int u = round * SR + ((tid + i * kThreads) >> kShiftV);
+            col_v[i] = cols[u < n_union ? u : 0];
+        }
+    };
+    auto fetch_rows = [&](int round) {  // needs col_k / col_v of the same sub-round
+        const uint4_t zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int i = 0; i < NK; ++i) {
+            const int sidx = tid + i * kThreads;
+            const int u = round * SR + (sidx >> kShiftK), sl = sidx & ((1 << kShiftK) - 1);
+            const bool real = u < n_union && 8 * sl < d_qk;
+            const uint4_t x = *reinterpret_cast<const uint4_t *>(k + (size_t)col_k[i] * d_qk + (real ? 8 * sl : 0));
+            stage_k[i] = real ? x : zero;
+        }
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int sidx = tid + i * kThreads;
+            const int u = round * SR + (sidx >> kShiftV), sl = sidx & ((1 << kShiftV) - 1);
+            const bool real = u < n_union && 8 * sl < d_v;
+            const uint4_t x = *reinterpret_cast<const uint4_t *>(v + (size_t)col_v[i] * d_v + (real ? 8 * sl : 0));
+            stage_v[i] = real ? x : zero;
+        }
+        if (tid < kRows * SS) stage_m = (unsigned)masks[round * kMaskWords + tid];
+    };
+    auto commit = [&]() {  // the parked sub-round into LDS (rows past the union and slices past d as zeros)
+#pragma unroll
+        for (int i = 0; i < NK; ++i) {
+            const int sidx = tid + i * kThreads;
+            *reinterpret_cast<uint4_t *>(kbuf + (sidx >> kShiftK) * PITCH + 8 * (sidx & ((1 << kShiftK) - 1))) = stage_k[i];
+        }
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int sidx = tid + i * kThreads;
+            *reinterpret_cast<uint4_t *>(vbuf + (sidx >> kShiftV) * PITCH + 8 * (sidx & ((1 << kShiftV) - 1))) = stage_v[i];
+        }
+        if (tid < kRows * SS) maskbuf[tid] = stage_m;
+    };
+
+    fetch_cols(0);
+    const int q_first = 16 * wave;
+    const long long q_global = (long long)row_first * V + q_first;
+    const long long q_limit = (long long)row_last * V;
+    half8_t qb[KS];
+    load_q16<KS>(qb, q, q_global, q_limit, d_qk, c, g);
+    if (n_rounds > 0) fetch_rows(0);
+    if (n_rounds > 1) fetch_cols(1);
+    const float s2a = __builtin_fabsf(s2);  // the maximum is tracked on raw dot products: a negative scale moves into Q
+    if (s2 < 0.f) {
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) {
+            uint4_t bits = __builtin_bit_cast(uint4_t, qb[kk]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) bits[i] ^= 0x80008000u;
+            qb[kk] = __builtin_bit_cast(half8_t, bits);
+        }
+    }
+    const unsigned *mrow = maskbuf + ((q_first + c) / V) * SS;
+    const half_t *k_lane = kbuf + c * PITCH + 8 * g;
+    const half_t *v_lane = vbuf + 4 * g * PITCH + col_off;
+    const float neg_inf = -__builtin_inff();
+    constexpr unsigned kLaneBits = 0x000F000Fu;
+    const half8_t ones = {1, 1, 1, 1, 1, 1, 1, 1};
+    float4_t acc[CPL];
+#pragma unroll
+    for (int cc = 0; cc < CPL; ++cc) acc[cc] = float4_t{0.f, 0.f, 0.f, 0.f};
+    float4_t lacc = {0.f, 0.f, 0.f, 0.f};
+    float mx_run = neg_inf;
+
+    for (int round = 0; round < n_rounds; ++round) {
+        if (round > 0) __syncthreads();  // every wave is done with the previous sub-round's rows and masks
+        commit();
+        __syncthreads();
+        if (round + 1 < n_rounds) fetch_rows(round + 1);  // in flight during the arithmetic below
+        if (round + 2 < n_rounds) fetch_cols(round + 2);
+        const int n_here = (n_union - round * SR) < SR ? (n_union - round * SR) : SR;
+        const int n_steps = (n_here + 31) >> 5;
+
+        // scores of the sub-round, kept raw; the maximum over the pairs the mask holds
+        float4_t sacc[SS][2];
+        unsigned act = 0, full = 0;
+        float mx_raw = neg_inf;
+#pragma unroll
+        for (int t = 0; t < SS; ++t) {
+            sacc[t][0] = sacc[t][1] = float4_t{0.f, 0.f, 0.f, 0.f};
+            if (t < n_steps) {
+                const unsigned word = mrow[t];
+                if (__builtin_amdgcn_ballot_w64(word != 0u) != 0ull) {
+                    act |= 1u << t;
+                    const unsigned wg = word >> (4 * g);
+                    half8_t a[2][KS];
+                    load_k_step<KS, PITCH>(a, k_lane, t);
+                    scores_step<KS>(sacc[t], a, qb);
+                    if (__builtin_amdgcn_ballot_w64((wg & kLaneBits) != kLaneBits) == 0ull) {
+                        full |= 1u << t;
+#pragma unroll
+                        for (int u = 0; u < 2; ++u)
+                            mx_raw = fmaxf(fmaxf(mx_raw, fmaxf(sacc[t][u][0], sacc[t][u][1])),
+                                           fmaxf(sacc[t][u][2], sacc[t][u][3]));
+                    } else {
+#pragma unroll
+                        for (int u = 0; u < 2; ++u)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                mx_raw = fmaxf(mx_raw, select_bit(wg, 16 * u + e, sacc[t][u][e], neg_inf));
+                    }
+                }
+            }
+        }
+        act = __builtin_amdgcn_readfirstlane(act);
+        full = __builtin_amdgcn_readfirstlane(full);
+        mx_raw = fmaxf(mx_raw, partner<16>(mx_raw));  // scalar row c lives in the four lanes (c, g = 0..3)
+        mx_raw = fmaxf(mx_raw, partner<32>(mx_raw));
+        const float mx_new = fmaxf(mx_run, mx_raw);
+        const float neg_mx = mx_new == neg_inf ? 0.f : -(mx_new * s2a);
+        if (round > 0) {
+            // bring what the earlier sub-rounds accumulated to the new maximum
+            const float f = mx_new == neg_inf ? 1.f
+                            : (mx_run == neg_inf ? 0.f : __builtin_amdgcn_exp2f((mx_run - mx_new) * s2a));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float fe = from_lane(f, (4 * g + e) & 15);  // accumulator register e of lane (c, g) is scalar row 4g + e
+                lacc[e] *= fe;
+#pragma unroll
+                for (int cc = 0; cc < CPL; ++cc) acc[cc][e] *= fe;
+            }
+        }
+        mx_run = mx_new;
+
+        // probabilities (masked-out pairs exact zeros), then P V and the row sums
+#pragma unroll
+        for (int t = 0; t < SS; ++t) {
+            if ((act >> t) & 1u) {
+                half8_t p;
+                if ((full >> t) & 1u) {
+#pragma unroll
+                    for (int u = 0; u < 2; ++u)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            p[4 * u + e] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf(sacc[t][u][e], s2a, neg_mx));
+                } else {
+                    const unsigned wg = mrow[t] >> (4 * g);
+#pragma unroll
+                    for (int u = 0; u < 2; ++u)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const float bias = select_bit(wg, 16 * u + e, neg_mx, neg_inf);
+                            p[4 * u + e] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf(sacc[t][u][e], s2a, bias));
+                        }
+                }
+                RowChunk<CPL> rows[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) rows[e].load(v_lane + (32 * t + (e < 4 ? e : 12 + e)) * PITCH);
+#pragma unroll
+                for (int pp = 0; pp < CPL / 2; ++pp) {
+                    uint4_t even, odd;
+#pragma unroll
+                    for (int qq = 0; qq < 4; ++qq) {
+                        even[qq] = pack_lo(rows[2 * qq].dword(pp), rows[2 * qq + 1].dword(pp));
+                        odd[qq] = pack_hi(rows[2 * qq].dword(pp), rows[2 * qq + 1].dword(pp));
+                    }
+                    acc[2 * pp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(p, __builtin_bit_cast(half8_t, even), acc[2 * pp], 0, 0, 0);
+                    acc[2 * pp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(p, __builtin_bit_cast(half8_t, odd), acc[2 * pp + 1], 0, 0, 0);
+                }
+                lacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(p, ones, lacc, 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const long long row = q_global + 4 * g + e;
+        if (row < q_limit && col_ok) {
+            const float norm = lacc[e] > 0.f ? 1.f / lacc[e] : 0.f;  // a row with no column attends to nothing: zeros
+            float tmp[CPL];
+#pragma unroll
+            for (int cc = 0; cc < CPL; ++cc) tmp[cc] = acc[cc][e] * norm;
+            store_converted<half_t, CPL>(out + (size_t)row * d_v + col0, tmp);
+        }
+    }
+}
+
+// 32-bit words of one round of row masks of a workgroup: `rows` vector rows x `steps` words, padded to 16 bytes.
+static int union_mask_words(int rows, int steps) { return (rows * steps + 3) & ~3; }
+
+// Launch shape of the union kernels for a request of `rows` vector rows per workgroup.
 struct UnionShape {
-    int waves;   // 16 scalar rows each
-    int rows;    // vector rows per workgroup actually used
-    int u_max;   // distinct columns a workgroup can hold in LDS
+    int waves;    // 16 scalar rows each
+    int rows;     // vector rows per workgroup actually used
+    bool stream;  // planned launch of eight waves: the streamed kernel
+    int u_max;    // ranks of the union in LDS at once
+    int rounds;   // rounds of u_max ranks a workgroup can take (1 unless streamed)
+    int steps;    // mask words per vector row and round
     size_t lds;
     size_t plan_lds;  // LDS of the plan kernel for this shape
 };
 
-// plan_rounds: 0 for launches that rebuild the union, else the rounds of the plan (1..kMaxPlanRounds).
-static bool union_shape(UnionShape &s, int vec_length, int n, int d_qk, int d_v, int rows, int plan_rounds)
+static bool union_shape(UnionShape &s, int vec_length, int n, int d_qk, int d_v, int rows, bool planned)
 {
-    if (plan_rounds < 0 || plan_rounds > kMaxPlanRounds) return false;
-    // Half of a CU's LDS per workgroup, so that two workgroups overlap each other's memory phases (wide heads:
-    // one workgroup per CU, all of it).  With a plan the column bitmap, its prefix sums and the column list
-    // stay out of the attention kernel's LDS.
-    const bool planned = plan_rounds > 0;
-    const int ks = d_qk <= 32 ? 1 : (d_qk <= 64 ? 2 : 4);
-    const int cpl = d_v <= 64 ? 4 : 8;
-    const size_t budget = (union_wide(ks, cpl) ? 152 : (planned ? 80 : 72)) * 1024;
     const int rpw = 16 / vec_length;
     s.waves = ceil_div(rows < 1 ? 1 : rows, rpw);
     if (s.waves > 8) s.waves = 8;
     s.rows = s.waves * rpw;
+    s.stream = planned && s.waves == 8;
+    const int ks = d_qk <= 32 ? 1 : (d_qk <= 64 ? 2 : 4);
+    const int cpl = d_v <= 64 ? 4 : 8;
+    const size_t row_bytes = (size_t)union_pitch(ks, cpl) * sizeof(half_t);
     const int n_words = (((n + 31) / 32) + 3) & ~3;
-    const size_t mask = (size_t)union_mask_words(s.rows) * sizeof(unsigned);
-    const size_t build = 2 * (size_t)n_words * sizeof(unsigned) + 16 * sizeof(int) + mask;  // + one int per column
-    const size_t fixed = planned ? mask : build;
-    const size_t per_union_row = (size_t)union_pitch(ks, cpl) * sizeof(half_t) + (planned ? 0 : sizeof(int));
+    const size_t bitmaps = 2 * (size_t)n_words * sizeof(unsigned) + 16 * sizeof(int);  // what build_union adds
+    if (s.stream) {
+        s.u_max = kStreamRanks;
+        s.rounds = kStreamRounds;
+        s.steps = kStreamSteps;
+        const size_t mask = (size_t)union_mask_words(s.rows, s.steps) * sizeof(unsigned);
+        s.lds = mask + 2 * (size_t)s.u_max * row_bytes;  // masks of one sub-round, K rows and V rows side by side
+        s.plan_lds = bitmaps + s.rounds * (mask + (size_t)s.u_max * sizeof(int));
+        return s.plan_lds <= 160 * 1024;
+    }
+    // Half of a CU's LDS per workgroup, so that two workgroups overlap each other's memory phases (wide heads:
+    // one workgroup per CU, all of it).  With a plan the column bitmap, its prefix sums and the column list
+    // stay out of the attention kernel's LDS.
+    s.rounds = 1;
+    s.steps = kUnionSteps;
+    const size_t budget = (union_wide(ks, cpl) ? 152 : (planned ? 80 : 72)) * 1024;
+    const size_t mask = (size_t)union_mask_words(s.rows, s.steps) * sizeof(unsigned);
+    const size_t fixed = planned ? mask : bitmaps + mask;
+    const size_t per_union_row = row_bytes + (planned ? 0 : sizeof(int));
     if (fixed + 32 * per_union_row > budget) return false;  // the column bitmap alone fills the budget
     s.u_max = (int)((budget - fixed) / per_union_row) & ~31;
     if (s.u_max > 32 * kUnionSteps) s.u_max = 32 * kUnionSteps;
-    // the plan kernel holds the bitmap, the masks of every round and the column list of one workgroup in LDS
-    s.plan_lds = planned ? build + (plan_rounds - 1) * mask + (size_t)plan_rounds * s.u_max * sizeof(int) : 0;
-    if (s.plan_lds > 160 * 1024) return false;
     s.lds = fixed + (size_t)s.u_max * per_union_row;
-    return true;
+    s.plan_lds = planned ? bitmaps + mask + (size_t)s.u_max * sizeof(int) : 0;
+    return s.plan_lds <= 160 * 1024;
 }
 
 static bool union_dims_ok(int d_qk, int d_v)
@@ -819,7 +1059,7 @@ static bool union_dims_ok(int d_qk, int d_v)
 }
 
 struct UnionLaunch {
-    int m_vec, n, d_qk, d_v, rows, plan_rounds;
+    int m_vec, n, d_qk, d_v, rows;
     const int *row_offsets, *col_indices, *plan;
     const half_t *q, *k, *v;
     half_t *out;
@@ -829,43 +1069,52 @@ struct UnionLaunch {
     long long stride_v;
 };
 
-template <int V, int KS, int CPL, int MODE>
+template <int V, int KS, int CPL, bool PLANNED>
 static int launch_one(const UnionLaunch &a)
 {
     UnionShape s;
-    if (!union_shape(s, V, a.n, a.d_qk, a.d_v, a.rows, a.plan_rounds)) return hipErrorNotSupported;
-    auto kernel = sparse_attention_union_kernel<V, KS, CPL, MODE>;
-    static std::atomic<unsigned long long> lds_allowed{0};
+    if (!union_shape(s, V, a.n, a.d_qk, a.d_v, a.rows, PLANNED)) return hipErrorNotSupported;
+    static std::atomic<unsigned long long> lds_allowed{0}, stream_lds_allowed{0};
+    const dim3 grid((unsigned)ceil_div(a.m_vec, s.rows), (unsigned)a.batch->count);
+    if (PLANNED && s.stream) {
+        auto kernel = sparse_attention_stream_kernel<V, KS, CPL>;
+        const hipError_t attr = allow_large_lds(reinterpret_cast<const void *>(kernel), 160 * 1024, stream_lds_allowed);
+        if (attr != hipSuccess) return (int)attr;
+        hipLaunchKernelGGL(kernel, grid, dim3(512), s.lds, a.stream, a.m_vec, a.n, a.d_qk, a.d_v, a.row_offsets,
+                           a.col_indices, a.plan, a.q, a.k, a.v, a.out, a.batch->stride_a, a.batch->stride_b,
+                           a.stride_v, a.batch->stride_out, a.scale);
+        return (int)hipGetLastError();
+    }
+    auto kernel = sparse_attention_union_kernel<V, KS, CPL, PLANNED>;
     const hipError_t attr = allow_large_lds(reinterpret_cast<const void *>(kernel), 160 * 1024, lds_allowed);
     if (attr != hipSuccess) return (int)attr;
-    const int blocks = ceil_div(a.m_vec, s.rows);
-    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)a.batch->count), dim3(64 * s.waves), s.lds, a.stream,
-                       a.m_vec, a.n, a.d_qk, a.d_v, s.u_max, a.plan_rounds, a.row_offsets, a.col_indices, a.plan, a.q,
-                       a.k, a.v, a.out, a.batch->stride_a, a.batch->stride_b, a.stride_v, a.batch->stride_out, a.scale);
+    hipLaunchKernelGGL(kernel, grid, dim3(64 * s.waves), s.lds, a.stream, a.m_vec, a.n, a.d_qk, a.d_v, s.u_max,
+                       a.row_offsets, a.col_indices, a.plan, a.q, a.k, a.v, a.out, a.batch->stride_a,
+                       a.batch->stride_b, a.stride_v, a.batch->stride_out, a.scale);
     return (int)hipGetLastError();
 }
 
-template <int V, int MODE>
+template <int V, bool PLANNED>
 static int launch_shape(const UnionLaunch &a)
 {
     if (a.d_v <= 64) {
-        if (a.d_qk <= 32) return launch_one<V, 1, 4, MODE>(a);
-        if (a.d_qk <= 64) return launch_one<V, 2, 4, MODE>(a);
-        return launch_one<V, 4, 4, MODE>(a);
+        if (a.d_qk <= 32) return launch_one<V, 1, 4, PLANNED>(a);
+        if (a.d_qk <= 64) return launch_one<V, 2, 4, PLANNED>(a);
+        return launch_one<V, 4, 4, PLANNED>(a);
     }
-    if (a.d_qk <= 32) return launch_one<V, 1, 8, MODE>(a);
-    if (a.d_qk <= 64) return launch_one<V, 2, 8, MODE>(a);
-    return launch_one<V, 4, 8, MODE>(a);
+    if (a.d_qk <= 32) return launch_one<V, 1, 8, PLANNED>(a);
+    if (a.d_qk <= 64) return launch_one<V, 2, 8, PLANNED>(a);
+    return launch_one<V, 4, 8, PLANNED>(a);
 }
 
-template <int MODE>
+template <bool PLANNED>
 static int launch_v(int vec_length, const UnionLaunch &a)
 {
     switch (vec_length) {
-    case 1: return launch_shape<1, MODE>(a);
-    case 2: return launch_shape<2, MODE>(a);
-    case 4: return launch_shape<4, MODE>(a);
-    case 8: return launch_shape<8, MODE>(a);
+    case 1: return launch_shape<1, PLANNED>(a);
+    case 2: return launch_shape<2, PLANNED>(a);
+    case 4: return launch_shape<4, PLANNED>(a);
+    case 8: return launch_shape<8, PLANNED>(a);
     default: return hipErrorInvalidValue;
     }
 }
@@ -876,56 +1125,54 @@ static bool union_supported(int vec_length, int n, int d_qk, int d_v)
     return n >= 0 && n <= 1024 * 1024 && union_dims_ok(d_qk, d_v);  // the column bitmap lives in LDS
 }
 
-int sparse_attention_union_capacity(int vec_length, int n, int d_qk, int d_v, int rows, int plan_rounds, int *rows_used)
+int sparse_attention_union_capacity(int vec_length, int n, int d_qk, int d_v, int rows, bool with_plan, int *rows_used)
 {
     UnionShape s;
     if (!union_supported(vec_length, n, d_qk, d_v) || d_v % 8 != 0) return 0;
-    if (!union_shape(s, vec_length, n, d_qk, d_v, rows, plan_rounds)) return 0;
+    if (!union_shape(s, vec_length, n, d_qk, d_v, rows, with_plan)) return 0;
     if (rows_used) *rows_used = s.rows;
-    return plan_rounds > 1 ? plan_rounds * s.u_max : s.u_max;
+    return s.rounds * s.u_max;
 }
 
-long long sparse_attention_plan_bytes(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, int plan_rounds)
+long long sparse_attention_plan_bytes(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows)
 {
     UnionShape s;
-    if (m_vec < 0 || plan_rounds < 1 || !union_supported(vec_length, n, d_qk, d_v)) return 0;
-    if (!union_shape(s, vec_length, n, d_qk, d_v, rows, plan_rounds)) return 0;
-    const long long stride = 4 + plan_rounds * ((long long)union_mask_words(s.rows) + s.u_max);
+    if (m_vec < 0 || !union_supported(vec_length, n, d_qk, d_v)) return 0;
+    if (!union_shape(s, vec_length, n, d_qk, d_v, rows, true)) return 0;
+    const long long stride = 4 + s.rounds * ((long long)union_mask_words(s.rows, s.steps) + s.u_max);
     return (long long)sizeof(int) * (kPlanHeader + stride * ceil_div(m_vec, s.rows));
 }
 
-int launch_sparse_attention_plan(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, int plan_rounds,
-                                 const int *row_offsets, const int *col_indices, int *plan, long long plan_bytes,
-                                 hipStream_t stream)
+int launch_sparse_attention_plan(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, const int *row_offsets,
+                                 const int *col_indices, int *plan, long long plan_bytes, hipStream_t stream)
 {
     UnionShape s;
-    if (plan_rounds < 1 || !union_supported(vec_length, n, d_qk, d_v)) return hipErrorNotSupported;
-    if (!union_shape(s, vec_length, n, d_qk, d_v, rows, plan_rounds)) return hipErrorNotSupported;
-    const long long need = sparse_attention_plan_bytes(m_vec, vec_length, n, d_qk, d_v, rows, plan_rounds);
+    if (!union_supported(vec_length, n, d_qk, d_v)) return hipErrorNotSupported;
+    if (!union_shape(s, vec_length, n, d_qk, d_v, rows, true)) return hipErrorNotSupported;
+    const long long need = sparse_attention_plan_bytes(m_vec, vec_length, n, d_qk, d_v, rows);
     if (plan_bytes < need) return hipErrorInvalidValue;
     if (m_vec == 0) return hipSuccess;
     static std::atomic<unsigned long long> lds_allowed{0};
-    const hipError_t attr = allow_large_lds(reinterpret_cast<const void *>(sparse_attention_plan_kernel), 160 * 1024, lds_allowed);
+    const hipError_t attr = allow_large_lds(reinterpret_cast<const void *>(sparse_attention_plan_kernel), 160 * 1024,
+                                            lds_allowed);
     if (attr != hipSuccess) return (int)attr;
     hipLaunchKernelGGL(sparse_attention_plan_kernel, dim3((unsigned)ceil_div(m_vec, s.rows)), dim3(256), s.plan_lds,
-                       stream, m_vec, vec_length, n, s.rows, s.u_max, plan_rounds, row_offsets, col_indices, plan);
+                       stream, m_vec, vec_length, n, s.rows, s.u_max, s.rounds, s.steps, row_offsets, col_indices, plan);
     return (int)hipGetLastError();
 }
 
-int launch_sparse_attention_union(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, int plan_rounds,
-                                  const int *row_offsets, const int *col_indices, const int *plan, const half_t *q,
-                                  const half_t *k, const half_t *v, half_t *out, float scale, hipStream_t stream,
-                                  const Batch &batch, long long stride_v)
+int launch_sparse_attention_union(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, const int *row_offsets,
+                                  const int *col_indices, const int *plan, const half_t *q, const half_t *k,
+                                  const half_t *v, half_t *out, float scale, hipStream_t stream, const Batch &batch,
+                                  long long stride_v)
 {
     if (m_vec == 0 || batch.count == 0 || d_v == 0) return hipSuccess;
     if (batch.count > 65535) return hipErrorNotSupported;
     if (!union_supported(vec_length, n, d_qk, d_v)) return hipErrorNotSupported;
-    if (!plan) plan_rounds = 0;
-    const UnionLaunch a = {m_vec, n, d_qk, d_v, rows, plan_rounds, row_offsets, col_indices, plan, q, k, v, out,
+    const UnionLaunch a = {m_vec, n, d_qk, d_v, rows, row_offsets, col_indices, plan, q, k, v, out,
                            scale, stream, &batch, stride_v};
-    if (plan_rounds > 1) return launch_v<2>(vec_length, a);
-    if (plan_rounds == 1) return launch_v<1>(vec_length, a);
-    return launch_v<0>(vec_length, a);
+    if (plan) return launch_v<true>(vec_length, a);
+    return launch_v<false>(vec_length, a);
 }
 
 }  // namespace vs

@@ -254,15 +254,14 @@ int launch_sparse_attention(int m_vec, int vec_length, int d_qk, int d_v, const 
                             const int *row_offsets, const int *col_indices, const half_t *q, const half_t *k,
                             const half_t *v, half_t *out, float scale, hipStream_t stream, const Batch &batch,
                             long long stride_v);
-int launch_sparse_attention_union(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, int plan_rounds,
-                                  const int *row_offsets, const int *col_indices, const int *plan, const half_t *q,
-                                  const half_t *k, const half_t *v, half_t *out, float scale, hipStream_t stream,
-                                  const Batch &batch, long long stride_v);
-long long sparse_attention_plan_bytes(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, int plan_rounds);
-int launch_sparse_attention_plan(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, int plan_rounds,
-                                 const int *row_offsets, const int *col_indices, int *plan, long long plan_bytes,
-                                 hipStream_t stream);
-int sparse_attention_union_capacity(int vec_length, int n, int d_qk, int d_v, int rows, int plan_rounds, int *rows_used);
+int launch_sparse_attention_union(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, const int *row_offsets,
+                                  const int *col_indices, const int *plan, const half_t *q, const half_t *k,
+                                  const half_t *v, half_t *out, float scale, hipStream_t stream, const Batch &batch,
+                                  long long stride_v);
+long long sparse_attention_plan_bytes(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows);
+int launch_sparse_attention_plan(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows, const int *row_offsets,
+                                 const int *col_indices, int *plan, long long plan_bytes, hipStream_t stream);
+int sparse_attention_union_capacity(int vec_length, int n, int d_qk, int d_v, int rows, bool with_plan, int *rows_used);
 int launch_sparse_softmax(int m_vec, int vec_length, const int *row_indices, const int *row_offsets,
                           const half_t *values_in, half_t *values_out, float scale, hipStream_t stream,
                           const Batch &batch = Batch());

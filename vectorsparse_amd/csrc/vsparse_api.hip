@@ -291,13 +291,11 @@ int vs_wmma_spmm_softmax_f16_batched(int batch, int m_vec, int vec_length, int k
 int vs_sparse_attention_f16(int batch, int m_vec, int vec_length, int n, int d_qk, int d_v, const int *row_indices,
                             const int *row_offsets, const int *col_indices, const void *q, long long stride_q,
                             const void *k, long long stride_k, const void *v, long long stride_v, void *out,
-                            long long stride_out, float scale, int rows_per_workgroup, const void *plan, int plan_rounds,
-                            void *stream)
+                            long long stride_out, float scale, int rows_per_workgroup, const void *plan, void *stream)
 {
     if (batch < 0 || m_vec < 0 || n < 0 || d_qk < 0 || d_v < 0 || !vec_ok(vec_length)) return VS_ERROR_INVALID_VALUE;
     if (rows_per_workgroup < 0 || rows_per_workgroup > 128) return VS_ERROR_INVALID_VALUE;
-    if (plan && (rows_per_workgroup < 2 || !aligned(plan, 16) || plan_rounds < 1 || plan_rounds > 4))
-        return VS_ERROR_INVALID_VALUE;
+    if (plan && (rows_per_workgroup < 2 || !aligned(plan, 16))) return VS_ERROR_INVALID_VALUE;
     if (batch == 0 || m_vec == 0 || d_v == 0) return VS_SUCCESS;
     if (!row_indices || !row_offsets || !q || !out) return VS_ERROR_INVALID_VALUE;
     if (n > 0 && (!k || !v)) return VS_ERROR_INVALID_VALUE;
@@ -305,8 +303,8 @@ int vs_sparse_attention_f16(int batch, int m_vec, int vec_length, int n, int d_q
     if (!stride_ok(stride_q, 8) || !stride_ok(stride_k, 8) || !stride_ok(stride_v, 8) || !stride_ok(stride_out, 8))
         return VS_ERROR_INVALID_VALUE;
     if (rows_per_workgroup > 1)  // union-gather kernel: pays off when neighbouring rows share columns
-        return vs::launch_sparse_attention_union(m_vec, vec_length, n, d_qk, d_v, rows_per_workgroup, plan_rounds,
-                                                 row_offsets, col_indices, static_cast<const int *>(plan), static_cast<const half_t *>(q), static_cast<const half_t *>(k),
+        return vs::launch_sparse_attention_union(m_vec, vec_length, n, d_qk, d_v, rows_per_workgroup, row_offsets,
+                                                 col_indices, static_cast<const int *>(plan), static_cast<const half_t *>(q), static_cast<const half_t *>(k),
                                                  static_cast<const half_t *>(v), static_cast<half_t *>(out), scale,
                                                  static_cast<hipStream_t>(stream),
                                                  make_batch(batch, stride_q, stride_k, stride_out), stride_v);
@@ -317,33 +315,29 @@ int vs_sparse_attention_f16(int batch, int m_vec, int vec_length, int n, int d_q
                                        stride_v);
 }
 
-long long vs_sparse_attention_plan_bytes(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows_per_workgroup,
-                                         int plan_rounds)
+long long vs_sparse_attention_plan_bytes(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows_per_workgroup)
 {
     if (m_vec < 0 || n < 0 || !vec_ok(vec_length) || rows_per_workgroup < 2 || rows_per_workgroup > 128) return 0;
-    if (plan_rounds < 1 || plan_rounds > 4) return 0;
-    return vs::sparse_attention_plan_bytes(m_vec, vec_length, n, d_qk, d_v, rows_per_workgroup, plan_rounds);
+    return vs::sparse_attention_plan_bytes(m_vec, vec_length, n, d_qk, d_v, rows_per_workgroup);
 }
 
 int vs_sparse_attention_plan(int m_vec, int vec_length, int n, int d_qk, int d_v, int rows_per_workgroup,
-                             int plan_rounds, const int *row_offsets, const int *col_indices, void *plan,
-                             long long plan_bytes, void *stream)
+                             const int *row_offsets, const int *col_indices, void *plan, long long plan_bytes,
+                             void *stream)
 {
     if (m_vec < 0 || n < 0 || !vec_ok(vec_length) || rows_per_workgroup < 2 || rows_per_workgroup > 128)
         return VS_ERROR_INVALID_VALUE;
-    if (plan_rounds < 1 || plan_rounds > 4) return VS_ERROR_INVALID_VALUE;
     if (!plan || !aligned(plan, 16) || (m_vec > 0 && !row_offsets)) return VS_ERROR_INVALID_VALUE;
-    return vs::launch_sparse_attention_plan(m_vec, vec_length, n, d_qk, d_v, rows_per_workgroup, plan_rounds,
-                                            row_offsets, col_indices, static_cast<int *>(plan), plan_bytes,
+    return vs::launch_sparse_attention_plan(m_vec, vec_length, n, d_qk, d_v, rows_per_workgroup, row_offsets,
+                                            col_indices, static_cast<int *>(plan), plan_bytes,
                                             static_cast<hipStream_t>(stream));
 }
 
-int vs_sparse_attention_union_capacity(int vec_length, int n, int d_qk, int d_v, int rows_per_workgroup, int plan_rounds,
+int vs_sparse_attention_union_capacity(int vec_length, int n, int d_qk, int d_v, int rows_per_workgroup, int with_plan,
                                        int *rows_used)
 {
     if (!vec_ok(vec_length) || n < 0 || rows_per_workgroup < 2 || rows_per_workgroup > 128) return 0;
-    if (plan_rounds < 0 || plan_rounds > 4) return 0;
-    return vs::sparse_attention_union_capacity(vec_length, n, d_qk, d_v, rows_per_workgroup, plan_rounds, rows_used);
+    return vs::sparse_attention_union_capacity(vec_length, n, d_qk, d_v, rows_per_workgroup, with_plan != 0, rows_used);
 }
 
 int vs_sparse_softmax_f16(int batch, int m_vec, int vec_length, const int *row_indices, const int *row_offsets,

@@ -156,13 +156,12 @@ def spmm_softmax_batched(m_vec, vec_length, k, n, row_indices, row_offsets, colu
 
 
 def sparse_attention(m_vec, vec_length, n, row_indices, row_offsets, col_indices, q, k, v, out=None, scale=None,
-                     stream=None, rows_per_workgroup=0, plan=None, plan_rounds=None):
+                     stream=None, rows_per_workgroup=0, plan=None):
     """Single-launch fixed-mask attention: out = softmax(scale * mask(q k^T)) v.
 
     q: [heads, m, d_qk], k: [heads, n, d_qk], v: [heads, n, d_v] (or 2-D for one head), fp16.
     rows_per_workgroup: 0 / 1 = one vector row per workgroup; >= 2 = union-gather kernel for masks whose
-    neighbouring rows share columns, optionally with a plan from `sparse_attention_plan` (whose number of
-    rounds travels with the plan tensor unless plan_rounds says otherwise).
+    neighbouring rows share columns, optionally (and much faster) with a plan from `sparse_attention_plan`.
     """
     if q.dim() == 2:
         q, k, v = q.unsqueeze(0), k.unsqueeze(0), v.unsqueeze(0)
@@ -176,13 +175,11 @@ def sparse_attention(m_vec, vec_length, n, row_indices, row_offsets, col_indices
         out = torch.empty((heads, m, d_v), dtype=torch.float16, device=q.device)
     for t, nm in ((q, "q"), (k, "k"), (v, "v"), (out, "out")):
         _expect_batched(t, torch.float16, nm)
-    if plan_rounds is None:
-        plan_rounds = getattr(plan, "plan_rounds", 1)
     st = _lib.lib().vs_sparse_attention_f16(heads, m_vec, vec_length, n, d_qk, d_v, _ptr(row_indices),
                                             _ptr(row_offsets), _ptr(col_indices), _ptr(q), _stride(q, heads),
                                             _ptr(k), _stride(k, heads), _ptr(v), _stride(v, heads), _ptr(out),
                                             _stride(out, heads), float(scale), int(rows_per_workgroup),
-                                            _ptr(plan), int(plan_rounds), _stream(stream))
+                                            _ptr(plan), _stream(stream))
     _lib.check(st, "vs_sparse_attention_f16")
     return out
 
@@ -233,19 +230,16 @@ def _expect_batched(t, dtype, name):
         raise ValueError("%s must be contiguous in its trailing dimensions" % name)
 
 
-def sparse_attention_plan(m_vec, vec_length, n, d_qk, d_v, rows_per_workgroup, row_offsets, col_indices, stream=None,
-                          plan_rounds=1):
-    """Analyse a fixed mask once for the union-gather kernel: returns the plan (a device byte tensor, its
-    `plan_rounds` attribute set) that `sparse_attention(..., rows_per_workgroup=..., plan=...)` reads instead
-    of rebuilding it per launch.  plan_rounds 2..4: unions of that many times the LDS capacity, in rounds."""
-    size = _lib.lib().vs_sparse_attention_plan_bytes(m_vec, vec_length, n, d_qk, d_v, rows_per_workgroup, plan_rounds)
+def sparse_attention_plan(m_vec, vec_length, n, d_qk, d_v, rows_per_workgroup, row_offsets, col_indices, stream=None):
+    """Analyse a fixed mask once for the union-gather kernel: returns the plan (a device byte tensor) that
+    `sparse_attention(..., rows_per_workgroup=..., plan=...)` reads instead of rebuilding it per launch."""
+    size = _lib.lib().vs_sparse_attention_plan_bytes(m_vec, vec_length, n, d_qk, d_v, rows_per_workgroup)
     if size <= 0:
         raise _lib.VSparseError("vs_sparse_attention_plan_bytes: shape not supported by the union kernel")
     plan = torch.empty(size, dtype=torch.uint8, device=row_offsets.device)
-    st = _lib.lib().vs_sparse_attention_plan(m_vec, vec_length, n, d_qk, d_v, rows_per_workgroup, plan_rounds,
-                                             _ptr(row_offsets), _ptr(col_indices), _ptr(plan), size, _stream(stream))
+    st = _lib.lib().vs_sparse_attention_plan(m_vec, vec_length, n, d_qk, d_v, rows_per_workgroup, _ptr(row_offsets),
+                                             _ptr(col_indices), _ptr(plan), size, _stream(stream))
     _lib.check(st, "vs_sparse_attention_plan")
-    plan.plan_rounds = int(plan_rounds)
     return plan
 
 
@@ -263,65 +257,61 @@ class SparseAttention:
         self._plans = {}
         self._rows = {}
 
-    def union_shape(self, d_qk, d_v):
-        """(rows per workgroup, plan rounds) of the single-launch kernel with these head widths (cached)."""
+    def union_rows(self, d_qk, d_v):
+        """Rows per workgroup for the single-launch kernel with these head widths (cached per shape)."""
         key = (int(d_qk), int(d_v))
         if key not in self._rows:
-            self._rows[key] = self._union_shape(self.mask, *key)
+            self._rows[key] = self._union_rows(self.mask, *key)
         return self._rows[key]
-
-    def union_rows(self, d_qk, d_v):
-        """Rows per workgroup for the single-launch kernel with these head widths."""
-        return self.union_shape(d_qk, d_v)[0]
 
     def plan(self, d_qk, d_v):
         """Device plan of the union kernel for these head widths (built on first use), or None."""
         key = (int(d_qk), int(d_v))
-        rows, rounds = self.union_shape(*key)
+        rows = self.union_rows(*key)
         if rows < 2:
             return None
         if key not in self._plans:
             p = self.prob
             self._plans[key] = sparse_attention_plan(p.m_vec, p.vec_length, p.n, key[0], key[1], rows,
-                                                     p.row_offsets, p.column_indices, plan_rounds=rounds)
+                                                     p.row_offsets, p.column_indices)
         return self._plans[key]
 
     @staticmethod
-    def _union_shape(mask, d_qk, d_v, min_fill=0.4):
-        """(vector rows per workgroup, plan rounds) for the single-launch kernel: the largest block of
-        consecutive rows whose distinct columns fit the library's capacity for this shape in every block -
-        in LDS at once if possible, else in up to four rounds - and whose dense tile (rows x union) is at
-        least `min_fill` full (banded, blocky or strided masks), else (1, 1): one row per workgroup, any mask.
+    def _union_rows(mask, d_qk, d_v, min_fill=0.4):
+        """Vector rows per workgroup for the single-launch kernel: the largest block of consecutive rows
+        whose distinct columns stay within the library's capacity for this shape (with a plan) in every block
+        and whose dense tile (rows x union) is at least `min_fill` full (banded, blocky or strided masks),
+        else 1 (one row per workgroup, any mask).
 
         Every workgroup gathers its whole union, so small workgroups pay the gather for few rows: measured
-        on MI355X (16 heads, 4096 x 4096 band + strided masks) eight waves in two rounds beat four waves in
-        one (40 us against 53 us), two waves beat the per-row kernel only for V <= 4 (132 us against 165 us
-        at V = 4, 133 us against 99 us at V = 8) and a single wave only for V = 1 (385 us against 481 us)."""
+        on MI355X (16 heads, 4096 x 4096 band + strided masks whose unions only fit small blocks) two waves
+        beat the per-row kernel only for V <= 4 (132 us against 165 us at V = 4, 133 us against 99 us at
+        V = 8) and a single wave only for V = 1 (385 us against 481 us)."""
         ro, ci = mask.row_offsets, mask.column_indices
         if mask.m_vec == 0 or mask.nnz_vec == 0:
-            return 1, 1
+            return 1
         per_wave = 16 // mask.vec_length
         min_waves = {1: 1, 2: 2, 4: 2, 8: 4}[mask.vec_length]
-        capacity = _lib.lib().vs_sparse_attention_union_capacity
         for waves in (8, 4, 2, 1):
             if waves < min_waves:
                 break
             used = ctypes.c_int(0)
-            if capacity(mask.vec_length, mask.n, d_qk, d_v, waves * per_wave, 1, ctypes.addressof(used)) <= 0:
-                continue
+            cap = _lib.lib().vs_sparse_attention_union_capacity(mask.vec_length, mask.n, d_qk, d_v, waves * per_wave,
+                                                                1, ctypes.addressof(used))
             rows = used.value
-            if rows != waves * per_wave:
+            if cap <= 0 or rows != waves * per_wave:
                 continue
-            unions = [np.unique(ci[ro[first]:ro[min(first + rows, mask.m_vec)]]).size
-                      for first in range(0, mask.m_vec, rows)]
-            tile = sum(u * (min(first + rows, mask.m_vec) - first)
-                       for u, first in zip(unions, range(0, mask.m_vec, rows)))
-            if mask.nnz_vec < min_fill * tile:
-                continue
-            for rounds in (1, 2, 3, 4):
-                if 0 < max(unions) <= capacity(mask.vec_length, mask.n, d_qk, d_v, rows, rounds, None):
-                    return rows, rounds
-        return 1, 1
+            fits, tile = True, 0
+            for first in range(0, mask.m_vec, rows):
+                last = min(first + rows, mask.m_vec)
+                union = np.unique(ci[ro[first]:ro[last]]).size
+                if union > cap:
+                    fits = False
+                    break
+                tile += union * (last - first)
+            if fits and mask.nnz_vec >= min_fill * tile:
+                return rows
+        return 1
 
     def forward(self, q, k, v, scale=None, kernel="wmma", stream=None, scores=None, out=None, fused=None):
         """q, k, v: fp16 [heads, seq, d] on the device.  Returns fp16 [heads, seq, d].
@@ -350,7 +340,7 @@ class SparseAttention:
             return sparse_attention(p.m_vec, p.vec_length, p.n, p.row_indices, p.row_offsets, p.column_indices,
                                     q, k, v, out=out, scale=scale, stream=stream,
                                     rows_per_workgroup=self.union_rows(q.shape[2], v.shape[2]),
-                                    plan=self.plan(q.shape[2], v.shape[2]))  # the plan carries its rounds
+                                    plan=self.plan(q.shape[2], v.shape[2]))
         sddmm_batched(p.m_vec, d, p.n, p.nnz_vec, p.row_indices, p.row_offsets, p.column_indices, q, k, scores,
                       p.vec_length, kernel=kernel, stream=stream)
         if fused:
