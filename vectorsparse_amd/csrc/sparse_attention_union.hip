@@ -35,8 +35,8 @@
 //      and the V rows (transposed in registers with v_perm_b32, as in the SpMM kernel) are read in that
 //      same order.  One more MFMA per step with an all-ones B operand yields the row sums of the rounded
 //      p in exactly the accumulator layout, so normalising needs no cross-lane traffic.
-// A plan of several rounds lets a workgroup take a union that does not fit LDS at once: steps 2 (the copy)
-// to C run once per round of u_max ranks, with the maximum and the sums carried across the rounds.
+// Planned launches of eight waves do not hold the union at once: sparse_attention_stream_kernel below runs
+// steps 2 (the copy) to C per sub-round of 128 ranks, the next sub-round's rows on their way meanwhile.
 #include "vs_common.hpp"
 
 namespace vs {
@@ -798,29 +798,19 @@ sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
     const int n_union = plan_ok ? rec[0] : 0x7fffffff;
     const int *masks = rec + 4;
     const int *cols = rec + 4 + kStreamRounds * kMaskWords;
-    if (n_union > u_cap || d_v % 8 != 0) {
-        per_row_block<V, KS, CPL>(row_first, row_last, wave, 8, row_offsets, col_indices, q, k, v, out, d_qk, d_v, s2,
-                                  c, g, col_off);
-        return;
-    }
-    const int n_rounds = (n_union + SR - 1) / SR;
 
     // What a thread fetches per sub-round: NK slices of K rows, NV slices of V rows (thread t takes slices
     // t, t + 512, ...: consecutive threads read consecutive 16 bytes of a row) and one mask word.
     int col_k[NK], col_v[NV];
     uint4_t stage_k[NK], stage_v[NV];
     unsigned stage_m = 0;
-    auto fetch_cols = [&](int round) {  // column numbers of sub-round `round` (0 past the union: row 0, unused)
+    // column numbers of sub-round `round` < kStreamRounds (the plan lists 0 past the union: row 0, unused), which
+    // do not wait for the union's size
+    auto fetch_cols = [&](int round) {
 #pragma unroll
-        for (int i = 0; i < NK; ++i) {
-            const int u = round * SR + ((tid + i * kThreads) >> kShiftK);
-            col_k[i] = cols[u < n_union ? u : 0];
-        }
+        for (int i = 0; i < NK; ++i) col_k[i] = cols[round * SR + ((tid + i * kThreads) >> kShiftK)];
 #pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            const int u = round * SR + ((tid + i * kThreads) >> kShiftV);
-            col_v[i] = cols[u < n_union ? u : 0];
-        }
+        for (int i = 0; i < NV; ++i) col_v[i] = cols[round * SR + ((tid + i * kThreads) >> kShiftV)];
     };
     auto fetch_rows = [&](int round) {  // needs col_k / col_v of the same sub-round
         const uint4_t zero = {0u, 0u, 0u, 0u};
@@ -856,7 +846,13 @@ sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
         if (tid < kRows * SS) maskbuf[tid] = stage_m;
     };
 
-    fetch_cols(0);
+    fetch_cols(0);  // requested together with the union's size
+    if (n_union > u_cap || d_v % 8 != 0) {
+        per_row_block<V, KS, CPL>(row_first, row_last, wave, 8, row_offsets, col_indices, q, k, v, out, d_qk, d_v, s2,
+                                  c, g, col_off);
+        return;
+    }
+    const int n_rounds = (n_union + SR - 1) / SR;
     const int q_first = 16 * wave;
     const long long q_global = (long long)row_first * V + q_first;
     const long long q_limit = (long long)row_last * V;
