@@ -562,3 +562,32 @@ def test_attention_random_cases(gpu, seed):
         out = layer.forward(qd, kd, vd, scale=scale, fused=fused)
         torch.cuda.synchronize()
         _check_layer(out.cpu().numpy(), ref, what + " layer fused=%s" % fused)
+
+
+def test_streamed_kernel_falls_back_on_oversized_unions(gpu):
+    """Blocks of rows whose union exceeds what a plan lists (scattered columns over a long sequence): the
+    streamed kernel's workgroups take the per-row path; a mask that mixes such blocks with banded ones runs
+    both paths in one launch."""
+    V, seq, d = 8, 4096, 64
+    scattered = cv.uniform_pattern(seq // V, seq, 0.9, seed=11, vec_length=V)
+    band = cv.band_strided_pattern(seq, V, band_half_width=64, stride=128)
+    # first half of the rows banded, second half scattered
+    half = band.m_vec // 2
+    lengths = np.concatenate([np.diff(band.row_offsets)[:half], np.diff(scattered.row_offsets)[half:]])
+    offsets = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    columns = np.concatenate([band.column_indices[:band.row_offsets[half]],
+                              scattered.column_indices[scattered.row_offsets[half]:]])
+    mixed = cv.ColVecCSR(band.m_vec, seq, V, offsets, columns).validate()
+    rng = np.random.default_rng(12)
+    q, k, v = (rng.standard_normal((1, seq, d)).astype(np.float16) for _ in range(3))
+    qd, kd, vd = (torch.from_numpy(x).cuda() for x in (q, k, v))
+    for name, mask in (("scattered", scattered), ("mixed", mixed)):
+        unions = _unions(mask, 16)
+        assert max(unions) > _capacity(V, seq, d, d, 16, 1)
+        assert (min(unions) <= 512) == (name == "mixed")
+        prob = ops.DeviceProblem(mask)
+        plan = ops.sparse_attention_plan(mask.m_vec, V, seq, d, d, 16, prob.row_offsets, prob.column_indices)
+        out = ops.sparse_attention(mask.m_vec, V, seq, prob.row_indices, prob.row_offsets, prob.column_indices,
+                                   qd, kd, vd, scale=0.125, rows_per_workgroup=16, plan=plan)
+        torch.cuda.synchronize()
+        _check_layer(out.cpu().numpy(), _dense_attention(mask, q, k, v, 0.125), name)
