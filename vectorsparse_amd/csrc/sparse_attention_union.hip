@@ -609,10 +609,9 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max,
     const half_t *v_lane = buf + 4 * g * PITCH + col_off;
     const float neg_inf = -__builtin_inff();
 
-    // ---- A. per wave: 16 scalar rows against the n_steps steps of ranks in buf; maximum (joined with mx_run,
-    // the maximum of earlier rounds), then masked exponentials.  Returns the new maximum of the lane's scalar
-    // row c (raw dot products); act = steps in which at least one row of the wave holds a column (uniform).
-    auto scores = [&](int n_steps, float mx_run, half8_t (&p)[kUnionSteps], unsigned &act) {
+    // ---- A. per wave: 16 scalar rows against the n_steps steps of ranks in buf; maximum, then masked
+    // exponentials; act = steps in which at least one row of the wave holds a column (uniform).
+    auto scores = [&](int n_steps, half8_t (&p)[kUnionSteps], unsigned &act) {
         constexpr unsigned kLaneBits = 0x000F000Fu;  // after the shift by 4g: the lane's 4 + 4 ranks of a step
         unsigned full = 0;  // steps in which every lane's rows hold all of the lane's ranks: no masking needed
         float mx_raw = neg_inf;
@@ -647,8 +646,7 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max,
         full = __builtin_amdgcn_readfirstlane(full);
         mx_raw = fmaxf(mx_raw, partner<16>(mx_raw));  // scalar row c lives in the four lanes (c, g = 0..3)
         mx_raw = fmaxf(mx_raw, partner<32>(mx_raw));
-        const float mx_new = fmaxf(mx_run, mx_raw);
-        const float neg_mx = mx_new == neg_inf ? 0.f : -(mx_new * s2a);  // a row with no column: every exponent stays -inf
+        const float neg_mx = mx_raw == neg_inf ? 0.f : -(mx_raw * s2a);  // a row with no column: every exponent stays -inf
 #pragma unroll
         for (int t = 0; t < kUnionSteps; ++t) {
             p[t] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
@@ -676,7 +674,6 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max,
                 }
             }
         }
-        return mx_new;
     };
 
     // ---- C. P V and the row sums against the V rows in buf (one wave owns its rows: nothing to reduce)
@@ -718,7 +715,7 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max,
         __syncthreads();
         half8_t p[kUnionSteps];
         unsigned act;
-        scores(n_steps, neg_inf, p, act);
+        scores(n_steps, p, act);
         __syncthreads();
         gather(v, d_v, kShiftV, 0, n_union, n_steps);  // V rows over the K rows
         __syncthreads();
