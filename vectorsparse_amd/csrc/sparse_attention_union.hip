@@ -809,36 +809,42 @@ sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
 #pragma unroll
         for (int i = 0; i < NV; ++i) col_v[i] = cols[round * SR + ((tid + i * kThreads) >> kShiftV)];
     };
+    // Requests only: nothing here reads what the loads return, so the wave goes on to the arithmetic at once.
+    // Slices past the union or past d read the start of a valid row and are replaced by zeros in commit().
     auto fetch_rows = [&](int round) {  // needs col_k / col_v of the same sub-round
-        const uint4_t zero = {0u, 0u, 0u, 0u};
 #pragma unroll
         for (int i = 0; i < NK; ++i) {
             const int sidx = tid + i * kThreads;
             const int u = round * SR + (sidx >> kShiftK), sl = sidx & ((1 << kShiftK) - 1);
             const bool real = u < n_union && 8 * sl < d_qk;
-            const uint4_t x = *reinterpret_cast<const uint4_t *>(k + (size_t)col_k[i] * d_qk + (real ? 8 * sl : 0));
-            stage_k[i] = real ? x : zero;
+            stage_k[i] = *reinterpret_cast<const uint4_t *>(k + (size_t)col_k[i] * d_qk + (real ? 8 * sl : 0));
         }
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int sidx = tid + i * kThreads;
             const int u = round * SR + (sidx >> kShiftV), sl = sidx & ((1 << kShiftV) - 1);
             const bool real = u < n_union && 8 * sl < d_v;
-            const uint4_t x = *reinterpret_cast<const uint4_t *>(v + (size_t)col_v[i] * d_v + (real ? 8 * sl : 0));
-            stage_v[i] = real ? x : zero;
+            stage_v[i] = *reinterpret_cast<const uint4_t *>(v + (size_t)col_v[i] * d_v + (real ? 8 * sl : 0));
         }
         if (tid < kRows * SS) stage_m = (unsigned)masks[round * kMaskWords + tid];
     };
-    auto commit = [&]() {  // the parked sub-round into LDS (rows past the union and slices past d as zeros)
+    // The parked sub-round `round` into LDS; rows past the union and slices past d as zeros, so the arithmetic
+    // never meets stale bits.
+    auto commit = [&](int round) {
+        const uint4_t zero = {0u, 0u, 0u, 0u};
 #pragma unroll
         for (int i = 0; i < NK; ++i) {
             const int sidx = tid + i * kThreads;
-            *reinterpret_cast<uint4_t *>(kbuf + (sidx >> kShiftK) * PITCH + 8 * (sidx & ((1 << kShiftK) - 1))) = stage_k[i];
+            const int u = sidx >> kShiftK, sl = sidx & ((1 << kShiftK) - 1);
+            const bool real = round * SR + u < n_union && 8 * sl < d_qk;
+            *reinterpret_cast<uint4_t *>(kbuf + u * PITCH + 8 * sl) = real ? stage_k[i] : zero;
         }
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int sidx = tid + i * kThreads;
-            *reinterpret_cast<uint4_t *>(vbuf + (sidx >> kShiftV) * PITCH + 8 * (sidx & ((1 << kShiftV) - 1))) = stage_v[i];
+            const int u = sidx >> kShiftV, sl = sidx & ((1 << kShiftV) - 1);
+            const bool real = round * SR + u < n_union && 8 * sl < d_v;
+            *reinterpret_cast<uint4_t *>(vbuf + u * PITCH + 8 * sl) = real ? stage_v[i] : zero;
         }
         if (tid < kRows * SS) maskbuf[tid] = stage_m;
     };
@@ -881,7 +887,7 @@ sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
 
     for (int round = 0; round < n_rounds; ++round) {
         if (round > 0) __syncthreads();  // every wave is done with the previous sub-round's rows and masks
-        commit();
+        commit(round);
         __syncthreads();
         if (round + 1 < n_rounds) fetch_rows(round + 1);  // in flight during the arithmetic below
         if (round + 2 < n_rounds) fetch_cols(round + 2);
