@@ -277,6 +277,10 @@ def main():
 
     _, dense_attn_ms = time_graph(torch, dense_attention, 5, 2)
     attn_flops = 2.0 * amask.nnz * heads * dim * 2
+    # the same layer with a plain 513-wide window (unions of up to 634 columns per 16 vector rows)
+    wmask = cv.band_strided_pattern(seq, 8, band_half_width=256, stride=seq)
+    wlayer = ops.SparseAttention(wmask)
+    _, window_ms = time_graph(torch, lambda: wlayer.forward(q, kk_, vv, out=ctx), attn_steps, 3)
 
     cold_ms = time_cold(torch, step)
     cold_dense_ms = time_cold(torch, lambda: torch.matmul(Ad, Bd, out=dense_out))
@@ -311,6 +315,8 @@ def main():
             "speedup_vs_dense_gemm": dense_ms / ev_ms,
             "cold_cache_launch_us": cold_ms * 1e3,
             "cold_cache_dense_gemm_us": cold_dense_ms * 1e3,
+            "attention_window513": {"layer_ms": window_ms, "density": 1.0 - wmask.sparsity,
+                                    "tflops": 2.0 * wmask.nnz * heads * dim * 2 / (window_ms * 1e-3) * 1e-12},
             "attention_config5": {"layer_ms": attn_ms, "density": 1.0 - amask.sparsity,
                                   "tflops": attn_flops / (attn_ms * 1e-3) * 1e-12,
                                   "dense_masked_attention_ms": dense_attn_ms,
