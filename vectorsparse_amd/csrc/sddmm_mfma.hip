@@ -277,7 +277,7 @@ static int launch_one(int m_vec, int k, int nonzeros_vec, const int *row_indices
             return (int)hipGetLastError();
         }
     }
-    const int slots = sddmm_auto_slots(m_vec * batch.count, nonzeros_vec * batch.count, 16 * GRP);
+    const int slots = sddmm_auto_slots((long long)m_vec * batch.count, (long long)nonzeros_vec * batch.count, 16 * GRP);
     const long long waves = (long long)m_vec * slots;
     const long long blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
@@ -304,15 +304,16 @@ static int launch_ks(int m_vec, int k, int nonzeros_vec, const int *row_indices,
 // capped so that the launch stays near the number of wave slots of the chip.  A wave that finds no
 // super-group of its own exits after two scalar loads; what it costs is its share of a workgroup
 // dispatch, which is why workgroups are eight waves wide.
-int sddmm_auto_slots(int m_vec, int nonzeros_vec, int group)
+int sddmm_auto_slots(long long m_vec, long long nonzeros_vec, int group)
 {
     int slots = options().sddmm_slots;
     if (slots > 0) return slots;
-    const long long avg = ((long long)nonzeros_vec + m_vec - 1) / (m_vec > 0 ? m_vec : 1);
-    const int avg_groups = (int)((avg + group - 1) / group);
-    const int want = ceil_div(8192, m_vec > 0 ? m_vec : 1);
-    slots = 2 * avg_groups < want ? 2 * avg_groups : want;
-    return slots < 1 ? 1 : slots;
+    if (m_vec < 1) m_vec = 1;
+    const long long avg = (nonzeros_vec + m_vec - 1) / m_vec;
+    const long long avg_groups = (avg + group - 1) / group;
+    const long long want = (8192 + m_vec - 1) / m_vec;
+    const long long pick = 2 * avg_groups < want ? 2 * avg_groups : want;
+    return pick < 1 ? 1 : (int)pick;
 }
 
 template <typename OutT>

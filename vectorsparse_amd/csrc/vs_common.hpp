@@ -212,7 +212,7 @@ inline hipError_t allow_large_lds(const void *kernel, int bytes, std::atomic<uns
 }
 
 // Waves per vector row for the SDDMM kernels; `group` = nonzero vectors a wave covers per step.
-int sddmm_auto_slots(int m_vec, int nonzeros_vec, int group);
+int sddmm_auto_slots(long long m_vec, long long nonzeros_vec, int group);  // rows and nonzero vectors of the whole batch
 
 // Batched launches: problem b of `count` uses operand pointers advanced by b * stride (in elements);
 // the sparsity pattern (row_indices, row_offsets, column indices) is shared by the whole batch.
