@@ -224,7 +224,7 @@ def main():
             for _ in range(10):
                 layer.forward(q, kk_, vv, out=ctx)
             info["algorithmic_bytes"] = 4 * heads * seq * dim * 2      # q, k, v read once, out written once
-            info["rows_per_workgroup"] = layer.union_rows(dim, dim)
+            info["rows_per_workgroup"] = layer.union_rows(dim, dim, heads)
             info["nonzero_vectors"] = int(amask.nnz_vec)
         torch.cuda.synchronize()
         print(json.dumps(info))

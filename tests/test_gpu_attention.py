@@ -134,7 +134,7 @@ def test_softmax_fused_into_spmm(gpu, V, N):
 
 
 def test_fused_and_unfused_layers_agree(gpu):
-    V, heads, seq, d = 8, 4, 1024, 64
+    V, heads, seq, d = 8, 16, 1024, 64
     mask = cv.band_strided_pattern(seq, V, band_half_width=128, stride=128)
     layer = ops.SparseAttention(mask)
     g = torch.Generator(device="cuda").manual_seed(1)
@@ -144,11 +144,14 @@ def test_fused_and_unfused_layers_agree(gpu):
     rms = float(np.sqrt(np.mean(b * b)))
     assert float(np.max(np.abs(a - b))) <= 1e-2 * rms
     # the default: one launch where blocks of rows share their columns, two launches where they do not
-    assert layer.union_rows(d, d) >= 2
+    assert layer.union_rows(d, d, heads) == 128 // V
     assert torch.equal(layer.forward(q, k, v), layer.forward(q, k, v, fused="layer"))
     scattered = ops.SparseAttention(cv.uniform_pattern(seq // V, seq, 0.9, seed=2, vec_length=V))
-    assert scattered.union_rows(d, d) == 1
+    assert scattered.union_rows(d, d, heads) == 1
     assert torch.equal(scattered.forward(q, k, v), scattered.forward(q, k, v, fused=True))
+    # few heads: a launch of few workgroups is as long as its longest workgroup, and the two launches win
+    assert layer.union_rows(d, d, 2) == 1
+    assert torch.equal(layer.forward(q[:2], k[:2], v[:2]), layer.forward(q[:2], k[:2], v[:2], fused=True))
 
 
 def test_attention_steps_match_the_oracle_chain(gpu):
@@ -265,8 +268,8 @@ def test_union_gather_on_structured_and_random_masks(gpu, V):
             torch.cuda.synchronize()
             _check_layer(out.cpu().numpy(), ref, "%s mask V%d rows%d" % (name, V, rows))
             assert torch.equal(out, again)      # deterministic
-        planned = ops.SparseAttention(mask).union_rows(d, d)
-        assert (planned > 1) if name == "band" else (planned == 1)
+        if name == "band":
+            assert ops.SparseAttention(mask).union_rows(d, d) == 128 // V
 
 
 def _with_empty_rows(mask, first, last):
@@ -353,10 +356,11 @@ def test_planned_launch_streams_large_unions(gpu, V, seq, half_width, stride, di
         _check_layer(planned.cpu().numpy(), ref, "V%d scale %g streamed" % (V, scale))
         assert torch.equal(planned, again)
     layer = ops.SparseAttention(mask)
-    assert layer.union_rows(d_qk, d_v) == rows            # the host-side choice counts on the streamed kernel
-    out = layer.forward(qd, kd, vd, scale=0.125)
+    assert layer.union_rows(d_qk, d_v, 16) == rows        # the host-side choice counts on the streamed kernel
+    out = layer.forward(*(x.repeat(8, 1, 1) for x in (qd, kd, vd)), scale=0.125)     # sixteen heads
     torch.cuda.synchronize()
-    _check_layer(out.cpu().numpy(), _dense_attention(mask, q, k, v, 0.125), "V%d layer streamed" % V)
+    _check_layer(out[:2].cpu().numpy(), _dense_attention(mask, q, k, v, 0.125), "V%d layer streamed" % V)
+    assert torch.equal(out[:2], out[14:])
 
 
 @pytest.mark.parametrize("V", [1, 8])

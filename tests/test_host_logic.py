@@ -25,8 +25,11 @@ def test_attention_launch_shape_follows_the_mask():
     # every vector length fills its waves with 16 scalar rows
     for V in (1, 2, 4):
         assert rows_for(cv.band_strided_pattern(2048, V, band_half_width=128, stride=128), 64, 64) == 128 // V
-    # scattered columns: a dense tile over the union would be mostly masked out -> one row per workgroup
+    # a narrow band: the tile over the union is mostly masked out, yet the union is short
+    assert rows_for(cv.band_strided_pattern(4096, 8, band_half_width=4, stride=4096), 64, 64) == 16
+    # scattered columns: unions beyond the capacity -> the two launches
     scattered = cv.uniform_pattern(512, 4096, 0.9, seed=3, vec_length=8)
+    assert _largest_union(scattered, 16) > 2048
     assert rows_for(scattered, 64, 64) == 1
     # head widths the union kernel does not take
     assert rows_for(band, 64, 36) == 1
@@ -35,28 +38,24 @@ def test_attention_launch_shape_follows_the_mask():
     assert rows_for(empty, 64, 64) == 1
 
 
-def _moving_blocks(m_vec, n, V, rows_per_block, width=600, step=700):
-    """Every vector row holds `width` consecutive columns; the window jumps by `step` every rows_per_block rows."""
-    lengths = np.full(m_vec, width, dtype=np.int64)
-    offsets = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
-    cols = np.concatenate([np.arange(width) + step * ((r // rows_per_block) % 11) for r in range(m_vec)])
-    return cv.ColVecCSR(m_vec, n, V, offsets, cols.astype(np.int32)).validate()
-
-
-def test_small_workgroups_only_where_they_beat_the_per_row_kernel():
-    """Masks whose dense tile is full enough only over small blocks of rows: two waves are taken for V <= 4,
-    never for V = 8."""
+def test_attention_launch_shape_weighs_union_columns_against_nonzeros():
+    """The streamed kernel pays per union column, the two launches per nonzero (measured on MI355X, 16 heads x
+    4096: V = 8 uniform random masks switch between 99.5 % and 99.8 % sparsity, V = 1 takes the single launch
+    whenever 128 rows' columns fit), and a launch of few workgroups is as long as its longest workgroup."""
     rows_for = ops.SparseAttention._union_rows
-    # V = 4, the window jumps every 4 rows: tiles of 32 and 16 rows are 1/8 and 1/4 full, tiles of 8 rows (two
-    # waves) half full, and their 480 columns fit LDS at once
-    mask = _moving_blocks(256, 8192, 4, rows_per_block=4, width=240, step=300)
-    assert _largest_union(mask, 8) == 480
-    assert rows_for(mask, 64, 64) == 8
-    # V = 8, the window jumps every 2 rows: only tiles of 4 rows (two waves) would be full enough - but two
-    # waves lose to the per-row kernel at V = 8
-    mask = _moving_blocks(256, 8192, 8, rows_per_block=2, width=240, step=300)
-    assert _largest_union(mask, 4) == 480
-    assert rows_for(mask, 64, 64) == 1
+    for sparsity, want in ((0.98, 1), (0.99, 1), (0.998, 16)):
+        mask = cv.uniform_pattern(512, 4096, sparsity, seed=7, vec_length=8)
+        assert _largest_union(mask, 16) <= 2048
+        assert rows_for(mask, 64, 64) == want, sparsity
+    sparse_v1 = cv.uniform_pattern(4096, 4096, 0.998, seed=7, vec_length=1)
+    assert _largest_union(sparse_v1, 128) <= 2048 and rows_for(sparse_v1, 64, 64) == 128
+    # the same mask with 16 heads and with 2: 32 workgroups of 900 columns each lose to the two launches
+    small = cv.uniform_pattern(2048, 2048, 0.995, seed=7, vec_length=1)
+    assert rows_for(small, 64, 64, heads=64) == 128
+    assert rows_for(small, 64, 64, heads=2) == 1
+    # wider heads run one workgroup per CU: the switch comes earlier
+    mask = cv.uniform_pattern(512, 4096, 0.995, seed=7, vec_length=8)
+    assert rows_for(mask, 128, 128) == 1
 
 
 def test_device_problem_reads_the_row_statistics():

@@ -257,61 +257,75 @@ class SparseAttention:
         self._plans = {}
         self._rows = {}
 
-    def union_rows(self, d_qk, d_v):
-        """Rows per workgroup for the single-launch kernel with these head widths (cached per shape)."""
-        key = (int(d_qk), int(d_v))
+    def union_rows(self, d_qk, d_v, heads=16):
+        """Rows per workgroup for the single-launch kernel with these head widths and head count (cached)."""
+        key = (int(d_qk), int(d_v), int(heads))
         if key not in self._rows:
             self._rows[key] = self._union_rows(self.mask, *key)
         return self._rows[key]
 
-    def plan(self, d_qk, d_v):
+    def plan(self, d_qk, d_v, heads=16):
         """Device plan of the union kernel for these head widths (built on first use), or None."""
-        key = (int(d_qk), int(d_v))
-        rows = self.union_rows(*key)
+        rows = self.union_rows(d_qk, d_v, heads)
         if rows < 2:
             return None
+        key = (int(d_qk), int(d_v), rows)
         if key not in self._plans:
             p = self.prob
             self._plans[key] = sparse_attention_plan(p.m_vec, p.vec_length, p.n, key[0], key[1], rows,
                                                      p.row_offsets, p.column_indices)
         return self._plans[key]
 
-    @staticmethod
-    def _union_rows(mask, d_qk, d_v, min_fill=0.4):
-        """Vector rows per workgroup for the single-launch kernel: the largest block of consecutive rows
-        whose distinct columns stay within the library's capacity for this shape (with a plan) in every block
-        and whose dense tile (rows x union) is at least `min_fill` full (banded, blocky or strided masks),
-        else 1 (one row per workgroup, any mask).
+    # Cost model of the row choice below, in us per layer, fitted on MI355X (2..64 heads x 1024..16384 rows, band,
+    # band + strided and uniform random masks of 8..960 nonzero vectors per row).  A streamed workgroup (128
+    # scalar rows) alone on its CU takes 3.5 + 0.0235 * (union columns), two sharing a CU 7 + 0.04 * columns
+    # each; heads wider than 64 run one workgroup per CU at 6 + 0.037 * columns.  SDDMM followed by the
+    # softmax-fused SpMM takes 6 us plus, per 16 heads, a per vector row and b per nonzero vector (ns, by vector
+    # length; 1.3 a and 1.7 b for the wider heads).
+    _TWO_LAUNCH_NS = {8: (19.5, 0.35), 4: (15.6, 0.29), 2: (13.2, 0.25), 1: (12.0, 0.22)}
 
-        Every workgroup gathers its whole union, so small workgroups pay the gather for few rows: measured
-        on MI355X (16 heads, 4096 x 4096 band + strided masks whose unions only fit small blocks) two waves
-        beat the per-row kernel only for V <= 4 (132 us against 165 us at V = 4, 133 us against 99 us at
-        V = 8) and a single wave only for V = 1 (385 us against 481 us)."""
+    @staticmethod
+    def _union_rows(mask, d_qk, d_v, heads=16):
+        """Vector rows per workgroup for the single-launch kernel: workgroups of eight waves (128 scalar rows,
+        which stream the union of their columns through LDS) when every block's distinct columns stay within
+        the library's capacity for this shape and the cost model above puts the launch below the two-launch
+        path, else 1 (the two launches, any mask).
+
+        The streamed kernel pays per union column, the two launches per nonzero: measured (us per layer, 16
+        heads x 4096, d = 64) a +-4 band takes 12.5 against 18.6 (V = 8) and 12.7 against 63.7 (V = 1), a
+        uniform random mask at 99.8 % sparsity 10.8 against 17.8, at 99.5 % 20.8 against 19.3, at 98 % 54.8
+        against 31.3 (V = 8).  A launch of few workgroups is bound by the longest of them (2 heads x 2048,
+        V = 1, 98 % random: 47.9 us streamed against 10.6 us), hence the head count.  Smaller workgroups (the
+        kernel that holds the union at once) were slower than eight waves on every mask where both apply
+        (+-4 .. +-64 bands: four waves 17.6 .. 27.1 us, eight waves 12.5 .. 15.3 us), so they are left to
+        callers that ask for them."""
         ro, ci = mask.row_offsets, mask.column_indices
         if mask.m_vec == 0 or mask.nnz_vec == 0:
             return 1
-        per_wave = 16 // mask.vec_length
-        min_waves = {1: 1, 2: 2, 4: 2, 8: 4}[mask.vec_length]
-        for waves in (8, 4, 2, 1):
-            if waves < min_waves:
-                break
-            used = ctypes.c_int(0)
-            cap = _lib.lib().vs_sparse_attention_union_capacity(mask.vec_length, mask.n, d_qk, d_v, waves * per_wave,
-                                                                1, ctypes.addressof(used))
-            rows = used.value
-            if cap <= 0 or rows != waves * per_wave:
-                continue
-            fits, tile = True, 0
-            for first in range(0, mask.m_vec, rows):
-                last = min(first + rows, mask.m_vec)
-                union = np.unique(ci[ro[first]:ro[last]]).size
-                if union > cap:
-                    fits = False
-                    break
-                tile += union * (last - first)
-            if fits and mask.nnz_vec >= min_fill * tile:
-                return rows
-        return 1
+        used = ctypes.c_int(0)
+        want = 128 // mask.vec_length
+        cap = _lib.lib().vs_sparse_attention_union_capacity(mask.vec_length, mask.n, d_qk, d_v, want, 1,
+                                                            ctypes.addressof(used))
+        rows = used.value
+        if cap <= 0 or rows != want:
+            return 1
+        unions = [np.unique(ci[ro[first]:ro[min(first + rows, mask.m_vec)]]).size
+                  for first in range(0, mask.m_vec, rows)]
+        longest = max(unions)
+        if longest > cap:
+            return 1
+        wide = d_qk > 64 or d_v > 64
+        if wide:
+            alone = 6.0 + 0.037 * longest
+            busy = sum(6.0 + 0.037 * u for u in unions) * heads / 256.0
+        else:
+            alone = 3.5 + 0.0235 * longest
+            busy = sum(7.0 + 0.04 * u for u in unions) * heads / 512.0
+        per_row, per_nonzero = SparseAttention._TWO_LAUNCH_NS[mask.vec_length]
+        if wide:
+            per_row, per_nonzero = 1.3 * per_row, 1.7 * per_nonzero
+        two_launches = 6.0 + (per_row * mask.m_vec + per_nonzero * mask.nnz_vec) * (heads / 16.0) * 1e-3
+        return rows if max(alone, busy) <= two_launches else 1
 
     def forward(self, q, k, v, scale=None, kernel="wmma", stream=None, scores=None, out=None, fused=None):
         """q, k, v: fp16 [heads, seq, d] on the device.  Returns fp16 [heads, seq, d].
@@ -335,12 +349,12 @@ class SparseAttention:
             if kernel != "wmma":
                 fused = False
             else:
-                fused = "layer" if self.union_rows(q.shape[2], v.shape[2]) >= 2 else True
+                fused = "layer" if self.union_rows(q.shape[2], v.shape[2], heads) >= 2 else True
         if fused == "layer":
             return sparse_attention(p.m_vec, p.vec_length, p.n, p.row_indices, p.row_offsets, p.column_indices,
                                     q, k, v, out=out, scale=scale, stream=stream,
-                                    rows_per_workgroup=self.union_rows(q.shape[2], v.shape[2]),
-                                    plan=self.plan(q.shape[2], v.shape[2]))
+                                    rows_per_workgroup=self.union_rows(q.shape[2], v.shape[2], heads),
+                                    plan=self.plan(q.shape[2], v.shape[2], heads))
         sddmm_batched(p.m_vec, d, p.n, p.nnz_vec, p.row_indices, p.row_offsets, p.column_indices, q, k, scores,
                       p.vec_length, kernel=kernel, stream=stream)
         if fused:
