@@ -36,7 +36,8 @@
 //      same order.  One more MFMA per step with an all-ones B operand yields the row sums of the rounded
 //      p in exactly the accumulator layout, so normalising needs no cross-lane traffic.
 // Planned launches of eight waves do not hold the union at once: sparse_attention_stream_kernel below runs
-// steps 2 (the copy) to C per sub-round of 128 ranks, the next sub-round's rows on their way meanwhile.
+// steps 2 (the copy) to C per sub-round of 128 ranks, the next sub-round's rows on their way meanwhile, with
+// the V rows transposed while they are copied (one transposition per workgroup instead of one per wave).
 #include "vs_common.hpp"
 
 namespace vs {
@@ -736,12 +737,37 @@ sparse_attention_union_kernel(int m_vec, int n, int d_qk, int d_v, int u_max,
     }
 }
 
-// Planned launches of eight waves stream the union through LDS in sub-rounds of kStreamRanks ranks, K and V
-// rows side by side: the rows, row masks and column numbers of the NEXT sub-round are requested before the
-// current one is computed and parked in registers meanwhile, so after the first sub-round no wave waits for
-// a gather.  A sub-round is short enough to keep its raw scores in registers: the K rows are read and
-// multiplied once, not twice.  Maximum and sums run across the sub-rounds as in flash attention, so a
+// Planned launches of eight waves stream the union through LDS in sub-rounds of kStreamRanks ranks, K rows
+// and V columns side by side: the rows, row masks and column numbers of the NEXT sub-round are requested
+// before the current one is computed and parked in registers meanwhile, so after the first sub-round no wave
+// waits for a gather.  A sub-round is short enough to keep its raw scores in registers: the K rows are read
+// and multiplied once, not twice.  Maximum and sums run across the sub-rounds as in flash attention, so a
 // workgroup takes unions of up to kStreamRounds * kStreamRanks columns.
+//
+// The kernel is bound by vector-ALU instructions (softmax arithmetic and operand shuffles), so two things
+// are kept out of the waves' inner loop.  The V rows of a sub-round go to LDS transposed, in the order the
+// P V MFMA wants its B operand - the transposition is done once per workgroup while the rows are written, not
+// once per wave while they are read.  And the mask enters the scores as the accumulators' start value (0 or
+// -inf), so neither the maximum nor the exponentials look at it again.
+constexpr int kStreamVPitch = kStreamRanks + 8;  // halves between consecutive V columns in LDS
+typedef int int2_t __attribute__((ext_vector_type(2)));
+
+// Where rank r of a sub-round sits inside a V column: lane (c, g) multiplies ranks 16u + 4g + e (u < 2,
+// e < 4) of a 32-rank step, which this order puts into 16 consecutive bytes.
+__device__ __forceinline__ int stream_v_slot(int r) { return (r & ~31) | (((r >> 2) & 3) << 3) | (((r >> 4) & 1) << 2) | (r & 3); }
+
+// First rank of pair `pair` (0 .. kStreamRanks / 2) in the order the threads take them: consecutive pairs differ
+// in the bits that choose the 32-bit word inside a 16-byte chunk (e bit 1, then u), so the 32 lanes of a
+// transposed write hit 32 different banks.
+__device__ __forceinline__ int stream_v_pair_rank(int pair)
+{
+    return ((pair & 1) << 1) | (((pair >> 1) & 1) << 4) | (((pair >> 2) & 3) << 2) | ((pair >> 4) << 5);
+}
+
+// Offset in halves of 8-rank chunk `chunk` of V column `col`; chunks are permuted by column so that neither
+// the transposed writes (lanes of a quad: columns 8 apart) nor the reads (lanes: columns CPL apart) collide.
+__device__ __forceinline__ int stream_v_offset(int col, int chunk) { return col * kStreamVPitch + ((chunk ^ ((col >> 3) & 7)) << 3); }
+
 template <int V, int KS, int CPL>
 __global__ void __launch_bounds__(512, union_wide(KS, CPL) ? 2 : 4)
 sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
@@ -756,7 +782,7 @@ sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
     v += blockIdx.y * stride_v;
     out += blockIdx.y * stride_out;
     constexpr int RPW = 16 / V;
-    constexpr int PITCH = union_pitch(KS, CPL);
+    constexpr int PITCH = 32 * KS + 8;                              // halves between consecutive K rows in LDS
     constexpr int SS = kStreamSteps;
     constexpr int SR = kStreamRanks;
     constexpr int kThreads = 512;
@@ -765,15 +791,15 @@ sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
     constexpr int kShiftK = KS == 1 ? 2 : (KS == 2 ? 3 : 4);        // 4 * KS slices of 8 halves per K row
     constexpr int kShiftV = CPL == 4 ? 3 : 4;                       // 2 * CPL slices per V row
     constexpr int NK = (SR << kShiftK) / kThreads;                  // 16-byte slices per thread and sub-round
-    constexpr int NV = (SR << kShiftV) / kThreads;
+    constexpr int NV = ((SR / 2) << kShiftV) / kThreads;            // pairs of V slices (two consecutive ranks)
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     extern __shared__ __align__(16) unsigned char smem[];
     unsigned *maskbuf = reinterpret_cast<unsigned *>(smem);        // [kRows][SS] masks of the sub-round in LDS
-    half_t *kbuf = reinterpret_cast<half_t *>(maskbuf + kRows * SS);
-    half_t *vbuf = kbuf + SR * PITCH;
+    half_t *kbuf = reinterpret_cast<half_t *>(maskbuf + kRows * SS);  // [SR][PITCH]
+    half_t *vbuf = kbuf + SR * PITCH;                                 // [16 * CPL columns][kStreamVPitch]
 
     int bx = blockIdx.x;
     if ((gridDim.x & 7) == 0) bx = (bx & 7) * (gridDim.x >> 3) + (bx >> 3);  // a run of row blocks per XCD
@@ -781,7 +807,7 @@ sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
     const int row_last = (row_first + kRows) < m_vec ? (row_first + kRows) : m_vec;
     const int c = lane & 15;
     const int g = lane >> 4;
-    const float s2 = scale * kLog2e;
+    float s2 = scale * kLog2e;
     const int col0 = c * CPL;
     const bool col_ok = col0 < d_v;
     const int col_off = col_ok ? col0 : 0;
@@ -796,10 +822,12 @@ sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
     const int *masks = rec + 4;
     const int *cols = rec + 4 + kStreamRounds * kMaskWords;
 
-    // What a thread fetches per sub-round: NK slices of K rows, NV slices of V rows (thread t takes slices
-    // t, t + 512, ...: consecutive threads read consecutive 16 bytes of a row) and one mask word.
-    int col_k[NK], col_v[NV];
-    uint4_t stage_k[NK], stage_v[NV];
+    // What a thread fetches per sub-round: NK slices of K rows (thread t takes slices t, t + 512, ...:
+    // consecutive threads read consecutive 16 bytes of a row), NV times the same slice of the V rows of two
+    // consecutive ranks, and one mask word.
+    int col_k[NK];
+    int2_t col_v[NV];
+    uint4_t stage_k[NK], stage_v[NV][2];
     unsigned stage_m = 0;
     // column numbers of sub-round `round` < kStreamRounds (the plan lists 0 past the union: row 0, unused), which
     // do not wait for the union's size
@@ -807,7 +835,8 @@ sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
 #pragma unroll
         for (int i = 0; i < NK; ++i) col_k[i] = cols[round * SR + ((tid + i * kThreads) >> kShiftK)];
 #pragma unroll
-        for (int i = 0; i < NV; ++i) col_v[i] = cols[round * SR + ((tid + i * kThreads) >> kShiftV)];
+        for (int i = 0; i < NV; ++i)
+            col_v[i] = *reinterpret_cast<const int2_t *>(cols + round * SR + stream_v_pair_rank((tid + i * kThreads) >> kShiftV));
     };
     // Requests only: nothing here reads what the loads return, so the wave goes on to the arithmetic at once.
     // Slices past the union or past d read the start of a valid row and are replaced by zeros in commit().
@@ -822,14 +851,16 @@ sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int sidx = tid + i * kThreads;
-            const int u = round * SR + (sidx >> kShiftV), sl = sidx & ((1 << kShiftV) - 1);
-            const bool real = u < n_union && 8 * sl < d_v;
-            stage_v[i] = *reinterpret_cast<const uint4_t *>(v + (size_t)col_v[i] * d_v + (real ? 8 * sl : 0));
+            const int u = round * SR + stream_v_pair_rank(sidx >> kShiftV), sl = sidx & ((1 << kShiftV) - 1);
+            const int off = (u < n_union && 8 * sl < d_v) ? 8 * sl : 0;
+            stage_v[i][0] = *reinterpret_cast<const uint4_t *>(v + (size_t)col_v[i][0] * d_v + off);
+            stage_v[i][1] = *reinterpret_cast<const uint4_t *>(v + (size_t)col_v[i][1] * d_v + off);
         }
         if (tid < kRows * SS) stage_m = (unsigned)masks[round * kMaskWords + tid];
     };
     // The parked sub-round `round` into LDS; rows past the union and slices past d as zeros, so the arithmetic
-    // never meets stale bits.
+    // never meets stale bits.  V goes in transposed: a thread holds 8 columns of two consecutive ranks and
+    // writes, per column, the two ranks as one 32-bit word.
     auto commit = [&](int round) {
         const uint4_t zero = {0u, 0u, 0u, 0u};
 #pragma unroll
@@ -842,9 +873,17 @@ sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int sidx = tid + i * kThreads;
-            const int u = sidx >> kShiftV, sl = sidx & ((1 << kShiftV) - 1);
-            const bool real = round * SR + u < n_union && 8 * sl < d_v;
-            *reinterpret_cast<uint4_t *>(vbuf + u * PITCH + 8 * sl) = real ? stage_v[i] : zero;
+            const int r0 = stream_v_pair_rank(sidx >> kShiftV), sl = sidx & ((1 << kShiftV) - 1);
+            const bool wide_enough = 8 * sl < d_v;
+            const uint4_t first = (wide_enough && round * SR + r0 < n_union) ? stage_v[i][0] : zero;
+            const uint4_t second = (wide_enough && round * SR + r0 + 1 < n_union) ? stage_v[i][1] : zero;
+            const int slot = stream_v_slot(r0);
+            half_t *dst = vbuf + stream_v_offset(8 * sl, slot >> 3) + (slot & 7);  // columns 8 sl .. 8 sl + 7 share their chunk order
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj) {
+                *reinterpret_cast<uint32_t *>(dst + (2 * jj) * kStreamVPitch) = pack_lo(first[jj], second[jj]);
+                *reinterpret_cast<uint32_t *>(dst + (2 * jj + 1) * kStreamVPitch) = pack_hi(first[jj], second[jj]);
+            }
         }
         if (tid < kRows * SS) maskbuf[tid] = stage_m;
     };
@@ -863,7 +902,15 @@ sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
     load_q16<KS>(qb, q, q_global, q_limit, d_qk, c, g);
     if (n_rounds > 0) fetch_rows(0);
     if (n_rounds > 1) fetch_cols(1);
-    const float s2a = __builtin_fabsf(s2);  // the maximum is tracked on raw dot products: a negative scale moves into Q
+    // The maximum is tracked on raw dot products and masked-out pairs are -inf before the scale is applied, so
+    // the scale the exponentials see must be positive: a negative one moves into Q, a zero one becomes Q = 0
+    // (every pair of the mask then weighs the same, which is what a zero scale means).
+    if (s2 == 0.f) {
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) qb[kk] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        s2 = 1.f;
+    }
+    const float s2a = __builtin_fabsf(s2);
     if (s2 < 0.f) {
 #pragma unroll
         for (int kk = 0; kk < KS; ++kk) {
@@ -875,7 +922,6 @@ sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
     }
     const unsigned *mrow = maskbuf + ((q_first + c) / V) * SS;
     const half_t *k_lane = kbuf + c * PITCH + 8 * g;
-    const half_t *v_lane = vbuf + 4 * g * PITCH + col_off;
     const float neg_inf = -__builtin_inff();
     constexpr unsigned kLaneBits = 0x000F000Fu;
     const half8_t ones = {1, 1, 1, 1, 1, 1, 1, 1};
@@ -894,9 +940,9 @@ sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
         const int n_here = (n_union - round * SR) < SR ? (n_union - round * SR) : SR;
         const int n_steps = (n_here + 31) >> 5;
 
-        // scores of the sub-round, kept raw; the maximum over the pairs the mask holds
+        // scores of the sub-round, kept raw, masked-out pairs -inf; their maximum
         float4_t sacc[SS][2];
-        unsigned act = 0, full = 0;
+        unsigned act = 0;
         float mx_raw = neg_inf;
 #pragma unroll
         for (int t = 0; t < SS; ++t) {
@@ -908,77 +954,57 @@ sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
                     const unsigned wg = word >> (4 * g);
                     half8_t a[2][KS];
                     load_k_step<KS, PITCH>(a, k_lane, t);
-                    scores_step<KS>(sacc[t], a, qb);
-                    if (__builtin_amdgcn_ballot_w64((wg & kLaneBits) != kLaneBits) == 0ull) {
-                        full |= 1u << t;
-#pragma unroll
-                        for (int u = 0; u < 2; ++u)
-                            mx_raw = fmaxf(fmaxf(mx_raw, fmaxf(sacc[t][u][0], sacc[t][u][1])),
-                                           fmaxf(sacc[t][u][2], sacc[t][u][3]));
-                    } else {
+                    if (__builtin_amdgcn_ballot_w64((wg & kLaneBits) != kLaneBits) != 0ull) {
 #pragma unroll
                         for (int u = 0; u < 2; ++u)
 #pragma unroll
-                            for (int e = 0; e < 4; ++e)
-                                mx_raw = fmaxf(mx_raw, select_bit(wg, 16 * u + e, sacc[t][u][e], neg_inf));
+                            for (int e = 0; e < 4; ++e) sacc[t][u][e] = select_bit(wg, 16 * u + e, 0.f, neg_inf);
+                    }
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) {
+#pragma unroll
+                        for (int kk = 0; kk < KS; ++kk)
+                            sacc[t][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u][kk], qb[kk], sacc[t][u], 0, 0, 0);
+                        mx_raw = fmaxf(fmaxf(mx_raw, fmaxf(sacc[t][u][0], sacc[t][u][1])), fmaxf(sacc[t][u][2], sacc[t][u][3]));
                     }
                 }
             }
         }
         act = __builtin_amdgcn_readfirstlane(act);
-        full = __builtin_amdgcn_readfirstlane(full);
         mx_raw = fmaxf(mx_raw, partner<16>(mx_raw));  // scalar row c lives in the four lanes (c, g = 0..3)
         mx_raw = fmaxf(mx_raw, partner<32>(mx_raw));
         const float mx_new = fmaxf(mx_run, mx_raw);
         const float neg_mx = mx_new == neg_inf ? 0.f : -(mx_new * s2a);
         if (round > 0) {
-            // bring what the earlier sub-rounds accumulated to the new maximum
+            // bring what the earlier sub-rounds accumulated to the new maximum, unless no row's maximum moved
             const float f = mx_new == neg_inf ? 1.f
                             : (mx_run == neg_inf ? 0.f : __builtin_amdgcn_exp2f((mx_run - mx_new) * s2a));
+            if (__builtin_amdgcn_ballot_w64(f != 1.f) != 0ull) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float fe = from_lane(f, (4 * g + e) & 15);  // accumulator register e of lane (c, g) is scalar row 4g + e
-                lacc[e] *= fe;
+                for (int e = 0; e < 4; ++e) {
+                    const float fe = from_lane(f, (4 * g + e) & 15);  // accumulator register e of lane (c, g) is scalar row 4g + e
+                    lacc[e] *= fe;
 #pragma unroll
-                for (int cc = 0; cc < CPL; ++cc) acc[cc][e] *= fe;
+                    for (int cc = 0; cc < CPL; ++cc) acc[cc][e] *= fe;
+                }
             }
         }
         mx_run = mx_new;
 
-        // probabilities (masked-out pairs exact zeros), then P V and the row sums
+        // probabilities (exp2(-inf) = 0 for masked-out pairs), then P V and the row sums
 #pragma unroll
         for (int t = 0; t < SS; ++t) {
             if ((act >> t) & 1u) {
                 half8_t p;
-                if ((full >> t) & 1u) {
 #pragma unroll
-                    for (int u = 0; u < 2; ++u)
+                for (int u = 0; u < 2; ++u)
 #pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            p[4 * u + e] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf(sacc[t][u][e], s2a, neg_mx));
-                } else {
-                    const unsigned wg = mrow[t] >> (4 * g);
+                    for (int e = 0; e < 4; ++e)
+                        p[4 * u + e] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf(sacc[t][u][e], s2a, neg_mx));
 #pragma unroll
-                    for (int u = 0; u < 2; ++u)
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const float bias = select_bit(wg, 16 * u + e, neg_mx, neg_inf);
-                            p[4 * u + e] = (half_t)__builtin_amdgcn_exp2f(__builtin_fmaf(sacc[t][u][e], s2a, bias));
-                        }
-                }
-                RowChunk<CPL> rows[8];
-#pragma unroll
-                for (int e = 0; e < 8; ++e) rows[e].load(v_lane + (32 * t + (e < 4 ? e : 12 + e)) * PITCH);
-#pragma unroll
-                for (int pp = 0; pp < CPL / 2; ++pp) {
-                    uint4_t even, odd;
-#pragma unroll
-                    for (int qq = 0; qq < 4; ++qq) {
-                        even[qq] = pack_lo(rows[2 * qq].dword(pp), rows[2 * qq + 1].dword(pp));
-                        odd[qq] = pack_hi(rows[2 * qq].dword(pp), rows[2 * qq + 1].dword(pp));
-                    }
-                    acc[2 * pp] = __builtin_amdgcn_mfma_f32_16x16x32_f16(p, __builtin_bit_cast(half8_t, even), acc[2 * pp], 0, 0, 0);
-                    acc[2 * pp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(p, __builtin_bit_cast(half8_t, odd), acc[2 * pp + 1], 0, 0, 0);
+                for (int cc = 0; cc < CPL; ++cc) {
+                    const half8_t b = *reinterpret_cast<const half8_t *>(vbuf + stream_v_offset(col_off + cc, 4 * t + g));
+                    acc[cc] = __builtin_amdgcn_mfma_f32_16x16x32_f16(p, b, acc[cc], 0, 0, 0);
                 }
                 lacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(p, ones, lacc, 0, 0, 0);
             }
@@ -1029,7 +1055,8 @@ static bool union_shape(UnionShape &s, int vec_length, int n, int d_qk, int d_v,
         s.rounds = kStreamRounds;
         s.steps = kStreamSteps;
         const size_t mask = (size_t)union_mask_words(s.rows, s.steps) * sizeof(unsigned);
-        s.lds = mask + 2 * (size_t)s.u_max * row_bytes;  // masks of one sub-round, K rows and V rows side by side
+        // masks of one sub-round, its K rows and its V columns (transposed) side by side
+        s.lds = mask + (size_t)s.u_max * (32 * ks + 8) * sizeof(half_t) + (size_t)16 * cpl * kStreamVPitch * sizeof(half_t);
         s.plan_lds = bitmaps + s.rounds * (mask + (size_t)s.u_max * sizeof(int));
         return s.plan_lds <= 160 * 1024;
     }
