@@ -141,6 +141,22 @@ def test_fp32_output_overload(gpu, kernel):
     assert_parity(got, _oracle(pat, B), "fp32 out " + kernel)
 
 
+@pytest.mark.parametrize("V", [1, 2, 4, 8])
+@pytest.mark.parametrize("kernel", ["wmma", "cuda"])
+def test_subnormal_values_keep_exact_products(gpu, kernel, V):
+    """fp16 subnormals times large rhs entries: every product is exact in fp32 (the host loop's arithmetic,
+    spmm_benchmark.cpp:79-81), so the fp32 output equals the count of nonzeros times 2^-10 exactly - on MFMA,
+    on v_fma_mix_f32 (V = 1) and on v_dot2_f32_f16 (V >= 2) alike; a path that flushed them would return zeros."""
+    pat = cv.uniform_pattern(16, 96, 0.5, seed=41, vec_length=V)
+    vals = np.full((pat.nnz_vec, V), 2.0 ** -20, dtype=np.float16)
+    pat = cv.ColVecCSR(pat.m_vec, pat.n, V, pat.row_offsets, pat.column_indices, vals)
+    B = np.full((96, 64), 1024.0, dtype=np.float16)
+    got = _run(pat, B, kernel, out_dtype=torch.float32)
+    want = np.repeat(np.diff(pat.row_offsets), V).astype(np.float32)[:, None] * np.float32(2.0 ** -10)
+    assert np.array_equal(got, np.broadcast_to(want, got.shape))
+    assert np.array_equal(_oracle(pat, B), got)
+
+
 def test_launch_shape_overrides_keep_parity(gpu):
     pat = cv.random_values(cv.binomial_pattern(16, 1024, 0.8, seed=31, vec_length=8), seed=32)
     B = cv.dense_uniform(1024, 256, seed=33)

@@ -1,8 +1,9 @@
 // Fine-grained SpMM on the fp16 vector ALU (replaces src/cuda_spmm.cu of the reference).
 //
 // A V x 1 vector times a gathered rhs row is a rank-1 update, not a dense contraction, so
-// this path keeps it on the vector ALU: one mixed-precision v_fma_mix_f32 per multiply-add
-// (fp16 operands, exact product, fp32 accumulate).  The reference rounds every product to fp16
+// this path keeps it on the vector ALU: mixed-precision multiply-adds with fp16 operands, exact
+// products and fp32 accumulation - v_fma_mix_f32 for V = 1, v_dot2_f32_f16 over pairs of
+// nonzeros for V >= 2 (half the instructions per multiply-add).  The reference rounds every product to fp16
 // first (src/spmm_utils/compute_utils.h:45); that rounding alone costs up to ~9e-2 of the
 // 1e-2 relative-error budget against the host loop on near-zero outputs, so it is not
 // reproduced.  Work item = (vector row, tile of TN = 8*LR dense columns); a wave is G = 64/LR groups
@@ -13,23 +14,22 @@
 
 namespace vs {
 
+// The V halves of one nonzero vector as 32-bit words, two halves per word (V = 1: the low half of one word).
 template <int V>
-__device__ __forceinline__ void load_values(half_t (&dst)[V], const half_t *p)
+__device__ __forceinline__ void load_values(uint32_t (&dst)[V > 1 ? V / 2 : 1], const half_t *p)
 {
     if constexpr (V == 8) {
-        const half8_t t = *reinterpret_cast<const half8_t *>(p);
+        const uint4_t t = *reinterpret_cast<const uint4_t *>(p);
 #pragma unroll
-        for (int v = 0; v < 8; ++v) dst[v] = t[v];
+        for (int i = 0; i < 4; ++i) dst[i] = t[i];
     } else if constexpr (V == 4) {
-        const half4_t t = *reinterpret_cast<const half4_t *>(p);
-#pragma unroll
-        for (int v = 0; v < 4; ++v) dst[v] = t[v];
-    } else if constexpr (V == 2) {
-        const half2_t t = *reinterpret_cast<const half2_t *>(p);
+        const uint2_t t = *reinterpret_cast<const uint2_t *>(p);
         dst[0] = t[0];
         dst[1] = t[1];
+    } else if constexpr (V == 2) {
+        dst[0] = *reinterpret_cast<const uint32_t *>(p);
     } else {
-        dst[0] = p[0];
+        dst[0] = *reinterpret_cast<const uint16_t *>(p);
     }
 }
 
@@ -70,7 +70,7 @@ spmm_valu_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
     constexpr int U = 4;
     for (int j0 = beg + (wave * G + g) * U; j0 < end; j0 += n_waves * G * U) {
         int col[U];
-        half_t a[U][V];
+        uint32_t a[U][V > 1 ? V / 2 : 1];  // the vector's halves, two per word (V = 1: one half in the low bits)
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int j = j0 + u;
@@ -80,18 +80,42 @@ spmm_valu_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
             load_values<V>(a[u], values + (size_t)jc * V);
             if (!valid) {
 #pragma unroll
-                for (int v = 0; v < V; ++v) a[u][v] = (half_t)0.f;
+                for (int i = 0; i < (V > 1 ? V / 2 : 1); ++i) a[u][i] = 0u;
             }
         }
-        half8_t b[U];
+        uint4_t b[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) b[u] = *reinterpret_cast<const half8_t *>(rhs_col + (size_t)col[u] * n_cols);
+        for (int u = 0; u < U; ++u) b[u] = *reinterpret_cast<const uint4_t *>(rhs_col + (size_t)col[u] * n_cols);
+        if constexpr (V == 1) {
+            // one multiply-add per column and nonzero: nothing to pair up
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
+            for (int u = 0; u < U; ++u) {
+                const float av = (float)__builtin_bit_cast(half2_t, a[u][0])[0];
+                const half8_t bu = __builtin_bit_cast(half8_t, b[u]);
 #pragma unroll
-            for (int v = 0; v < V; ++v) {
+                for (int c = 0; c < 8; ++c) acc[0][c] = __builtin_fmaf(av, (float)bu[c], acc[0][c]);
+            }
+        } else {
+            // Two nonzeros at a time on v_dot2_f32_f16 (two exact products and the accumulator summed in fp32 by
+            // one instruction): the values of the two vectors and the two gathered rows are interleaved with
+            // v_perm_b32 first - V + 8 shuffles buy 8 V instructions instead of 16 V.
 #pragma unroll
-                for (int c = 0; c < 8; ++c) acc[v][c] = __builtin_fmaf((float)a[u][v], (float)b[u][c], acc[v][c]);
+            for (int u = 0; u < U; u += 2) {
+                half2_t av[V], bv[8];
+#pragma unroll
+                for (int i = 0; i < V / 2; ++i) {
+                    av[2 * i] = __builtin_bit_cast(half2_t, pack_lo(a[u][i], a[u + 1][i]));
+                    av[2 * i + 1] = __builtin_bit_cast(half2_t, pack_hi(a[u][i], a[u + 1][i]));
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    bv[2 * i] = __builtin_bit_cast(half2_t, pack_lo(b[u][i], b[u + 1][i]));
+                    bv[2 * i + 1] = __builtin_bit_cast(half2_t, pack_hi(b[u][i], b[u + 1][i]));
+                }
+#pragma unroll
+                for (int v = 0; v < V; ++v)
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) acc[v][c] = __builtin_amdgcn_fdot2(av[v], bv[c], acc[v][c], false);
             }
         }
     }
