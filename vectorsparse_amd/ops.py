@@ -246,9 +246,11 @@ def sparse_attention_plan(m_vec, vec_length, n, d_qk, d_v, rows_per_workgroup, r
 class SparseAttention:
     """One fixed-mask sparse attention layer: SDDMM (QK^T on the mask) -> row softmax -> SpMM (P V).
 
-    The mask is a column-vector CSR pattern over [seq, seq] shared by all heads; the three steps are
-    one batched launch each, chained on one stream with no host synchronisation and no re-layout (the
-    SDDMM output layout is the SpMM value layout).
+    The mask is a column-vector CSR pattern over [seq, seq] shared by all heads.  `forward` runs the layer as
+    one launch (scores and probabilities never leave the chip), as two (SDDMM, then the SpMM with the softmax
+    folded in) or as the three operators, one batched launch each, chained on one stream with no host
+    synchronisation and no re-layout (the SDDMM output layout is the SpMM value layout); by default it
+    picks the faster of the first two for the mask, the head widths and the head count.
     """
 
     def __init__(self, mask, device="cuda", sort=True):
@@ -332,10 +334,11 @@ class SparseAttention:
 
         fused: "layer" runs the whole layer in one launch with scores and probabilities kept in LDS; True
         folds only the softmax into the SpMM launch (two launches, raw scores go through memory); False runs
-        the three operators one after the other.  Default on the MFMA path: "layer" when the mask lets blocks
-        of rows share their columns (the union kernel: 2-3x faster than the alternatives), else True - on
-        masks without such structure the single launch gathers K / V rows per row and is 10-60 % slower
-        than the two launches (16 heads x 4096, uniform random masks, 90-98 % sparse, V = 1..8).
+        the three operators one after the other.  Default on the MFMA path: "layer" when the cost model of
+        `_union_rows` puts the streamed union kernel ahead (banded, blocky, strided and very sparse masks: 1.5-15x
+        faster than the alternatives), else True - on masks without shared columns the single launch gathers
+        K / V rows per row and is 10-60 % slower than the two launches (16 heads x 4096, uniform random masks,
+        90-98 % sparse, V = 1..8).
         """
         p = self.prob
         heads, seq, d = q.shape
