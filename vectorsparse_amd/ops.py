@@ -24,8 +24,15 @@ def _ptr(t):
     return t.data_ptr()
 
 
+# torch's raw-handle getter when this torch has it: torch.cuda.current_stream() builds a Stream object per call
+# (2.8 us on the host against 0.1 us, measured; an eager SpMM launch is 3.8 us of GPU time)
+_raw_current_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(stream):
     if stream is None:
+        if _raw_current_stream is not None:
+            return _raw_current_stream(torch.cuda.current_device())
         return torch.cuda.current_stream().cuda_stream
     if isinstance(stream, torch.cuda.Stream):
         return stream.cuda_stream
