@@ -40,46 +40,45 @@ def _stream(stream):
 
 
 def _expect(t, dtype, name):
-    if isinstance(t, torch.Tensor):
-        if t.dtype != dtype:
-            raise TypeError("%s must be %s, got %s" % (name, dtype, t.dtype))
-        if not t.is_cuda:
-            raise ValueError("%s must live in device memory" % name)
-        if not t.is_contiguous():
-            raise ValueError("%s must be contiguous" % name)
+    """Type / placement / layout check of a tensor argument; returns its device address (raw addresses pass)."""
+    if t is None or type(t) is int:
+        return t
+    if t.dtype is not dtype:
+        raise TypeError("%s must be %s, got %s" % (name, dtype, t.dtype))
+    if not t.is_cuda:
+        raise ValueError("%s must live in device memory" % name)
+    if not t.is_contiguous():
+        raise ValueError("%s must be contiguous" % name)
+    return t.data_ptr()
 
 
 def _spmm(entry, m_vec, vec_length, k, n, row_indices, row_offsets, column_indices, values, rhs_matrix,
           output_matrix, stream):
-    for t, nm in ((row_indices, "row_indices"), (row_offsets, "row_offsets"), (column_indices, "column_indices")):
-        _expect(t, torch.int32, nm)
-    _expect(values, torch.float16, "values")
-    _expect(rhs_matrix, torch.float16, "rhs_matrix")
-    f32 = isinstance(output_matrix, torch.Tensor) and output_matrix.dtype == torch.float32
-    if not f32:
-        _expect(output_matrix, torch.float16, "output_matrix")
-    fn = getattr(_lib.lib(), entry + ("_f32out" if f32 else ""))
-    st = fn(m_vec, vec_length, k, n, _ptr(row_indices), _ptr(row_offsets), _ptr(column_indices), _ptr(values),
-            _ptr(rhs_matrix), _ptr(output_matrix), _stream(stream))
-    _lib.check(st, entry)
+    f32 = isinstance(output_matrix, torch.Tensor) and output_matrix.dtype is torch.float32
+    fn = getattr(_lib.lib(), entry + "_f32out" if f32 else entry)
+    st = fn(m_vec, vec_length, k, n, _expect(row_indices, torch.int32, "row_indices"),
+            _expect(row_offsets, torch.int32, "row_offsets"), _expect(column_indices, torch.int32, "column_indices"),
+            _expect(values, torch.float16, "values"), _expect(rhs_matrix, torch.float16, "rhs_matrix"),
+            _expect(output_matrix, torch.float32 if f32 else torch.float16, "output_matrix"), _stream(stream))
+    if st:
+        _lib.check(st, entry)
     return output_matrix
 
 
 def _sddmm(entry, m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices, lhs_matrix, rhs_matrix,
            output_values, vec_length, stream, algorithm=None):
-    for t, nm in ((row_indices, "row_indices"), (row_offsets, "row_offsets"), (col_indices, "col_indices")):
-        _expect(t, torch.int32, nm)
-    _expect(lhs_matrix, torch.float16, "lhs_matrix")
-    _expect(rhs_matrix, torch.float16, "rhs_matrix")
-    f32 = isinstance(output_values, torch.Tensor) and output_values.dtype == torch.float32
-    if not f32:
-        _expect(output_values, torch.float16, "output_values")
-    fn = getattr(_lib.lib(), entry + ("_f32out" if f32 else ""))
-    args = [m_vec, k, n, nonzeros_vec, _ptr(row_indices), _ptr(row_offsets), _ptr(col_indices), _ptr(lhs_matrix),
-            _ptr(rhs_matrix), _ptr(output_values), vec_length, _stream(stream)]
+    f32 = isinstance(output_values, torch.Tensor) and output_values.dtype is torch.float32
+    fn = getattr(_lib.lib(), entry + "_f32out" if f32 else entry)
+    args = [m_vec, k, n, nonzeros_vec, _expect(row_indices, torch.int32, "row_indices"),
+            _expect(row_offsets, torch.int32, "row_offsets"), _expect(col_indices, torch.int32, "col_indices"),
+            _expect(lhs_matrix, torch.float16, "lhs_matrix"), _expect(rhs_matrix, torch.float16, "rhs_matrix"),
+            _expect(output_values, torch.float32 if f32 else torch.float16, "output_values"), vec_length,
+            _stream(stream)]
     if algorithm is not None:
         args.append(algorithm)
-    _lib.check(fn(*args), entry)
+    st = fn(*args)
+    if st:
+        _lib.check(st, entry)
     return output_values
 
 
