@@ -17,7 +17,8 @@
  *
  * Conventions shared by all device entry points
  *   - all array pointers are DEVICE pointers owned by the caller; nothing is
- *     retained after return; no workspace; no allocation inside the library;
+ *     retained after return; no allocation inside the library; no workspace
+ *     except where an entry point takes one as an argument;
  *   - the output is fully overwritten (alpha = 1, beta = 0), including the
  *     rows of empty vector rows, and nothing outside it is written;
  *   - the launch is asynchronous on `stream` (a hipStream_t; NULL = default
@@ -65,6 +66,33 @@ int vs_wmma_spmm_f16_f32out(int m_vec, int vec_length, int k, int n,
                             const int *row_indices, const int *row_offsets,
                             const int *column_indices, const void *values,
                             const void *rhs_matrix, float *output_matrix, void *stream);
+
+/*
+ * The same operator (spmm::wmmaSpmm, include/wmma_spmm.cuh:15-21 and :7-13) on a schedule that balances
+ * skewed row lengths across the whole chip, which the reference's SortedRowSwizzle
+ * (include/bm_test_utils.h:200-215) only approximates by reordering whole rows: the nonzero range is cut
+ * into equal runs, one wave per (run, column tile) and sixteen runs per workgroup; a row that crosses run
+ * boundaries is computed in segments whose fp32 partial tiles are added in ascending order - inside a
+ * workgroup through LDS, across workgroups through `workspace` by a second launch (no atomics; deterministic; the result does not depend on row_indices, which may be null and is ignored).
+ * nonzeros_vec must equal row_offsets[m_vec] (the host cannot read it from device memory).
+ * workspace: device memory, 16-byte aligned, workspace_bytes long, owned by the caller, contents undefined
+ * before and after, not shared between calls that may overlap.  vs_wmma_spmm_workspace_bytes() returns the
+ * size that lets the library pick its preferred run length (0 when one workgroup takes everything); a smaller
+ * workspace - even none - is accepted and makes the runs longer (fewer waves, same results up to the
+ * order of the fp32 summation).  Other requirements as vs_wmma_spmm_f16.  Faster than vs_wmma_spmm_f16 when
+ * a few rows hold a large share of the nonzeros; slower on uniform rows.
+ */
+long long vs_wmma_spmm_workspace_bytes(int m_vec, int vec_length, int k, int n, int nonzeros_vec);
+int vs_wmma_spmm_f16_ws(int m_vec, int vec_length, int k, int n, int nonzeros_vec,
+                        const int *row_indices, const int *row_offsets,
+                        const int *column_indices, const void *values,
+                        const void *rhs_matrix, void *output_matrix,
+                        void *workspace, long long workspace_bytes, void *stream);
+int vs_wmma_spmm_f16_f32out_ws(int m_vec, int vec_length, int k, int n, int nonzeros_vec,
+                               const int *row_indices, const int *row_offsets,
+                               const int *column_indices, const void *values,
+                               const void *rhs_matrix, float *output_matrix,
+                               void *workspace, long long workspace_bytes, void *stream);
 
 /*
  * Replaces spmm::cudaSpmm(half in, half out) — include/cuda_spmm.cuh:15-21,
@@ -284,7 +312,9 @@ void vs_sorted_row_swizzle(int rows, const int *row_offsets, int *row_indices);
 /*
  * Launch-shape tuning knob (process-wide, not thread-safe against concurrent
  * launches).  Names: "spmm_waves" (waves per workgroup, 0 = automatic),
- * "spmm_cols_per_lane" (4, 8, 0 = automatic), "sddmm_slots" (waves per
+ * "spmm_cols_per_lane" (4, 8, 0 = automatic), "spmm_flat_piece" (nonzero vectors
+ * per wave of the split-row SpMM, rounded up to 32, 0 = automatic), "spmm_flat_waves"
+ * (its waves per workgroup, 1..16, 0 = automatic), "sddmm_slots" (waves per
  * vector row, 0 = automatic), "sddmm_block_waves" (1..16, 0 = automatic),
  * "sddmm_flat_supers" (super-groups per wave of algorithm 2, 1..16, 0 = automatic),
  * "attention_waves" (1..8, 0 = automatic), "attention_chunk" (nonzero vectors per

@@ -13,8 +13,8 @@ EXE = os.path.join(ROOT, "tests", "cxx", "reference_call_sites")
 
 
 def test_cxx_program_through_the_shim(gpu):
-    if not os.path.exists(EXE):
-        pytest.skip("tests/cxx/reference_call_sites is not built (python -m vectorsparse_amd.build)")
+    # a missing executable is a failure, not a skip: it is the only C++-caller evidence for the shim
+    assert os.path.exists(EXE), "tests/cxx/reference_call_sites is not built (python -m vectorsparse_amd.build)"
     proc = subprocess.run([EXE], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
     print(proc.stdout)
     assert proc.returncode == 0, proc.stdout

@@ -216,3 +216,16 @@ def test_algorithm_2_batched_equals_unbatched(gpu):
         one = prob.sddmm(A[h], B[h], algorithm=1)
         torch.cuda.synchronize()
         assert torch.equal(out[h], one), "head %d" % h
+
+
+@pytest.mark.parametrize("kernel", ["wmma", "cuda"])
+@pytest.mark.parametrize("out_dtype", [torch.float16, torch.float32])
+def test_empty_contraction_writes_zeros(gpu, kernel, out_dtype):
+    # k == 0: every sampled output is an empty sum (Host_sddmm, include/bm_test_utils.h:171-193, leaves 0)
+    pat = cv.binomial_pattern(12, 80, 0.7, seed=3, vec_length=4)
+    A = np.zeros((pat.m, 0), dtype=np.float16)
+    B = np.zeros((80, 0), dtype=np.float16)
+    got = _run(pat, A, B, kernel, out_dtype=out_dtype)
+    assert got.shape == (pat.nnz,) and not got.any()
+    ref = co.sddmm_host_ref_f32(pat.m_vec, 0, 4, pat.row_offsets, pat.column_indices, A, B)
+    assert np.array_equal(ref, got.astype(np.float32))

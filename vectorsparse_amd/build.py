@@ -9,7 +9,8 @@ import sys
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_HERE, "libvsparse.so")
-SOURCES = ["vsparse_api.hip", "spmm_mfma.hip", "spmm_valu.hip", "sddmm_mfma.hip", "sddmm_valu.hip",
+OBJ_DIR = os.path.join(_HERE, "build")
+SOURCES = ["vsparse_api.hip", "spmm_mfma.hip", "spmm_mfma_flat.hip", "spmm_valu.hip", "sddmm_mfma.hip", "sddmm_valu.hip",
            "sparse_softmax.hip", "sparse_attention.hip",
            "sparse_attention_union.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -20,8 +21,7 @@ FLAGS = [
 ]
 
 
-def build(verbose=False):
-    cmd = [HIPCC] + FLAGS + ["-o", LIB_PATH] + [os.path.join(CSRC, s) for s in SOURCES]
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -32,6 +32,29 @@ def build(verbose=False):
         raise RuntimeError("hipcc failed:\n" + out)
     if verbose and out.strip():
         print(out)
+
+
+def _stale(src, obj):
+    if not os.path.exists(obj):
+        return True
+    newest = max(os.path.getmtime(p) for p in [src, os.path.join(CSRC, "vs_common.hpp"),
+                                               os.path.join(os.path.dirname(_HERE), "include", "vsparse.h")])
+    return os.path.getmtime(obj) < newest
+
+
+def build(verbose=False, jobs=None, incremental=False):
+    """Compile every source to an object (in parallel: the translation units are independent) and link.
+    incremental: recompile only the sources that are newer than their objects (or whose shared headers are)."""
+    from concurrent.futures import ThreadPoolExecutor
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    compile_flags = [f for f in FLAGS if f != "-shared"]
+    objects = [os.path.join(OBJ_DIR, s.replace(".hip", ".o")) for s in SOURCES]
+    cmds = [[HIPCC] + compile_flags + ["-c", os.path.join(CSRC, s), "-o", o] for s, o in zip(SOURCES, objects)
+            if not incremental or _stale(os.path.join(CSRC, s), o)]
+    jobs = jobs or max(1, min(len(cmds), os.cpu_count() or 1, 16))
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        list(pool.map(lambda c: _run(c, verbose), cmds))
+    _run([HIPCC, "--offload-arch=gfx950", "-fPIC", "-shared", "-o", LIB_PATH] + objects, verbose)
     return LIB_PATH
 
 
@@ -52,6 +75,6 @@ def build_cxx_caller(verbose=False):
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    print(build(verbose=True, incremental="--incremental" in sys.argv))
     print(build_cxx_caller(verbose=True))
     sys.exit(0)

@@ -18,46 +18,10 @@
 //     with the sparse vectors as the 16 x 32 A operand (rows v >= V are zero).
 //   The accumulator of lane (cs, g), register e, MFMA c is out[4g + e][tile*TN + cs*CPL + c], i.e.
 //   CPL consecutive outputs per (lane, e): one vector store each.
+#include "spmm_mfma_step.hpp"
 #include "vs_common.hpp"
 
 namespace vs {
-
-// The V halves of one nonzero vector, fetched with one load.
-template <int V>
-__device__ __forceinline__ void load_vector(half_t (&dst)[V], const half_t *p)
-{
-    if constexpr (V == 8) {
-        const half8_t t = *reinterpret_cast<const half8_t *>(p);
-#pragma unroll
-        for (int v = 0; v < 8; ++v) dst[v] = t[v];
-    } else if constexpr (V == 4) {
-        const half4_t t = *reinterpret_cast<const half4_t *>(p);
-#pragma unroll
-        for (int v = 0; v < 4; ++v) dst[v] = t[v];
-    } else if constexpr (V == 2) {
-        const half2_t t = *reinterpret_cast<const half2_t *>(p);
-        dst[0] = t[0];
-        dst[1] = t[1];
-    } else {
-        dst[0] = p[0];
-    }
-}
-
-__device__ __forceinline__ void wave_lds_fence()
-{
-    // LDS operations of one wave execute in order; this only stops the compiler from moving
-    // LDS accesses of different lanes' data across the hand-off point.
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-}
-
-constexpr int kStep = 32;  // nonzero vectors per MFMA step
-
-template <int V>
-constexpr int stage_bytes()
-{
-    return kStep * (int)sizeof(int) + V * kStep * (int)sizeof(half_t);  // indices + transposed vectors
-}
 
 // SOFTMAX: the sparse values are raw scores and the kernel multiplies by softmax_row(scale * values)
 // instead: a pre-pass finds each scalar row's maximum, the staging step turns every score into
@@ -161,37 +125,9 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
             }
         }
         wave_lds_fence();
-        const int4_t i_lo = *reinterpret_cast<const int4_t *>(idx_s + 8 * g);
-        const int4_t i_hi = *reinterpret_cast<const int4_t *>(idx_s + 8 * g + 4);
-        half8_t a = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (cs < V) a = *reinterpret_cast<const half8_t *>(vec_s + cs * kStep + 8 * g);
-        wave_lds_fence();
-
-        RowChunk<CPL> chunk[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int col = e < 4 ? i_lo[e] : i_hi[e - 4];
-            if constexpr (IDX32) {
-                // rhs has fewer than 2^31 elements: 32-bit offsets from a uniform base
-                chunk[e].load(rhs + ((uint32_t)col * (uint32_t)n_cols + col_off));
-            } else {
-                chunk[e].load(rhs + ((size_t)col * n_cols + col_off));
-            }
-        }
-        if (base + stride < end) fetch(base + stride);
-#pragma unroll
-        for (int p = 0; p < CPL / 2; ++p) {
-            uint4_t even, odd;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                even[q] = pack_lo(chunk[2 * q].dword(p), chunk[2 * q + 1].dword(p));
-                odd[q] = pack_hi(chunk[2 * q].dword(p), chunk[2 * q + 1].dword(p));
-            }
-            const half8_t b_even = __builtin_bit_cast(half8_t, even);
-            const half8_t b_odd = __builtin_bit_cast(half8_t, odd);
-            acc[2 * p] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b_even, acc[2 * p], 0, 0, 0);
-            acc[2 * p + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b_odd, acc[2 * p + 1], 0, 0, 0);
-        }
+        spmm_mfma_step<V, CPL, IDX32>(idx_s, vec_s, rhs, n_cols, col_off, cs, g, acc, [&] {
+            if (base + stride < end) fetch(base + stride);
+        });
     }
 
     if constexpr (SOFTMAX) {

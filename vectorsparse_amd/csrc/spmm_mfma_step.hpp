@@ -1,0 +1,133 @@
+// One 32-vector step of the SpMM tile loop on fp16 MFMA, shared by the row-per-workgroup kernel and the
+// kernel that splits the nonzero range (src/wmma_spmm.cu:77-90 of the reference is the loop this replaces).
+#pragma once
+#include "vs_common.hpp"
+
+namespace vs {
+
+constexpr int kStep = 32;  // nonzero vectors per MFMA step
+
+// Wave-private staging slot in LDS: 32 column indices, then the 32 vectors transposed to [v][nonzero].
+template <int V>
+constexpr int stage_bytes()
+{
+    return kStep * (int)sizeof(int) + V * kStep * (int)sizeof(half_t);
+}
+
+// The V halves of one nonzero vector, fetched with one load.
+template <int V>
+__device__ __forceinline__ void load_vector(half_t (&dst)[V], const half_t *p)
+{
+    if constexpr (V == 8) {
+        const half8_t t = *reinterpret_cast<const half8_t *>(p);
+#pragma unroll
+        for (int v = 0; v < 8; ++v) dst[v] = t[v];
+    } else if constexpr (V == 4) {
+        const half4_t t = *reinterpret_cast<const half4_t *>(p);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) dst[v] = t[v];
+    } else if constexpr (V == 2) {
+        const half2_t t = *reinterpret_cast<const half2_t *>(p);
+        dst[0] = t[0];
+        dst[1] = t[1];
+    } else {
+        dst[0] = p[0];
+    }
+}
+
+__device__ __forceinline__ void wave_lds_fence()
+{
+    // LDS operations of one wave execute in order; this only stops the compiler from moving
+    // LDS accesses of different lanes' data across the hand-off point.
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+// Consumes the staged step: lane (cs = lane % 16, g = lane / 16) reads its eight column indices and its
+// slice of the transposed vectors from the wave's slot, gathers CPL consecutive halves of the eight rhs rows
+// at column offset `col_off` (element offset of the lane's first column inside a row), calls `prefetch()`
+// with those loads in flight, transposes the CPL x 8 block with v_perm_b32 and issues CPL MFMAs:
+// acc[c][e] += sum_j vec[4g + e][j] * rhs[col_j][col_off + c].
+template <int V, int CPL, bool IDX32, typename Prefetch>
+__device__ __forceinline__ void spmm_mfma_step(const int *idx_s, const half_t *vec_s, const half_t *rhs, int n_cols,
+                                               uint32_t col_off, int cs, int g, float4_t (&acc)[CPL],
+                                               Prefetch &&prefetch)
+{
+    const int4_t i_lo = *reinterpret_cast<const int4_t *>(idx_s + 8 * g);
+    const int4_t i_hi = *reinterpret_cast<const int4_t *>(idx_s + 8 * g + 4);
+    half8_t a = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (cs < V) a = *reinterpret_cast<const half8_t *>(vec_s + cs * kStep + 8 * g);
+    wave_lds_fence();
+
+    RowChunk<CPL> chunk[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const int col = e < 4 ? i_lo[e] : i_hi[e - 4];
+        if constexpr (IDX32) {
+            // rhs has fewer than 2^31 elements: 32-bit offsets from a uniform base
+            chunk[e].load(rhs + ((uint32_t)col * (uint32_t)n_cols + col_off));
+        } else {
+            chunk[e].load(rhs + ((size_t)col * n_cols + col_off));
+        }
+    }
+    prefetch();
+#pragma unroll
+    for (int p = 0; p < CPL / 2; ++p) {
+        uint4_t even, odd;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            even[q] = pack_lo(chunk[2 * q].dword(p), chunk[2 * q + 1].dword(p));
+            odd[q] = pack_hi(chunk[2 * q].dword(p), chunk[2 * q + 1].dword(p));
+        }
+        const half8_t b_even = __builtin_bit_cast(half8_t, even);
+        const half8_t b_odd = __builtin_bit_cast(half8_t, odd);
+        acc[2 * p] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b_even, acc[2 * p], 0, 0, 0);
+        acc[2 * p + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b_odd, acc[2 * p + 1], 0, 0, 0);
+    }
+}
+
+// Last index i in [0, rows] with offsets[i] <= pos (of equal offsets, i.e. empty rows, the last one): the row
+// that holds nonzero `pos` when pos < offsets[rows].  64-ary search, one probe per lane and round (two dependent
+// loads for up to 4095 rows); every lane of the wave must be active and gets the same answer.
+__device__ __forceinline__ int find_row_of(const int *__restrict__ offsets, int rows, int pos, int lane)
+{
+    int lo = 0, span = rows + 1;
+    do {
+        const int step = (span + 63) >> 6;
+        const int idx = lo + lane * step;
+        const int probe = idx < lo + span ? offsets[idx] : 0x7fffffff;
+        const int below = __builtin_popcountll(__builtin_amdgcn_ballot_w64(probe <= pos));  // a prefix of the lanes
+        const int k = below > 0 ? below - 1 : 0;
+        lo += k * step;
+        span = span - k * step < step ? span - k * step : step;
+    } while (span > 1);
+    return lo;
+}
+
+// The same search, returning the probes of its last round as a window over the offsets: on return lane l holds
+// offsets[base + l] (0x7fffffff past offsets[rows]) and the row found is base + first, so that the caller can walk
+// on from there (row base + i runs from lane i to lane i + 1) without another load.
+__device__ __forceinline__ int find_row_window(const int *__restrict__ offsets, int rows, int pos, int lane,
+                                               int &base, int &first)
+{
+    int lo = 0, span = rows + 1;
+    for (;;) {
+        const int step = (span + 63) >> 6;
+        // the last round (step 1) probes 64 consecutive offsets whatever is left of the span: the offsets are
+        // ascending, so the entries past the span are greater than pos and do not change the count
+        const int idx = lo + lane * step;
+        const bool inside = step == 1 ? idx <= rows : idx < lo + span;
+        const int probe = inside ? offsets[idx] : 0x7fffffff;
+        const int below = __builtin_popcountll(__builtin_amdgcn_ballot_w64(probe <= pos));  // a prefix of the lanes
+        const int k = below > 0 ? below - 1 : 0;
+        if (step == 1) {
+            base = lo;
+            first = k;
+            return probe;
+        }
+        lo += k * step;
+        span = span - k * step < step ? span - k * step : step;
+    }
+}
+
+}  // namespace vs

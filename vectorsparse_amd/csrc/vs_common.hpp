@@ -187,6 +187,8 @@ __device__ __forceinline__ void store_converted<float, 1>(float *dst, const floa
 struct Options {
     int spmm_waves = 0;
     int spmm_cols_per_lane = 0;
+    int spmm_flat_piece = 0;    // split-row SpMM: nonzero vectors per wave (rounded up to 32), 0 = automatic
+    int spmm_flat_waves = 0;    // split-row SpMM: waves per workgroup, 0 = automatic
     int sddmm_slots = 0;
     int sddmm_block_waves = 0;
     int sddmm_flat_supers = 0;  // flat MFMA SDDMM (algorithm 2): super-groups per wave, 0 = automatic
@@ -245,6 +247,17 @@ int launch_sddmm_valu(int m_vec, int k, int n, int nonzeros_vec, const int *row_
                       const int *row_offsets, const int *col_indices, const half_t *lhs,
                       const half_t *rhs, OutT *out, int vec_length, hipStream_t stream,
                       const Batch &batch = Batch());
+
+// Writes `bytes` zero bytes to each of `batch` buffers `stride_bytes` apart (a kernel, not a memset node, so that
+// callers may capture the call into a HIP graph).
+int launch_zero_fill(void *out, long long bytes, long long stride_bytes, int batch, hipStream_t stream);
+
+// Split-row SpMM (csrc/spmm_mfma_flat.hip): `workspace` holds the fp32 partial tiles of rows longer than a piece.
+template <typename OutT>
+int launch_spmm_mfma_flat(int m_vec, int vec_length, int k, int n, int nonzeros_vec, const int *row_offsets,
+                          const int *column_indices, const half_t *values, const half_t *rhs, OutT *out,
+                          float *workspace, long long workspace_bytes, hipStream_t stream);
+long long spmm_flat_workspace_bytes(int vec_length, int k, int nonzeros_vec);
 
 int launch_spmm_softmax_mfma(int m_vec, int vec_length, int k, int n, const int *row_indices,
                              const int *row_offsets, const int *column_indices, const half_t *scores,

@@ -16,9 +16,42 @@ Options &options()
 }
 }  // namespace vs
 
+namespace vs {
+
+// Zeros for `bytes` bytes (whole 32-bit words, then the odd bytes) of each of gridDim.y buffers.
+__global__ void zero_fill_kernel(unsigned char *out, long long bytes, long long stride_bytes)
+{
+    unsigned char *dst = out + (long long)blockIdx.y * stride_bytes;
+    const long long words = bytes >> 2;
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < words; i += (long long)gridDim.x * blockDim.x)
+        reinterpret_cast<uint32_t *>(dst)[i] = 0u;
+    if (blockIdx.x == 0 && threadIdx.x < (bytes & 3)) dst[(words << 2) + threadIdx.x] = 0;
+}
+
+int launch_zero_fill(void *out, long long bytes, long long stride_bytes, int batch, hipStream_t stream)
+{
+    if (batch > 65535) return hipErrorNotSupported;
+    if (bytes <= 0 || batch <= 0) return hipSuccess;
+    long long blocks = (bytes / 4 + 255) / 256;
+    blocks = blocks < 1 ? 1 : (blocks > 1024 ? 1024 : blocks);
+    hipLaunchKernelGGL(zero_fill_kernel, dim3((unsigned)blocks, (unsigned)batch), dim3(256), 0, stream,
+                       static_cast<unsigned char *>(out), bytes, stride_bytes);
+    return (int)hipGetLastError();
+}
+
+}  // namespace vs
+
 namespace {
 
 using vs::half_t;
+
+// The contraction is empty (k == 0): every sampled output of SDDMM is an empty sum.
+int sddmm_zero_outputs(void *out, long long nonzeros_vec, int vec_length, size_t out_elem, int batch,
+                       long long stride_out_elems, hipStream_t stream)
+{
+    return vs::launch_zero_fill(out, nonzeros_vec * vec_length * (long long)out_elem,
+                                stride_out_elems * (long long)out_elem, batch, stream);
+}
 
 bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
@@ -34,7 +67,8 @@ int check_spmm(int m_vec, int vec_length, int k, int n, const int *row_indices, 
     // allocation); the host cannot see the pattern, so only the dense operand is required here.
     (void)column_indices;
     if (n > 0 && !rhs) return VS_ERROR_INVALID_VALUE;
-    if (!aligned(values, 2 * (size_t)vec_length) || !aligned(rhs, 16) || !aligned(out, 8 * out_elem))
+    (void)out_elem;
+    if (!aligned(values, 2 * (size_t)vec_length) || !aligned(rhs, 16) || !aligned(out, 16))
         return VS_ERROR_INVALID_VALUE;
     return VS_SUCCESS;
 }
@@ -45,7 +79,8 @@ int check_sddmm(int m_vec, int k, int n, int nonzeros_vec, const int *row_indice
 {
     if (m_vec < 0 || k < 0 || n < 0 || nonzeros_vec < 0 || !vec_ok(vec_length)) return VS_ERROR_INVALID_VALUE;
     if (m_vec == 0 || nonzeros_vec == 0) return VS_SUCCESS;
-    if (!row_indices || !row_offsets || !col_indices || !lhs || !rhs || !out) return VS_ERROR_INVALID_VALUE;
+    if (!row_indices || !row_offsets || !col_indices || !out) return VS_ERROR_INVALID_VALUE;
+    if (k > 0 && (!lhs || !rhs)) return VS_ERROR_INVALID_VALUE;  // k == 0: the dense operands are empty
     if (!aligned(out, out_elem * (size_t)vec_length)) return VS_ERROR_INVALID_VALUE;
     if (k % 8 == 0 && (!aligned(lhs, 16) || !aligned(rhs, 16))) return VS_ERROR_INVALID_VALUE;
     return VS_SUCCESS;
@@ -91,6 +126,56 @@ int vs_wmma_spmm_f16_f32out(int m_vec, int vec_length, int k, int n, const int *
                                        output_matrix, static_cast<hipStream_t>(stream));
 }
 
+long long vs_wmma_spmm_workspace_bytes(int m_vec, int vec_length, int k, int n, int nonzeros_vec)
+{
+    (void)n;
+    if (m_vec < 0 || k < 0 || nonzeros_vec < 0 || !vec_ok(vec_length)) return 0;
+    return vs::spmm_flat_workspace_bytes(vec_length, k, nonzeros_vec);
+}
+
+static int check_spmm_ws(int nonzeros_vec, const int *column_indices, const void *values, const void *workspace,
+                         long long workspace_bytes)
+{
+    if (nonzeros_vec < 0 || workspace_bytes < 0) return VS_ERROR_INVALID_VALUE;
+    if (nonzeros_vec > 0 && (!column_indices || !values)) return VS_ERROR_INVALID_VALUE;
+    if (workspace_bytes > 0 && (!workspace || !aligned(workspace, 16))) return VS_ERROR_INVALID_VALUE;
+    return VS_SUCCESS;
+}
+
+int vs_wmma_spmm_f16_ws(int m_vec, int vec_length, int k, int n, int nonzeros_vec, const int *row_indices,
+                        const int *row_offsets, const int *column_indices, const void *values,
+                        const void *rhs_matrix, void *output_matrix, void *workspace, long long workspace_bytes,
+                        void *stream)
+{
+    static const int identity[1] = {0};  // the swizzle is not used by this schedule; only its presence was checked
+    int st = check_spmm(m_vec, vec_length, k, n, row_indices ? row_indices : identity, row_offsets, column_indices,
+                        values, rhs_matrix, output_matrix, sizeof(half_t));
+    if (st == VS_SUCCESS) st = check_spmm_ws(nonzeros_vec, column_indices, values, workspace, workspace_bytes);
+    if (st != VS_SUCCESS) return st;
+    return vs::launch_spmm_mfma_flat<half_t>(m_vec, vec_length, k, n, nonzeros_vec, row_offsets, column_indices,
+                                             static_cast<const half_t *>(values),
+                                             static_cast<const half_t *>(rhs_matrix),
+                                             static_cast<half_t *>(output_matrix), static_cast<float *>(workspace),
+                                             workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int vs_wmma_spmm_f16_f32out_ws(int m_vec, int vec_length, int k, int n, int nonzeros_vec, const int *row_indices,
+                               const int *row_offsets, const int *column_indices, const void *values,
+                               const void *rhs_matrix, float *output_matrix, void *workspace,
+                               long long workspace_bytes, void *stream)
+{
+    static const int identity[1] = {0};
+    int st = check_spmm(m_vec, vec_length, k, n, row_indices ? row_indices : identity, row_offsets, column_indices,
+                        values, rhs_matrix, output_matrix, sizeof(float));
+    if (st == VS_SUCCESS) st = check_spmm_ws(nonzeros_vec, column_indices, values, workspace, workspace_bytes);
+    if (st != VS_SUCCESS) return st;
+    return vs::launch_spmm_mfma_flat<float>(m_vec, vec_length, k, n, nonzeros_vec, row_offsets, column_indices,
+                                            static_cast<const half_t *>(values),
+                                            static_cast<const half_t *>(rhs_matrix), output_matrix,
+                                            static_cast<float *>(workspace), workspace_bytes,
+                                            static_cast<hipStream_t>(stream));
+}
+
 int vs_cuda_spmm_f16(int m_vec, int vec_length, int k, int n, const int *row_indices, const int *row_offsets,
                      const int *column_indices, const void *values, const void *rhs_matrix, void *output_matrix,
                      void *stream)
@@ -123,6 +208,8 @@ int vs_wmma_sddmm_f16(int m_vec, int k, int n, int nonzeros_vec, const int *row_
     int st = check_sddmm(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices, lhs_matrix, rhs_matrix,
                          output_values, vec_length, sizeof(half_t));
     if (st != VS_SUCCESS) return st;
+    if (k == 0 && m_vec > 0)
+        return sddmm_zero_outputs(output_values, nonzeros_vec, vec_length, sizeof(half_t), 1, 0, static_cast<hipStream_t>(stream));
     vs::Batch one;
     one.algorithm = algorithm;
     return vs::launch_sddmm_mfma<half_t>(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices,
@@ -141,6 +228,8 @@ int vs_wmma_sddmm_f16_f32out(int m_vec, int k, int n, int nonzeros_vec, const in
     int st = check_sddmm(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices, lhs_matrix, rhs_matrix,
                          output_values, vec_length, sizeof(float));
     if (st != VS_SUCCESS) return st;
+    if (k == 0 && m_vec > 0)
+        return sddmm_zero_outputs(output_values, nonzeros_vec, vec_length, sizeof(float), 1, 0, static_cast<hipStream_t>(stream));
     vs::Batch one;
     one.algorithm = algorithm;
     return vs::launch_sddmm_mfma<float>(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices,
@@ -156,6 +245,8 @@ int vs_cuda_sddmm_f16(int m_vec, int k, int n, int nonzeros_vec, const int *row_
     int st = check_sddmm(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices, lhs_matrix, rhs_matrix,
                          output_values, vec_length, sizeof(half_t));
     if (st != VS_SUCCESS) return st;
+    if (k == 0 && m_vec > 0)
+        return sddmm_zero_outputs(output_values, nonzeros_vec, vec_length, sizeof(half_t), 1, 0, static_cast<hipStream_t>(stream));
     return vs::launch_sddmm_valu<half_t>(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices,
                                          static_cast<const half_t *>(lhs_matrix),
                                          static_cast<const half_t *>(rhs_matrix),
@@ -170,6 +261,8 @@ int vs_cuda_sddmm_f16_f32out(int m_vec, int k, int n, int nonzeros_vec, const in
     int st = check_sddmm(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices, lhs_matrix, rhs_matrix,
                          output_values, vec_length, sizeof(float));
     if (st != VS_SUCCESS) return st;
+    if (k == 0 && m_vec > 0)
+        return sddmm_zero_outputs(output_values, nonzeros_vec, vec_length, sizeof(float), 1, 0, static_cast<hipStream_t>(stream));
     return vs::launch_sddmm_valu<float>(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices,
                                         static_cast<const half_t *>(lhs_matrix),
                                         static_cast<const half_t *>(rhs_matrix), output_values, vec_length,
@@ -238,6 +331,10 @@ int vs_wmma_sddmm_f16_batched(int batch, int m_vec, int k, int n, int nonzeros_v
     int st = check_sddmm(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices, lhs_matrix, rhs_matrix,
                          output_values, vec_length, sizeof(half_t));
     if (st != VS_SUCCESS) return st;
+    if (k == 0 && m_vec > 0) {
+        if (!stride_ok(stride_output, vec_length)) return VS_ERROR_INVALID_VALUE;
+        return sddmm_zero_outputs(output_values, nonzeros_vec, vec_length, sizeof(half_t), batch, stride_output, static_cast<hipStream_t>(stream));
+    }
     if (!stride_ok(stride_lhs, 8) || !stride_ok(stride_rhs, 8) || !stride_ok(stride_output, vec_length))
         return VS_ERROR_INVALID_VALUE;
     vs::Batch many = make_batch(batch, stride_lhs, stride_rhs, stride_output);
@@ -258,6 +355,10 @@ int vs_cuda_sddmm_f16_batched(int batch, int m_vec, int k, int n, int nonzeros_v
     int st = check_sddmm(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices, lhs_matrix, rhs_matrix,
                          output_values, vec_length, sizeof(half_t));
     if (st != VS_SUCCESS) return st;
+    if (k == 0 && m_vec > 0) {
+        if (!stride_ok(stride_output, vec_length)) return VS_ERROR_INVALID_VALUE;
+        return sddmm_zero_outputs(output_values, nonzeros_vec, vec_length, sizeof(half_t), batch, stride_output, static_cast<hipStream_t>(stream));
+    }
     const long long in_mult = (k % 8 == 0) ? 8 : 1;
     if (!stride_ok(stride_lhs, in_mult) || !stride_ok(stride_rhs, in_mult) || !stride_ok(stride_output, vec_length))
         return VS_ERROR_INVALID_VALUE;
@@ -383,6 +484,11 @@ int vs_set_option(const char *name, int value)
     } else if (std::strcmp(name, "spmm_cols_per_lane") == 0) {
         if (value != 0 && value != 4 && value != 8) return VS_ERROR_INVALID_VALUE;
         o.spmm_cols_per_lane = value;
+    } else if (std::strcmp(name, "spmm_flat_piece") == 0) {
+        o.spmm_flat_piece = value;
+    } else if (std::strcmp(name, "spmm_flat_waves") == 0) {
+        if (value > 16) return VS_ERROR_INVALID_VALUE;
+        o.spmm_flat_waves = value;
     } else if (std::strcmp(name, "sddmm_slots") == 0) {
         o.sddmm_slots = value;
     } else if (std::strcmp(name, "sddmm_flat_supers") == 0) {

@@ -100,6 +100,32 @@ class spmm:
                      values, rhs_matrix, output_matrix, stream)
 
 
+def spmm_workspace_bytes(m_vec, vec_length, k, n, nonzeros_vec):
+    """Preferred workspace size of `spmm_split_rows` for this problem (0: no row can be split)."""
+    return int(_lib.lib().vs_wmma_spmm_workspace_bytes(m_vec, vec_length, k, n, nonzeros_vec))
+
+
+def spmm_split_rows(m_vec, vec_length, k, n, nonzeros_vec, row_offsets, column_indices, values, rhs_matrix,
+                    output_matrix, workspace=None, stream=None, row_indices=None):
+    """wmmaSpmm on the schedule that splits the nonzero range instead of the rows (skewed row lengths).
+
+    workspace: a device tensor (any dtype) for the partial tiles of rows that cross workgroups, or None (one
+    workgroup then takes everything).  Returns output_matrix.
+    """
+    f32 = output_matrix.dtype is torch.float32
+    entry = "vs_wmma_spmm_f16_f32out_ws" if f32 else "vs_wmma_spmm_f16_ws"
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    st = getattr(_lib.lib(), entry)(
+        m_vec, vec_length, k, n, nonzeros_vec, _expect(row_indices, torch.int32, "row_indices"),
+        _expect(row_offsets, torch.int32, "row_offsets"), _expect(column_indices, torch.int32, "column_indices"),
+        _expect(values, torch.float16, "values"), _expect(rhs_matrix, torch.float16, "rhs_matrix"),
+        _expect(output_matrix, torch.float32 if f32 else torch.float16, "output_matrix"), _ptr(workspace), ws_bytes,
+        _stream(stream))
+    if st:
+        _lib.check(st, entry)
+    return output_matrix
+
+
 class sddmm:
     """Namespace ``sddmm`` of the reference: D = (A[m x k] * B[n x k]^T) sampled on a column-vector CSR mask."""
 
@@ -409,17 +435,26 @@ class DeviceProblem:
         self.row_indices = torch.from_numpy(swz).to(device)
         self.row_offsets = torch.from_numpy(np.ascontiguousarray(pattern.row_offsets)).to(device)
         self.column_indices = torch.from_numpy(np.ascontiguousarray(pattern.column_indices)).to(device)
+        self._workspace = None  # partial tiles of the split-row SpMM, allocated on first use
         self.values = None
         if pattern.values is not None:
             self.values = torch.from_numpy(np.ascontiguousarray(pattern.values)).to(device)
 
-    def spmm(self, rhs_matrix, kernel="wmma", out_dtype=torch.float16, out=None, stream=None, row_length_hint=False):
+    def spmm(self, rhs_matrix, kernel="wmma", out_dtype=torch.float16, out=None, stream=None, row_length_hint=False,
+             split_rows=False):
         """SpMM through the reference-shaped entry points; with row_length_hint (fp16 output only) through the
         batched entry point with batch = 1, which also takes the pattern's nonzero count and longest row and
-        sizes its workgroups by the real row lengths instead of by n."""
+        sizes its workgroups by the real row lengths instead of by n; with split_rows (MFMA path) on the
+        schedule that cuts the nonzero range into equal pieces, with a workspace this object owns."""
         k = rhs_matrix.shape[1]
         if out is None:
             out = torch.empty((self.m_vec * self.vec_length, k), dtype=out_dtype, device=rhs_matrix.device)
+        if split_rows and kernel == "wmma":
+            need = spmm_workspace_bytes(self.m_vec, self.vec_length, k, self.n, self.nnz_vec)
+            if self._workspace is None or self._workspace.numel() < need:
+                self._workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=rhs_matrix.device)
+            return spmm_split_rows(self.m_vec, self.vec_length, k, self.n, self.nnz_vec, self.row_offsets,
+                                   self.column_indices, self.values, rhs_matrix, out, self._workspace, stream)
         if row_length_hint and out.dtype == torch.float16:
             spmm_batched(self.m_vec, self.vec_length, k, self.n, self.row_indices, self.row_offsets,
                          self.column_indices, self.values, rhs_matrix, out.unsqueeze(0), kernel=kernel, stream=stream,
