@@ -95,6 +95,24 @@ int vs_wmma_spmm_f16_f32out_ws(int m_vec, int vec_length, int k, int n, int nonz
                                void *workspace, long long workspace_bytes, void *stream);
 
 /*
+ * vs_wmma_spmm_f16_ws without the workspace argument, for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the partial tiles go to a
+ * static device array of vs_wmma_spmm_noalloc_scratch_bytes() = 16 MiB that the library holds on every GPU it
+ * runs on until the process ends.  The call allocates and frees nothing.  It has no counterpart in the
+ * reference.  Same results, bit for bit, as vs_wmma_spmm_f16_ws with a workspace of that size.
+ * Size limit: vec_length * (k rounded up to a multiple of 128) <= 32768 (the array must hold the partial tiles
+ * of 64 pieces); beyond it the call returns 801 (hipErrorNotSupported) and launches nothing.
+ * Every call on a GPU shares that GPU's array: calls that may overlap on one GPU (different streams, different
+ * threads) race on it and must be serialised by the caller.  Nothing in the array has to be cleared between
+ * calls (every partial tile that is read was written by the same call).
+ */
+long long vs_wmma_spmm_noalloc_scratch_bytes(void);
+int vs_wmma_spmm_f16_noalloc(int m_vec, int vec_length, int k, int n, int nonzeros_vec,
+                             const int *row_indices, const int *row_offsets,
+                             const int *column_indices, const void *values,
+                             const void *rhs_matrix, void *output_matrix, void *stream);
+
+/*
  * Replaces spmm::cudaSpmm(half in, half out) — include/cuda_spmm.cuh:15-21,
  * src/cuda_spmm.cu:316-325.  Fine-grained path on the fp16 vector ALU
  * (mixed-precision FMA: exact fp16 x fp16 products, fp32 accumulate).  The

@@ -1,0 +1,81 @@
+"""`vs_wmma_spmm_f16_noalloc`: the split-row SpMM with its workspace in a static device array of the library.
+Through the C ABI, against `vs_wmma_spmm_f16_ws` with a caller workspace of the same size (bit for bit) and
+against the CPU oracle; two calls in a row, the second on a smaller problem, so that whatever the first call left
+in the array must not leak into the second."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle as co
+from vectorsparse_amd import _lib
+from vectorsparse_amd import colvec_csr as cv
+from util import assert_parity
+
+pytestmark = pytest.mark.gpu
+
+
+def _problem(m_vec, n, V, N, seed, longest):
+    rng = np.random.default_rng(seed)
+    lengths = np.minimum((rng.pareto(1.5, m_vec) + 0.3) * 60, n).astype(np.int64)
+    lengths[m_vec // 3] = longest      # a row that spans many pieces
+    lengths[m_vec // 2] = 0
+    ro, ci = cv._pattern_from_lengths(rng, m_vec, n, lengths)
+    pat = cv.random_values(cv.ColVecCSR(m_vec, n, V, ro, ci).validate(), seed=seed + 1)
+    return pat, cv.dense_uniform(n, N, seed=seed + 2)
+
+
+def _device(pat, B):
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    return d(pat.row_offsets), d(pat.column_indices), d(pat.values), d(B)
+
+
+def test_two_calls_in_a_row_match_the_workspace_entry_point(gpu):
+    L = _lib.lib()
+    scratch = L.vs_wmma_spmm_noalloc_scratch_bytes()
+    assert scratch == 16 << 20
+    workspace = torch.empty(scratch, dtype=torch.uint8, device="cuda")
+    # the first problem splits many rows across pieces; the second is smaller in every dimension
+    for (m_vec, n, V, N, seed, longest) in ((512, 4096, 8, 256, 1, 4096), (96, 1024, 8, 128, 2, 1000)):
+        pat, B = _problem(m_vec, n, V, N, seed, longest)
+        ro, ci, vals, Bd = _device(pat, B)
+        assert L.vs_wmma_spmm_workspace_bytes(m_vec, V, N, n, pat.nnz_vec) > 0, "the case must use the scratch"
+        pad = 64
+        buf = torch.full((pat.m + 2 * pad, N), 4321.0, dtype=torch.float16, device="cuda")
+        got = buf[pad:pad + pat.m]
+        want = torch.full((pat.m, N), -1.0, dtype=torch.float16, device="cuda")
+        st = L.vs_wmma_spmm_f16_noalloc(m_vec, V, N, n, pat.nnz_vec, 0, ro.data_ptr(), ci.data_ptr(), vals.data_ptr(),
+                                        Bd.data_ptr(), got.data_ptr(), 0)
+        assert st == 0, L.vs_status_string(st)
+        st = L.vs_wmma_spmm_f16_ws(m_vec, V, N, n, pat.nnz_vec, 0, ro.data_ptr(), ci.data_ptr(), vals.data_ptr(),
+                                   Bd.data_ptr(), want.data_ptr(), workspace.data_ptr(), scratch, 0)
+        assert st == 0, L.vs_status_string(st)
+        torch.cuda.synchronize()
+        host = buf.cpu().numpy()
+        assert np.all(host[:pad] == 4321.0) and np.all(host[pad + pat.m:] == 4321.0), "wrote outside the output"
+        assert np.array_equal(host[pad:pad + pat.m].view(np.uint16), want.cpu().numpy().view(np.uint16)), \
+            "static scratch and caller workspace give different bits"
+        ref = co.spmm_host_ref_f32(m_vec, V, N, n, pat.row_offsets, pat.column_indices, pat.values, B)
+        assert_parity(host[pad:pad + pat.m], ref, "no-alloc entry point, %d rows" % m_vec)
+        assert np.array_equal(ro.cpu().numpy(), pat.row_offsets) and np.array_equal(ci.cpu().numpy(), pat.column_indices)
+
+
+def test_sizes_beyond_the_scratch_are_rejected(gpu):
+    L = _lib.lib()
+    pat, B = _problem(16, 256, 8, 4224, 3, 200)      # 8 * 4224 > 32768
+    ro, ci, vals, Bd = _device(pat, B)
+    out = torch.full((pat.m, 4224), 9.0, dtype=torch.float16, device="cuda")
+    st = L.vs_wmma_spmm_f16_noalloc(16, 8, 4224, 256, pat.nnz_vec, 0, ro.data_ptr(), ci.data_ptr(), vals.data_ptr(),
+                                    Bd.data_ptr(), out.data_ptr(), 0)
+    assert st == 801 and b"limit" in L.vs_status_string(st)
+    torch.cuda.synchronize()
+    assert bool((out == 9.0).all()), "a rejected call must not launch anything"
+    # at the limit it runs
+    pat, B = _problem(16, 256, 8, 4096, 4, 200)
+    ro, ci, vals, Bd = _device(pat, B)
+    out = torch.empty((pat.m, 4096), dtype=torch.float16, device="cuda")
+    st = L.vs_wmma_spmm_f16_noalloc(16, 8, 4096, 256, pat.nnz_vec, 0, ro.data_ptr(), ci.data_ptr(), vals.data_ptr(),
+                                    Bd.data_ptr(), out.data_ptr(), 0)
+    assert st == 0
+    torch.cuda.synchronize()
+    ref = co.spmm_host_ref_f32(16, 8, 4096, 256, pat.row_offsets, pat.column_indices, pat.values, B)
+    assert_parity(out.cpu().numpy(), ref, "no-alloc entry point at its size limit")

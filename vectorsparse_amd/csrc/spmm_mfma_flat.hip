@@ -383,6 +383,47 @@ int launch_spmm_mfma_flat(int m_vec, int vec_length, int k, int n, int nonzeros_
     }
 }
 
+// Library-owned scratch for the entry point that allocates nothing: the workspace of the split-row schedule in a
+// static device array (every GPU the library runs on holds its own copy at its own address until the process
+// ends).  Host code must not use the array's name as an address: it is resolved once per device.
+constexpr long long kScratchBytes = 16LL << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+static std::atomic<void *> scratch_of_device[64];
+
+long long spmm_flat_scratch_bytes() { return kScratchBytes; }
+
+// The current device's copy of `scratch` (resolved on the first call on that device, with it current).
+static int scratch_address(float **address)
+{
+    int device = 0;
+    hipError_t st = hipGetDevice(&device);
+    if (st != hipSuccess) return (int)st;
+    if (device < 0 || device >= 64) return hipErrorNotSupported;
+    void *p = scratch_of_device[device].load(std::memory_order_acquire);
+    if (!p) {
+        st = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (st != hipSuccess) return (int)st;
+        if (!p) return hipErrorInvalidSymbol;
+        scratch_of_device[device].store(p, std::memory_order_release);
+    }
+    *address = static_cast<float *>(p);
+    return hipSuccess;
+}
+
+int launch_spmm_mfma_flat_static(int m_vec, int vec_length, int k, int n, int nonzeros_vec, const int *row_offsets,
+                                 const int *column_indices, const half_t *values, const half_t *rhs, half_t *out,
+                                 hipStream_t stream)
+{
+    // the scratch must hold the partial tiles of at least 64 pieces, or the schedule degenerates
+    const long long k_pad = (long long)ceil_div(k, 128) * 128;
+    if (64LL * 2 * vec_length * k_pad * (long long)sizeof(float) > kScratchBytes) return hipErrorNotSupported;
+    float *ws = nullptr;
+    const int st = scratch_address(&ws);
+    if (st != hipSuccess) return st;
+    return launch_spmm_mfma_flat<half_t>(m_vec, vec_length, k, n, nonzeros_vec, row_offsets, column_indices, values, rhs,
+                                         out, ws, kScratchBytes, stream);
+}
+
 template int launch_spmm_mfma_flat<half_t>(int, int, int, int, int, const int *, const int *, const half_t *,
                                            const half_t *, half_t *, float *, long long, hipStream_t);
 template int launch_spmm_mfma_flat<float>(int, int, int, int, int, const int *, const int *, const half_t *,

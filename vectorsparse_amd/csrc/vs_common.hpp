@@ -258,6 +258,11 @@ int launch_spmm_mfma_flat(int m_vec, int vec_length, int k, int n, int nonzeros_
                           const int *column_indices, const half_t *values, const half_t *rhs, OutT *out,
                           float *workspace, long long workspace_bytes, hipStream_t stream);
 long long spmm_flat_workspace_bytes(int vec_length, int k, int nonzeros_vec);
+// The same schedule with the workspace in a library-owned static device array (no allocation anywhere).
+int launch_spmm_mfma_flat_static(int m_vec, int vec_length, int k, int n, int nonzeros_vec, const int *row_offsets,
+                                 const int *column_indices, const half_t *values, const half_t *rhs, half_t *out,
+                                 hipStream_t stream);
+long long spmm_flat_scratch_bytes();
 
 int launch_spmm_softmax_mfma(int m_vec, int vec_length, int k, int n, const int *row_indices,
                              const int *row_offsets, const int *column_indices, const half_t *scores,

@@ -97,7 +97,7 @@ const char *vs_status_string(int status)
     switch (status) {
     case VS_SUCCESS: return "success";
     case VS_ERROR_INVALID_VALUE: return "invalid value (null pointer, negative size, misaligned operand, or unsupported vec_length/algorithm)";
-    case VS_ERROR_NOT_SUPPORTED: return "shape not supported by the selected path";
+    case VS_ERROR_NOT_SUPPORTED: return "shape not supported by the selected path (or beyond the size limit of an entry point that allocates nothing)";
     default: return hipGetErrorString(static_cast<hipError_t>(status));
     }
 }
@@ -158,6 +158,23 @@ int vs_wmma_spmm_f16_ws(int m_vec, int vec_length, int k, int n, int nonzeros_ve
                                              static_cast<half_t *>(output_matrix), static_cast<float *>(workspace),
                                              workspace_bytes, static_cast<hipStream_t>(stream));
 }
+
+int vs_wmma_spmm_f16_noalloc(int m_vec, int vec_length, int k, int n, int nonzeros_vec, const int *row_indices,
+                             const int *row_offsets, const int *column_indices, const void *values,
+                             const void *rhs_matrix, void *output_matrix, void *stream)
+{
+    static const int identity[1] = {0};
+    int st = check_spmm(m_vec, vec_length, k, n, row_indices ? row_indices : identity, row_offsets, column_indices,
+                        values, rhs_matrix, output_matrix, sizeof(half_t));
+    if (st == VS_SUCCESS) st = check_spmm_ws(nonzeros_vec, column_indices, values, nullptr, 0);
+    if (st != VS_SUCCESS) return st;
+    return vs::launch_spmm_mfma_flat_static(m_vec, vec_length, k, n, nonzeros_vec, row_offsets, column_indices,
+                                            static_cast<const half_t *>(values),
+                                            static_cast<const half_t *>(rhs_matrix),
+                                            static_cast<half_t *>(output_matrix), static_cast<hipStream_t>(stream));
+}
+
+long long vs_wmma_spmm_noalloc_scratch_bytes(void) { return vs::spmm_flat_scratch_bytes(); }
 
 int vs_wmma_spmm_f16_f32out_ws(int m_vec, int vec_length, int k, int n, int nonzeros_vec, const int *row_indices,
                                const int *row_offsets, const int *column_indices, const void *values,
