@@ -330,7 +330,11 @@ void vs_sorted_row_swizzle(int rows, const int *row_offsets, int *row_indices);
 /*
  * Launch-shape tuning knob (process-wide, not thread-safe against concurrent
  * launches).  Names: "spmm_waves" (waves per workgroup, 0 = automatic),
- * "spmm_cols_per_lane" (4, 8, 0 = automatic), "spmm_flat_piece" (nonzero vectors
+ * "spmm_cols_per_lane" (4, 8, 0 = automatic), "spmm_gather" (how the MFMA SpMM
+ * brings the gathered rows of the dense operand to the matrix cores: 1 = through
+ * registers and an in-register transpose, 2 = global -> LDS loads and transposing LDS
+ * reads, k % 8 == 0 only; 0 = automatic, which is 1: 2 measured 10-18 % slower),
+ * "spmm_flat_piece" (nonzero vectors
  * per wave of the split-row SpMM, rounded up to 32, 0 = automatic), "spmm_flat_waves"
  * (its waves per workgroup, 1..16, 0 = automatic), "sddmm_slots" (waves per
  * vector row, 0 = automatic), "sddmm_block_waves" (1..16, 0 = automatic),

@@ -246,3 +246,34 @@ def test_longest_row_hint_on_heavy_tailed_rows(gpu):
         torch.cuda.synchronize()
         assert_parity(plain.cpu().numpy(), ref, "heavy tail, reference-shaped entry")
         assert_parity(hinted.cpu().numpy(), ref, "heavy tail, hinted")
+
+
+@pytest.mark.parametrize("V", [1, 2, 4, 8])
+def test_lds_dma_gather_variant_keeps_parity(gpu, V):
+    """The variant of the MFMA kernel whose gathered rows go global -> LDS directly and reach the MFMA through
+    transposing LDS reads (option spmm_gather = 2): same contract, every wave count, ragged rows, dense-width
+    edges, and the same bits for any row swizzle."""
+    lengths = np.array([0, 1, 15, 16, 17, 0, 31, 33, 64, 65, 300, 2, 0, 128, 7, 0], dtype=np.int64)
+    rng = np.random.default_rng(5)
+    ro, ci = cv._pattern_from_lengths(rng, len(lengths), 320, lengths)
+    ragged = cv.random_values(cv.ColVecCSR(len(lengths), 320, V, ro, ci).validate(), seed=6)
+    big = cv.random_values(cv.binomial_pattern(512 // V, 4608, 0.9, seed=1, vec_length=V), seed=101)
+    try:
+        _lib.set_option("spmm_gather", 2)
+        for N in (8, 72, 128, 192, 1000):
+            B = cv.dense_uniform(320, N, seed=N)
+            ref = _oracle(ragged, B)
+            for waves in (0, 1, 3, 16):
+                _lib.set_option("spmm_waves", waves)
+                got = _run(ragged, B, "wmma")
+                assert_parity(got, ref, "dma gather V%d N%d waves %d" % (V, N, waves))
+        _lib.set_option("spmm_waves", 0)
+        B = cv.dense_uniform(4608, 256, seed=201)
+        a = _run(big, B, "wmma", sort=False)
+        b = _run(big, B, "wmma", sort=True)
+        assert_parity(a, _oracle(big, B), "dma gather config-2 shape V%d" % V)
+        assert np.array_equal(a.view(np.uint16), b.view(np.uint16)), "row swizzle changed the bits"
+        assert_parity(_run(big, B, "wmma", out_dtype=torch.float32), _oracle(big, B), "dma gather fp32 out")
+    finally:
+        _lib.set_option("spmm_gather", 0)
+        _lib.set_option("spmm_waves", 0)

@@ -186,15 +186,27 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
             float sum[CPL];
 #pragma unroll
             for (int c = 0; c < CPL; ++c) sum[c] = 0.f;
-            for (int w = 0; w < active; ++w) {
-                const float *src = partial + (size_t)w * V * TN + v * TN + cs2 * CPL;
+            // four partial tiles are requested at once (a wave past `active` contributes an exact zero) and added
+            // in wave order: one LDS round trip per four waves instead of one per wave
+            for (int w0 = 0; w0 < active; w0 += 4) {
+                float4_t x[4][CPL / 4];
 #pragma unroll
-                for (int c4 = 0; c4 < CPL / 4; ++c4) {
-                    const float4_t x = *reinterpret_cast<const float4_t *>(src + 4 * c4);
-                    sum[4 * c4] += x[0];
-                    sum[4 * c4 + 1] += x[1];
-                    sum[4 * c4 + 2] += x[2];
-                    sum[4 * c4 + 3] += x[3];
+                for (int i = 0; i < 4; ++i) {
+                    const int w = w0 + i < active ? w0 + i : active - 1;
+                    const float *src = partial + (size_t)w * V * TN + v * TN + cs2 * CPL;
+#pragma unroll
+                    for (int c4 = 0; c4 < CPL / 4; ++c4) x[i][c4] = *reinterpret_cast<const float4_t *>(src + 4 * c4);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const bool keep = w0 + i < active;
+#pragma unroll
+                    for (int c4 = 0; c4 < CPL / 4; ++c4) {
+                        sum[4 * c4] += keep ? x[i][c4][0] : 0.f;
+                        sum[4 * c4 + 1] += keep ? x[i][c4][1] : 0.f;
+                        sum[4 * c4 + 2] += keep ? x[i][c4][2] : 0.f;
+                        sum[4 * c4 + 3] += keep ? x[i][c4][3] : 0.f;
+                    }
                 }
             }
             if constexpr (SOFTMAX) {
@@ -275,6 +287,8 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
     constexpr int kTargetBlocks = 256;   // one workgroup per CU at least
     constexpr int kTargetWaves = 4096;
     int cpl = options().spmm_cols_per_lane;
+    const bool use_dma = !SOFTMAX && options().spmm_gather == 2 && k % 8 == 0;
+    if (use_dma) cpl = 8;
     if (cpl != 4 && cpl != 8) {
         const long long blocks128 = (long long)m_vec * ceil_div(k, 128) * batch.count;
         cpl = (k % 8 == 0 && k > 64 && blocks128 >= kTargetBlocks) ? 8 : 4;  // k <= 64 fits one 64-column tile
@@ -320,6 +334,11 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
     }
     if (waves < 1) waves = 1;
     if (waves > 16) waves = 16;
+    if constexpr (!SOFTMAX) {
+        if (use_dma)
+            return launch_spmm_mfma_dma<OutT>(m_vec, vec_length, k, n, waves, row_indices, row_offsets, column_indices,
+                                              values, rhs, out, stream, batch);
+    }
     if (cpl == 8)
         return launch_v<8, SOFTMAX, OutT>(vec_length, m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
     return launch_v<4, SOFTMAX, OutT>(vec_length, m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);

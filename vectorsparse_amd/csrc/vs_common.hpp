@@ -187,6 +187,7 @@ __device__ __forceinline__ void store_converted<float, 1>(float *dst, const floa
 struct Options {
     int spmm_waves = 0;
     int spmm_cols_per_lane = 0;
+    int spmm_gather = 0;        // 1 = gathered rows through registers, 2 = through LDS-DMA loads, 0 = automatic
     int spmm_flat_piece = 0;    // split-row SpMM: nonzero vectors per wave (rounded up to 32), 0 = automatic
     int spmm_flat_waves = 0;    // split-row SpMM: waves per workgroup, 0 = automatic
     int sddmm_slots = 0;
@@ -233,6 +234,10 @@ template <typename OutT>
 int launch_spmm_mfma(int m_vec, int vec_length, int k, int n, const int *row_indices,
                      const int *row_offsets, const int *column_indices, const half_t *values,
                      const half_t *rhs, OutT *out, hipStream_t stream, const Batch &batch = Batch());
+template <typename OutT>
+int launch_spmm_mfma_dma(int m_vec, int vec_length, int k, int n, int waves, const int *row_indices,
+                         const int *row_offsets, const int *column_indices, const half_t *values, const half_t *rhs,
+                         OutT *out, hipStream_t stream, const Batch &batch);
 template <typename OutT>
 int launch_spmm_valu(int m_vec, int vec_length, int k, int n, const int *row_indices,
                      const int *row_offsets, const int *column_indices, const half_t *values,

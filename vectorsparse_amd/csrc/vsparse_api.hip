@@ -501,6 +501,9 @@ int vs_set_option(const char *name, int value)
     } else if (std::strcmp(name, "spmm_cols_per_lane") == 0) {
         if (value != 0 && value != 4 && value != 8) return VS_ERROR_INVALID_VALUE;
         o.spmm_cols_per_lane = value;
+    } else if (std::strcmp(name, "spmm_gather") == 0) {
+        if (value > 2) return VS_ERROR_INVALID_VALUE;
+        o.spmm_gather = value;
     } else if (std::strcmp(name, "spmm_flat_piece") == 0) {
         o.spmm_flat_piece = value;
     } else if (std::strcmp(name, "spmm_flat_waves") == 0) {
