@@ -53,8 +53,10 @@ const char *vs_status_string(int status);
  * Replaces spmm::wmmaSpmm(half in, half out) — include/wmma_spmm.cuh:15-21,
  * src/wmma_spmm.cu:400-409.  fp16 MFMA with fp32 accumulate.
  * vec_length in {2, 4, 8} as in the reference (1 is accepted as well).
- * Requirements: k % 4 == 0; `values` aligned to 2*vec_length bytes,
- * `rhs_matrix` and `output_matrix` aligned to 16 bytes.
+ * Requirements: `values` aligned to 2*vec_length bytes, `rhs_matrix` and
+ * `output_matrix` aligned to 16 bytes.  Any k >= 1 (the reference assumes
+ * k % 64 == 0 and reads / writes past the operands otherwise, src/wmma_spmm.cu:362);
+ * k % 4 != 0 takes a slower kernel that moves the dense operands half by half.
  */
 int vs_wmma_spmm_f16(int m_vec, int vec_length, int k, int n,
                      const int *row_indices, const int *row_offsets,
@@ -119,7 +121,8 @@ int vs_wmma_spmm_f16_noalloc(int m_vec, int vec_length, int k, int n, int nonzer
  * reference rounds each product to fp16 (src/spmm_utils/compute_utils.h:45);
  * that rounding is deliberately not reproduced because it alone breaks the
  * 1e-2 relative-error contract against the host loop.
- * vec_length in {1, 2, 4, 8}.  Same alignment rules; k % 8 == 0.
+ * vec_length in {1, 2, 4, 8}.  Same alignment rules; any k >= 1 (k % 8 != 0 takes a
+ * slower kernel that moves the dense operands half by half).
  */
 int vs_cuda_spmm_f16(int m_vec, int vec_length, int k, int n,
                      const int *row_indices, const int *row_offsets,

@@ -101,17 +101,35 @@ def test_all_rows_empty(gpu, kernel):
     assert got.shape == (64, 64) and not got.any()
 
 
-@pytest.mark.parametrize("N", [8, 24, 64, 72, 136, 512, 1000])
+@pytest.mark.parametrize("N", [1, 3, 4, 8, 12, 24, 30, 64, 66, 72, 136, 147, 512, 1000, 1001])
 @pytest.mark.parametrize("kernel", ["wmma", "cuda"])
 def test_dense_width_edges(gpu, N, kernel):
+    # any dense width on both paths (the reference has no bounds check at all, src/wmma_spmm.cu:362-384): widths
+    # that are not a multiple of 4 (MFMA) / 8 (fine-grained) take the kernels that move the operands half by half;
+    # odd widths make every row of B and of the output start at an odd half
     pat = cv.random_values(cv.binomial_pattern(24, 200, 0.8, seed=N, vec_length=8), seed=N + 1)
     B = cv.dense_uniform(200, N, seed=N + 2)
-    assert_parity(_run(pat, B, kernel), _oracle(pat, B), "N=%d %s" % (N, kernel))
+    ref = _oracle(pat, B)
+    assert_parity(_run(pat, B, kernel), ref, "N=%d %s" % (N, kernel))
+    if N in (3, 30, 147, 1001):
+        assert_parity(_run(pat, B, kernel, out_dtype=torch.float32, sort=True), ref, "N=%d %s fp32 out" % (N, kernel))
+
+
+@pytest.mark.parametrize("V", [1, 2, 4])
+@pytest.mark.parametrize("kernel", ["wmma", "cuda"])
+def test_odd_dense_widths_every_vector_length(gpu, V, kernel):
+    lengths = np.array([0, 1, 15, 33, 64, 65, 300, 2, 0, 7], dtype=np.int64)
+    rng = np.random.default_rng(5)
+    ro, ci = cv._pattern_from_lengths(rng, len(lengths), 320, lengths)
+    pat = cv.random_values(cv.ColVecCSR(len(lengths), 320, V, ro, ci).validate(), seed=6)
+    for N in (5, 66, 131):
+        B = cv.dense_uniform(320, N, seed=N)
+        assert_parity(_run(pat, B, kernel), _oracle(pat, B), "V%d N=%d %s" % (V, N, kernel))
 
 
 def test_dense_width_multiple_of_4_on_mfma_path(gpu):
     pat = cv.random_values(cv.binomial_pattern(24, 100, 0.7, seed=3, vec_length=4), seed=4)
-    for N in (4, 12, 68, 132):
+    for N in (4, 12, 68, 132, 2, 6, 70):
         B = cv.dense_uniform(100, N, seed=N)
         assert_parity(_run(pat, B, "wmma"), _oracle(pat, B), "N=%d wmma" % N)
 

@@ -26,7 +26,9 @@ namespace vs {
 // SOFTMAX: the sparse values are raw scores and the kernel multiplies by softmax_row(scale * values)
 // instead: a pre-pass finds each scalar row's maximum, the staging step turns every score into
 // exp2(s*x - max) (and sums them), and the accumulated tile is divided by the row sum at the end.
-template <int V, int CPL, bool SOFTMAX, bool IDX32, typename OutT>
+// RAGGED: the dense width is not a multiple of CPL (rows of the dense operand and of the output start at any 2-byte
+// boundary, the last chunk of a row is cut): chunks are fetched and stored half by half.
+template <int V, int CPL, bool SOFTMAX, bool IDX32, typename OutT, bool RAGGED = false>
 __global__ void __launch_bounds__(1024)
 spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
                  const int *__restrict__ row_offsets, const int *__restrict__ column_indices,
@@ -51,8 +53,9 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
     const int cs = lane & 15;
     const int g = lane >> 4;
     const int col0 = tile * TN + cs * CPL;
-    const bool col_ok = col0 < n_cols;  // n_cols % CPL == 0: a lane's chunk is all in or all out
+    const bool col_ok = col0 < n_cols;  // n_cols % CPL == 0 unless RAGGED: a lane's chunk is all in or all out
     const uint32_t col_off = col_ok ? col0 : 0;
+    const int valid = !col_ok ? 0 : (n_cols - col0 < CPL ? n_cols - col0 : CPL);  // RAGGED: halves of the chunk that exist
 
     int *idx_s = reinterpret_cast<int *>(smem + (size_t)wave * kStage);
     half_t *vec_s = reinterpret_cast<half_t *>(idx_s + kStep);  // [V][kStep]
@@ -125,9 +128,9 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
             }
         }
         wave_lds_fence();
-        spmm_mfma_step<V, CPL, IDX32>(idx_s, vec_s, rhs, n_cols, col_off, cs, g, acc, [&] {
+        spmm_mfma_step<V, CPL, IDX32, RAGGED>(idx_s, vec_s, rhs, n_cols, col_off, cs, g, acc, [&] {
             if (base + stride < end) fetch(base + stride);
-        });
+        }, valid);
     }
 
     if constexpr (SOFTMAX) {
@@ -150,7 +153,10 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
                 float tmp[CPL];
 #pragma unroll
                 for (int c = 0; c < CPL; ++c) tmp[c] = acc[c][e] * norm;
-                store_converted<OutT, CPL>(out + ((size_t)row * V + v) * n_cols + col0, tmp);
+                if constexpr (RAGGED)
+                    store_ragged<OutT, CPL>(out + ((size_t)row * V + v) * n_cols + col0, tmp, valid);
+                else
+                    store_converted<OutT, CPL>(out + ((size_t)row * V + v) * n_cols + col0, tmp);
             }
         }
         return;
@@ -216,7 +222,10 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
 #pragma unroll
                 for (int c = 0; c < CPL; ++c) sum[c] *= norm;
             }
-            store_converted<OutT, CPL>(out + ((size_t)row * V + v) * n_cols + col, sum);
+            if constexpr (RAGGED)
+                store_ragged<OutT, CPL>(out + ((size_t)row * V + v) * n_cols + col, sum, n_cols - col);
+            else
+                store_converted<OutT, CPL>(out + ((size_t)row * V + v) * n_cols + col, sum);
         }
     }
 }
@@ -247,6 +256,23 @@ static int launch_idx(int m_vec, int k, int n, int waves, const int *row_indices
     hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)batch.count), dim3(64 * waves), lds, stream,
                        k, n_tiles, row_indices, row_offsets, column_indices, values, rhs, out,
                        batch.stride_a, batch.stride_b, batch.stride_out, scale);
+    return (int)hipGetLastError();
+}
+
+// Dense widths that are not a multiple of 4: the half-by-half variant of the 64-column-tile kernel.
+template <int V, typename OutT>
+static int launch_ragged(int m_vec, int k, int waves, const int *row_indices, const int *row_offsets,
+                         const int *column_indices, const half_t *values, const half_t *rhs, OutT *out,
+                         hipStream_t stream, const Batch &batch)
+{
+    constexpr int TN = 64;
+    const int n_tiles = ceil_div(k, TN);
+    const long long blocks = (long long)m_vec * n_tiles;
+    if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
+    const size_t lds = (size_t)waves * stage_bytes<V>() + (waves > 1 ? (size_t)waves * V * (TN + 1) * sizeof(float) : 0);
+    hipLaunchKernelGGL((spmm_mfma_kernel<V, 4, false, false, OutT, true>), dim3((unsigned)blocks, (unsigned)batch.count),
+                       dim3(64 * waves), lds, stream, k, n_tiles, row_indices, row_offsets, column_indices, values, rhs,
+                       out, batch.stride_a, batch.stride_b, batch.stride_out, 1.f);
     return (int)hipGetLastError();
 }
 
@@ -283,7 +309,8 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
                       const half_t *rhs, OutT *out, hipStream_t stream, const Batch &batch, float scale)
 {
     if (m_vec == 0 || k == 0 || batch.count == 0) return hipSuccess;
-    if (k % 4 != 0 || batch.count > 65535) return hipErrorNotSupported;
+    if (batch.count > 65535) return hipErrorNotSupported;
+    if (SOFTMAX && k % 4 != 0) return hipErrorNotSupported;
     constexpr int kTargetBlocks = 256;   // one workgroup per CU at least
     constexpr int kTargetWaves = 4096;
     int cpl = options().spmm_cols_per_lane;
@@ -294,6 +321,8 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
         cpl = (k % 8 == 0 && k > 64 && blocks128 >= kTargetBlocks) ? 8 : 4;  // k <= 64 fits one 64-column tile
     }
     if (cpl == 8 && k % 8 != 0) cpl = 4;
+    const bool ragged = k % 4 != 0;
+    if (ragged) cpl = 4;
     const long long blocks = (long long)m_vec * ceil_div(k, 16 * cpl) * batch.count;
     int waves = options().spmm_waves;
     if (waves <= 0) {
@@ -335,6 +364,16 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
     if (waves < 1) waves = 1;
     if (waves > 16) waves = 16;
     if constexpr (!SOFTMAX) {
+        if (ragged) {
+            if (waves > 8) waves = 8;  // 8 x 2.7 KB of LDS stay below the default limit of dynamic LDS
+            switch (vec_length) {
+            case 1: return launch_ragged<1, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
+            case 2: return launch_ragged<2, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
+            case 4: return launch_ragged<4, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
+            case 8: return launch_ragged<8, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
+            default: return hipErrorInvalidValue;
+            }
+        }
         if (use_dma)
             return launch_spmm_mfma_dma<OutT>(m_vec, vec_length, k, n, waves, row_indices, row_offsets, column_indices,
                                               values, rhs, out, stream, batch);

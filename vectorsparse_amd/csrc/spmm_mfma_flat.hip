@@ -414,6 +414,8 @@ int launch_spmm_mfma_flat_static(int m_vec, int vec_length, int k, int n, int no
                                  const int *column_indices, const half_t *values, const half_t *rhs, half_t *out,
                                  hipStream_t stream)
 {
+    if (m_vec == 0 || k == 0) return hipSuccess;
+    if (k % 4 != 0) return hipErrorNotSupported;
     // the scratch must hold the partial tiles of at least 64 pieces, or the schedule degenerates
     const long long k_pad = (long long)ceil_div(k, 128) * 128;
     if (64LL * 2 * vec_length * k_pad * (long long)sizeof(float) > kScratchBytes) return hipErrorNotSupported;

@@ -48,10 +48,11 @@ __device__ __forceinline__ void wave_lds_fence()
 // at column offset `col_off` (element offset of the lane's first column inside a row), calls `prefetch()`
 // with those loads in flight, transposes the CPL x 8 block with v_perm_b32 and issues CPL MFMAs:
 // acc[c][e] += sum_j vec[4g + e][j] * rhs[col_j][col_off + c].
-template <int V, int CPL, bool IDX32, typename Prefetch>
+// RAGGED: the dense width is not a multiple of CPL; `valid` (0..CPL) halves of the lane's chunk exist.
+template <int V, int CPL, bool IDX32, bool RAGGED = false, typename Prefetch>
 __device__ __forceinline__ void spmm_mfma_step(const int *idx_s, const half_t *vec_s, const half_t *rhs, int n_cols,
                                                uint32_t col_off, int cs, int g, float4_t (&acc)[CPL],
-                                               Prefetch &&prefetch)
+                                               Prefetch &&prefetch, int valid = CPL)
 {
     const int4_t i_lo = *reinterpret_cast<const int4_t *>(idx_s + 8 * g);
     const int4_t i_hi = *reinterpret_cast<const int4_t *>(idx_s + 8 * g + 4);
@@ -63,7 +64,9 @@ __device__ __forceinline__ void spmm_mfma_step(const int *idx_s, const half_t *v
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         const int col = e < 4 ? i_lo[e] : i_hi[e - 4];
-        if constexpr (IDX32) {
+        if constexpr (RAGGED) {
+            load_ragged<CPL>(chunk[e], rhs + ((size_t)col * n_cols + col_off), valid);
+        } else if constexpr (IDX32) {
             // rhs has fewer than 2^31 elements: 32-bit offsets from a uniform base
             chunk[e].load(rhs + ((uint32_t)col * (uint32_t)n_cols + col_off));
         } else {

@@ -33,7 +33,9 @@ __device__ __forceinline__ void load_values(uint32_t (&dst)[V > 1 ? V / 2 : 1], 
     }
 }
 
-template <int V, int LR, typename OutT>
+// RAGGED: the dense width is not a multiple of 8 (rows of the dense operand and of the output start at any 2-byte
+// boundary, the last chunk of a row is cut): chunks are fetched and stored half by half.
+template <int V, int LR, typename OutT, bool RAGGED = false>
 __global__ void __launch_bounds__(1024)
 spmm_valu_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
                  const int *__restrict__ row_offsets, const int *__restrict__ column_indices,
@@ -57,8 +59,9 @@ spmm_valu_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
     const int cl = lane % LR;
     const int g = lane / LR;
     const int col0 = tile * TN + cl * 8;
-    const bool col_ok = col0 < n_cols;  // n_cols % 8 == 0
+    const bool col_ok = col0 < n_cols;  // n_cols % 8 == 0 unless RAGGED
     const half_t *rhs_col = rhs + (col_ok ? col0 : 0);
+    const int valid = !col_ok ? 0 : (n_cols - col0 < 8 ? n_cols - col0 : 8);  // RAGGED: halves of the chunk that exist
 
     float acc[V][8];
 #pragma unroll
@@ -85,7 +88,15 @@ spmm_valu_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
         }
         uint4_t b[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) b[u] = *reinterpret_cast<const uint4_t *>(rhs_col + (size_t)col[u] * n_cols);
+        for (int u = 0; u < U; ++u) {
+            if constexpr (RAGGED) {
+                RowChunk<8> chunk;
+                load_ragged<8>(chunk, rhs_col + (size_t)col[u] * n_cols, valid);
+                b[u] = chunk.d;
+            } else {
+                b[u] = *reinterpret_cast<const uint4_t *>(rhs_col + (size_t)col[u] * n_cols);
+            }
+        }
         if constexpr (V == 1) {
             // one multiply-add per column and nonzero: nothing to pair up
 #pragma unroll
@@ -123,8 +134,12 @@ spmm_valu_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
     if (n_waves * G == 1) {
         if (col_ok) {
 #pragma unroll
-            for (int v = 0; v < V; ++v)
-                store_converted<OutT, 8>(out + ((size_t)row * V + v) * n_cols + col0, acc[v]);
+            for (int v = 0; v < V; ++v) {
+                if constexpr (RAGGED)
+                    store_ragged<OutT, 8>(out + ((size_t)row * V + v) * n_cols + col0, acc[v], valid);
+                else
+                    store_converted<OutT, 8>(out + ((size_t)row * V + v) * n_cols + col0, acc[v]);
+            }
         }
         return;
     }
@@ -159,11 +174,14 @@ spmm_valu_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
             sum[0] += x[0]; sum[1] += x[1]; sum[2] += x[2]; sum[3] += x[3];
             sum[4] += y[0]; sum[5] += y[1]; sum[6] += y[2]; sum[7] += y[3];
         }
-        store_converted<OutT, 8>(out + ((size_t)row * V + v) * n_cols + col, sum);
+        if constexpr (RAGGED)
+            store_ragged<OutT, 8>(out + ((size_t)row * V + v) * n_cols + col, sum, n_cols - col);
+        else
+            store_converted<OutT, 8>(out + ((size_t)row * V + v) * n_cols + col, sum);
     }
 }
 
-template <int V, int LR, typename OutT>
+template <int V, int LR, typename OutT, bool RAGGED = false>
 static int launch_one(int m_vec, int k, int waves, const int *row_indices, const int *row_offsets,
                       const int *column_indices, const half_t *values, const half_t *rhs, OutT *out,
                       hipStream_t stream, const Batch &batch)
@@ -178,7 +196,7 @@ static int launch_one(int m_vec, int k, int waves, const int *row_indices, const
     if (waves > max_waves) waves = max_waves;
     if (waves < 1) waves = 1;
     const size_t lds = (waves * G > 1) ? (size_t)waves * G * V * TN * sizeof(float) : 0;
-    hipLaunchKernelGGL((spmm_valu_kernel<V, LR, OutT>), dim3((unsigned)blocks, (unsigned)batch.count),
+    hipLaunchKernelGGL((spmm_valu_kernel<V, LR, OutT, RAGGED>), dim3((unsigned)blocks, (unsigned)batch.count),
                        dim3(64 * waves), lds, stream, k, n_tiles, row_indices, row_offsets, column_indices, values,
                        rhs, out, batch.stride_a, batch.stride_b, batch.stride_out);
     return (int)hipGetLastError();
@@ -198,6 +216,8 @@ static int launch_lr(int m_vec, int k, int waves, const int *row_indices, const 
                      const int *column_indices, const half_t *values, const half_t *rhs, OutT *out,
                      hipStream_t stream, const Batch &batch)
 {
+    if (k % 8 != 0)  // any dense width: the half-by-half variant, 16 lanes (128 columns) per tile
+        return launch_one<V, 16, OutT, true>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
     const int lr = valu_tile_lanes(m_vec, k, batch.count);
     if (lr == 8) return launch_one<V, 8, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
     if (lr == 16) return launch_one<V, 16, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
@@ -212,7 +232,7 @@ int launch_spmm_valu(int m_vec, int vec_length, int k, int n, const int *row_ind
 {
     (void)n;
     if (m_vec == 0 || k == 0 || batch.count == 0) return hipSuccess;
-    if (k % 8 != 0 || batch.count > 65535) return hipErrorNotSupported;
+    if (batch.count > 65535) return hipErrorNotSupported;
     int waves = options().spmm_waves;
     if (waves <= 0) {
         const int lr = valu_tile_lanes(m_vec, k, batch.count);

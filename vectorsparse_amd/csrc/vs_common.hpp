@@ -80,6 +80,20 @@ struct RowChunk<4> {
     __device__ __forceinline__ uint32_t dword(int i) const { return d[i]; }
 };
 
+// The same chunk when the dense width is not a multiple of the chunk: rows then start at any 2-byte boundary and
+// the last chunk of a row is cut, so the halves are fetched one by one and those at or past `valid` read as zero.
+template <int CPL>
+__device__ __forceinline__ void load_ragged(RowChunk<CPL> &chunk, const half_t *p, int valid)
+{
+    const uint16_t *h = reinterpret_cast<const uint16_t *>(p);
+#pragma unroll
+    for (int i = 0; i < CPL / 2; ++i) {
+        const uint32_t lo = 2 * i < valid ? h[2 * i] : 0u;
+        const uint32_t hi = 2 * i + 1 < valid ? h[2 * i + 1] : 0u;
+        chunk.d[i] = lo | (hi << 16);
+    }
+}
+
 // Row-major lane order -> MFMA lane order for a 16-row x 64-byte block: lane (c = lane % 16, g = lane / 16)
 // takes the four registers of lane 4c + g (`src_lane_bytes` = (4c + g) * 4) through the LDS crossbar.
 __device__ __forceinline__ half8_t to_mfma_order(const uint4_t &x, int src_lane_bytes)
@@ -181,6 +195,15 @@ template <>
 __device__ __forceinline__ void store_converted<float, 1>(float *dst, const float *src)
 {
     dst[0] = src[0];
+}
+
+// The first `valid` of Count consecutive outputs, converted and stored one by one (no alignment assumed).
+template <typename OutT, int Count>
+__device__ __forceinline__ void store_ragged(OutT *dst, const float *src, int valid)
+{
+#pragma unroll
+    for (int i = 0; i < Count; ++i)
+        if (i < valid) dst[i] = (OutT)src[i];
 }
 
 // Process-wide launch-shape overrides (0 = automatic).
