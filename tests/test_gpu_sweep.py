@@ -39,6 +39,7 @@ def test_sweep_over_a_matrix_list(gpu, tmp_path, op):
     assert {r["bm"] for r in rows} == set(names[:2])
     assert {float(r["sparsity"]) for r in rows} == {0.8, 0.95}
     assert all(float(r["us"]) > 0 and float(r["speedup"]) > 0 for r in rows)
+    assert all(r["verified"] == "1" and float(r["max_rel_err"]) <= 1e-2 for r in rows), "every point is checked"
     for r in rows:
         k = int(r["N"] if op == "spmm" else r["K"])
         for kernel in (r["kernel"], "dense"):

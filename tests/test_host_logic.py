@@ -3,8 +3,9 @@ host-only capacity query."""
 import numpy as np
 import pytest
 
+from oracle import c_oracle as co
 from vectorsparse_amd import colvec_csr as cv
-from vectorsparse_amd import ops
+from vectorsparse_amd import ops, sweep
 
 
 def _largest_union(mask, rows):
@@ -139,3 +140,21 @@ def test_plot_reads_the_sweep_result_file(tmp_path):
     assert len(means) == 8
     assert means[("mma", 8, 256)] == pytest.approx((2.0, 4.0))      # sqrt(1 * 4), sqrt(2 * 8)
     assert means[("fpu", 2, 64)] == pytest.approx((1.0, 2.0))
+
+
+def test_the_sweep_check_catches_a_wrong_result():
+    """The driver's verification must fail on a result that is wrong in one sampled row."""
+    pat = sweep.spmm_grid_pattern(64, 256, 0.9, 8)
+    B = cv.dense_uniform(256, 64, seed=1)
+    ref = co.spmm_host_ref_f32(pat.m_vec, 8, 64, 256, pat.row_offsets, pat.column_indices, pat.values, B)
+    assert sweep.verify_spmm(pat, B, ref.astype(np.float16))[0]
+    bad = ref.astype(np.float16).copy()
+    bad[0, 5] += np.float16(1.0)
+    assert not sweep.verify_spmm(pat, B, bad)[0]
+    A = cv.dense_normal(64, 32, seed=2)
+    R = cv.dense_normal(256, 32, seed=3)
+    good = co.sddmm_host_ref_f32(pat.m_vec, 32, 8, pat.row_offsets, pat.column_indices, A, R)
+    assert sweep.verify_sddmm(pat, A, R, good.astype(np.float16))[0]
+    worse = good.astype(np.float16).copy()
+    worse[3] = -worse[3] + np.float16(2.0)
+    assert not sweep.verify_sddmm(pat, A, R, worse)[0]

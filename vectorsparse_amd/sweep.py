@@ -16,6 +16,11 @@ the entries [--start, --end) of --matrix-list (one path per line, relative to --
 reference's rn50_matrices.txt); the file's pattern is the sparse operand (SpMM) or the mask (SDDMM), --dimK
 the dense width / contraction length (job_launcher.py:41-50: a value <= 0 looks the layer up in --batchsizes,
 lines `layer,k`; --dimK-mul scales it), --dimV the vector lengths.
+Every point is verified before it is timed (the reference runs its own check on every benchmark it launches with
+func = 1, spmm_benchmark.cpp:206-225, sddmm_benchmark.cpp:279-301): one launch per kernel is compared with a
+float64 product on a sample of vector rows, by the reference's criterion (no element off by more than 0.5) and by
+the maximum relative error (denominator floored at 1e-2 rms); the result file carries `verified` and
+`max_rel_err` columns and the run ends with a non-zero status if any point failed.
 Durations are device time per launch (HIP events around a HIP-graph replay).  --csv-dir also writes one
 duration file per (benchmark, k, v, kernel) point under the names and in the record layout the reference's
 plot scripts read (file_name_server.py:6-45, :57-81), dense baseline included.
@@ -45,6 +50,70 @@ def spmm_bytes(pat, n_dense):
 def sddmm_bytes(pat, k):
     n_ref = int(np.unique(pat.column_indices[:pat.nnz_vec]).size)
     return 2 * pat.m * k + 2 * n_ref * k + 4 * pat.nnz_vec + 4 * (pat.m_vec + 1) + 4 * pat.m_vec + 2 * pat.nnz
+
+
+SDDMM_SIZES = (512, 1024, 2048, 4096)
+SDDMM_KS = (64, 128, 256)
+
+
+def spmm_grid_pattern(M, K, s, V):
+    """The synthetic SpMM point (M x K, sparsity s, vector length V): pattern with values, seeded by the point."""
+    from . import colvec_csr as cv
+    seed = (M * 1000003 + K * 10007 + int(round(s * 100)) * 101 + V) % (2 ** 31)
+    return cv.random_values(cv.uniform_pattern(M // V, K, s, seed, V), seed=V + 7)
+
+
+def sddmm_grid_pattern(M, s, V):
+    """The synthetic SDDMM mask (M x M, sparsity s, vector length V), seeded by the point."""
+    from . import colvec_csr as cv
+    seed = (M * 1000003 + int(round(s * 100)) * 101 + V) % (2 ** 31)
+    return cv.random_values(cv.uniform_pattern(M // V, M, s, seed, V), seed=V + 7)
+
+
+def sample_rows(m_vec, count=24):
+    """Vector rows a verification looks at: the first, the last and an even spread in between."""
+    if m_vec <= count:
+        return np.arange(m_vec)
+    return np.unique(np.linspace(0, m_vec - 1, count).round().astype(np.int64))
+
+
+def _verdict(got, ref):
+    got = np.asarray(got, dtype=np.float64).reshape(-1)
+    ref = np.asarray(ref, dtype=np.float64).reshape(-1)
+    if ref.size == 0:
+        return True, 0.0
+    floor = max(1e-2 * float(np.sqrt(np.mean(ref * ref))), 1e-30)
+    rel = float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), floor)))
+    ok = bool(np.all(np.isfinite(got))) and int(np.sum(np.abs(got - ref) > 0.5)) == 0 and rel <= 1e-2
+    return ok, rel
+
+
+def verify_spmm(pat, B, out_host):
+    """(passed, max relative error) of an SpMM result on a sample of vector rows against a float64 product."""
+    V = pat.vec_length
+    rows = sample_rows(pat.m_vec)
+    Bd = np.asarray(B, dtype=np.float64)
+    got, ref = [], []
+    for i in rows:
+        lo, hi = int(pat.row_offsets[i]), int(pat.row_offsets[i + 1])
+        vals = np.asarray(pat.values[lo:hi], dtype=np.float64).reshape(hi - lo, V)
+        ref.append(vals.T @ Bd[pat.column_indices[lo:hi]])
+        got.append(out_host[i * V:(i + 1) * V])
+    return _verdict(np.concatenate(got), np.concatenate(ref))
+
+
+def verify_sddmm(pat, A, B, out_host):
+    """(passed, max relative error) of an SDDMM result on a sample of vector rows against float64 dot products."""
+    V = pat.vec_length
+    rows = sample_rows(pat.m_vec)
+    Ad, Bd = np.asarray(A, dtype=np.float64), np.asarray(B, dtype=np.float64)
+    out_host = np.asarray(out_host).reshape(-1, V)
+    got, ref = [], []
+    for i in rows:
+        lo, hi = int(pat.row_offsets[i]), int(pat.row_offsets[i + 1])
+        ref.append(Bd[pat.column_indices[lo:hi]] @ Ad[i * V:(i + 1) * V].T)    # [nonzero][v]
+        got.append(out_host[lo:hi])
+    return _verdict(np.concatenate(got), np.concatenate(ref))
 
 
 def geomean(xs):
@@ -141,6 +210,7 @@ def main(argv=None):
                     help="SpMM through the batched entry point with the pattern's nonzero count and longest row "
                          "(workgroups sized by the real row lengths) instead of the reference-shaped entry points")
     ap.add_argument("--iters", type=int, default=100, help="launches per timed HIP-graph replay")
+    ap.add_argument("--no-verify", action="store_true", help="time without checking the results first")
     ap.add_argument("--csv-dir", default=None,
                     help="also write <csv-dir>/<spmm|sddmm>/<benchmark>_<kernel>_half_sort[_<alg>]_k<k>_v<v>.csv, one "
                          "profiler-style Duration record each, as the reference's plot scripts expect them")
@@ -172,28 +242,28 @@ def main(argv=None):
             for K in ks:
                 for s in ss:
                     def make(V, M=M, K=K, s=s):
-                        seed = (M * 1000003 + K * 10007 + int(round(s * 100)) * 101 + V) % (2 ** 31)
-                        return cv.uniform_pattern(M // V, K, s, seed, V)
+                        return spmm_grid_pattern(M, K, s, V)
                     cases.append(("synthetic/uniform/%g/m%d_k%d" % (s, M, K), s, make, widths))
     else:
-        sizes, ks, ss = ((512, 1024, 2048, 4096), (64, 128, 256), SPARSITIES) if not args.quick else \
+        sizes, ks, ss = (SDDMM_SIZES, SDDMM_KS, SPARSITIES) if not args.quick else \
             ((512, 2048), (64, 256), (0.7, 0.9, 0.98))
         widths = [k * args.dimK_mul for k in (int_list(args.dimK) if args.dimK else ks)]
         for M in sizes:
             for s in ss:
                 def make(V, M=M, s=s):
-                    seed = (M * 1000003 + int(round(s * 100)) * 101 + V) % (2 ** 31)
-                    return cv.uniform_pattern(M // V, M, s, seed, V)
+                    return sddmm_grid_pattern(M, s, V)
                 cases.append(("synthetic/uniform/%g/m%d_n%d" % (s, M, M), s, make, widths))
 
     def per_point(bm, dim_k, V, kernel, name, us):
         if args.csv_dir:
             write_duration_csv(duration_csv_path(args.csv_dir, bm, dim_k, V, kernel, args.op), name, us)
 
-    rows, dense_us = [], {}
+    rows, dense_us, failed = [], {}, 0
     for name, bucket, make, widths in cases:
         for V in vs:
-            pat = cv.random_values(make(V), seed=V + 7)
+            pat = make(V)
+            if pat.values is None:
+                pat = cv.random_values(pat, seed=V + 7)
             if pat.nnz_vec == 0:
                 continue
             M, n = pat.m, pat.n
@@ -202,8 +272,10 @@ def main(argv=None):
             for k in widths:
                 if spmm:
                     # C[M, k] = A_sparse[M, n] B[n, k]
-                    B = torch.from_numpy(cv.dense_uniform(n, k, seed=11)).cuda()
+                    B_host = cv.dense_uniform(n, k, seed=11)
+                    B = torch.from_numpy(B_host).cuda()
                     out = torch.empty((M, k), dtype=torch.float16, device="cuda")
+                    check = lambda: verify_spmm(pat, B_host, out.cpu().numpy())
                     if (M, n, k) not in dense_us:
                         A = torch.randn((M, n), dtype=torch.float16, device="cuda")
                         dense_us[(M, n, k)] = time_launches(torch, lambda: torch.matmul(A, B, out=out), args.iters)
@@ -216,6 +288,8 @@ def main(argv=None):
                     A = torch.randn((M, k), dtype=torch.float16, device="cuda")
                     B = torch.randn((n, k), dtype=torch.float16, device="cuda")
                     out = torch.empty((pat.nnz_vec, V), dtype=torch.float16, device="cuda")
+                    A_host, B_host = A.cpu().numpy(), B.cpu().numpy()
+                    check = lambda: verify_sddmm(pat, A_host, B_host, out.cpu().numpy())
                     if (M, n, k) not in dense_us:
                         full = torch.empty((M, n), dtype=torch.float16, device="cuda")
                         dense_us[(M, n, k)] = time_launches(torch, lambda: torch.matmul(A, B.t(), out=full), args.iters)
@@ -226,18 +300,35 @@ def main(argv=None):
                 dense = dense_us[(M, n, k)]
                 per_point(name, k, V, "dense", "hipblaslt_gemm_f16", dense)
                 for kern in ("wmma", "cuda"):
+                    verified, rel = "", float("nan")
+                    if not args.no_verify:
+                        out.fill_(float("nan"))
+                        run[kern]()
+                        torch.cuda.synchronize()
+                        ok, rel = check()
+                        verified = int(ok)
+                        if not ok:
+                            failed += 1
+                            print("VERIFICATION FAILED: %s k=%d V=%d %s max relative error %.3e" % (name, k, V, kern, rel),
+                                  flush=True)
                     us = time_launches(torch, run[kern], args.iters)
                     per_point(name, k, V, kern, names[kern], us)
                     rows.append({"op": args.op, "bm": name, "k": k, "M": M, "K": n if spmm else k, "N": k if spmm else n,
                                  "sparsity": round(s, 4), "V": V, "kernel": kern, "nnz_vec": pat.nnz_vec,
                                  "us": round(us, 3), "dense_us": round(dense, 3), "speedup": round(dense / us, 4),
-                                 "tflops": round(flops / us * 1e-6, 3), "gbs": round(nbytes / us * 1e-3, 1)})
+                                 "tflops": round(flops / us * 1e-6, 3), "gbs": round(nbytes / us * 1e-3, 1),
+                                 "verified": verified, "max_rel_err": "%.3e" % rel})
                 print("%s M=%d n=%d k=%d s=%.2f V=%d  wmma %.2f us  cuda %.2f us  dense %.2f us" % (
                     name, M, n, k, s, V, rows[-2]["us"], rows[-1]["us"], dense), flush=True)
     if not rows:
         raise SystemExit("nothing to run")
     report(args.out, rows, "SpMM: geometric-mean speed-up over dense fp16 GEMM (hipBLASLt)" if spmm else
            "SDDMM: geometric-mean speed-up over the dense fp16 product A B^T (hipBLASLt)")
+    if failed:
+        print("%d point(s) failed verification" % failed, flush=True)
+        return 1
+    if not args.no_verify:
+        print("all %d points verified" % len(rows), flush=True)
     return 0
 
 
