@@ -44,8 +44,10 @@ def sddmm_algorithmic_bytes(pat, k):
             + 2 * pat.nnz)
 
 
-def time_graph(torch, fn, steps, warmup):
-    """Capture `steps` calls of fn into a HIP graph; return (wall ms/step, event ms/step)."""
+def time_graph(torch, fn, steps, warmup, replays=7):
+    """Capture `steps` calls of fn into a HIP graph and replay it `replays` times; return the medians of
+    (wall ms/step, event ms/step).  One replay now and then runs at twice its usual time (clock ramp after an
+    idle gap) and a single replay of a short graph carries its fixed start-up cost, so no single replay is used."""
     for _ in range(max(warmup, 1)):
         fn()
     torch.cuda.synchronize()
@@ -61,16 +63,22 @@ def time_graph(torch, fn, steps, warmup):
             fn()
     graph.replay()  # untimed: first replay uploads the graph
     torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    e0.record()
-    graph.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
+    walls, events = [], []
+    for _ in range(max(1, replays)):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        walls.append((t1 - t0) * 1e3 / steps)
+        events.append(e0.elapsed_time(e1) / steps)
+    walls.sort()
+    events.sort()
+    return walls[len(walls) // 2], events[len(events) // 2]
 
 
 def time_cold(torch, fn, samples=20):
@@ -93,17 +101,42 @@ def time_cold(torch, fn, samples=20):
     return times[len(times) // 2]
 
 
-def measured_traffic(path):
-    """HBM-side bytes per launch of the headline kernel, from the committed rocprofv3 --pmc summary
-    (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a copy of known size)."""
+def kernel_source_tag(*names):
+    """First 16 hex digits of the SHA-256 of the kernel sources a counter summary belongs to."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in names:
+        with open(os.path.join(ROOT, "vectorsparse_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+SPMM_SOURCES = ("spmm_mfma.hip", "spmm_mfma_step.hpp", "vs_common.hpp")
+SDDMM_SOURCES = ("sddmm_mfma.hip", "vs_common.hpp")
+
+
+def measured_traffic(path, sources):
+    """(HBM-side bytes per launch, note) of a kernel from the committed rocprofv3 --pmc summary (FETCH_SIZE and
+    WRITE_SIZE, each scaled by what the same counter reads for a copy of known size).  The summary names the
+    kernel sources it was measured on (`kernel_source_tag`); when they have changed since, the figure is stale
+    and None is returned with a note saying so."""
+    value, tag = None, None
     try:
         with open(path) as f:
             for ln in f:
                 if ln.startswith("traffic_bytes_per_launch"):
-                    return float(ln.split()[1])
+                    value = float(ln.split()[1])
+                elif ln.startswith("kernel_source_tag"):
+                    tag = ln.split()[1]
     except OSError:
-        pass
-    return None
+        return None, "no counter summary at %s" % os.path.relpath(path, ROOT)
+    now = kernel_source_tag(*sources)
+    if value is None:
+        return None, "no traffic figure in %s" % os.path.relpath(path, ROOT)
+    if tag != now:
+        return None, "%s was measured on kernel sources %s, the sources are now %s: stale, not reported" % (
+            os.path.relpath(path, ROOT), tag, now)
+    return value, "from %s (kernel sources %s)" % (os.path.relpath(path, ROOT), now)
 
 
 def time_eager(torch, fn, steps, warmup):
@@ -150,17 +183,37 @@ def cpu_baseline(pat, B, n_dense, flops, budget_s=12.0):
     }
 
 
+PMC_MODES = ["spmm", "spmm_largest", "spmm_dma", "spmm_split_rows", "sddmm", "attention", "attention_window"]
+
+
+def largest_sweep_point(cv):
+    """The largest single-GPU point of the ResNet-50-shaped sweep: M = 2048, K = 4608, N = 256, V = 8, 90 %."""
+    pat = cv.random_values(cv.uniform_pattern(2048 // 8, 4608, 0.9, seed=3, vec_length=8), seed=4)
+    return pat, cv.dense_uniform(4608, 256, seed=5)
+
+
+def skewed_point(cv, np):
+    """Pareto-distributed row lengths (mean about 280 vectors, the longest row dense), 1024 vector rows x 4608."""
+    rng = np.random.default_rng(0)
+    m_vec, K = 1024, 4608
+    lengths = np.minimum((rng.pareto(1.5, m_vec) + 0.3) * 150, K).astype(np.int64)
+    lengths = lengths[rng.permutation(m_vec)]
+    ro, ci = cv._pattern_from_lengths(rng, m_vec, K, lengths)
+    return cv.random_values(cv.ColVecCSR(m_vec, K, 8, ro, ci), 1), cv.dense_uniform(K, 256, seed=2)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--pmc", nargs="?", const="spmm", default=None, choices=["spmm", "sddmm", "attention", "attention_window"],
+    ap.add_argument("--pmc", nargs="?", const="spmm", default=None, choices=PMC_MODES,
                     help="counter-collection mode for `rocprofv3 --pmc`: a 64 MiB device copy of known size "
-                         "(calibration), then a few eager launches of one kernel (the headline SpMM, the "
-                         "config-4 SDDMM, the config-5 attention layer with its plan, or the same layer with a "
-                         "plain 513-wide window mask, whose unions of up to 634 columns are streamed through LDS), nothing else")
+                         "(calibration), then ten eager launches of one kernel and nothing else: the headline SpMM "
+                         "(config 2), the largest sweep point (2048 x 4608 at 90 %%), config 2 on the LDS-DMA gather "
+                         "variant, the split-row SpMM on Pareto-distributed rows, the config-4 SDDMM, the config-5 "
+                         "attention layer with its plan, or that layer with a plain 513-wide window mask")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the SpMM/SDDMM path has no multi-GPU leg (rows shard with no "
@@ -170,6 +223,7 @@ def main():
     import numpy as np
     import torch
 
+    from vectorsparse_amd import _lib
     from vectorsparse_amd import colvec_csr as cv
     from vectorsparse_amd import ops
 
@@ -191,6 +245,16 @@ def main():
     def step():
         prob.spmm(Bd, kernel="wmma", out=out)
 
+    # ---- SDDMM companion point (config 4: M = N = 2048, K = 64, V = 8, 90 %)
+    mask = cv.uniform_pattern(2048 // 8, 2048, 0.9, seed=4, vec_length=8)
+    lhs = torch.from_numpy(cv.dense_normal(2048, 64, seed=14)).cuda()
+    rhs = torch.from_numpy(cv.dense_normal(2048, 64, seed=24)).cuda()
+    sprob = ops.DeviceProblem(mask)
+    sout = torch.empty((mask.nnz_vec, 8), dtype=torch.float16, device="cuda")
+
+    def sddmm_step():
+        sprob.sddmm(lhs, rhs, kernel="wmma", out=sout)
+
     if args.pmc:
         src = torch.zeros(32 * 1024 * 1024, dtype=torch.float16, device="cuda")   # 64 MiB read + 64 MiB written
         dst = torch.empty_like(src)
@@ -198,19 +262,37 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         info = {"pmc_mode": args.pmc, "copy_bytes_each_way": src.numel() * 2}
-        if args.pmc == "spmm":
+        if args.pmc in ("spmm", "spmm_dma"):
+            if args.pmc == "spmm_dma":
+                _lib.set_option("spmm_gather", 2)
             for _ in range(10):
                 step()
             info["algorithmic_bytes"] = alg_bytes
-        elif args.pmc == "sddmm":
-            mask = cv.uniform_pattern(2048 // 8, 2048, 0.9, seed=4, vec_length=8)
-            lhs = torch.from_numpy(cv.dense_normal(2048, 64, seed=14)).cuda()
-            rhs = torch.from_numpy(cv.dense_normal(2048, 64, seed=24)).cuda()
-            sprob = ops.DeviceProblem(mask)
-            sout = torch.empty((mask.nnz_vec, 8), dtype=torch.float16, device="cuda")
+            info["kernel_source_tag"] = kernel_source_tag(*SPMM_SOURCES)
+        elif args.pmc == "spmm_largest":
+            lpat, lB = largest_sweep_point(cv)
+            lprob = ops.DeviceProblem(lpat, sort=True)
+            lBd = torch.from_numpy(lB).cuda()
+            lout = torch.empty((lpat.m, 256), dtype=torch.float16, device="cuda")
             for _ in range(10):
-                sprob.sddmm(lhs, rhs, kernel="wmma", out=sout)
+                lprob.spmm(lBd, kernel="wmma", out=lout)
+            info["algorithmic_bytes"] = spmm_algorithmic_bytes(lpat, 256)
+            info["nonzero_vectors"] = int(lpat.nnz_vec)
+            info["kernel_source_tag"] = kernel_source_tag(*SPMM_SOURCES)
+        elif args.pmc == "spmm_split_rows":
+            kpat, kB = skewed_point(cv, np)
+            kprob = ops.DeviceProblem(kpat, sort=True)
+            kBd = torch.from_numpy(kB).cuda()
+            kout = torch.empty((kpat.m, 256), dtype=torch.float16, device="cuda")
+            for _ in range(10):
+                kprob.spmm(kBd, kernel="wmma", out=kout, split_rows=True)
+            info["algorithmic_bytes"] = spmm_algorithmic_bytes(kpat, 256)
+            info["nonzero_vectors"] = int(kpat.nnz_vec)
+        elif args.pmc == "sddmm":
+            for _ in range(10):
+                sddmm_step()
             info["algorithmic_bytes"] = sddmm_algorithmic_bytes(mask, 64)
+            info["kernel_source_tag"] = kernel_source_tag(*SDDMM_SOURCES)
         else:
             heads, seq, dim = 16, 4096, 64
             if args.pmc == "attention_window":
@@ -245,20 +327,51 @@ def main():
     max_rel = float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), floor)))
     errors = int(np.sum(np.abs(got - ref) > 0.5))
 
+    # ---- the dispatch floor of the headline launch: a kernel that does nothing on the same grid.  No kernel of
+    # that shape finishes sooner, so algorithmic bytes / this time is the ceiling of `roofline.frac` on config 2.
+    floor_lib = _lib.lib()
+
+
+    def probe(threads):  # on whatever stream is current at the call (the capture stream inside time_graph)
+        return lambda: floor_lib.vs_launch_floor_probe(256, threads, torch.cuda.current_stream().cuda_stream)
+
+    _, floor_ms = time_graph(torch, probe(1024), args.steps, args.warmup)
+    _, floor_small_ms = time_graph(torch, probe(64), args.steps, args.warmup)
+
     # ---- dense fp16 GEMM (hipBLASLt through torch) on the same M x K x N, same timing method
     Ad = torch.randn((M, K), dtype=torch.float16, device="cuda")
     dense_out = torch.empty((M, N), dtype=torch.float16, device="cuda")
     _, dense_ms = time_graph(torch, lambda: torch.matmul(Ad, Bd, out=dense_out), args.steps, args.warmup)
 
-    # ---- SDDMM companion point (config 4: M = N = 2048, K = 64, V = 8, 90 %)
-    mask = cv.uniform_pattern(2048 // 8, 2048, 0.9, seed=4, vec_length=8)
-    lhs = torch.from_numpy(cv.dense_normal(2048, 64, seed=14)).cuda()
-    rhs = torch.from_numpy(cv.dense_normal(2048, 64, seed=24)).cuda()
-    sprob = ops.DeviceProblem(mask)
-    sout = torch.empty((mask.nnz_vec, 8), dtype=torch.float16, device="cuda")
-    _, sddmm_ms = time_graph(torch, lambda: sprob.sddmm(lhs, rhs, kernel="wmma", out=sout), args.steps, args.warmup)
+    # ---- the largest single-GPU point of the sweep (2048 x 4608 x 256, 90 %): the end where the roofline counts
+    lpat, lB = largest_sweep_point(cv)
+    lprob = ops.DeviceProblem(lpat, sort=True)
+    lBd = torch.from_numpy(lB).cuda()
+    lout = torch.empty((lpat.m, 256), dtype=torch.float16, device="cuda")
+    _, large_ms = time_graph(torch, lambda: lprob.spmm(lBd, kernel="wmma", out=lout), args.steps, args.warmup)
+    large_bytes = spmm_algorithmic_bytes(lpat, 256)
+    lA = torch.randn((lpat.m, 4608), dtype=torch.float16, device="cuda")
+    _, large_dense_ms = time_graph(torch, lambda: torch.matmul(lA, lBd, out=lout), args.steps, args.warmup)
+
+    # ---- skewed rows: reference-shaped entry, batched entry with the row-length hints, split-row schedule
+    kpat, kB = skewed_point(cv, np)
+    kprob = ops.DeviceProblem(kpat, sort=True)
+    kBd = torch.from_numpy(kB).cuda()
+    kout = torch.empty((kpat.m, 256), dtype=torch.float16, device="cuda")
+    skew_steps = max(20, args.steps // 4)
+    _, skew_plain_ms = time_graph(torch, lambda: kprob.spmm(kBd, out=kout), skew_steps, 3)
+    _, skew_hint_ms = time_graph(torch, lambda: kprob.spmm(kBd, out=kout, row_length_hint=True), skew_steps, 3)
+    _, skew_split_ms = time_graph(torch, lambda: kprob.spmm(kBd, out=kout, split_rows=True), skew_steps, 3)
+    upat = cv.random_values(cv.uniform_pattern(kpat.m_vec, kpat.n, 1 - kpat.nnz_vec / (kpat.m_vec * kpat.n), 1, 8), 1)
+    uprob = ops.DeviceProblem(upat, sort=True)
+    _, skew_uniform_ms = time_graph(torch, lambda: uprob.spmm(kBd, out=kout), skew_steps, 3)
+
+    # ---- SDDMM config 4
+    _, sddmm_ms = time_graph(torch, sddmm_step, args.steps, args.warmup)
     sddmm_flops = 2.0 * mask.nnz * 64
     sddmm_bytes = sddmm_algorithmic_bytes(mask, 64)
+    full = torch.empty((2048, 2048), dtype=torch.float16, device="cuda")
+    _, sddmm_dense_ms = time_graph(torch, lambda: torch.matmul(lhs, rhs.t(), out=full), args.steps, args.warmup)
 
     # ---- fixed-mask sparse attention layer (config 5: 16 heads, seq 4096, d 64, V = 8 band + strided mask)
     heads, seq, dim = 16, 4096, 64
@@ -275,18 +388,32 @@ def main():
         s_ = torch.matmul(q, kk_.transpose(1, 2))
         return torch.matmul(torch.softmax(s_ * 0.125, dim=-1), vv)
 
-    _, dense_attn_ms = time_graph(torch, dense_attention, 5, 2)
+    _, dense_attn_ms = time_graph(torch, dense_attention, 5, 2, replays=3)
     attn_flops = 2.0 * amask.nnz * heads * dim * 2
     # the same layer with a plain 513-wide window (unions of up to 634 columns per 16 vector rows)
     wmask = cv.band_strided_pattern(seq, 8, band_half_width=256, stride=seq)
     wlayer = ops.SparseAttention(wmask)
     _, window_ms = time_graph(torch, lambda: wlayer.forward(q, kk_, vv, out=ctx), attn_steps, 3)
 
+    # ---- cold caches (how the reference measures: Nsight --cache-control all)
     cold_ms = time_cold(torch, step)
     cold_dense_ms = time_cold(torch, lambda: torch.matmul(Ad, Bd, out=dense_out))
+    cold_large_ms = time_cold(torch, lambda: lprob.spmm(lBd, kernel="wmma", out=lout), samples=10)
+    cold_sddmm_ms = time_cold(torch, sddmm_step, samples=10)
+    cold_attn_ms = time_cold(torch, lambda: layer.forward(q, kk_, vv, scores=scores, out=ctx), samples=10)
 
     achieved = alg_bytes / (ev_ms * 1e-3) * 1e-9
-    traffic = measured_traffic(os.path.join(ROOT, "profiles", "spmm_mfma_config2_pmc.txt"))
+    traffic, traffic_note = measured_traffic(os.path.join(ROOT, "profiles", "spmm_mfma_config2_pmc.txt"), SPMM_SOURCES)
+    large_traffic, _ = measured_traffic(os.path.join(ROOT, "profiles", "spmm_mfma_largest_pmc.txt"), SPMM_SOURCES)
+    sddmm_traffic, sddmm_note = measured_traffic(os.path.join(ROOT, "profiles", "sddmm_mfma_config4_pmc.txt"), SDDMM_SOURCES)
+
+    def hbm(nbytes, ms, traffic_bytes=None, **more):
+        gbs = nbytes / (ms * 1e-3) * 1e-9
+        d = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+             "traffic": traffic_bytes, "algorithmic_bytes": nbytes, "avg_launch_us": ms * 1e3}
+        d.update(more)
+        return d
+
     line = {
         "metric": "SpMM effective TFLOP/s (2*nnz*N), fp16 V=8, 90% sparse",
         "value": flops / (wall_ms * 1e-3) * 1e-12,
@@ -302,28 +429,47 @@ def main():
         "data": "synthetic",
         "config": {"workload": "config2: single SpMM M=512 K=4608 N=256 V=8 sparsity=0.9 (binomial rows), "
                                "sorted row swizzle, fp16 out / fp32 accumulate",
-                   "nnz_vec": pat.nnz_vec, "launch": "HIP graph of `steps` operator calls"},
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                     "kernel": "spmm_mfma_kernel<V=8>", "algorithmic_bytes": alg_bytes,
-                     "avg_launch_us": ev_ms * 1e3},
+                   "nnz_vec": pat.nnz_vec,
+                   "launch": "HIP graph of `steps` operator calls, median of 7 replays"},
+        "roofline": hbm(alg_bytes, ev_ms, traffic, kernel="spmm_mfma_kernel<V=8>", traffic_note=traffic_note,
+                        caches="warm: the 3.2 MB working set stays in the Infinity Cache between launches (the L2s "
+                               "start every launch cold); see extra.cold_cache",
+                        frac_cold=alg_bytes / (cold_ms * 1e-3) * 1e-9 / HBM_PEAK_GBS,
+                        ceiling_frac=alg_bytes / (floor_ms * 1e-3) * 1e-9 / HBM_PEAK_GBS,
+                        ceiling_note="a kernel that does nothing on this launch's grid (256 workgroups of 1024 threads) "
+                                     "takes extra.launch_floor.empty_grid_us: the HBM-roofline time of config 2 "
+                                     "(0.40 us) is a quarter of it, so frac cannot exceed ceiling_frac on this config"),
         "parity": {"max_rel_err": max_rel, "errors_gt_0.5": errors},
         "extra": {
             "eager_ms_per_step": eager_wall_ms,
             "batched_entry_with_nonzero_count_ms": hinted_ms,
             "dense_gemm_ms": dense_ms,
             "speedup_vs_dense_gemm": dense_ms / ev_ms,
-            "cold_cache_launch_us": cold_ms * 1e3,
-            "cold_cache_dense_gemm_us": cold_dense_ms * 1e3,
+            "launch_floor": {"empty_grid_us": floor_ms * 1e3, "empty_grid_one_wave_per_workgroup_us": floor_small_ms * 1e3,
+                             "frac_of_floor": floor_ms / ev_ms},
+            "cold_cache": {"spmm_config2_us": cold_ms * 1e3, "dense_gemm_config2_us": cold_dense_ms * 1e3,
+                           "spmm_largest_us": cold_large_ms * 1e3, "sddmm_config4_us": cold_sddmm_ms * 1e3,
+                           "attention_config5_us": cold_attn_ms * 1e3},
+            "spmm_largest_sweep_point": dict(
+                hbm(large_bytes, large_ms, large_traffic),
+                workload="M=2048 K=4608 N=256 V=8 sparsity=0.9", tflops=2.0 * lpat.nnz * 256 / (large_ms * 1e-3) * 1e-12,
+                gather_tbs=lpat.nnz_vec * 512 / (large_ms * 1e-3) * 1e-12, dense_gemm_us=large_dense_ms * 1e3,
+                speedup_vs_dense_gemm=large_dense_ms / large_ms),
+            "spmm_skewed_rows": {"workload": "1024 vector rows x 4608, Pareto row lengths (mean %.0f, longest %d), N=256"
+                                             % (kpat.nnz_vec / kpat.m_vec, int(np.diff(kpat.row_offsets).max())),
+                                 "reference_entry_us": skew_plain_ms * 1e3, "hinted_batched_entry_us": skew_hint_ms * 1e3,
+                                 "split_rows_entry_us": skew_split_ms * 1e3,
+                                 "uniform_rows_same_nonzeros_us": skew_uniform_ms * 1e3},
+            "sddmm_config4_k64": dict(
+                hbm(sddmm_bytes, sddmm_ms, sddmm_traffic, traffic_note=sddmm_note, kernel="sddmm_mfma_kernel<V=8>"),
+                ms=sddmm_ms, tflops=sddmm_flops / (sddmm_ms * 1e-3) * 1e-12, dense_product_us=sddmm_dense_ms * 1e3,
+                speedup_vs_dense=sddmm_dense_ms / sddmm_ms),
             "attention_window513": {"layer_ms": window_ms, "density": 1.0 - wmask.sparsity,
                                     "tflops": 2.0 * wmask.nnz * heads * dim * 2 / (window_ms * 1e-3) * 1e-12},
             "attention_config5": {"layer_ms": attn_ms, "density": 1.0 - amask.sparsity,
                                   "tflops": attn_flops / (attn_ms * 1e-3) * 1e-12,
                                   "dense_masked_attention_ms": dense_attn_ms,
                                   "speedup_vs_dense": dense_attn_ms / attn_ms},
-            "sddmm_config4_k64": {"ms": sddmm_ms, "tflops": sddmm_flops / (sddmm_ms * 1e-3) * 1e-12,
-                                  "hbm_gbs": sddmm_bytes / (sddmm_ms * 1e-3) * 1e-9,
-                                  "hbm_frac": sddmm_bytes / (sddmm_ms * 1e-3) * 1e-9 / HBM_PEAK_GBS},
         },
     }
     if not args.no_cpu:

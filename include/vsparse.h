@@ -331,6 +331,14 @@ void vs_identity_row_swizzle(int rows, int *row_indices);
 void vs_sorted_row_swizzle(int rows, const int *row_offsets, int *row_indices);
 
 /*
+ * Measurement aid: launches a kernel that does nothing on a grid of `blocks` workgroups of
+ * `threads_per_block` threads (1..1024), asynchronously on `stream`.  Timing it prices the dispatch
+ * floor of a launch shape, below which no kernel of that shape can finish.  No counterpart in the
+ * reference.
+ */
+int vs_launch_floor_probe(int blocks, int threads_per_block, void *stream);
+
+/*
  * Launch-shape tuning knob (process-wide, not thread-safe against concurrent
  * launches).  Names: "spmm_waves" (waves per workgroup, 0 = automatic),
  * "spmm_cols_per_lane" (4, 8, 0 = automatic), "spmm_gather" (how the MFMA SpMM
@@ -340,7 +348,8 @@ void vs_sorted_row_swizzle(int rows, const int *row_offsets, int *row_indices);
  * "spmm_flat_piece" (nonzero vectors
  * per wave of the split-row SpMM, rounded up to 32, 0 = automatic), "spmm_flat_waves"
  * (its waves per workgroup, 1..16, 0 = automatic), "sddmm_slots" (waves per
- * vector row, 0 = automatic), "sddmm_block_waves" (1..16, 0 = automatic),
+ * vector row, 0 = automatic), "sddmm_group" (16-vector groups per wave step of the
+ * MFMA SDDMM: 1, 2, 4, 0 = automatic), "sddmm_block_waves" (1..16, 0 = automatic),
  * "sddmm_flat_supers" (super-groups per wave of algorithm 2, 1..16, 0 = automatic),
  * "attention_waves" (1..8, 0 = automatic), "attention_chunk" (nonzero vectors per
  * LDS chunk of the one-row-per-workgroup attention kernel, 0 = automatic).

@@ -41,6 +41,7 @@ SIGNATURES = {
     "vs_sparse_softmax_f16": ([_int] * 3 + [_vp] * 2 + [_vp, _ll, _vp, _ll, ctypes.c_float, _vp], _int),
     "vs_identity_row_swizzle": ([_int, _vp], None),
     "vs_sorted_row_swizzle": ([_int, _vp, _vp], None),
+    "vs_launch_floor_probe": ([_int, _int, _vp], _int),
     "vs_set_option": ([ctypes.c_char_p, _int], _int),
 }
 

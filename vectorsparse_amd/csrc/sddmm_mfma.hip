@@ -277,7 +277,7 @@ static int launch_one(int m_vec, int k, int nonzeros_vec, const int *row_indices
             return (int)hipGetLastError();
         }
     }
-    const int slots = sddmm_auto_slots((long long)m_vec * batch.count, (long long)nonzeros_vec * batch.count, 16 * GRP);
+    const int slots = sddmm_auto_slots((long long)m_vec * batch.count, (long long)nonzeros_vec * batch.count, 16 * GRP, true);
     const long long waves = (long long)m_vec * slots;
     const long long blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
@@ -287,32 +287,72 @@ static int launch_one(int m_vec, int k, int nonzeros_vec, const int *row_indices
     return (int)hipGetLastError();
 }
 
+// Vectors per wave step (16 * GRP): as many as the registers allow for the contraction length while the mask is
+// large enough to fill the chip with such waves, fewer on small masks so that the launch has about 4096 working
+// waves (a wave's time is one chain of dependent loads whatever its step holds, so on a small mask more, lighter
+// waves finish sooner).
+static int sddmm_group(int k, long long nonzeros_vec)
+{
+    const int forced = options().sddmm_group;
+    int grp = k <= 64 ? 4 : (k <= 128 ? 2 : 1);
+    if (forced == 1 || forced == 2 || forced == 4) return forced < grp ? forced : grp;
+    while (grp > 1 && nonzeros_vec / (16 * grp) < 4096) grp >>= 1;
+    return grp;
+}
+
+template <int V, int KS, typename OutT>
+static int launch_grp(int grp, int m_vec, int k, int nonzeros_vec, const int *row_indices, const int *row_offsets,
+                      const int *col_indices, const half_t *lhs, const half_t *rhs, OutT *out, hipStream_t stream,
+                      const Batch &batch)
+{
+    if constexpr (KS <= 2) {
+        if (grp == 4) return launch_one<V, KS, 4, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    }
+    if constexpr (KS <= 4) {
+        if (grp >= 2) return launch_one<V, KS, 2, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    }
+    return launch_one<V, KS, 1, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+}
+
 template <int V, typename OutT>
 static int launch_ks(int m_vec, int k, int nonzeros_vec, const int *row_indices, const int *row_offsets,
                      const int *col_indices, const half_t *lhs, const half_t *rhs, OutT *out, hipStream_t stream,
                       const Batch &batch)
 {
-    if (k <= 32) return launch_one<V, 1, 4, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
-    if (k <= 64) return launch_one<V, 2, 4, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
-    if (k <= 128) return launch_one<V, 4, 2, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    const int grp = sddmm_group(k, (long long)nonzeros_vec * batch.count);
+    if (k <= 32) return launch_grp<V, 1, OutT>(grp, m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    if (k <= 64) return launch_grp<V, 2, OutT>(grp, m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
+    if (k <= 128) return launch_grp<V, 4, OutT>(grp, m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
     if (k <= 256) return launch_one<V, 8, 1, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
     return launch_one<V, 0, 4, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
 }
 
-// Waves per vector row.  Waves are independent (no reduction): twice as many as an average row has
-// super-groups, so that a row twice the average still gets one super-group per wave (longer rows loop),
-// capped so that the launch stays near the number of wave slots of the chip.  A wave that finds no
-// super-group of its own exits after two scalar loads; what it costs is its share of a workgroup
-// dispatch, which is why workgroups are eight waves wide.
-int sddmm_auto_slots(long long m_vec, long long nonzeros_vec, int group)
+// Waves per vector row.  Waves are independent (no reduction).  A wave that finds no super-group of its own exits
+// after two scalar loads; what it costs is its share of a workgroup dispatch, which is why workgroups are eight
+// waves wide.  Rows with more super-groups than waves loop.
+// MFMA kernel: one wave per super-group of an average row, capped so that the launch has about 2048 to 4096 waves
+// (eight per row up to 512 rows; measured on masks of 512 to 4096 rows and columns, K = 64 and 128, 70 to 95 %
+// sparse: within 5 % of the best choice, where the rule below was 10 to 30 % off because half of its waves found
+// nothing to do).
+// Fine-grained kernel: twice as many as an average row has super-groups, so that a row twice the average still
+// gets one super-group per wave, capped near the number of wave slots of the chip (it gains from up to 32 waves
+// per row on the denser masks: 2048 x 2048 at 70 %, K = 128, 9.1 us against 12.1 us with eight).
+int sddmm_auto_slots(long long m_vec, long long nonzeros_vec, int group, bool mfma)
 {
     int slots = options().sddmm_slots;
     if (slots > 0) return slots;
     if (m_vec < 1) m_vec = 1;
     const long long avg = (nonzeros_vec + m_vec - 1) / m_vec;
     const long long avg_groups = (avg + group - 1) / group;
-    const long long want = (8192 + m_vec - 1) / m_vec;
-    const long long pick = 2 * avg_groups < want ? 2 * avg_groups : want;
+    long long pick;
+    if (mfma) {
+        long long cap = m_vec <= 1024 ? 2048 / m_vec : 8192 / m_vec;
+        if (m_vec <= 1024 && cap < 8) cap = 8;
+        pick = avg_groups < cap ? avg_groups : cap;
+    } else {
+        const long long want = (8192 + m_vec - 1) / m_vec;
+        pick = 2 * avg_groups < want ? 2 * avg_groups : want;
+    }
     return pick < 1 ? 1 : (int)pick;
 }
 

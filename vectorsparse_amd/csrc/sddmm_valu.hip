@@ -156,7 +156,7 @@ static int launch_one(int m_vec, int k, int nonzeros_vec, const int *row_indices
                       const Batch &batch)
 {
     constexpr int kWavesPerBlock = 4;
-    const int slots = sddmm_auto_slots((long long)m_vec * batch.count, (long long)nonzeros_vec * batch.count, 64 / LK);
+    const int slots = sddmm_auto_slots((long long)m_vec * batch.count, (long long)nonzeros_vec * batch.count, 64 / LK, false);
     const long long waves = (long long)m_vec * slots;
     const long long blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks > 0x7fffffffLL) return hipErrorNotSupported;

@@ -215,6 +215,7 @@ struct Options {
     int spmm_flat_waves = 0;    // split-row SpMM: waves per workgroup, 0 = automatic
     int sddmm_slots = 0;
     int sddmm_block_waves = 0;
+    int sddmm_group = 0;        // MFMA SDDMM: 16-vector groups per wave step (1, 2, 4), 0 = automatic
     int sddmm_flat_supers = 0;  // flat MFMA SDDMM (algorithm 2): super-groups per wave, 0 = automatic
     int attention_waves = 0;
     int attention_chunk = 0;
@@ -238,7 +239,7 @@ inline hipError_t allow_large_lds(const void *kernel, int bytes, std::atomic<uns
 }
 
 // Waves per vector row for the SDDMM kernels; `group` = nonzero vectors a wave covers per step.
-int sddmm_auto_slots(long long m_vec, long long nonzeros_vec, int group);  // rows and nonzero vectors of the whole batch
+int sddmm_auto_slots(long long m_vec, long long nonzeros_vec, int group, bool mfma);  // rows and nonzero vectors of the whole batch
 
 // Batched launches: problem b of `count` uses operand pointers advanced by b * stride (in elements);
 // the sparsity pattern (row_indices, row_offsets, column indices) is shared by the whole batch.

@@ -28,6 +28,9 @@ __global__ void zero_fill_kernel(unsigned char *out, long long bytes, long long 
     if (blockIdx.x == 0 && threadIdx.x < (bytes & 3)) dst[(words << 2) + threadIdx.x] = 0;
 }
 
+// A kernel that does nothing: what a launch of a given shape costs before any work.
+__global__ void floor_probe_kernel() {}
+
 int launch_zero_fill(void *out, long long bytes, long long stride_bytes, int batch, hipStream_t stream)
 {
     if (batch > 65535) return hipErrorNotSupported;
@@ -491,6 +494,14 @@ void vs_sorted_row_swizzle(int rows, const int *row_offsets, int *row_indices)
     });
 }
 
+int vs_launch_floor_probe(int blocks, int threads_per_block, void *stream)
+{
+    if (blocks < 1 || threads_per_block < 1 || threads_per_block > 1024) return VS_ERROR_INVALID_VALUE;
+    hipLaunchKernelGGL(vs::floor_probe_kernel, dim3((unsigned)blocks), dim3((unsigned)threads_per_block), 0,
+                       static_cast<hipStream_t>(stream));
+    return (int)hipGetLastError();
+}
+
 int vs_set_option(const char *name, int value)
 {
     if (!name || value < 0) return VS_ERROR_INVALID_VALUE;
@@ -514,6 +525,9 @@ int vs_set_option(const char *name, int value)
     } else if (std::strcmp(name, "sddmm_flat_supers") == 0) {
         if (value > 16) return VS_ERROR_INVALID_VALUE;
         o.sddmm_flat_supers = value;
+    } else if (std::strcmp(name, "sddmm_group") == 0) {
+        if (value != 0 && value != 1 && value != 2 && value != 4) return VS_ERROR_INVALID_VALUE;
+        o.sddmm_group = value;
     } else if (std::strcmp(name, "sddmm_block_waves") == 0) {
         if (value > 16) return VS_ERROR_INVALID_VALUE;
         o.sddmm_block_waves = value;
