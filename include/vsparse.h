@@ -287,14 +287,17 @@ int vs_wmma_spmm_softmax_f16_batched(int batch, int m_vec, int vec_length, int k
  * With a plan, workgroups of eight waves (rows_per_workgroup >= 128 / vec_length) stream their union
  * through LDS 128 columns at a time with the next columns' K / V rows already on their way, keeping the
  * running maximum and sums of flash attention: the fastest path, and one that takes unions of up to 2048
- * columns.  A plan made for another shape is detected and ignored (every workgroup then takes the per-row
- * path: correct, slower).
+ * columns.  plan_bytes is the size of the plan buffer: it must be at least
+ * vs_sparse_attention_plan_bytes() for THIS shape (else 1, hipErrorInvalidValue, and no launch), so that the
+ * kernels never read past it whatever it holds.  A plan made for another shape is detected and ignored
+ * (every workgroup then takes the per-row path: correct, slower).
  */
 int vs_sparse_attention_f16(int batch, int m_vec, int vec_length, int n, int d_qk, int d_v,
                             const int *row_indices, const int *row_offsets, const int *col_indices,
                             const void *q, long long stride_q, const void *k, long long stride_k,
                             const void *v, long long stride_v, void *out, long long stride_out,
-                            float scale, int rows_per_workgroup, const void *plan, void *stream);
+                            float scale, int rows_per_workgroup, const void *plan, long long plan_bytes,
+                            void *stream);
 
 /*
  * Analysis step for rows_per_workgroup >= 2 of vs_sparse_attention_f16: writes into `plan` (device memory,
@@ -339,8 +342,14 @@ void vs_sorted_row_swizzle(int rows, const int *row_offsets, int *row_indices);
 int vs_launch_floor_probe(int blocks, int threads_per_block, void *stream);
 
 /*
- * Launch-shape tuning knob (process-wide, not thread-safe against concurrent
- * launches).  Names: "spmm_waves" (waves per workgroup, 0 = automatic),
+ * Launch-shape tuning knobs.  vs_set_option sets the process-wide default (not
+ * synchronised: set it before launching from several threads).
+ * vs_set_thread_option sets the value for the calling thread only: from its first
+ * call on, that thread's launches use its own copy of the options (initialised
+ * from the process-wide values at that moment) until vs_clear_thread_options().
+ * Launch shapes are decided on the host inside each call, so a thread can also
+ * change its options between two calls on different streams - every call sees
+ * exactly what its thread last set, whatever other threads do.  Names: "spmm_waves" (waves per workgroup, 0 = automatic),
  * "spmm_cols_per_lane" (4, 8, 0 = automatic), "spmm_gather" (how the MFMA SpMM
  * brings the gathered rows of the dense operand to the matrix cores: 1 = through
  * registers and an in-register transpose, 2 = global -> LDS loads and transposing LDS
@@ -358,6 +367,8 @@ int vs_launch_floor_probe(int blocks, int threads_per_block, void *stream);
  * (src/wmma_spmm.cu:396).
  */
 int vs_set_option(const char *name, int value);
+int vs_set_thread_option(const char *name, int value);
+void vs_clear_thread_options(void);
 
 #ifdef __cplusplus
 }

@@ -197,15 +197,35 @@ def _dense_attention(mask, q, k, v, scale):
     return out
 
 
-def _check_layer(got, ref, what):
-    # end-to-end bound for a chain with fp16 operands in both MFMA stages and an fp16 result: every element
-    # within 1e-2 of max(|ref|, rms(ref)) - relative for the large outputs (an fp16 result of magnitude 13 rms
-    # carries half an ulp = 0.5e-2 rms of rounding alone), absolute at 1e-2 rms for those near zero
+OBSERVED = {"loose": 0.0, "strict": 0.0}
+
+
+def _check_layer(got, ref, what, kind="chain"):
+    # End-to-end bounds for a chain with fp16 operands in both MFMA stages, fp16 probabilities and an fp16 result.
+    # loose: |err| / max(|ref|, rms(ref)) - relative for the large outputs, absolute at the scale of a typical
+    # output for those near zero; strict: the per-operator metric of tests/util.py, |err| / max(|ref|, 1e-2 rms),
+    # which for a chain is dominated by the outputs that cancel to near zero.  Both are printed; the limits (LIMITS
+    # below) are about twice the largest values observed over this file's cases on MI355X.
     ref = np.asarray(ref, dtype=np.float64)
+    got = got.astype(np.float64)
     rms = float(np.sqrt(np.mean(ref * ref)))
-    err = float(np.max(np.abs(got.astype(np.float64) - ref) / np.maximum(np.abs(ref), rms)))
+    loose = float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), rms)))
+    strict = float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), 1e-2 * rms)))
+    OBSERVED["loose"] = max(OBSERVED["loose"], loose)
+    OBSERVED["strict"] = max(OBSERVED["strict"], strict)
+    print("attention parity %-60s loose %.3e  strict %.3e" % (what, loose, strict))
     assert np.all(np.isfinite(got)), what
-    assert err <= 1e-2, "%s: max |err| / max(|ref|, rms) = %.3e" % (what, err)
+    loose_limit, strict_limit = LIMITS[kind]
+    assert loose <= loose_limit, "%s: max |err| / max(|ref|, rms) = %.3e > %.1e" % (what, loose, loose_limit)
+    assert strict <= strict_limit, "%s: max |err| / max(|ref|, 1e-2 rms) = %.3e > %.2f" % (what, strict, strict_limit)
+
+
+# Largest values observed over this file's cases on MI355X -> limit (about twice the observation):
+#   single-launch kernels (per-row, union, streamed; scores and probabilities stay on the chip):
+#       loose 1.4e-3, strict 8.1e-2  ->  3e-3, 0.17
+#   chains with fp16 scores / probabilities in memory (SDDMM -> softmax -> SpMM, softmax-fused SpMM, and
+#   whatever `forward` picks): loose 7.0e-3, strict 0.33  ->  1e-2 (the contract's figure), 0.7
+LIMITS = {"single": (3e-3, 0.17), "chain": (1e-2, 0.7)}
 
 
 @pytest.mark.parametrize("V", [1, 2, 4, 8])
@@ -239,7 +259,7 @@ def test_single_launch_attention(gpu, V, dims):
             host = pad.cpu().numpy()
             assert np.all(host[:, :8] == 3.0) and np.all(host[:, 8 + mask.m:] == 3.0), "wrote outside the output"
             _check_layer(host[:, 8:8 + mask.m], ref,
-                         "V%d dqk%d dv%d chunk%d waves%d rows%d" % (V, d_qk, d_v, chunk, waves, rows))
+                         "V%d dqk%d dv%d chunk%d waves%d rows%d" % (V, d_qk, d_v, chunk, waves, rows), kind="single")
             for i in np.nonzero(lengths == 0)[0]:
                 assert not host[:, 8 + i * V:8 + (i + 1) * V].any(), "an empty row must produce zeros"
     finally:
@@ -266,7 +286,7 @@ def test_union_gather_on_structured_and_random_masks(gpu, V):
             again = ops.sparse_attention(mask.m_vec, V, seq, prob.row_indices, prob.row_offsets,
                                          prob.column_indices, qd, kd, vd, scale=0.125, rows_per_workgroup=rows)
             torch.cuda.synchronize()
-            _check_layer(out.cpu().numpy(), ref, "%s mask V%d rows%d" % (name, V, rows))
+            _check_layer(out.cpu().numpy(), ref, "%s mask V%d rows%d" % (name, V, rows), kind="single")
             assert torch.equal(out, again)      # deterministic
         if name == "band":
             assert ops.SparseAttention(mask).union_rows(d, d) == 128 // V
@@ -316,8 +336,8 @@ def test_plan_raises_the_union_capacity(gpu, V, seq, half_width, stride, rows):
     rebuilt = ops.sparse_attention(*args, scale=0.125, rows_per_workgroup=rows)
     out = layer.forward(qd, kd, vd, scale=0.125)
     torch.cuda.synchronize()
-    _check_layer(planned.cpu().numpy(), ref, "V%d planned" % V)
-    _check_layer(rebuilt.cpu().numpy(), ref, "V%d rebuilt" % V)
+    _check_layer(planned.cpu().numpy(), ref, "V%d planned" % V, kind="single")
+    _check_layer(rebuilt.cpu().numpy(), ref, "V%d rebuilt" % V, kind="single")
     _check_layer(out.cpu().numpy(), ref, "V%d layer" % V)
     assert not torch.equal(planned, rebuilt)              # different summation orders: the paths did differ
 
@@ -353,7 +373,7 @@ def test_planned_launch_streams_large_unions(gpu, V, seq, half_width, stride, di
         planned = ops.sparse_attention(*args, scale=scale, rows_per_workgroup=rows, plan=plan)
         again = ops.sparse_attention(*args, scale=scale, rows_per_workgroup=rows, plan=plan)
         torch.cuda.synchronize()
-        _check_layer(planned.cpu().numpy(), ref, "V%d scale %g streamed" % (V, scale))
+        _check_layer(planned.cpu().numpy(), ref, "V%d scale %g streamed" % (V, scale), kind="single")
         assert torch.equal(planned, again)
     layer = ops.SparseAttention(mask)
     assert layer.union_rows(d_qk, d_v, 16) == rows        # the host-side choice counts on the streamed kernel
@@ -387,22 +407,34 @@ def test_planned_launch_equals_unplanned(gpu, V):
             plan = ops.sparse_attention_plan(mask.m_vec, V, seq, d, d, rows, prob.row_offsets, prob.column_indices)
             planned = ops.sparse_attention(*args, scale=0.125, rows_per_workgroup=rows, plan=plan)
             torch.cuda.synchronize()
-            _check_layer(planned.cpu().numpy(), ref, "%s V%d rows%d planned" % (name, V, rows))
+            _check_layer(planned.cpu().numpy(), ref, "%s V%d rows%d planned" % (name, V, rows), kind="single")
             # a planned launch holds more columns per workgroup: same bits unless some union fits only then
             built, held = _capacity(V, seq, d, d, rows, 0), _capacity(V, seq, d, d, rows, 1)
             streamed = rows == 128 // V
             if not streamed and not any(built < u <= held for u in _unions(mask, rows)):
                 assert torch.equal(plain, planned), "%s V%d rows%d" % (name, V, rows)
             else:
-                _check_layer(plain.cpu().numpy(), ref, "%s V%d rows%d rebuilt" % (name, V, rows))
+                _check_layer(plain.cpu().numpy(), ref, "%s V%d rows%d rebuilt" % (name, V, rows), kind="single")
         # a negative scale (sign handled inside the kernel) through the same paths
         neg = ops.sparse_attention(*args, scale=-0.125, rows_per_workgroup=128 // V, plan=plan)
         torch.cuda.synchronize()
-        _check_layer(neg.cpu().numpy(), _dense_attention(mask, q, k, v, -0.125), "%s V%d negative scale" % (name, V))
+        _check_layer(neg.cpu().numpy(), _dense_attention(mask, q, k, v, -0.125), "%s V%d negative scale" % (name, V), kind="single")
+        # a plan made for another launch shape: rejected on the host when it is too small for this shape (the
+        # kernels read it at this shape's offsets before they can tell), detected in the kernel and ignored when
+        # it is large enough
+        from vectorsparse_amd import _lib
         other = ops.sparse_attention_plan(mask.m_vec, V, seq, d, d, 16 // V, prob.row_offsets, prob.column_indices)
+        need = _lib.lib().vs_sparse_attention_plan_bytes(mask.m_vec, V, seq, d, d, 128 // V)
+        if other.numel() < need:
+            with pytest.raises(_lib.VSparseError):
+                ops.sparse_attention(*args, scale=0.125, rows_per_workgroup=128 // V, plan=other)
+            other = torch.cat([other, torch.zeros(need - other.numel(), dtype=torch.uint8, device="cuda")])
+        tiny = torch.zeros(64, dtype=torch.uint8, device="cuda")
+        with pytest.raises(_lib.VSparseError):
+            ops.sparse_attention(*args, scale=0.125, rows_per_workgroup=128 // V, plan=tiny)
         out = ops.sparse_attention(*args, scale=0.125, rows_per_workgroup=128 // V, plan=other)
         torch.cuda.synchronize()
-        _check_layer(out.cpu().numpy(), ref, "%s V%d foreign plan" % (name, V))
+        _check_layer(out.cpu().numpy(), ref, "%s V%d foreign plan" % (name, V), kind="single")
 
 
 def _lib_set(name, value):
@@ -472,8 +504,8 @@ def test_union_kernel_on_awkward_shapes(gpu):
         host = pad.cpu().numpy()
         assert np.all(host[:, :8] == 5.0) and np.all(host[:, 8 + mask.m:] == 5.0), what + ": wrote outside the output"
         if np.sqrt(np.mean(ref * ref)) > 0:
-            _check_layer(host[:, 8:8 + mask.m], ref, what)
-            _check_layer(planned.cpu().numpy(), ref, what + " planned")
+            _check_layer(host[:, 8:8 + mask.m], ref, what, kind="single")
+            _check_layer(planned.cpu().numpy(), ref, what + " planned", kind="single")
         else:
             assert not host[:, 8:8 + mask.m].any() and not planned.cpu().numpy().any(), what
 
@@ -504,8 +536,8 @@ def test_config5_full_size(gpu):
                                    qd, kd, vd, scale=0.125)
     chain = layer.forward(qd, kd, vd, fused=False)        # SDDMM -> softmax -> SpMM, three launches
     torch.cuda.synchronize()
-    _check_layer(out.cpu().numpy(), ref, "config 5, union kernel with plan")
-    _check_layer(per_row.cpu().numpy(), ref, "config 5, per-row kernel")
+    _check_layer(out.cpu().numpy(), ref, "config 5, union kernel with plan", kind="single")
+    _check_layer(per_row.cpu().numpy(), ref, "config 5, per-row kernel", kind="single")
     _check_layer(chain.cpu().numpy(), ref, "config 5, three operators")
 
 
@@ -548,19 +580,19 @@ def test_attention_random_cases(gpu, seed):
     what = "seed %d V%d seq %d d %d/%d" % (seed, V, seq, d_qk, d_v)
     out = ops.sparse_attention(*args, scale=scale)
     torch.cuda.synchronize()
-    _check_layer(out.cpu().numpy(), ref, what + " per row")
+    _check_layer(out.cpu().numpy(), ref, what + " per row", kind="single")
     for rows in (16 // V, 128 // V):
         if rows < 2:
             continue
         out = ops.sparse_attention(*args, scale=scale, rows_per_workgroup=rows)
         torch.cuda.synchronize()
-        _check_layer(out.cpu().numpy(), ref, what + " rows %d rebuilt" % rows)
+        _check_layer(out.cpu().numpy(), ref, what + " rows %d rebuilt" % rows, kind="single")
         if _capacity(V, seq, d_qk, d_v, rows, 1) > 0:
             plan = ops.sparse_attention_plan(mask.m_vec, V, seq, d_qk, d_v, rows, prob.row_offsets,
                                              prob.column_indices)
             out = ops.sparse_attention(*args, scale=scale, rows_per_workgroup=rows, plan=plan)
             torch.cuda.synchronize()
-            _check_layer(out.cpu().numpy(), ref, what + " rows %d planned" % rows)
+            _check_layer(out.cpu().numpy(), ref, what + " rows %d planned" % rows, kind="single")
     layer = ops.SparseAttention(mask)
     for fused in (None, True, False):
         out = layer.forward(qd, kd, vd, scale=scale, fused=fused)
@@ -594,4 +626,4 @@ def test_streamed_kernel_falls_back_on_oversized_unions(gpu):
         out = ops.sparse_attention(mask.m_vec, V, seq, prob.row_indices, prob.row_offsets, prob.column_indices,
                                    qd, kd, vd, scale=0.125, rows_per_workgroup=16, plan=plan)
         torch.cuda.synchronize()
-        _check_layer(out.cpu().numpy(), _dense_attention(mask, q, k, v, 0.125), name)
+        _check_layer(out.cpu().numpy(), _dense_attention(mask, q, k, v, 0.125), name, kind="single")

@@ -168,6 +168,25 @@ def test_sddmm_c_equals_numpy_bitwise_and_float64_brute_force(V):
     assert np.array_equal(c.view(np.uint16), mt.view(np.uint16))
 
 
+def test_sddmm_accumulates_along_k_in_ascending_order_fp32():
+    # Host_sddmm adds the products of one output in ascending l, in fp32 (include/bm_test_utils.h:181-186):
+    # 2048 followed by 4096 terms of 2^-13 loses every small term (each is below half an ulp of 2048), the same
+    # terms in descending l keep their sum 0.5.  A pairwise or reversed accumulation fails one of the two.
+    K = 4097
+    A = np.full((1, K), 2.0 ** -13, np.float16)
+    A[0, 0] = 2048.0
+    B = np.ones((1, K), np.float16)
+    ro = np.array([0, 1], np.int32)
+    ci = np.array([0], np.int32)
+    out = co.sddmm_host_ref_f32(1, K, 1, ro, ci, A, B)
+    assert out[0] == np.float32(2048.0)
+    rev = co.sddmm_host_ref_f32(1, K, 1, ro, ci, A[:, ::-1].copy(), B)
+    assert rev[0] == np.float32(2048.5)
+    # the fp16 flavour rounds that fp32 sum once
+    assert co.sddmm_host_ref_f16(1, K, 1, ro, ci, A[:, ::-1].copy(), B)[0] == np.float16(2048.0)   # 2048.5 -> even
+    assert no.sddmm_host_ref(1, K, 1, ro, ci, A, B)[0] == np.float16(2048.0)
+
+
 def test_sddmm_full_mask_is_dense_product_and_layout():
     V, m_vec, n, K = 2, 3, 5, 8
     ro = (np.arange(m_vec + 1) * n).astype(np.int32)

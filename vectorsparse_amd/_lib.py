@@ -33,7 +33,7 @@ SIGNATURES = {
     "vs_wmma_spmm_softmax_f16_batched": ([_int] * 7 + [_vp] * 3 + [_vp, _ll, _vp, _ll, _vp, _ll, ctypes.c_float, _vp],
                                          _int),
     "vs_sparse_attention_f16": ([_int] * 6 + [_vp] * 3 + [_vp, _ll, _vp, _ll, _vp, _ll, _vp, _ll, ctypes.c_float, _int,
-                                 _vp, _vp],
+                                 _vp, _ll, _vp],
                                 _int),
     "vs_sparse_attention_union_capacity": ([_int] * 6 + [_vp], _int),
     "vs_sparse_attention_plan_bytes": ([_int] * 6, _ll),
@@ -43,6 +43,8 @@ SIGNATURES = {
     "vs_sorted_row_swizzle": ([_int, _vp, _vp], None),
     "vs_launch_floor_probe": ([_int, _int, _vp], _int),
     "vs_set_option": ([ctypes.c_char_p, _int], _int),
+    "vs_set_thread_option": ([ctypes.c_char_p, _int], _int),
+    "vs_clear_thread_options": ([], None),
 }
 
 _lib = None
@@ -78,4 +80,22 @@ def check(status, where):
 
 
 def set_option(name, value):
+    """Process-wide launch-shape override (0 = automatic)."""
     check(lib().vs_set_option(name.encode(), int(value)), "vs_set_option(%s)" % name)
+
+
+class thread_options:
+    """Launch-shape overrides for the calls the current thread makes inside the `with` block, e.g.
+    `with thread_options(spmm_waves=4): prob.spmm(...)`.  Other threads are not affected."""
+
+    def __init__(self, **values):
+        self.values = values
+
+    def __enter__(self):
+        for name, value in self.values.items():
+            check(lib().vs_set_thread_option(name.encode(), int(value)), "vs_set_thread_option(%s)" % name)
+        return self
+
+    def __exit__(self, *exc):
+        lib().vs_clear_thread_options()
+        return False

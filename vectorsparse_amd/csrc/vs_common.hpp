@@ -206,7 +206,7 @@ __device__ __forceinline__ void store_ragged(OutT *dst, const float *src, int va
         if (i < valid) dst[i] = (OutT)src[i];
 }
 
-// Process-wide launch-shape overrides (0 = automatic).
+// Launch-shape overrides (0 = automatic).
 struct Options {
     int spmm_waves = 0;
     int spmm_cols_per_lane = 0;
@@ -220,7 +220,7 @@ struct Options {
     int attention_waves = 0;
     int attention_chunk = 0;
 };
-Options &options();
+const Options &options();  // the calling thread's overrides if it has set any, else the process-wide ones
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 

@@ -9,11 +9,14 @@
 #include "vs_common.hpp"
 
 namespace vs {
-Options &options()
-{
-    static Options opts;
-    return opts;
-}
+// Launch-shape overrides: a process-wide default, and a per-thread copy that replaces it for the calls a thread
+// makes once that thread has set one of its own (launch shapes are decided on the host inside the call, so two
+// threads - or one thread between two calls - never see each other's choices).
+static Options g_options;
+static thread_local Options t_options;
+static thread_local bool t_options_active = false;
+
+const Options &options() { return t_options_active ? t_options : g_options; }
 }  // namespace vs
 
 namespace vs {
@@ -412,11 +415,18 @@ int vs_wmma_spmm_softmax_f16_batched(int batch, int m_vec, int vec_length, int k
 int vs_sparse_attention_f16(int batch, int m_vec, int vec_length, int n, int d_qk, int d_v, const int *row_indices,
                             const int *row_offsets, const int *col_indices, const void *q, long long stride_q,
                             const void *k, long long stride_k, const void *v, long long stride_v, void *out,
-                            long long stride_out, float scale, int rows_per_workgroup, const void *plan, void *stream)
+                            long long stride_out, float scale, int rows_per_workgroup, const void *plan,
+                            long long plan_bytes, void *stream)
 {
     if (batch < 0 || m_vec < 0 || n < 0 || d_qk < 0 || d_v < 0 || !vec_ok(vec_length)) return VS_ERROR_INVALID_VALUE;
     if (rows_per_workgroup < 0 || rows_per_workgroup > 128) return VS_ERROR_INVALID_VALUE;
     if (plan && (rows_per_workgroup < 2 || !aligned(plan, 16))) return VS_ERROR_INVALID_VALUE;
+    // the kernels read the plan at offsets that follow from THIS launch's shape before they know whether it is
+    // theirs: a buffer too small for this shape is rejected here, whatever it holds
+    if (plan && (d_qk <= 0 || d_v <= 0 ||
+                 plan_bytes < vs::sparse_attention_plan_bytes(m_vec, vec_length, n, d_qk, d_v, rows_per_workgroup) ||
+                 vs::sparse_attention_plan_bytes(m_vec, vec_length, n, d_qk, d_v, rows_per_workgroup) <= 0))
+        return VS_ERROR_INVALID_VALUE;
     if (batch == 0 || m_vec == 0 || d_v == 0) return VS_SUCCESS;
     if (!row_indices || !row_offsets || !q || !out) return VS_ERROR_INVALID_VALUE;
     if (n > 0 && (!k || !v)) return VS_ERROR_INVALID_VALUE;
@@ -502,10 +512,9 @@ int vs_launch_floor_probe(int blocks, int threads_per_block, void *stream)
     return (int)hipGetLastError();
 }
 
-int vs_set_option(const char *name, int value)
+static int set_option_field(vs::Options &o, const char *name, int value)
 {
     if (!name || value < 0) return VS_ERROR_INVALID_VALUE;
-    vs::Options &o = vs::options();
     if (std::strcmp(name, "spmm_waves") == 0) {
         if (value > 16) return VS_ERROR_INVALID_VALUE;
         o.spmm_waves = value;
@@ -536,11 +545,23 @@ int vs_set_option(const char *name, int value)
         o.attention_waves = value;
     } else if (std::strcmp(name, "attention_chunk") == 0) {
         o.attention_chunk = value;
-
     } else {
         return VS_ERROR_INVALID_VALUE;
     }
     return VS_SUCCESS;
 }
+
+int vs_set_option(const char *name, int value) { return set_option_field(vs::g_options, name, value); }
+
+int vs_set_thread_option(const char *name, int value)
+{
+    if (!vs::t_options_active) {
+        vs::t_options = vs::g_options;  // starts from the process-wide values as they are now
+        vs::t_options_active = true;
+    }
+    return set_option_field(vs::t_options, name, value);
+}
+
+void vs_clear_thread_options(void) { vs::t_options_active = false; }
 
 }  // extern "C"

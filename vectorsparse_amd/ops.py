@@ -211,7 +211,8 @@ def sparse_attention(m_vec, vec_length, n, row_indices, row_offsets, col_indices
                                             _ptr(row_offsets), _ptr(col_indices), _ptr(q), _stride(q, heads),
                                             _ptr(k), _stride(k, heads), _ptr(v), _stride(v, heads), _ptr(out),
                                             _stride(out, heads), float(scale), int(rows_per_workgroup),
-                                            _ptr(plan), _stream(stream))
+                                            _ptr(plan), 0 if plan is None else plan.numel() * plan.element_size(),
+                                            _stream(stream))
     _lib.check(st, "vs_sparse_attention_f16")
     return out
 
