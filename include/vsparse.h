@@ -75,10 +75,13 @@ int vs_wmma_spmm_f16_f32out(int m_vec, int vec_length, int k, int n,
  * (include/bm_test_utils.h:200-215) only approximates by reordering whole rows: the nonzero range is cut
  * into equal runs, one wave per (run, column tile) and sixteen runs per workgroup; a row that crosses run
  * boundaries is computed in segments whose fp32 partial tiles are added in ascending order - inside a
- * workgroup through LDS, across workgroups through `workspace` by a second launch (no atomics; deterministic; the result does not depend on row_indices, which may be null and is ignored).
+ * workgroup through LDS, across workgroups through `workspace` by whichever wave brings a row's last part (one
+ * launch, nobody waits, no atomics on the output; deterministic; the result does not depend on row_indices, which may be null and is ignored).
  * nonzeros_vec must equal row_offsets[m_vec] (the host cannot read it from device memory).
- * workspace: device memory, 16-byte aligned, workspace_bytes long, owned by the caller, contents undefined
- * before and after, not shared between calls that may overlap.  vs_wmma_spmm_workspace_bytes() returns the
+ * workspace: device memory, 16-byte aligned, workspace_bytes long, owned by the caller, ZERO-FILLED before its
+ * first use: it starts with arrival counters that every call finds at zero and leaves at zero (so no call
+ * spends a launch on clearing them); the rest is undefined before and after.  Not shared between calls that may
+ * overlap.  (Option "spmm_flat_launches" = 2 adds the parts in a second launch instead and uses no counters.)  vs_wmma_spmm_workspace_bytes() returns the
  * size that lets the library pick its preferred run length (0 when one workgroup takes everything); a smaller
  * workspace - even none - is accepted and makes the runs longer (fewer waves, same results up to the
  * order of the fp32 summation).  Other requirements as vs_wmma_spmm_f16.  Faster than vs_wmma_spmm_f16 when
@@ -106,7 +109,8 @@ int vs_wmma_spmm_f16_f32out_ws(int m_vec, int vec_length, int k, int n, int nonz
  * of 64 pieces); beyond it the call returns 801 (hipErrorNotSupported) and launches nothing.
  * Every call on a GPU shares that GPU's array: calls that may overlap on one GPU (different streams, different
  * threads) race on it and must be serialised by the caller.  Nothing in the array has to be cleared between
- * calls (every partial tile that is read was written by the same call).
+ * calls: it starts zeroed, every call leaves its arrival counters at zero, and every partial tile that is read
+ * was written by the same call.
  */
 long long vs_wmma_spmm_noalloc_scratch_bytes(void);
 int vs_wmma_spmm_f16_noalloc(int m_vec, int vec_length, int k, int n, int nonzeros_vec,
@@ -356,7 +360,8 @@ int vs_launch_floor_probe(int blocks, int threads_per_block, void *stream);
  * reads, k % 8 == 0 only; 0 = automatic, which is 1: 2 measured 10-18 % slower),
  * "spmm_flat_piece" (nonzero vectors
  * per wave of the split-row SpMM, rounded up to 32, 0 = automatic), "spmm_flat_waves"
- * (its waves per workgroup, 1..16, 0 = automatic), "sddmm_slots" (waves per
+ * (its waves per workgroup, 1..16, 0 = automatic), "spmm_flat_launches" (1 = partial tiles
+ * added inside the launch, 2 = by a second launch, 0 = automatic), "sddmm_slots" (waves per
  * vector row, 0 = automatic), "sddmm_group" (16-vector groups per wave step of the
  * MFMA SDDMM: 1, 2, 4, 0 = automatic), "sddmm_block_waves" (1..16, 0 = automatic),
  * "sddmm_flat_supers" (super-groups per wave of algorithm 2, 1..16, 0 = automatic),

@@ -19,7 +19,7 @@ def _oracle(pat, B):
                                 pat.column_indices, pat.values, B)
 
 
-def _run(pat, B, out_dtype=torch.float16, workspace="auto", piece=0, waves=0):
+def _run(pat, B, out_dtype=torch.float16, workspace="auto", piece=0, waves=0, launches=0):
     """One call with canaries round the output and round the workspace; returns the host copy of the output."""
     prob = ops.DeviceProblem(pat)
     Bd = torch.from_numpy(B).cuda()
@@ -30,11 +30,14 @@ def _run(pat, B, out_dtype=torch.float16, workspace="auto", piece=0, waves=0):
     try:
         _lib.set_option("spmm_flat_piece", piece)
         _lib.set_option("spmm_flat_waves", waves)
+        _lib.set_option("spmm_flat_launches", launches)
         need = ops.spmm_workspace_bytes(pat.m_vec, pat.vec_length, k, pat.n, pat.nnz_vec)
         ws_bytes = need if workspace == "auto" else int(workspace)
         guard = 4096
         ws_buf = torch.full((ws_bytes + 2 * guard,), 0x5A, dtype=torch.uint8, device="cuda")
         ws = ws_buf[guard:guard + ws_bytes] if ws_bytes else None
+        if ws is not None:
+            ws.zero_()   # the contract: zero before the first use; every call leaves it ready for the next
         for _ in range(2):  # the second call finds the workspace as the first left it
             out.fill_(777.0)
             ops.spmm_split_rows(pat.m_vec, pat.vec_length, k, pat.n, pat.nnz_vec, prob.row_offsets,
@@ -43,6 +46,7 @@ def _run(pat, B, out_dtype=torch.float16, workspace="auto", piece=0, waves=0):
     finally:
         _lib.set_option("spmm_flat_piece", 0)
         _lib.set_option("spmm_flat_waves", 0)
+        _lib.set_option("spmm_flat_launches", 0)
     host = buf.cpu().numpy()
     assert np.all(host[:pad] == 12345.0) and np.all(host[pad + pat.m:] == 12345.0), "wrote outside the output"
     wsh = ws_buf.cpu().numpy()
@@ -62,14 +66,15 @@ def _from_lengths(lengths, n, V, seed):
 @pytest.mark.parametrize("V", [1, 2, 4, 8])
 @pytest.mark.parametrize("piece", [0, 32, 64, 96, 512])
 @pytest.mark.parametrize("waves", [0, 1, 3])
-def test_ragged_empty_and_long_rows(gpu, V, piece, waves):
+@pytest.mark.parametrize("launches", [1, 2])
+def test_ragged_empty_and_long_rows(gpu, V, piece, waves, launches):
     # empty rows at the start, in the middle and at the end; rows of every tail length; rows that span many runs
     # and pieces; a row that starts exactly on a run boundary (the 64 in front of it ends nonzero 128)
     lengths = [0, 0, 1, 15, 16, 17, 0, 31, 33, 14, 0, 64, 65, 300, 2, 0, 128, 7, 640, 1, 0, 0]
     pat = _from_lengths(lengths, 640, V, seed=5)
     B = cv.dense_uniform(640, 192, seed=7)
-    got = _run(pat, B, piece=piece, waves=waves)
-    assert_parity(got, _oracle(pat, B), "split rows V%d run %d waves %d" % (V, piece, waves))
+    got = _run(pat, B, piece=piece, waves=waves, launches=launches)
+    assert_parity(got, _oracle(pat, B), "split rows V%d run %d waves %d launches %d" % (V, piece, waves, launches))
     for i in np.nonzero(np.asarray(lengths) == 0)[0]:
         assert not got[i * V:(i + 1) * V].any(), "empty vector row %d must be written as zeros" % i
 
@@ -99,6 +104,8 @@ def test_pareto_rows_with_a_dense_row(gpu, V):
     assert_parity(a, ref, "pareto rows, automatic pieces")
     b = _run(pat, B)
     assert np.array_equal(a.view(np.uint16), b.view(np.uint16)), "two runs differ"
+    c = _run(pat, B, launches=2)
+    assert np.array_equal(a.view(np.uint16), c.view(np.uint16)), "one launch and two launches add in the same order"
     assert_parity(_run(pat, B, out_dtype=torch.float32), ref, "pareto rows, fp32 out")
 
 

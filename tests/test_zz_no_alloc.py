@@ -33,7 +33,7 @@ def test_two_calls_in_a_row_match_the_workspace_entry_point(gpu):
     L = _lib.lib()
     scratch = L.vs_wmma_spmm_noalloc_scratch_bytes()
     assert scratch == 16 << 20
-    workspace = torch.empty(scratch, dtype=torch.uint8, device="cuda")
+    workspace = torch.zeros(scratch, dtype=torch.uint8, device="cuda")
     # the first problem splits many rows across pieces; the second is smaller in every dimension
     for (m_vec, n, V, N, seed, longest) in ((512, 4096, 8, 256, 1, 4096), (96, 1024, 8, 128, 2, 1000)):
         pat, B = _problem(m_vec, n, V, N, seed, longest)

@@ -12,13 +12,21 @@
 //     slot F[w]; the wave in whose run a row starts keeps that segment in its accumulators and, after the one
 //     barrier, adds the slots F[w+1], F[w+2], ... of the runs the row covers;
 //   * across workgroups through the workspace: the part of a row that a piece holds goes to slot T[c] (the row
-//     starts inside piece c) or F[c] (it started earlier), fp32.  A second launch adds T[c0] + F[c0+1] + ... for
-//     every row that crosses a piece boundary and writes its output rows.  (Adding them inside the first launch
-//     - the wave that brings a row's last part adds up - was measured at 1.5 to 4 times the time of the two
-//     launches: on this GPU every part then has to go through device-coherent stores or be followed by a
-//     write-back of the whole L2, because the eight L2s do not see each other's lines within a launch.)
-// The second launch also writes the zero rows of empty vector rows, which no wave of the first launch visits
-// (writing them from the walk costs the tile loop 24 registers and with them its occupancy).
+//     starts inside piece c) or F[c] (it started earlier), fp32.  A row that starts in piece c0 and ends in piece c1
+//     has c1 - c0 + 1 parts, added as T[c0] + F[c0+1] + ... + F[c1] in one of two ways:
+//     ONE_LAUNCH (default): every wave that has written a part counts itself in on the row's arrival counter (the
+//     one of piece c0: at most one row starts in a piece and leaves it) and the wave that arrives last adds the
+//     parts, writes the output rows and puts the counter back to zero.  Nobody waits for anybody and the sum is
+//     the same whoever arrives last.  The eight L2s of the chip do not see each other's lines within a launch,
+//     so the parts are written and read with the device-coherence bits of the cache policy set (buffer accesses
+//     with sc0 sc1, tracked by the compiler; the same accesses as inline assembly lost their data registers to
+//     reuse before the stores had read them) - an L2-wide write-back and invalidate around the counter
+//     (__threadfence) cost 60 us per launch instead of 1.
+//     Two launches: a second launch adds the parts; 1.5 to 2.5 us slower, no counters, and the route taken when
+//     the tiles would not fit 32-bit buffer offsets.
+// The zero rows of empty vector rows, which no wave's walk visits, are written by extra workgroups at the end of
+// the grid (ONE_LAUNCH) or by the second launch (writing them from the walk costs the tile loop 24 registers and
+// with them its occupancy).
 // The arithmetic of a step is the row-per-workgroup kernel's (spmm_mfma_step).  row_indices is not needed.
 #include "spmm_mfma_step.hpp"
 #include "vs_common.hpp"
@@ -61,6 +69,66 @@ __device__ __forceinline__ void tile_add(const float *tile_base, int pitch, int 
     }
 }
 
+// The same two for tiles in the workspace that waves on other CUs - and other XCDs, whose L2 is a different one -
+// read within the same launch: 128-bit buffer stores and loads with the device-coherence bits of the cache policy
+// set (sc0 sc1: written through to memory, read past the caches), so that no cache-wide write-back or invalidate
+// is needed around the arrival counter.  `tiles` is a buffer descriptor over the tile area of the workspace
+// (below 2^31 bytes), offsets are in bytes.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+constexpr int kCoherent = 1 | 16;  // cache policy bits: sc0, sc1
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_area(float *base)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(base, 0, 0x7fffffff, 0x00020000);
+}
+
+template <int V, int CPL>
+__device__ __forceinline__ void tile_store_coherent(__amdgpu_buffer_rsrc_t tiles, uint32_t tile_bytes, int pitch, int cs,
+                                                    int g, const float4_t (&acc)[CPL])
+{
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int v = 4 * g + e;
+        if (v < V) {
+#pragma unroll
+            for (int c4 = 0; c4 < CPL / 4; ++c4) {
+                const float4_t t = {acc[4 * c4][e], acc[4 * c4 + 1][e], acc[4 * c4 + 2][e], acc[4 * c4 + 3][e]};
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, t), tiles,
+                                                       tile_bytes + 4u * (uint32_t)(v * pitch + cs * CPL + 4 * c4), 0,
+                                                       kCoherent);
+            }
+        }
+    }
+}
+
+// adds the lane's part of a tile (rows 4g..4g+3 below V, its CPL columns) to acc
+template <int V, int CPL>
+__device__ __forceinline__ void tile_add_coherent(__amdgpu_buffer_rsrc_t tiles, uint32_t tile_bytes, int pitch, int cs,
+                                                  int g, float4_t (&acc)[CPL])
+{
+    float4_t part[4][CPL / 4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int v = 4 * g + e;
+#pragma unroll
+        for (int c4 = 0; c4 < CPL / 4; ++c4) {
+            part[e][c4] = float4_t{0.f, 0.f, 0.f, 0.f};
+            if (v < V)
+                part[e][c4] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(
+                                  tiles, tile_bytes + 4u * (uint32_t)(v * pitch + cs * CPL + 4 * c4), 0, kCoherent));
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int c4 = 0; c4 < CPL / 4; ++c4) {
+            acc[4 * c4][e] += part[e][c4][0];
+            acc[4 * c4 + 1][e] += part[e][c4][1];
+            acc[4 * c4 + 2][e] += part[e][c4][2];
+            acc[4 * c4 + 3][e] += part[e][c4][3];
+        }
+}
+
 // The lane's CPL outputs of the V scalar rows of vector row `row`, converted and stored.
 template <int V, int CPL, typename OutT>
 __device__ __forceinline__ void tile_to_output(OutT *out, int row, int n_cols, int col0, bool col_ok, int g,
@@ -78,9 +146,12 @@ __device__ __forceinline__ void tile_to_output(OutT *out, int row, int n_cols, i
     }
 }
 
-template <int V, int CPL, bool IDX32, typename OutT>
+// ONE_LAUNCH: the parts of rows that cross workgroups are added inside this launch by whichever wave brings a
+// row's last part (arrival counters at the start of the workspace, which every launch leaves at zero), and the
+// workgroups past `main_blocks` write the zero rows of empty vector rows; there is no second launch.
+template <int V, int CPL, bool IDX32, bool ONE_LAUNCH, typename OutT>
 __global__ void __launch_bounds__(1024)
-spmm_mfma_flat_kernel(int m_vec, int n_cols, int n_tiles, int nonzeros_vec, int sub,
+spmm_mfma_flat_kernel(int m_vec, int n_cols, int n_tiles, int nonzeros_vec, int sub, int main_blocks, int *counters,
                       const int *__restrict__ row_offsets, const int *__restrict__ column_indices,
                       const half_t *__restrict__ values, const half_t *__restrict__ rhs, OutT *__restrict__ out,
                       float *__restrict__ ws_base, int ws_pitch)
@@ -91,6 +162,19 @@ spmm_mfma_flat_kernel(int m_vec, int n_cols, int n_tiles, int nonzeros_vec, int 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n_waves = blockDim.x >> 6;
+    if constexpr (ONE_LAUNCH) {
+        if ((int)blockIdx.x >= main_blocks) {  // four vector rows per wave: zeros for the empty ones
+            const int first = (((int)blockIdx.x - main_blocks) * n_waves + wave) * 4;
+            const int quads = n_cols >> 2;  // n_cols % 4 == 0
+            for (int row = first; row < first + 4 && row < m_vec; ++row) {
+                if (row_offsets[row + 1] != row_offsets[row]) continue;
+                const float zeros[4] = {0.f, 0.f, 0.f, 0.f};
+                for (int item = lane; item < V * quads; item += 64)
+                    store_converted<OutT, 4>(out + (size_t)row * V * n_cols + 4 * (size_t)item, zeros);
+            }
+            return;
+        }
+    }
     const int tile = blockIdx.x % n_tiles;
     const int c = blockIdx.x / n_tiles;  // piece
     const long long piece = (long long)n_waves * sub;
@@ -114,7 +198,7 @@ spmm_mfma_flat_kernel(int m_vec, int n_cols, int n_tiles, int nonzeros_vec, int 
     for (int q = 0; q < CPL; ++q) acc[q] = float4_t{0.f, 0.f, 0.f, 0.f};
     bool has_t = false;   // the accumulators hold the first segment of a row that goes on past this run
     bool has_f = false;   // this run starts inside a row (its partial tile is in F[wave])
-    int t_row = 0, t_row_end = 0, f_row_end = 0;
+    int t_row = 0, t_row_end = 0, f_row = 0, f_row_beg = 0, f_row_end = 0;
 
     if (sb_ll < nonzeros_vec) {
         const int sb = (int)sb_ll;
@@ -180,6 +264,8 @@ spmm_mfma_flat_kernel(int m_vec, int n_cols, int n_tiles, int nonzeros_vec, int 
             } else if (row_beg < sb) {  // started in an earlier run (and may go on past this one)
                 tile_store<V, CPL>(f_mine, TN, cs, g, acc);
                 has_f = true;
+                f_row = row;
+                f_row_beg = row_beg;
                 f_row_end = row_end;
             } else {  // starts here and goes on: the run's last segment, kept in the accumulators
                 has_t = true;
@@ -193,23 +279,73 @@ spmm_mfma_flat_kernel(int m_vec, int n_cols, int n_tiles, int nonzeros_vec, int 
     }
     __syncthreads();
 
+    // Parts of rows that leave the piece go to the workspace.  ONE_LAUNCH: `pending` = this wave has written one and
+    // counts itself in on the row's counter (the counter of the piece the row starts in; at most one row starts
+    // in a piece and leaves it).
+    bool pending = false;
+    int p_row = 0, p_first = 0, p_last = 0;  // the row, the piece it starts in, the piece it ends in
     if (has_t) {
         const long long stop = t_row_end < ce ? t_row_end : ce;
         const int last = (int)((stop - 1 - cb) / sub);  // the last run of this piece that holds nonzeros of the row
         for (int w = wave + 1; w <= last; ++w) tile_add<V, CPL>(f_tiles + (size_t)w * V * TN, TN, cs, g, acc);
-        if (t_row_end <= ce)  // the row ends inside the piece: this is all of it
+        if (t_row_end <= ce) {  // the row ends inside the piece: this is all of it
             tile_to_output<V, CPL, OutT>(out, t_row, n_cols, col0, col_ok, g, acc);
-        else
+        } else if constexpr (ONE_LAUNCH) {
+            tile_store_coherent<V, CPL>(tile_area(ws_base), (uint32_t)(((size_t)2 * c + 1) * ws_tile + tile * TN) * 4u, ws_pitch,
+                                        cs, g, acc);
+            pending = true;
+            p_row = t_row;
+            p_first = c;
+            p_last = (int)((t_row_end - 1) / piece);
+        } else {
             tile_store<V, CPL>(ws + ((size_t)2 * c + 1) * ws_tile, ws_pitch, cs, g, acc);
+        }
     }
-    if (wave == 0 && has_f) {  // the piece starts inside a row: its part of that row goes to F[c]
-        float4_t sum[CPL];
+    for (int round = 0; round < 2; ++round) {
+        if (round == 1) {
+            // the piece starts inside a row: its part of that row goes to F[c] (wave 0, after its own T part)
+            pending = false;
+            if (wave == 0 && has_f) {
+                float4_t sum[CPL];
 #pragma unroll
-        for (int q = 0; q < CPL; ++q) sum[q] = float4_t{0.f, 0.f, 0.f, 0.f};
-        const long long stop = f_row_end < ce ? f_row_end : ce;
-        const int last = (int)((stop - 1 - cb) / sub);
-        for (int w = 0; w <= last; ++w) tile_add<V, CPL>(f_tiles + (size_t)w * V * TN, TN, cs, g, sum);
-        tile_store<V, CPL>(ws + (size_t)2 * c * ws_tile, ws_pitch, cs, g, sum);
+                for (int q = 0; q < CPL; ++q) sum[q] = float4_t{0.f, 0.f, 0.f, 0.f};
+                const long long stop = f_row_end < ce ? f_row_end : ce;
+                const int last = (int)((stop - 1 - cb) / sub);
+                for (int w = 0; w <= last; ++w) tile_add<V, CPL>(f_tiles + (size_t)w * V * TN, TN, cs, g, sum);
+                if constexpr (ONE_LAUNCH) {
+                    tile_store_coherent<V, CPL>(tile_area(ws_base), (uint32_t)((size_t)2 * c * ws_tile + tile * TN) * 4u, ws_pitch,
+                                                cs, g, sum);
+                    pending = true;
+                    p_row = f_row;
+                    p_first = (int)(f_row_beg / piece);
+                    p_last = (int)((f_row_end - 1) / piece);
+                } else {
+                    tile_store<V, CPL>(ws + (size_t)2 * c * ws_tile, ws_pitch, cs, g, sum);
+                }
+            }
+        }
+        if constexpr (ONE_LAUNCH) {
+            if (!pending) continue;
+            int *counter = counters + (size_t)p_first * n_tiles + tile;
+            // the part's stores have completed (they go through to memory) before the count says so
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            __builtin_amdgcn_s_waitcnt(0);
+            int arrived = 0;
+            if (lane == 0) arrived = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            arrived = __builtin_amdgcn_readfirstlane(arrived);
+            if (arrived != p_last - p_first) continue;  // parts are still to come: whoever brings the last adds up
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // the parts are read after the count was seen
+            float4_t total[CPL];
+#pragma unroll
+            for (int q = 0; q < CPL; ++q) total[q] = float4_t{0.f, 0.f, 0.f, 0.f};
+            // T of the first piece, then F of the others, in ascending order
+            for (int pc = p_first; pc <= p_last; ++pc)
+                tile_add_coherent<V, CPL>(tile_area(ws_base),
+                                          (uint32_t)(((size_t)2 * pc + (pc == p_first ? 1 : 0)) * ws_tile + tile * TN) * 4u,
+                                          ws_pitch, cs, g, total);
+            tile_to_output<V, CPL, OutT>(out, p_row, n_cols, col0, col_ok, g, total);
+            if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+        }
     }
 }
 
@@ -266,7 +402,15 @@ spmm_flat_fixup_kernel(int m_vec, int n_cols, long long piece, int n_pieces, con
 
 namespace {
 
+// The workspace starts with one arrival counter per (piece, column tile), rounded up to 256 bytes, followed by the
+// tiles F and T of every piece.
+inline long long flat_counter_bytes(long long n_pieces, int n_tiles)
+{
+    return (n_pieces * n_tiles * (long long)sizeof(int) + 255) / 256 * 256;
+}
+
 struct FlatShape {
+    bool one_launch;  // cross-workgroup parts added inside the launch (arrival counters) instead of by a second one
     int cpl;       // columns per lane (tile of 16*cpl dense columns)
     int waves;     // runs (= waves) per piece (= workgroup)
     int sub;       // nonzero vectors per run
@@ -274,11 +418,11 @@ struct FlatShape {
     int ws_pitch;  // floats per row of a workspace tile: the dense width rounded up to whole tiles
 };
 
-// Launch shape: sixteen runs per piece, runs of three to eight steps sized so that the launch holds about 3600
-// waves (measured on Pareto-distributed rows of mean 280, 256 to 4096 vector rows x 4608, N = 256: five steps
-// best at 1024 rows, eight at 4096, three to four at 256; twelve thousand waves of two steps cost 1.6 times as
-// much, because every wave pays its row search before its first gather); longer runs (fewer, larger pieces) when
-// the workspace cannot hold two partial tiles per piece.
+// Launch shape: eight runs per piece, runs of four to eight steps sized so that the launch holds about 3600
+// waves (measured on Pareto-distributed rows of mean 280, 256 to 4096 vector rows x 4608, N = 256: four steps
+// best at 256 rows, five at 1024, eight at 4096; twelve thousand waves of two steps cost 1.6 times as much,
+// because every wave pays its row search before its first gather; sixteen runs per piece 0 to 15 % behind eight);
+// longer runs (fewer, larger pieces) when the workspace cannot hold two partial tiles per piece.
 bool flat_shape(int vec_length, int k, int nonzeros_vec, long long workspace_bytes, FlatShape &s)
 {
     const Options &o = options();
@@ -291,28 +435,59 @@ bool flat_shape(int vec_length, int k, int nonzeros_vec, long long workspace_byt
     const int n_tiles = ceil_div(k, 16 * cpl);
     s.cpl = cpl;
     s.ws_pitch = n_tiles * 16 * cpl;
-    s.waves = o.spmm_flat_waves > 0 ? o.spmm_flat_waves : 16;
+    s.waves = o.spmm_flat_waves > 0 ? o.spmm_flat_waves : 8;
+    s.one_launch = o.spmm_flat_launches != 2;  // (and the tile area below 2 GiB: 32-bit buffer offsets, see below)
     long long sub = o.spmm_flat_piece > 0 ? o.spmm_flat_piece : ((long long)nonzeros_vec * n_tiles + 3583) / 3584;
     sub = (sub + kStep - 1) / kStep * kStep;
     if (o.spmm_flat_piece <= 0) {
-        if (sub < 3 * kStep) sub = 3 * kStep;
+        if (sub < 4 * kStep) sub = 4 * kStep;
         if (sub > 8 * kStep) sub = 8 * kStep;
     }
     const long long slot_bytes = 2LL * vec_length * s.ws_pitch * (long long)sizeof(float);  // T and F of one piece
     for (;;) {
         const long long piece = sub * s.waves;
         const long long n_pieces = ((long long)nonzeros_vec + piece - 1) / piece;
-        if (n_pieces <= 1 || n_pieces * slot_bytes <= workspace_bytes) {
+        if (n_pieces <= 1 || flat_counter_bytes(n_pieces, n_tiles) + n_pieces * slot_bytes <= workspace_bytes) {
             s.sub = (int)sub;
             s.n_pieces = (int)n_pieces;
+            if (n_pieces * slot_bytes >= (1LL << 31)) s.one_launch = false;
             return true;
         }
         if (sub >= (1LL << 30)) return false;
-        const long long fit = workspace_bytes / slot_bytes;  // pieces the workspace can hold (>= 0)
+        const long long fit = (workspace_bytes - 256) / (slot_bytes + 4 * n_tiles);  // pieces the workspace can hold
         long long grown = fit > 1 ? ((long long)nonzeros_vec + fit - 1) / fit : (long long)nonzeros_vec;
         grown = ((grown + s.waves - 1) / s.waves + kStep - 1) / kStep * kStep;
         sub = grown > sub ? grown : sub + kStep;
     }
+}
+
+template <int V, int CPL, bool IDX32, bool ONE_LAUNCH, typename OutT>
+int launch_flat_kernel(int m_vec, int k, int nonzeros_vec, const FlatShape &s, const int *row_offsets,
+                       const int *column_indices, const half_t *values, const half_t *rhs, OutT *out, float *workspace,
+                       hipStream_t stream)
+{
+    const int n_tiles = ceil_div(k, 16 * CPL);
+    const long long main_blocks = (long long)s.n_pieces * n_tiles;
+    const long long zero_blocks = ONE_LAUNCH ? ceil_div(m_vec, 4 * s.waves) : 0;
+    if (main_blocks + zero_blocks > 0x7fffffffLL) return hipErrorNotSupported;
+    int *counters = reinterpret_cast<int *>(workspace);
+    float *tiles = reinterpret_cast<float *>(reinterpret_cast<unsigned char *>(workspace) +
+                                             (s.n_pieces > 1 ? flat_counter_bytes(s.n_pieces, n_tiles) : 0));
+    const size_t lds = (size_t)s.waves * (stage_bytes<V>() + (size_t)V * 16 * CPL * sizeof(float));
+    auto kernel = spmm_mfma_flat_kernel<V, CPL, IDX32, ONE_LAUNCH, OutT>;
+    static std::atomic<unsigned long long> lds_allowed{0};
+    const hipError_t attr = allow_large_lds(reinterpret_cast<const void *>(kernel), 96 * 1024, lds_allowed);
+    if (attr != hipSuccess) return (int)attr;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(main_blocks + zero_blocks)), dim3(64 * s.waves), lds, stream, m_vec, k,
+                       n_tiles, nonzeros_vec, s.sub, (int)main_blocks, counters, row_offsets, column_indices, values, rhs,
+                       out, tiles, s.ws_pitch);
+    const hipError_t st = hipGetLastError();
+    if (st != hipSuccess || ONE_LAUNCH) return (int)st;
+    const long long fix_blocks = (long long)(s.n_pieces - 1) + ceil_div(m_vec, 4);
+    if (fix_blocks > 0x7fffffffLL) return hipErrorNotSupported;
+    hipLaunchKernelGGL((spmm_flat_fixup_kernel<V, OutT>), dim3((unsigned)fix_blocks), dim3(256), 0, stream, m_vec, k,
+                       (long long)s.sub * s.waves, s.n_pieces, row_offsets, tiles, s.ws_pitch, out);
+    return (int)hipGetLastError();
 }
 
 template <int V, int CPL, bool IDX32, typename OutT>
@@ -320,23 +495,11 @@ int launch_flat_idx(int m_vec, int k, int nonzeros_vec, const FlatShape &s, cons
                     const int *column_indices, const half_t *values, const half_t *rhs, OutT *out, float *ws,
                     hipStream_t stream)
 {
-    const int n_tiles = ceil_div(k, 16 * CPL);
-    const long long blocks = (long long)s.n_pieces * n_tiles;
-    if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
-    const size_t lds = (size_t)s.waves * (stage_bytes<V>() + (size_t)V * 16 * CPL * sizeof(float));
-    auto kernel = spmm_mfma_flat_kernel<V, CPL, IDX32, OutT>;
-    static std::atomic<unsigned long long> lds_allowed{0};
-    const hipError_t attr = allow_large_lds(reinterpret_cast<const void *>(kernel), 96 * 1024, lds_allowed);
-    if (attr != hipSuccess) return (int)attr;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(64 * s.waves), lds, stream, m_vec, k, n_tiles,
-                       nonzeros_vec, s.sub, row_offsets, column_indices, values, rhs, out, ws, s.ws_pitch);
-    const hipError_t st = hipGetLastError();
-    if (st != hipSuccess) return (int)st;
-    const long long fix_blocks = (long long)(s.n_pieces - 1) + ceil_div(m_vec, 4);
-    if (fix_blocks > 0x7fffffffLL) return hipErrorNotSupported;
-    hipLaunchKernelGGL((spmm_flat_fixup_kernel<V, OutT>), dim3((unsigned)fix_blocks), dim3(256), 0, stream, m_vec, k,
-                       (long long)s.sub * s.waves, s.n_pieces, row_offsets, ws, s.ws_pitch, out);
-    return (int)hipGetLastError();
+    if (s.one_launch)
+        return launch_flat_kernel<V, CPL, IDX32, true, OutT>(m_vec, k, nonzeros_vec, s, row_offsets, column_indices, values,
+                                                             rhs, out, ws, stream);
+    return launch_flat_kernel<V, CPL, IDX32, false, OutT>(m_vec, k, nonzeros_vec, s, row_offsets, column_indices, values,
+                                                          rhs, out, ws, stream);
 }
 
 template <int V, typename OutT>
@@ -360,7 +523,9 @@ long long spmm_flat_workspace_bytes(int vec_length, int k, int nonzeros_vec)
     if (k <= 0 || nonzeros_vec <= 0) return 0;
     FlatShape s;
     if (!flat_shape(vec_length, k, nonzeros_vec, 0x7fffffffffffffffLL, s)) return 0;
-    return s.n_pieces > 1 ? 2LL * s.n_pieces * vec_length * s.ws_pitch * (long long)sizeof(float) : 0;
+    if (s.n_pieces <= 1) return 0;
+    return flat_counter_bytes(s.n_pieces, s.ws_pitch / (16 * s.cpl)) +
+           2LL * s.n_pieces * vec_length * s.ws_pitch * (long long)sizeof(float);
 }
 
 template <typename OutT>

@@ -212,6 +212,7 @@ struct Options {
     int spmm_cols_per_lane = 0;
     int spmm_gather = 0;        // 1 = gathered rows through registers, 2 = through LDS-DMA loads, 0 = automatic
     int spmm_flat_piece = 0;    // split-row SpMM: nonzero vectors per wave (rounded up to 32), 0 = automatic
+    int spmm_flat_launches = 0; // split-row SpMM: 1 = parts added inside the launch, 2 = by a second launch, 0 = automatic
     int spmm_flat_waves = 0;    // split-row SpMM: waves per workgroup, 0 = automatic
     int sddmm_slots = 0;
     int sddmm_block_waves = 0;

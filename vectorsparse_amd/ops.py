@@ -109,8 +109,9 @@ def spmm_split_rows(m_vec, vec_length, k, n, nonzeros_vec, row_offsets, column_i
                     output_matrix, workspace=None, stream=None, row_indices=None):
     """wmmaSpmm on the schedule that splits the nonzero range instead of the rows (skewed row lengths).
 
-    workspace: a device tensor (any dtype) for the partial tiles of rows that cross workgroups, or None (one
-    workgroup then takes everything).  Returns output_matrix.
+    workspace: a device tensor (any dtype), zero-filled before its first use (it starts with arrival counters
+    that every call leaves at zero), for the partial tiles of rows that cross workgroups; or None (one workgroup
+    then takes everything).  Returns output_matrix.
     """
     f32 = output_matrix.dtype is torch.float32
     entry = "vs_wmma_spmm_f16_f32out_ws" if f32 else "vs_wmma_spmm_f16_ws"
@@ -453,7 +454,7 @@ class DeviceProblem:
         if split_rows and kernel == "wmma":
             need = spmm_workspace_bytes(self.m_vec, self.vec_length, k, self.n, self.nnz_vec)
             if self._workspace is None or self._workspace.numel() < need:
-                self._workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=rhs_matrix.device)
+                self._workspace = torch.zeros(max(need, 16), dtype=torch.uint8, device=rhs_matrix.device)
             return spmm_split_rows(self.m_vec, self.vec_length, k, self.n, self.nnz_vec, self.row_offsets,
                                    self.column_indices, self.values, rhs_matrix, out, self._workspace, stream)
         if row_length_hint and out.dtype == torch.float16:
