@@ -77,6 +77,22 @@ def test_device_problem_reads_the_row_statistics():
     assert tiny.longest_row_vec == 0 and not tiny.skewed
 
 
+def test_split_row_choice_follows_the_row_lengths():
+    """The rule behind DeviceProblem.spmm(split_rows=None), on the row-length shapes it was measured on."""
+    pays = ops.split_rows_pays
+    # one dense row among rows of a hundred vectors: pays at every row count
+    for m_vec in (64, 256, 1024, 2048):
+        assert pays(m_vec, 4608 + 100 * (m_vec - 1), 4608)
+    # uniform lengths: never
+    for m_vec in (64, 1024):
+        assert not pays(m_vec, 461 * m_vec, 461)
+    # longest row at 15 mean lengths (Pareto): only for small matrices
+    assert pays(128, 128 * 300, 4500) and pays(256, 256 * 300, 4500)
+    assert not pays(512, 512 * 300, 4500) and not pays(1024, 1024 * 300, 4500)
+    # too small to matter, and degenerate shapes
+    assert not pays(8, 400, 300) and not pays(0, 0, 0)
+
+
 def test_sweep_benchmark_selection(tmp_path):
     """The sweep driver's file handling (job_launcher.py:25-50): list files, ranges, layer widths, buckets."""
     from vectorsparse_amd import sweep

@@ -74,7 +74,19 @@ def build_cxx_caller(verbose=False):
     return exe
 
 
+def build_probes(verbose=False):
+    """Compile csrc/probes/machine_probe.hip (launch floor, dependent-load latency, gather ceiling of the GPU) to
+    vectorsparse_amd/probes/machine_probe; run it on a GPU box to get the floors DESIGN.md prices the kernels by."""
+    out_dir = os.path.join(_HERE, "probes")
+    os.makedirs(out_dir, exist_ok=True)
+    exe = os.path.join(out_dir, "machine_probe")
+    _run([HIPCC, "-O3", "--offload-arch=gfx950", "-std=c++17", "-Wno-unused-value",
+          os.path.join(CSRC, "probes", "machine_probe.hip"), "-o", exe], verbose)
+    return exe
+
+
 if __name__ == "__main__":
     print(build(verbose=True, incremental="--incremental" in sys.argv))
     print(build_cxx_caller(verbose=True))
+    print(build_probes(verbose=True))
     sys.exit(0)

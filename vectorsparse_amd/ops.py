@@ -420,6 +420,19 @@ def SortedRowSwizzle(rows, row_offsets):
     return out
 
 
+def split_rows_pays(m_vec, nonzeros_vec, longest_row_vec):
+    """Whether the split-row SpMM schedule is expected to beat the row-per-workgroup one with row-length hints.
+    Measured at N = 256, V = 8, rows of up to 4608 vectors: a row of 25 or more mean lengths (one dense row among
+    short ones) holds its single workgroup per tile for 13-22 us where the split schedule needs 10-15 us whatever
+    the row count; milder skew (8 mean lengths and up: Pareto or lognormal lengths) pays only while the matrix has
+    at most 256 vector rows (10.6-12.8 us against 11.8-13.9 us), larger ones keep the chip busy with whole rows
+    (13.7 against 15.8 us at 512 rows).  Uniform and binomial lengths never pay (a third to twice slower)."""
+    if m_vec <= 0 or nonzeros_vec < 8192:
+        return False
+    ratio = longest_row_vec * m_vec / float(nonzeros_vec)
+    return ratio >= 25.0 or (ratio >= 8.0 and m_vec <= 256)
+
+
 class DeviceProblem:
     """Device-resident operands of one SpMM / SDDMM problem (caller-owned buffers, as in BmFN)."""
 
@@ -447,10 +460,15 @@ class DeviceProblem:
         """SpMM through the reference-shaped entry points; with row_length_hint (fp16 output only) through the
         batched entry point with batch = 1, which also takes the pattern's nonzero count and longest row and
         sizes its workgroups by the real row lengths instead of by n; with split_rows (MFMA path) on the
-        schedule that cuts the nonzero range into equal pieces, with a workspace this object owns."""
+        schedule that cuts the nonzero range into equal pieces, with a workspace this object owns.
+        split_rows=None chooses between those two from the row lengths (see split_rows_pays)."""
         k = rhs_matrix.shape[1]
         if out is None:
             out = torch.empty((self.m_vec * self.vec_length, k), dtype=out_dtype, device=rhs_matrix.device)
+        if split_rows is None:
+            split_rows = kernel == "wmma" and k % 4 == 0 and split_rows_pays(self.m_vec, self.nnz_vec,
+                                                                            self.longest_row_vec)
+            row_length_hint = True
         if split_rows and kernel == "wmma":
             need = spmm_workspace_bytes(self.m_vec, self.vec_length, k, self.n, self.nnz_vec)
             if self._workspace is None or self._workspace.numel() < need:
