@@ -93,6 +93,30 @@ def test_ragged_rows_and_empty_rows(gpu, V, kernel):
         assert not got[i * V:(i + 1) * V].any(), "empty vector row %d must be written as zeros" % i
 
 
+@pytest.mark.parametrize("V", [1, 2, 4, 8])
+@pytest.mark.parametrize("steps", [1, 2, 4])
+@pytest.mark.parametrize("cpl", [4, 8])
+def test_steps_in_flight_variants_keep_parity(gpu, V, steps, cpl):
+    """The MFMA kernel with one, two or four 32-vector steps of gathered rows in flight per wave: rows that end
+    inside a block (1, 33, 65, 127, 129 vectors), empty rows, rows of many blocks, and every wave count - including
+    more waves than a row has blocks."""
+    lengths = np.array([0, 1, 33, 64, 65, 0, 127, 128, 129, 300, 2, 0, 700, 7, 96, 0], dtype=np.int64)
+    n = 768
+    rng = np.random.default_rng(50 + V)
+    ro, ci = cv._pattern_from_lengths(rng, len(lengths), n, lengths)
+    pat = cv.random_values(cv.ColVecCSR(len(lengths), n, V, ro, ci).validate(), seed=51)
+    for N in (64, 136, 256):
+        B = cv.dense_uniform(n, N, seed=N)
+        ref = _oracle(pat, B)
+        for waves in (0, 1, 3, 8, 16):
+            with _lib.thread_options(spmm_steps=steps, spmm_cols_per_lane=cpl, spmm_waves=waves):
+                got = _run(pat, B, "wmma")
+                got32 = _run(pat, B, "wmma", out_dtype=torch.float32) if waves in (0, 3) else None
+            assert_parity(got, ref, "steps=%d cpl=%d waves=%d N=%d" % (steps, cpl, waves, N))
+            if got32 is not None:
+                assert_parity(got32, ref, "fp32 out, steps=%d cpl=%d waves=%d N=%d" % (steps, cpl, waves, N))
+
+
 @pytest.mark.parametrize("kernel", ["wmma", "cuda"])
 def test_all_rows_empty(gpu, kernel):
     pat = cv.ColVecCSR(8, 64, 8, np.zeros(9, np.int32), np.zeros(0, np.int32), np.zeros((0, 8), np.float16))

@@ -28,8 +28,10 @@ namespace vs {
 // exp2(s*x - max) (and sums them), and the accumulated tile is divided by the row sum at the end.
 // RAGGED: the dense width is not a multiple of CPL (rows of the dense operand and of the output start at any 2-byte
 // boundary, the last chunk of a row is cut): chunks are fetched and stored half by half.
-template <int V, int CPL, bool SOFTMAX, bool IDX32, typename OutT, bool RAGGED = false>
-__global__ void __launch_bounds__(1024)
+// S: 32-vector steps a wave keeps in flight at once (1, 2 or 4): its unit of work is a block of S steps whose 8 * S
+// row segments per lane are all requested before the first MFMA.
+template <int V, int CPL, bool SOFTMAX, bool IDX32, typename OutT, bool RAGGED = false, int S = 1>
+__global__ void __launch_bounds__(S * CPL >= 32 ? 256 : (S * CPL >= 16 ? 512 : 1024))
 spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
                  const int *__restrict__ row_offsets, const int *__restrict__ column_indices,
                  const half_t *__restrict__ values, const half_t *__restrict__ rhs,
@@ -41,9 +43,11 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
     out += blockIdx.y * stride_out;
     extern __shared__ __align__(16) unsigned char smem[];  // [W] staging slots, then [W][V][TN] partials
     constexpr int TN = 16 * CPL;
-    constexpr int kStage = stage_bytes<V>();
+    constexpr int kStage = S * stage_bytes<V>();
+    constexpr int kBlock = S * kStep;       // nonzero vectors per block
+    constexpr int F = (S + 1) / 2;          // vectors a lane fetches per block (lanes 0..31 only when S = 1)
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n_waves = blockDim.x >> 6;
     const int tile = blockIdx.x % n_tiles;
     const int slot = blockIdx.x / n_tiles;
@@ -58,9 +62,22 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
     const int valid = !col_ok ? 0 : (n_cols - col0 < CPL ? n_cols - col0 : CPL);  // RAGGED: halves of the chunk that exist
 
     int *idx_s = reinterpret_cast<int *>(smem + (size_t)wave * kStage);
-    half_t *vec_s = reinterpret_cast<half_t *>(idx_s + kStep);  // [V][kStep]
+    half_t *vec_s = reinterpret_cast<half_t *>(idx_s + kBlock);  // [V][kBlock]
     float *partial = reinterpret_cast<float *>(smem + (size_t)n_waves * kStage);
     float *sums_s = partial + (size_t)n_waves * V * TN;  // [W][V] softmax denominators (SOFTMAX only)
+
+    // Short rows do not need every wave: with fewer than two steps per wave the partial-tile reduction costs
+    // more than the split saves (S = 1); with S steps in flight a block is one round trip whatever its size, so
+    // every block gets its own wave - except that the barrier and the sum through LDS cost more than a second
+    // round trip, so a row of two blocks stays with one wave when the grid alone fills the chip (512 workgroups
+    // and more: 3.23 against 3.35 us on 256 rows of 102 vectors, N = 256; with 256 workgroups 2.78 against 2.64).
+    // The other waves end here: a workgroup barrier waits only for the waves that are still running, and a row
+    // of a single active wave needs neither barrier nor LDS for its result.
+    const int steps = (end - beg + kStep - 1) / kStep;
+    int active = S == 1 ? (steps + 1) >> 1 : (steps + S - 1) / S;
+    if (S > 1 && active == 2 && gridDim.x * gridDim.y >= 512) active = 1;
+    active = active < 1 ? 1 : (active > n_waves ? n_waves : active);
+    if (wave >= active) return;
 
     const float s2 = scale * kLog2e;
     float row_max[V], row_sum[V];
@@ -84,53 +101,69 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
 #pragma unroll
     for (int c = 0; c < CPL; ++c) acc[c] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    // Short rows do not need every wave: with fewer than two steps per wave the partial-tile
-    // reduction costs more than the split saves, so only `active` waves take steps.
-    const int steps = (end - beg + kStep - 1) / kStep;
-    int active = (steps + 1) >> 1;
-    active = active < 1 ? 1 : (active > n_waves ? n_waves : active);
-
     // The column index and the vector of the NEXT step are fetched into registers while the gathered
     // rows of the current step are in flight, so a wave pays one memory round trip per step, not two.
-    const int stride = kStep * active;
-    int base = beg + kStep * wave;
-    const bool has_work = wave < active && base < end;
-    int next_idx = 0;
-    bool next_valid = false;
-    half_t next_vec[V];
+    const int stride = kBlock * active;
+    int base = beg + kBlock * wave;
+    const bool has_work = base < end;
+    int next_idx[F];
+    bool next_valid[F];
+    half_t next_vec[F][V];
 #pragma unroll
-    for (int v = 0; v < V; ++v) next_vec[v] = (half_t)0.f;
+    for (int i = 0; i < F; ++i) {
+        next_idx[i] = 0;
+        next_valid[i] = false;
+#pragma unroll
+        for (int v = 0; v < V; ++v) next_vec[i][v] = (half_t)0.f;
+    }
     auto fetch = [&](int b) {
-        if (lane < kStep) {
-            const int j = b + lane;
-            next_valid = j < end;
-            // Slots past the row's end repeat its last vector with a zero value: the gather stays
-            // in bounds and contributes nothing.
-            const int jc = next_valid ? j : end - 1;
-            next_idx = column_indices[jc];
-            load_vector<V>(next_vec, values + (size_t)jc * V);
+#pragma unroll
+        for (int i = 0; i < F; ++i) {
+            if (64 * i + lane < kBlock) {
+                const int j = b + 64 * i + lane;
+                next_valid[i] = j < end;
+                // Slots past the row's end repeat its last vector with a zero value: the gather stays
+                // in bounds and contributes nothing.
+                const int jc = next_valid[i] ? j : end - 1;
+                next_idx[i] = column_indices[jc];
+                load_vector<V>(next_vec[i], values + (size_t)jc * V);
+            }
         }
     };
     if (has_work) fetch(base);
 
     for (; has_work && base < end; base += stride) {
-        if (lane < kStep) {
-            idx_s[lane] = next_idx;
 #pragma unroll
-            for (int v = 0; v < V; ++v) {
-                half_t staged = next_valid ? next_vec[v] : (half_t)0.f;
-                if constexpr (SOFTMAX) {
-                    const float p = next_valid ? __builtin_amdgcn_exp2f((float)next_vec[v] * s2 - row_max[v]) : 0.f;
-                    row_sum[v] += p;
-                    staged = (half_t)p;
+        for (int i = 0; i < F; ++i) {
+            const int at = 64 * i + lane;
+            if (at < kBlock) {
+                idx_s[at] = next_idx[i];
+#pragma unroll
+                for (int v = 0; v < V; ++v) {
+                    half_t staged = next_valid[i] ? next_vec[i][v] : (half_t)0.f;
+                    if constexpr (SOFTMAX) {
+                        const float p =
+                            next_valid[i] ? __builtin_amdgcn_exp2f((float)next_vec[i][v] * s2 - row_max[v]) : 0.f;
+                        row_sum[v] += p;
+                        staged = (half_t)p;
+                    }
+                    vec_s[v * kBlock + at] = staged;
                 }
-                vec_s[v * kStep + lane] = staged;
             }
         }
         wave_lds_fence();
-        spmm_mfma_step<V, CPL, IDX32, RAGGED>(idx_s, vec_s, rhs, n_cols, col_off, cs, g, acc, [&] {
-            if (base + stride < end) fetch(base + stride);
-        }, valid);
+        if constexpr (S == 1) {
+            spmm_mfma_step<V, CPL, IDX32, RAGGED>(idx_s, vec_s, rhs, n_cols, col_off, cs, g, acc, [&] {
+                if (base + stride < end) fetch(base + stride);
+            }, valid);
+        } else {
+            // A block that the row fills only in part still requests all its steps (the padding repeats one row
+            // segment, which stays in the L1): asking for fewer steps behind a uniform branch measured 5 % slower
+            // on short rows (the three code paths) and 4 % faster on long ones.
+            spmm_mfma_block<V, CPL, S, IDX32>(idx_s, vec_s, rhs, n_cols, col_off, cs, g, acc, [&] {
+                if (base + stride < end) fetch(base + stride);
+            });
+        }
     }
 
     if constexpr (SOFTMAX) {
@@ -138,7 +171,7 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
         for (int v = 0; v < V; ++v) row_sum[v] = wave_sum(row_sum[v]);
     }
 
-    if (n_waves == 1) {
+    if (active == 1) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const int v = 4 * g + e;
@@ -166,7 +199,7 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         const int v = 4 * g + e;
-        if (v < V && wave < active) {
+        if (v < V) {
 #pragma unroll
             for (int c4 = 0; c4 < CPL / 4; ++c4) {
                 float4_t t = {acc[4 * c4][e], acc[4 * c4 + 1][e], acc[4 * c4 + 2][e], acc[4 * c4 + 3][e]};
@@ -175,7 +208,7 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
         }
     }
     if constexpr (SOFTMAX) {
-        if (lane < V && wave < active) {
+        if (lane < V) {
             float mine_sum = 0.f;
 #pragma unroll
             for (int v = 0; v < V; ++v) mine_sum = (v == lane) ? row_sum[v] : mine_sum;
@@ -183,7 +216,7 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
         }
     }
     __syncthreads();
-    const int t = threadIdx.x;
+    const int t = threadIdx.x;  // V * 16 <= 128 threads add: waves 0 and 1, both among the active ones here
     if (t < V * 16) {
         const int v = t >> 4;
         const int cs2 = t & 15;
@@ -227,7 +260,7 @@ static int next_pow2(int x)
     return p;
 }
 
-template <int V, int CPL, bool SOFTMAX, bool IDX32, typename OutT>
+template <int V, int CPL, bool SOFTMAX, bool IDX32, typename OutT, int S = 1>
 static int launch_idx(int m_vec, int k, int n, int waves, const int *row_indices, const int *row_offsets,
                       const int *column_indices, const half_t *values, const half_t *rhs, OutT *out,
                       hipStream_t stream, const Batch &batch, float scale)
@@ -237,9 +270,9 @@ static int launch_idx(int m_vec, int k, int n, int waves, const int *row_indices
     const int n_tiles = ceil_div(k, TN);
     const long long blocks = (long long)m_vec * n_tiles;
     if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
-    const size_t lds = (size_t)waves * stage_bytes<V>() +
+    const size_t lds = (size_t)waves * S * stage_bytes<V>() +
                        (waves > 1 ? (size_t)waves * V * (TN + 1) * sizeof(float) : 0);
-    auto kernel = spmm_mfma_kernel<V, CPL, SOFTMAX, IDX32, OutT>;
+    auto kernel = spmm_mfma_kernel<V, CPL, SOFTMAX, IDX32, OutT, false, S>;
     static std::atomic<unsigned long long> lds_allowed{0};
     const hipError_t attr = allow_large_lds(reinterpret_cast<const void *>(kernel), 96 * 1024, lds_allowed);
     if (attr != hipSuccess) return (int)attr;
@@ -267,28 +300,38 @@ static int launch_ragged(int m_vec, int k, int waves, const int *row_indices, co
 }
 
 template <int V, int CPL, bool SOFTMAX, typename OutT>
-static int launch_one(int m_vec, int k, int n, int waves, const int *row_indices, const int *row_offsets,
-                      const int *column_indices, const half_t *values, const half_t *rhs, OutT *out,
-                      hipStream_t stream, const Batch &batch, float scale)
+static int launch_one(int m_vec, int k, int n, int waves, int in_flight, const int *row_indices,
+                      const int *row_offsets, const int *column_indices, const half_t *values, const half_t *rhs,
+                      OutT *out, hipStream_t stream, const Batch &batch, float scale)
 {
-    if ((long long)n * k < (1LL << 31))
+    if ((long long)n * k < (1LL << 31)) {
+        if constexpr (!SOFTMAX) {
+            // blocks of several steps in flight exist for the common case only: offsets that fit 32 bits
+            if (in_flight == 4)
+                return launch_idx<V, CPL, SOFTMAX, true, OutT, 4>(m_vec, k, n, waves, row_indices, row_offsets,
+                                                                   column_indices, values, rhs, out, stream, batch, scale);
+            if (in_flight >= 2)
+                return launch_idx<V, CPL, SOFTMAX, true, OutT, 2>(m_vec, k, n, waves, row_indices, row_offsets,
+                                                                   column_indices, values, rhs, out, stream, batch, scale);
+        }
         return launch_idx<V, CPL, SOFTMAX, true, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices,
                                                         values, rhs, out, stream, batch, scale);
+    }
     return launch_idx<V, CPL, SOFTMAX, false, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices,
                                                      values, rhs, out, stream, batch, scale);
 }
 
 template <int CPL, bool SOFTMAX, typename OutT>
-static int launch_v(int vec_length, int m_vec, int k, int n, int waves, const int *row_indices,
+static int launch_v(int vec_length, int m_vec, int k, int n, int waves, int in_flight, const int *row_indices,
                     const int *row_offsets, const int *column_indices, const half_t *values,
                     const half_t *rhs, OutT *out, hipStream_t stream, const Batch &batch,
                     float scale)
 {
     switch (vec_length) {
-    case 1: return launch_one<1, CPL, SOFTMAX, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
-    case 2: return launch_one<2, CPL, SOFTMAX, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
-    case 4: return launch_one<4, CPL, SOFTMAX, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
-    case 8: return launch_one<8, CPL, SOFTMAX, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
+    case 1: return launch_one<1, CPL, SOFTMAX, OutT>(m_vec, k, n, waves, in_flight, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
+    case 2: return launch_one<2, CPL, SOFTMAX, OutT>(m_vec, k, n, waves, in_flight, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
+    case 4: return launch_one<4, CPL, SOFTMAX, OutT>(m_vec, k, n, waves, in_flight, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
+    case 8: return launch_one<8, CPL, SOFTMAX, OutT>(m_vec, k, n, waves, in_flight, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
     default: return hipErrorInvalidValue;
     }
 }
@@ -314,32 +357,65 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
     const bool ragged = k % 4 != 0;
     if (ragged) cpl = 4;
     const long long blocks = (long long)m_vec * ceil_div(k, 16 * cpl) * batch.count;
+    // Steps of gathered rows a wave keeps in flight.  Two pay as soon as rows hold more than one step: the wave
+    // waits once for 64 vectors instead of twice (ResNet-shaped grid, 16 to 2304 vectors per row, N = 64 and 256:
+    // 5-20 % faster than one step at the best wave count of each; 3 % slower on rows of under 32 vectors).  Four
+    // pay 2-4 % more on large problems with 128-bit segments and cost up to 14 % on rows of one or two steps, so
+    // they are chosen only when the row lengths are known.  The unhinted entry takes the rows to hold a quarter of
+    // n: the kernel leaves the waves that a shorter row does not need idle at little cost (1.5 % per doubling
+    // of the workgroup beyond four waves), while too few waves for denser rows cost 10-18 %.
+    const bool hinted = batch.nonzeros_vec >= 0;
+    const int mean_steps = hinted ? ceil_div(ceil_div(batch.nonzeros_vec, m_vec), kStep) : ceil_div(n, 4 * kStep);
+    const int longest_steps = ceil_div(batch.longest_row_vec > 0 ? batch.longest_row_vec : 0, kStep);
+    // while the chip has room the workgroup of the longest row ends last, so that row sets the size
+    const int row_steps = longest_steps > mean_steps ? longest_steps : mean_steps;
+    const bool blocks_exist = !SOFTMAX && !ragged && !use_dma && (long long)n * k < (1LL << 31);
+    int in_flight = options().spmm_steps;
+    if (in_flight != 1 && in_flight != 2 && in_flight != 4) {
+        in_flight = row_steps >= 2 ? 2 : 1;
+        if (hinted && cpl == 8 && blocks >= 512 && mean_steps >= 8) in_flight = 4;
+    }
+    if (!blocks_exist) in_flight = 1;
     int waves = options().spmm_waves;
+    if (waves <= 0 && in_flight > 1) {
+        // One wave per block of the (estimated) row, as far as the launch stays resident at once; waves that a
+        // shorter row leaves without a block end at once.
+        const int row_blocks = ceil_div(row_steps, in_flight);
+        const int want = row_blocks <= 1 ? 1 : next_pow2(row_blocks);
+        const int registers = in_flight * cpl;                                 // in flight per lane, of 32 bits / 2
+        const int resident = (registers >= 32 ? 2 : registers >= 16 ? 3 : 5) * 1024;   // waves the chip holds at once
+        int room = 1;
+        while (2LL * room * blocks <= resident) room <<= 1;
+        waves = want < room ? want : room;
+        // A few rows far longer than the mean get at most sixteen steps per wave, as far as the waves this hands
+        // to every short row stay cheap (they end after reading their row's offsets).
+        if (hinted && longest_steps > 4 * mean_steps && longest_steps > 16) {
+            int cap = 16;
+            while (cap > 4 && blocks * cap > 16384) cap >>= 1;
+            int for_longest = next_pow2(ceil_div(longest_steps, 16));
+            if (for_longest > cap) for_longest = cap;
+            if (waves < for_longest) waves = for_longest;
+        }
+    }
     if (waves <= 0) {
         waves = next_pow2((int)((kTargetWaves + blocks - 1) / blocks));
-        if (batch.nonzeros_vec >= 0) {
+        if (hinted) {
             // Row lengths known: a wave is worth launching for about three 32-vector steps (measured over
             // the ResNet-shaped grid: within 0.4 % of the best power of two, 7 % better than sizing by n).
-            // While the chip has room (`waves` so far is the room per workgroup) the workgroup of the longest
-            // row ends last, so that row sets the size; idle waves of the shorter rows cost nothing then.
-            const int steps = ceil_div(ceil_div(batch.nonzeros_vec, m_vec), kStep);
-            const int longest_known = ceil_div(batch.longest_row_vec > 0 ? batch.longest_row_vec : 0, kStep);
-            const int sizing = longest_known > steps ? longest_known : steps;
-            const int by_rows = next_pow2(ceil_div(sizing > 0 ? sizing : 1, 3));
+            const int by_rows = next_pow2(ceil_div(row_steps > 0 ? row_steps : 1, 3));
             if (waves > by_rows) waves = by_rows;
             // a second wave per row pays on a full chip from about ten steps per row (256 to 2048 vector rows,
             // N = 256 to 1024: one wave 3-8 % ahead at 4 to 8 steps, two waves 3-10 % ahead at 12 and more)
-            if (waves < 2 && steps >= 10) waves = 2;
+            if (waves < 2 && mean_steps >= 10) waves = 2;
             // A few rows far longer than the mean: a wave takes about half a microsecond per step of a lone
             // long row, so that row gets at most sixteen steps per wave - as far as the idle waves this hands
-            // to every short row stay cheap (about half a nanosecond each: 16384 waves per launch, or four
-            // per row).  Measured on 1024 Pareto-distributed rows (mean 280, longest 4608 vectors, N = 256):
-            // 40 us with two waves per row, 15.8 us with the eight chosen here, 9.7 us for uniform rows.
-            const int longest = ceil_div(batch.longest_row_vec > 0 ? batch.longest_row_vec : 0, kStep);
-            if (longest > 4 * steps && longest > 16) {
+            // to every short row stay cheap (16384 waves per launch, or four per row).  Measured on 1024
+            // Pareto-distributed rows (mean 280, longest 4608 vectors, N = 256): 40 us with two waves per row,
+            // 15.8 us with the eight chosen here, 9.7 us for uniform rows.
+            if (longest_steps > 4 * mean_steps && longest_steps > 16) {
                 int cap = 16;
                 while (cap > 4 && blocks * cap > 16384) cap >>= 1;
-                int for_longest = next_pow2(ceil_div(longest, 16));
+                int for_longest = next_pow2(ceil_div(longest_steps, 16));
                 if (for_longest > cap) for_longest = cap;
                 if (waves < for_longest) waves = for_longest;
             }
@@ -353,6 +429,9 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
     }
     if (waves < 1) waves = 1;
     if (waves > 16) waves = 16;
+    // launch bounds of the variants with 64 / 128 registers of row segments in flight
+    if (in_flight * cpl >= 16 && waves > 8) waves = 8;
+    if (in_flight * cpl >= 32 && waves > 4) waves = 4;
     if constexpr (!SOFTMAX) {
         if (ragged) {
             if (waves > 8) waves = 8;  // 8 x 2.7 KB of LDS stay below the default limit of dynamic LDS
@@ -369,8 +448,8 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
                                               values, rhs, out, stream, batch);
     }
     if (cpl == 8)
-        return launch_v<8, SOFTMAX, OutT>(vec_length, m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
-    return launch_v<4, SOFTMAX, OutT>(vec_length, m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
+        return launch_v<8, SOFTMAX, OutT>(vec_length, m_vec, k, n, waves, in_flight, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
+    return launch_v<4, SOFTMAX, OutT>(vec_length, m_vec, k, n, waves, in_flight, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
 }
 
 template <typename OutT>

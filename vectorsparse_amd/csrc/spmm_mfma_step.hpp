@@ -49,7 +49,8 @@ __device__ __forceinline__ void wave_lds_fence()
 // with those loads in flight, transposes the CPL x 8 block with v_perm_b32 and issues CPL MFMAs:
 // acc[c][e] += sum_j vec[4g + e][j] * rhs[col_j][col_off + c].
 // RAGGED: the dense width is not a multiple of CPL; `valid` (0..CPL) halves of the lane's chunk exist.
-template <int V, int CPL, bool IDX32, bool RAGGED = false, typename Prefetch>
+// PITCH: halves between the staged vectors' rows (the slot may be laid out for a block of several steps).
+template <int V, int CPL, bool IDX32, bool RAGGED = false, int PITCH = kStep, typename Prefetch>
 __device__ __forceinline__ void spmm_mfma_step(const int *idx_s, const half_t *vec_s, const half_t *rhs, int n_cols,
                                                uint32_t col_off, int cs, int g, float4_t (&acc)[CPL],
                                                Prefetch &&prefetch, int valid = CPL)
@@ -57,7 +58,7 @@ __device__ __forceinline__ void spmm_mfma_step(const int *idx_s, const half_t *v
     const int4_t i_lo = *reinterpret_cast<const int4_t *>(idx_s + 8 * g);
     const int4_t i_hi = *reinterpret_cast<const int4_t *>(idx_s + 8 * g + 4);
     half8_t a = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (cs < V) a = *reinterpret_cast<const half8_t *>(vec_s + cs * kStep + 8 * g);
+    if (cs < V) a = *reinterpret_cast<const half8_t *>(vec_s + cs * PITCH + 8 * g);
     wave_lds_fence();
 
     RowChunk<CPL> chunk[8];
@@ -86,6 +87,56 @@ __device__ __forceinline__ void spmm_mfma_step(const int *idx_s, const half_t *v
         const half8_t b_odd = __builtin_bit_cast(half8_t, odd);
         acc[2 * p] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b_even, acc[2 * p], 0, 0, 0);
         acc[2 * p + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b_odd, acc[2 * p + 1], 0, 0, 0);
+    }
+}
+
+// S steps at once: the staged slot holds S * 32 column indices and the vectors as [v][S * 32]; all 8 * S row segments
+// of the lane are requested before the first MFMA, so the wave pays one memory round trip for S steps (at 2 * CPL / 4
+// registers per segment in flight).  Otherwise as spmm_mfma_step.
+template <int V, int CPL, int S, bool IDX32, int PITCH = S * kStep, typename Prefetch>
+__device__ __forceinline__ void spmm_mfma_block(const int *idx_s, const half_t *vec_s, const half_t *rhs, int n_cols,
+                                                uint32_t col_off, int cs, int g, float4_t (&acc)[CPL],
+                                                Prefetch &&prefetch)
+{
+    int4_t i_lo[S], i_hi[S];
+    half8_t a[S];
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+        i_lo[s] = *reinterpret_cast<const int4_t *>(idx_s + s * kStep + 8 * g);
+        i_hi[s] = *reinterpret_cast<const int4_t *>(idx_s + s * kStep + 8 * g + 4);
+        a[s] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        if (cs < V) a[s] = *reinterpret_cast<const half8_t *>(vec_s + cs * PITCH + s * kStep + 8 * g);
+    }
+    wave_lds_fence();
+
+    RowChunk<CPL> chunk[S][8];
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int col = e < 4 ? i_lo[s][e] : i_hi[s][e - 4];
+            if constexpr (IDX32)
+                chunk[s][e].load(rhs + ((uint32_t)col * (uint32_t)n_cols + col_off));
+            else
+                chunk[s][e].load(rhs + ((size_t)col * n_cols + col_off));
+        }
+    }
+    prefetch();
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+#pragma unroll
+        for (int p = 0; p < CPL / 2; ++p) {
+            uint4_t even, odd;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                even[q] = pack_lo(chunk[s][2 * q].dword(p), chunk[s][2 * q + 1].dword(p));
+                odd[q] = pack_hi(chunk[s][2 * q].dword(p), chunk[s][2 * q + 1].dword(p));
+            }
+            const half8_t b_even = __builtin_bit_cast(half8_t, even);
+            const half8_t b_odd = __builtin_bit_cast(half8_t, odd);
+            acc[2 * p] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[s], b_even, acc[2 * p], 0, 0, 0);
+            acc[2 * p + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[s], b_odd, acc[2 * p + 1], 0, 0, 0);
+        }
     }
 }
 
