@@ -362,7 +362,9 @@ int vs_launch_floor_probe(int blocks, int threads_per_block, void *stream);
  * "spmm_flat_piece" (nonzero vectors
  * per wave of the split-row SpMM, rounded up to 32, 0 = automatic), "spmm_flat_waves"
  * (its waves per workgroup, 1..16, 0 = automatic), "spmm_flat_launches" (1 = partial tiles
- * added inside the launch, 2 = by a second launch, 0 = automatic), "sddmm_slots" (waves per
+ * added inside the launch, 2 = by a second launch, 0 = automatic), "spmm_flat_shared" (1 = every
+ * row segment of the split-row SpMM starts a 32-vector step of its own, 2 = consecutive rows share
+ * steps, 0 = automatic), "sddmm_slots" (waves per
  * vector row, 0 = automatic), "sddmm_group" (16-vector groups per wave step of the
  * MFMA SDDMM: 1, 2, 4, 0 = automatic), "sddmm_block_waves" (1..16, 0 = automatic),
  * "sddmm_flat_supers" (super-groups per wave of algorithm 2, 1..16, 0 = automatic),

@@ -19,7 +19,7 @@ def _oracle(pat, B):
                                 pat.column_indices, pat.values, B)
 
 
-def _run(pat, B, out_dtype=torch.float16, workspace="auto", piece=0, waves=0, launches=0):
+def _run(pat, B, out_dtype=torch.float16, workspace="auto", piece=0, waves=0, launches=0, shared=0):
     """One call with canaries round the output and round the workspace; returns the host copy of the output."""
     prob = ops.DeviceProblem(pat)
     Bd = torch.from_numpy(B).cuda()
@@ -31,6 +31,7 @@ def _run(pat, B, out_dtype=torch.float16, workspace="auto", piece=0, waves=0, la
         _lib.set_option("spmm_flat_piece", piece)
         _lib.set_option("spmm_flat_waves", waves)
         _lib.set_option("spmm_flat_launches", launches)
+        _lib.set_option("spmm_flat_shared", shared)
         need = ops.spmm_workspace_bytes(pat.m_vec, pat.vec_length, k, pat.n, pat.nnz_vec)
         ws_bytes = need if workspace == "auto" else int(workspace)
         guard = 4096
@@ -47,6 +48,7 @@ def _run(pat, B, out_dtype=torch.float16, workspace="auto", piece=0, waves=0, la
         _lib.set_option("spmm_flat_piece", 0)
         _lib.set_option("spmm_flat_waves", 0)
         _lib.set_option("spmm_flat_launches", 0)
+        _lib.set_option("spmm_flat_shared", 0)
     host = buf.cpu().numpy()
     assert np.all(host[:pad] == 12345.0) and np.all(host[pad + pat.m:] == 12345.0), "wrote outside the output"
     wsh = ws_buf.cpu().numpy()
@@ -67,14 +69,16 @@ def _from_lengths(lengths, n, V, seed):
 @pytest.mark.parametrize("piece", [0, 32, 64, 96, 512])
 @pytest.mark.parametrize("waves", [0, 1, 3])
 @pytest.mark.parametrize("launches", [1, 2])
-def test_ragged_empty_and_long_rows(gpu, V, piece, waves, launches):
+@pytest.mark.parametrize("shared", [1, 2])
+def test_ragged_empty_and_long_rows(gpu, V, piece, waves, launches, shared):
     # empty rows at the start, in the middle and at the end; rows of every tail length; rows that span many runs
     # and pieces; a row that starts exactly on a run boundary (the 64 in front of it ends nonzero 128)
     lengths = [0, 0, 1, 15, 16, 17, 0, 31, 33, 14, 0, 64, 65, 300, 2, 0, 128, 7, 640, 1, 0, 0]
     pat = _from_lengths(lengths, 640, V, seed=5)
     B = cv.dense_uniform(640, 192, seed=7)
-    got = _run(pat, B, piece=piece, waves=waves, launches=launches)
-    assert_parity(got, _oracle(pat, B), "split rows V%d run %d waves %d launches %d" % (V, piece, waves, launches))
+    got = _run(pat, B, piece=piece, waves=waves, launches=launches, shared=shared)
+    assert_parity(got, _oracle(pat, B),
+                  "split rows V%d run %d waves %d launches %d shared %d" % (V, piece, waves, launches, shared))
     for i in np.nonzero(np.asarray(lengths) == 0)[0]:
         assert not got[i * V:(i + 1) * V].any(), "empty vector row %d must be written as zeros" % i
 
@@ -88,6 +92,24 @@ def test_all_rows_empty_and_single_row(gpu):
     B = cv.dense_uniform(2048, 128, seed=4)
     for waves in (1, 4, 16):
         assert_parity(_run(one, B, piece=64, waves=waves), _oracle(one, B), "single dense row, %d waves" % waves)
+
+
+@pytest.mark.parametrize("V", [1, 2, 4, 8])
+@pytest.mark.parametrize("shared", [1, 2])
+def test_many_short_rows_share_steps(gpu, V, shared):
+    """Rows of 0 to 40 vectors, more than sixty of them empty in a row (the offsets window of a wave moves on
+    several times inside one step), then long rows again: with shared steps up to 16 / V rows meet in one MFMA."""
+    rng = np.random.default_rng(70 + V)
+    lengths = np.concatenate([rng.integers(0, 41, 300), np.zeros(150, np.int64), [1, 0, 2, 500], np.zeros(70, np.int64),
+                              rng.integers(0, 9, 200), [900, 31, 32, 33]]).astype(np.int64)
+    pat = _from_lengths(lengths, 1024, V, seed=71)
+    B = cv.dense_uniform(1024, 136, seed=72)
+    ref = _oracle(pat, B)
+    for piece, waves in ((0, 0), (32, 2), (160, 5)):
+        got = _run(pat, B, piece=piece, waves=waves, shared=shared)
+        assert_parity(got, ref, "short rows V%d run %d waves %d shared %d" % (V, piece, waves, shared))
+        for i in np.nonzero(lengths == 0)[0]:
+            assert not got[i * V:(i + 1) * V].any(), "empty vector row %d must be written as zeros" % i
 
 
 @pytest.mark.parametrize("V", [2, 8])

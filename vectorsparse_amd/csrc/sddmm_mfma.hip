@@ -49,9 +49,15 @@ sddmm_mfma_kernel(int m_vec, int K, int slots, const int *__restrict__ row_indic
     if (wg >= (long long)m_vec * slots) return;
     const int slot = (int)(wg / slots);
     const int s = (int)(wg % slots);
+    // the row's extent is requested for the identity order together with the swizzle entry, and again only if
+    // the entry names another row: one dependent load less in the common case
     const int row = row_indices[slot];
-    const int beg = row_offsets[row];
-    const int end = row_offsets[row + 1];
+    int beg = row_offsets[slot];
+    int end = row_offsets[slot + 1];
+    if (row != slot) {
+        beg = row_offsets[row];
+        end = row_offsets[row + 1];
+    }
     const int n_super = (end - beg + SUPER - 1) / SUPER;
     if (s >= n_super) return;
     const int c = lane & 15;        // MFMA order: column (nonzero vector) index

@@ -90,6 +90,52 @@ __device__ __forceinline__ void spmm_mfma_step(const int *idx_s, const half_t *v
     }
 }
 
+// A step shared by up to 16 / V consecutive vector rows: MFMA row `cs` carries scalar row cs % V of the vector row in
+// group cs / V, which owns the staged slots [lo, hi) (per lane; the other slots read as zero for that row), so the
+// accumulator rows of group p add up that row's nonzeros only.  Otherwise as spmm_mfma_step.
+template <int V, int CPL, bool IDX32, typename Prefetch>
+__device__ __forceinline__ void spmm_mfma_step_shared(const int *idx_s, const half_t *vec_s, const half_t *rhs,
+                                                      int n_cols, uint32_t col_off, int cs, int g, float4_t (&acc)[CPL],
+                                                      int lo, int hi, Prefetch &&prefetch)
+{
+    const int4_t i_lo = *reinterpret_cast<const int4_t *>(idx_s + 8 * g);
+    const int4_t i_hi = *reinterpret_cast<const int4_t *>(idx_s + 8 * g + 4);
+    uint4_t a_bits = *reinterpret_cast<const uint4_t *>(vec_s + (cs % V) * kStep + 8 * g);
+    wave_lds_fence();
+    const uint32_t span = hi > lo ? (uint32_t)(hi - lo) : 0u;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        const uint32_t first = (uint32_t)(8 * g + 2 * d - lo);  // wraps to a large value below lo
+        const uint32_t keep = (first < span ? 0x0000ffffu : 0u) | (first + 1u < span ? 0xffff0000u : 0u);
+        a_bits[d] &= keep;
+    }
+    const half8_t a = __builtin_bit_cast(half8_t, a_bits);
+
+    RowChunk<CPL> chunk[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const int col = e < 4 ? i_lo[e] : i_hi[e - 4];
+        if constexpr (IDX32)
+            chunk[e].load(rhs + ((uint32_t)col * (uint32_t)n_cols + col_off));
+        else
+            chunk[e].load(rhs + ((size_t)col * n_cols + col_off));
+    }
+    prefetch();
+#pragma unroll
+    for (int p = 0; p < CPL / 2; ++p) {
+        uint4_t even, odd;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            even[q] = pack_lo(chunk[2 * q].dword(p), chunk[2 * q + 1].dword(p));
+            odd[q] = pack_hi(chunk[2 * q].dword(p), chunk[2 * q + 1].dword(p));
+        }
+        const half8_t b_even = __builtin_bit_cast(half8_t, even);
+        const half8_t b_odd = __builtin_bit_cast(half8_t, odd);
+        acc[2 * p] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b_even, acc[2 * p], 0, 0, 0);
+        acc[2 * p + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b_odd, acc[2 * p + 1], 0, 0, 0);
+    }
+}
+
 // S steps at once: the staged slot holds S * 32 column indices and the vectors as [v][S * 32]; all 8 * S row segments
 // of the lane are requested before the first MFMA, so the wave pays one memory round trip for S steps (at 2 * CPL / 4
 // registers per segment in flight).  Otherwise as spmm_mfma_step.

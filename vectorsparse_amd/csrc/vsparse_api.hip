@@ -532,6 +532,9 @@ static int set_option_field(vs::Options &o, const char *name, int value)
     } else if (std::strcmp(name, "spmm_flat_launches") == 0) {
         if (value > 2) return VS_ERROR_INVALID_VALUE;
         o.spmm_flat_launches = value;
+    } else if (std::strcmp(name, "spmm_flat_shared") == 0) {
+        if (value > 2) return VS_ERROR_INVALID_VALUE;
+        o.spmm_flat_shared = value;
     } else if (std::strcmp(name, "spmm_flat_waves") == 0) {
         if (value > 16) return VS_ERROR_INVALID_VALUE;
         o.spmm_flat_waves = value;
