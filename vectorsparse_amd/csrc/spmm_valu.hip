@@ -49,13 +49,30 @@ spmm_valu_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
     constexpr int G = 64 / LR;
     constexpr int TN = 8 * LR;
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n_waves = blockDim.x >> 6;
     const int tile = blockIdx.x % n_tiles;
     const int slot = blockIdx.x / n_tiles;
+    // the row's extent is requested for the identity order together with the swizzle entry, and again only if
+    // the entry names another row: one dependent load less in the common case
     const int row = row_indices[slot];
-    const int beg = row_offsets[row];
-    const int end = row_offsets[row + 1];
+    int beg = row_offsets[slot];
+    int end = row_offsets[slot + 1];
+    if (row != slot) {
+        beg = row_offsets[row];
+        end = row_offsets[row + 1];
+    }
+    constexpr int U = 4;  // nonzero vectors per group and turn, so that U gathered rows are in flight per lane
+    // Group p starts at nonzero beg + p * U: on a short row only the first few groups have any.  Waves that have
+    // neither a group with nonzeros nor a share of the final sum (V * LR items, one per thread) end here: a
+    // workgroup barrier waits only for the waves that still run.
+    int n_partials = (end - beg + U - 1) / U;
+    n_partials = n_partials < 1 ? 1 : (n_partials > n_waves * G ? n_waves * G : n_partials);
+    constexpr int kSumWaves = (V * LR + 63) / 64;
+    int alive_waves = (n_partials + G - 1) / G;
+    alive_waves = alive_waves < kSumWaves ? kSumWaves : alive_waves;
+    alive_waves = alive_waves < n_waves ? alive_waves : n_waves;
+    if (wave >= alive_waves) return;
     const int cl = lane % LR;
     const int g = lane / LR;
     const int col0 = tile * TN + cl * 8;
@@ -69,8 +86,8 @@ spmm_valu_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
 #pragma unroll
         for (int c = 0; c < 8; ++c) acc[v][c] = 0.f;
 
-    // U nonzero vectors per group and iteration, so that U gathered rows are in flight per lane
-    constexpr int U = 4;
+    // (fetching the next turn's column indices and values while the gathered rows of the current one are in flight
+    // costs 18 to 40 registers and measured 2-6 % slower over the ResNet-shaped grid)
     for (int j0 = beg + (wave * G + g) * U; j0 < end; j0 += n_waves * G * U) {
         int col[U];
         uint32_t a[U][V > 1 ? V / 2 : 1];  // the vector's halves, two per word (V = 1: one half in the low bits)
@@ -131,7 +148,7 @@ spmm_valu_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
         }
     }
 
-    if (n_waves * G == 1) {
+    if (n_waves * G == 1) {  // (deciding this by the row's length at run time instead measured 0.5 us slower)
         if (col_ok) {
 #pragma unroll
             for (int v = 0; v < V; ++v) {
@@ -144,10 +161,7 @@ spmm_valu_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
         return;
     }
 
-    // Group p starts at nonzero beg + p * U: on a short row only the first few groups had any, and only
-    // their partial tiles are written and summed (the others hold zeros).
-    int n_partials = (end - beg + U - 1) / U;
-    n_partials = n_partials < 1 ? 1 : (n_partials > n_waves * G ? n_waves * G : n_partials);
+    // only the partial tiles of the groups that had nonzeros are written and summed
     if (wave * G + g < n_partials) {
         float *mine = partial + (size_t)(wave * G + g) * V * TN;
 #pragma unroll
@@ -159,7 +173,7 @@ spmm_valu_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
         }
     }
     __syncthreads();
-    for (int item = threadIdx.x; item < V * LR; item += blockDim.x) {
+    for (int item = threadIdx.x; item < V * LR; item += 64 * alive_waves) {
         const int v = item / LR;
         const int cl2 = item % LR;
         const int col = tile * TN + cl2 * 8;
