@@ -3,7 +3,9 @@
 //   2. what a chain of dependent loads costs right after a launch (the row swizzle -> offsets -> indices ->
 //      gathered rows chain of the kernels);
 //   3. how fast random 256-byte segments of an L2-resident matrix can be gathered into the CUs, through
-//      registers, through global -> LDS loads, or both, with 4 to 32 segments in flight per 16-lane group.
+//      registers, through global -> LDS loads, or both, with 4 to 32 segments in flight per 16-lane group;
+//   4. what a launch costs that only writes its output (every lane one 16-byte store, no loads): the time a kernel
+//      waits for its last stores to be acknowledged.
 // Prints a short text report; times are medians of 7 replays of a graph of 100 launches.
 #include <hip/hip_runtime.h>
 
@@ -36,6 +38,13 @@ __global__ void __launch_bounds__(1024) chain_kernel(const int *__restrict__ tab
         for (int l = 0; l < L; ++l) idx = table[(idx + l * 1237) & mask];
         if (idx == 0x7fffffff || threadIdx.x == 0) out[blockIdx.x] = idx;
     }
+}
+
+// Every lane stores 16 bytes, nothing is loaded.
+__global__ void __launch_bounds__(1024) store_kernel(uint4_t *__restrict__ out)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    out[i] = uint4_t{(unsigned)i, 1u, 2u, 3u};
 }
 
 // REG segments per 16-lane group through registers plus DMA segments through LDS per iteration.
@@ -184,6 +193,17 @@ int main()
     gather_row<0, 16>("dma 16", stream, idx, rows, row_u4, n_idx, out);
     gather_row<8, 8>("reg 8 + dma 8", stream, idx, rows, row_u4, n_idx, out);
     gather_row<16, 16>("reg 16 + dma 16", stream, idx, rows, row_u4, n_idx, out);
+    printf("\n4. a kernel that only stores 16 bytes per lane, microseconds per launch\n");
+    {
+        uint4_t *dst;
+        CHECK(hipMalloc(&dst, (size_t)4096 * 1024 * 16));
+        for (int threads : {64, 256})
+            for (int blocks : {256, 1024, 4096}) {
+                const double us = graph_us(stream, [&](hipStream_t s) { hipLaunchKernelGGL(store_kernel, dim3(blocks), dim3(threads), 0, s, dst); });
+                printf("  %5d workgroups x %4d threads (%7.0f KB written): %.2f us\n", blocks, threads, blocks * threads * 16 / 1e3, us);
+            }
+        CHECK(hipFree(dst));
+    }
     CHECK(hipDeviceSynchronize());
     printf("\ndone\n");
     return 0;
