@@ -145,11 +145,15 @@ int vs_cuda_spmm_f16_f32out(int m_vec, int vec_length, int k, int n,
  * fp16 on store.  vec_length in {2, 4, 8} (1 accepted).  `algorithm` selects
  * among the reference's four Volta register/shuffle schedules (0..3); they
  * compute the same function, and so do the two schedules here, bit for bit:
- * 0 and 1 = a wave owns (vector row, slot) and walks that row's nonzeros, rows
+ * 1 = a wave owns (vector row, slot) and walks that row's nonzeros, rows
  * taken in row_indices order (best for rows of similar length); 2 = the waves
  * split the nonzero range itself, whatever rows it crosses (k <= 256; row
  * lengths may be arbitrarily skewed, row_indices is not used; slower on short
- * rows and small problems).  3 (the reference's timing-only hardware
+ * rows and small problems).  0 = automatic: schedule 1, except that masks of few
+ * nonzeros with vec_length <= 4 - which fill a quarter of a matrix-core tile or
+ * less - run on the fine-grained kernel of vs_cuda_sddmm_f16 (same function
+ * within the fp32-accumulation tolerance, not the same bits).
+ * 3 (the reference's timing-only hardware
  * simulation, whose results are wrong by design) is rejected with
  * hipErrorInvalidValue.
  * Requirements: k % 8 == 0 (the whole of k is contracted — the reference drops

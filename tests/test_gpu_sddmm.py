@@ -128,6 +128,24 @@ def test_algorithm_argument(gpu):
         _run(pat, A, B, "wmma", algorithm=3)
 
 
+@pytest.mark.parametrize("V", [1, 2, 4])
+def test_automatic_algorithm_takes_the_fine_grained_kernel_on_small_masks_of_short_vectors(gpu, V):
+    """algorithm 0 of the MFMA entry point: vectors of 1 to 4 rows fill at most a quarter of a matrix-core tile, so
+    a mask of few nonzeros goes to the fine-grained kernel (the bits of cudaSddmm), a large one stays on MFMA
+    (the bits of algorithm 1); both hold the oracle's tolerance."""
+    small = cv.uniform_pattern(64 // V, 512, 0.95, seed=40 + V, vec_length=V)
+    A = cv.dense_normal(small.m, 256, seed=41)
+    B = cv.dense_normal(512, 256, seed=42)
+    auto = _run(small, A, B, "wmma", algorithm=0)
+    assert_parity(auto, _oracle(small, A, B), "algorithm 0, small mask, V%d" % V)
+    assert np.array_equal(auto.view(np.uint16), _run(small, A, B, "cuda").view(np.uint16))
+    large = cv.uniform_pattern(2048 // V, 2048, 0.5, seed=43 + V, vec_length=V)   # beyond every limit
+    A = cv.dense_normal(large.m, 64, seed=44)
+    B = cv.dense_normal(2048, 64, seed=45)
+    auto = _run(large, A, B, "wmma", algorithm=0)
+    assert np.array_equal(auto.view(np.uint16), _run(large, A, B, "wmma", algorithm=1).view(np.uint16))
+
+
 def test_full_mask_equals_dense_product(gpu):
     V, m_vec, n, K = 8, 8, 96, 64
     ro = (np.arange(m_vec + 1) * n).astype(np.int32)

@@ -371,6 +371,19 @@ int launch_sddmm_mfma(int m_vec, int k, int n, int nonzeros_vec, const int *row_
     if (m_vec == 0 || nonzeros_vec == 0 || batch.count == 0) return hipSuccess;
     if (batch.count > 65535) return hipErrorNotSupported;
     if (k <= 0 || k % 8 != 0) return hipErrorNotSupported;
+    // algorithm 0 (automatic): vectors of 1, 2 or 4 rows fill 1/16 to 4/16 of an MFMA tile, and on masks of few
+    // nonzeros the fine-grained kernel (dot products on the vector ALU, reduced across lanes with DPP) is ahead:
+    // over the M = N = 512..4096, K = 64..256 grid by 5-40 % below these nonzero counts, behind above them.
+    if (batch.algorithm == 0 && vec_length <= 4) {
+        const long long total = (long long)nonzeros_vec * batch.count;
+        long long limit = 0;
+        if (vec_length == 1) limit = 800000;
+        else if (vec_length == 2) limit = k >= 256 ? 200000 : (k >= 128 ? 16000 : 0);
+        else limit = k >= 256 ? 16000 : (k >= 128 ? 8000 : 0);
+        if (total <= limit)
+            return launch_sddmm_valu<OutT>(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out,
+                                           vec_length, stream, batch);
+    }
     switch (vec_length) {
     case 1: return launch_ks<1, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);
     case 2: return launch_ks<2, OutT>(m_vec, k, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out, stream, batch);

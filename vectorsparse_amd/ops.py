@@ -487,12 +487,13 @@ class DeviceProblem:
     def sddmm(self, lhs_matrix, rhs_matrix, kernel="wmma", out_dtype=torch.float16, out=None, stream=None,
               algorithm=None):
         """SDDMM on the mask.  algorithm (MFMA path): 1 = a wave per (row, slot), 2 = waves split the nonzero
-        range (robust to skewed row lengths); None picks 2 for large, heavily skewed masks, else 1."""
+        range (robust to skewed row lengths), 0 = the library's choice between 1 and the fine-grained kernel (small
+        masks of short vectors); None picks 2 for large, heavily skewed masks, else 0."""
         k = lhs_matrix.shape[1]
         if out is None:
             out = torch.empty((self.nnz_vec, self.vec_length), dtype=out_dtype, device=lhs_matrix.device)
         if algorithm is None:
-            algorithm = 2 if (self.skewed and k <= 256) else 1
+            algorithm = 2 if (self.skewed and k <= 256) else 0
         if kernel == "wmma":
             return sddmm.wmmaSddmm(self.m_vec, k, self.n, self.nnz_vec, self.row_indices, self.row_offsets,
                                    self.column_indices, lhs_matrix, rhs_matrix, out, self.vec_length, stream,
