@@ -355,9 +355,17 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
     int cpl = options().spmm_cols_per_lane;
     const bool use_dma = !SOFTMAX && options().spmm_gather == 2 && k % 8 == 0;
     if (use_dma) cpl = 8;
+    const bool hinted = batch.nonzeros_vec >= 0;
+    const int mean_steps = hinted ? ceil_div(ceil_div(batch.nonzeros_vec, m_vec), kStep) : ceil_div(n, 4 * kStep);
+    const int longest_steps = ceil_div(batch.longest_row_vec > 0 ? batch.longest_row_vec : 0, kStep);
+    // a few rows far longer than the mean (known only to the batched entry points)
+    const bool skewed = hinted && longest_steps > 4 * mean_steps && longest_steps > 16;
     if (cpl != 4 && cpl != 8) {
         const long long blocks128 = (long long)m_vec * ceil_div(k, 128) * batch.count;
-        cpl = (k % 8 == 0 && k > 64 && blocks128 >= kTargetBlocks) ? 8 : 4;  // k <= 64 fits one 64-column tile
+        // Skewed rows keep the narrow tile until the grid is four workgroups per CU: the long rows then spread over
+        // twice the workgroups (256 rows, Pareto or one dense row among short ones, N = 256: 12.4 -> 11.4 us).
+        const long long enough = skewed ? 4 * kTargetBlocks : kTargetBlocks;
+        cpl = (k % 8 == 0 && k > 64 && blocks128 >= enough) ? 8 : 4;  // k <= 64 fits one 64-column tile
     }
     if (cpl == 8 && k % 8 != 0) cpl = 4;
     const bool ragged = k % 4 != 0;
@@ -370,16 +378,15 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
     // they are chosen only when the row lengths are known.  The unhinted entry takes the rows to hold a quarter of
     // n: the kernel leaves the waves that a shorter row does not need idle at little cost (1.5 % per doubling
     // of the workgroup beyond four waves), while too few waves for denser rows cost 10-18 %.
-    const bool hinted = batch.nonzeros_vec >= 0;
-    const int mean_steps = hinted ? ceil_div(ceil_div(batch.nonzeros_vec, m_vec), kStep) : ceil_div(n, 4 * kStep);
-    const int longest_steps = ceil_div(batch.longest_row_vec > 0 ? batch.longest_row_vec : 0, kStep);
     // while the chip has room the workgroup of the longest row ends last, so that row sets the size
     const int row_steps = longest_steps > mean_steps ? longest_steps : mean_steps;
     const bool blocks_exist = !SOFTMAX && !ragged && !use_dma && (long long)n * k < (1LL << 31);
     int in_flight = options().spmm_steps;
     if (in_flight != 1 && in_flight != 2 && in_flight != 4) {
         in_flight = row_steps >= 2 ? 2 : 1;
-        if (hinted && cpl == 8 && blocks >= 512 && mean_steps >= 8) in_flight = 4;
+        // (rows of unequal length end in half-empty blocks of 128: on log-normal and Pareto lengths four steps in
+        // flight were 10-25 % behind two)
+        if (hinted && cpl == 8 && blocks >= 512 && mean_steps >= 8 && 2 * longest_steps <= 3 * mean_steps) in_flight = 4;
     }
     if (!blocks_exist) in_flight = 1;
     int waves = options().spmm_waves;
@@ -398,9 +405,12 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
         waves = want < room ? want : room;
         // A few rows far longer than the mean get at most sixteen steps per wave, as far as the waves this hands
         // to every short row stay cheap (they end after reading their row's offsets).
-        if (hinted && longest_steps > 4 * mean_steps && longest_steps > 16) {
+        // (Where the average row itself fills more than six waves the budget is half: most of the waves then do
+        // work and crowd the chip - log-normal lengths, 1024 rows: 17.4 us with four waves, 20.5 us with eight.)
+        if (skewed) {
+            const long long budget = ceil_div(mean_steps, in_flight) <= 6 ? 16384 : 8192;
             int cap = 16;
-            while (cap > 4 && blocks * cap > 16384) cap >>= 1;
+            while (cap > 4 && blocks * cap > budget) cap >>= 1;
             int for_longest = next_pow2(ceil_div(longest_steps, 16));
             if (for_longest > cap) for_longest = cap;
             if (waves < for_longest) waves = for_longest;
@@ -421,7 +431,7 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
             // to every short row stay cheap (16384 waves per launch, or four per row).  Measured on 1024
             // Pareto-distributed rows (mean 280, longest 4608 vectors, N = 256): 40 us with two waves per row,
             // 15.8 us with the eight chosen here, 9.7 us for uniform rows.
-            if (longest_steps > 4 * mean_steps && longest_steps > 16) {
+            if (skewed) {
                 int cap = 16;
                 while (cap > 4 && blocks * cap > 16384) cap >>= 1;
                 int for_longest = next_pow2(ceil_div(longest_steps, 16));

@@ -422,15 +422,13 @@ def SortedRowSwizzle(rows, row_offsets):
 
 def split_rows_pays(m_vec, nonzeros_vec, longest_row_vec):
     """Whether the split-row SpMM schedule is expected to beat the row-per-workgroup one with row-length hints.
-    Measured at N = 256, V = 8, rows of up to 4608 vectors: a row of 25 or more mean lengths (one dense row among
-    short ones) holds its single workgroup per tile for 13-22 us where the split schedule needs 10-15 us whatever
-    the row count; milder skew (8 mean lengths and up: Pareto or lognormal lengths) pays only while the matrix has
-    at most 256 vector rows (10.6-12.8 us against 11.8-13.9 us), larger ones keep the chip busy with whole rows
-    (13.7 against 15.8 us at 512 rows).  Uniform and binomial lengths never pay (a third to twice slower)."""
+    Measured at N = 256, V = 8, rows of up to 4608 vectors, 64 to 2048 vector rows: a row of 25 or more mean lengths
+    (one dense row among short ones) holds its workgroups for 11.2-13.4 us where the split schedule needs 9.8-11.8 us;
+    on milder skew (Pareto or log-normal lengths, longest row 6 to 18 mean lengths) the hinted schedule is ahead at
+    every size (1024 Pareto rows: 14.5 against 18.2 us), and on uniform or binomial lengths by 1.5 to 2.5 times."""
     if m_vec <= 0 or nonzeros_vec < 8192:
         return False
-    ratio = longest_row_vec * m_vec / float(nonzeros_vec)
-    return ratio >= 25.0 or (ratio >= 8.0 and m_vec <= 256)
+    return longest_row_vec * m_vec >= 25.0 * nonzeros_vec
 
 
 class DeviceProblem:
