@@ -359,7 +359,10 @@ int vs_launch_floor_probe(int blocks, int threads_per_block, void *stream);
  * change its options between two calls on different streams - every call sees
  * exactly what its thread last set, whatever other threads do.  Names: "spmm_waves" (waves per workgroup, 0 = automatic),
  * "spmm_cols_per_lane" (4, 8, 0 = automatic), "spmm_steps" (32-vector steps of gathered
- * rows a wave of the MFMA SpMM keeps in flight: 1, 2, 4, 0 = automatic), "spmm_gather" (how the MFMA SpMM
+ * rows a wave of the MFMA SpMM keeps in flight: 1, 2, 4, 0 = automatic), "spmm_guard_waves"
+ * (MFMA SpMM through the entry points that do not know the row lengths, on grids that fill the
+ * chip by themselves: waves per workgroup kept for rows far longer than expected, 1 = none,
+ * 0 = automatic), "spmm_gather" (how the MFMA SpMM
  * brings the gathered rows of the dense operand to the matrix cores: 1 = through
  * registers and an in-register transpose, 2 = global -> LDS loads and transposing LDS
  * reads, k % 8 == 0 only; 0 = automatic, which is 1: 2 measured 10-18 % slower),

@@ -32,7 +32,7 @@ namespace vs {
 // row segments per lane are all requested before the first MFMA.
 template <int V, int CPL, bool SOFTMAX, bool IDX32, typename OutT, bool RAGGED = false, int S = 1>
 __global__ void __launch_bounds__(S * CPL >= 32 ? 256 : (S * CPL >= 16 ? 512 : 1024))
-spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
+spmm_mfma_kernel(int n_cols, int n_tiles, int per_wave_log2, const int *__restrict__ row_indices,
                  const int *__restrict__ row_offsets, const int *__restrict__ column_indices,
                  const half_t *__restrict__ values, const half_t *__restrict__ rhs,
                  OutT *__restrict__ out, long long stride_values, long long stride_rhs, long long stride_out,
@@ -80,8 +80,12 @@ spmm_mfma_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
     // The other waves end here: a workgroup barrier waits only for the waves that are still running, and a row
     // of a single active wave needs neither barrier nor LDS for its result.
     const int steps = (end - beg + kStep - 1) / kStep;
+    // per_wave_log2 > 0 (the grid alone fills the chip): a wave takes 2^per_wave_log2 blocks of a row one after the
+    // other, so that a row of the expected length keeps to the waves the chip has room for and only a row far longer
+    // than expected spreads over the rest of its workgroup.
     int active = S == 1 ? (steps + 1) >> 1 : (steps + S - 1) / S;
     if (S > 1 && active == 2 && gridDim.x * gridDim.y >= 512) active = 1;
+    if (S > 1) active = (active + (1 << per_wave_log2) - 1) >> per_wave_log2;
     active = active < 1 ? 1 : (active > n_waves ? n_waves : active);
     if (wave >= active) return;
 
@@ -269,9 +273,11 @@ static int next_pow2(int x)
 template <int V, int CPL, bool SOFTMAX, bool IDX32, typename OutT, int S = 1>
 static int launch_idx(int m_vec, int k, int n, int waves, const int *row_indices, const int *row_offsets,
                       const int *column_indices, const half_t *values, const half_t *rhs, OutT *out,
-                      hipStream_t stream, const Batch &batch, float scale)
+                      hipStream_t stream, const Batch &batch, float scale, int per_wave = 1)
 {
     (void)n;
+    int per_wave_log2 = 0;
+    while ((2 << per_wave_log2) <= per_wave) ++per_wave_log2;
     constexpr int TN = 16 * CPL;
     const int n_tiles = ceil_div(k, TN);
     const long long blocks = (long long)m_vec * n_tiles;
@@ -283,7 +289,7 @@ static int launch_idx(int m_vec, int k, int n, int waves, const int *row_indices
     const hipError_t attr = allow_large_lds(reinterpret_cast<const void *>(kernel), 96 * 1024, lds_allowed);
     if (attr != hipSuccess) return (int)attr;
     hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)batch.count), dim3(64 * waves), lds, stream,
-                       k, n_tiles, row_indices, row_offsets, column_indices, values, rhs, out,
+                       k, n_tiles, per_wave_log2, row_indices, row_offsets, column_indices, values, rhs, out,
                        batch.stride_a, batch.stride_b, batch.stride_out, scale);
     return (int)hipGetLastError();
 }
@@ -300,7 +306,7 @@ static int launch_ragged(int m_vec, int k, int waves, const int *row_indices, co
     if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
     const size_t lds = (size_t)waves * stage_bytes<V>() + (waves > 1 ? (size_t)waves * V * (TN + 1) * sizeof(float) : 0);
     hipLaunchKernelGGL((spmm_mfma_kernel<V, 4, false, false, OutT, true>), dim3((unsigned)blocks, (unsigned)batch.count),
-                       dim3(64 * waves), lds, stream, k, n_tiles, row_indices, row_offsets, column_indices, values, rhs,
+                       dim3(64 * waves), lds, stream, k, n_tiles, 0, row_indices, row_offsets, column_indices, values, rhs,
                        out, batch.stride_a, batch.stride_b, batch.stride_out, 1.f);
     return (int)hipGetLastError();
 }
@@ -310,15 +316,19 @@ static int launch_one(int m_vec, int k, int n, int waves, int in_flight, const i
                       const int *row_offsets, const int *column_indices, const half_t *values, const half_t *rhs,
                       OutT *out, hipStream_t stream, const Batch &batch, float scale)
 {
+    const int per_wave = in_flight >> 8;  // blocks a wave takes of one row, packed above the steps in flight
+    in_flight &= 255;
     if ((long long)n * k < (1LL << 31)) {
         if constexpr (!SOFTMAX) {
             // blocks of several steps in flight exist for the common case only: offsets that fit 32 bits
             if (in_flight == 4)
                 return launch_idx<V, CPL, SOFTMAX, true, OutT, 4>(m_vec, k, n, waves, row_indices, row_offsets,
-                                                                   column_indices, values, rhs, out, stream, batch, scale);
+                                                                   column_indices, values, rhs, out, stream, batch, scale,
+                                                                   per_wave);
             if (in_flight >= 2)
                 return launch_idx<V, CPL, SOFTMAX, true, OutT, 2>(m_vec, k, n, waves, row_indices, row_offsets,
-                                                                   column_indices, values, rhs, out, stream, batch, scale);
+                                                                   column_indices, values, rhs, out, stream, batch, scale,
+                                                                   per_wave);
         }
         return launch_idx<V, CPL, SOFTMAX, true, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices,
                                                         values, rhs, out, stream, batch, scale);
@@ -389,6 +399,7 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
         if (hinted && cpl == 8 && blocks >= 512 && mean_steps >= 8 && 2 * longest_steps <= 3 * mean_steps) in_flight = 4;
     }
     if (!blocks_exist) in_flight = 1;
+    int per_wave = 1;
     int waves = options().spmm_waves;
     if (waves <= 0 && in_flight > 1) {
         // One wave per block of the (estimated) row, as far as the launch stays resident at once; waves that a
@@ -403,6 +414,20 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
         int room = 1;
         while (2LL * room * blocks <= resident) room <<= 1;
         waves = want < room ? want : room;
+        // Row lengths unknown and the grid alone fills the chip: the workgroups still get a few waves, of which a
+        // row of the expected length uses `room` (a wave takes want / room of its blocks); a row far longer than
+        // expected spreads over all of them instead of holding one wave for the whole launch (1024 Pareto rows x
+        // 4608, N = 256: 39 -> 15 us with four waves, 23 us with two; one dense row among 1023 short ones 39 -> 14 us).
+        // The waves a row does not need end after reading the row's extent, but hold a wave slot until then:
+        // 0.3 us per thousand of them (binomial rows, 1024 x 4608: 14.1 -> 16.0 us with four, 14.6 us with two), so
+        // grids beyond 2048 workgroups get two.
+        int guard = options().spmm_guard_waves;
+        if (guard <= 0) guard = blocks <= 2048 ? 4 : 2;
+        if (!hinted && want > room && guard > room) {
+            const int launched = want < guard ? want : guard;
+            per_wave = want / room;
+            waves = launched;
+        }
         // A few rows far longer than the mean get at most sixteen steps per wave, as far as the waves this hands
         // to every short row stay cheap (they end after reading their row's offsets).
         // (Where the average row itself fills more than six waves the budget is half: most of the waves then do
@@ -467,8 +492,8 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
                                               values, rhs, out, stream, batch);
     }
     if (cpl == 8)
-        return launch_v<8, SOFTMAX, OutT>(vec_length, m_vec, k, n, waves, in_flight, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
-    return launch_v<4, SOFTMAX, OutT>(vec_length, m_vec, k, n, waves, in_flight, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
+        return launch_v<8, SOFTMAX, OutT>(vec_length, m_vec, k, n, waves, in_flight | (per_wave << 8), row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
+    return launch_v<4, SOFTMAX, OutT>(vec_length, m_vec, k, n, waves, in_flight | (per_wave << 8), row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
 }
 
 template <typename OutT>

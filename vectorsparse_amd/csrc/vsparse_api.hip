@@ -521,6 +521,9 @@ static int set_option_field(vs::Options &o, const char *name, int value)
     } else if (std::strcmp(name, "spmm_cols_per_lane") == 0) {
         if (value != 0 && value != 4 && value != 8) return VS_ERROR_INVALID_VALUE;
         o.spmm_cols_per_lane = value;
+    } else if (std::strcmp(name, "spmm_guard_waves") == 0) {
+        if (value > 16) return VS_ERROR_INVALID_VALUE;
+        o.spmm_guard_waves = value;
     } else if (std::strcmp(name, "spmm_steps") == 0) {
         if (value != 0 && value != 1 && value != 2 && value != 4) return VS_ERROR_INVALID_VALUE;
         o.spmm_steps = value;
