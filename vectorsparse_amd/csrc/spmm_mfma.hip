@@ -428,17 +428,22 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
             per_wave = want / room;
             waves = launched;
         }
-        // A few rows far longer than the mean get at most sixteen steps per wave, as far as the waves this hands
-        // to every short row stay cheap (they end after reading their row's offsets).
-        // (Where the average row itself fills more than six waves the budget is half: most of the waves then do
-        // work and crowd the chip - log-normal lengths, 1024 rows: 17.4 us with four waves, 20.5 us with eight.)
+        // A few rows far longer than the mean (lengths known): the average row keeps to the waves the chip has room
+        // for - a wave takes several of its blocks when the grid is full - and the longest row spreads over as many
+        // waves as its blocks ask for at that rate, within a budget of launched waves (the waves a row does not
+        // need end after reading its extent, at 0.3 us per thousand; where the average row itself fills more than
+        // six waves the budget is half - log-normal lengths, 1024 rows: 17.4 us with four waves, 20.5 us with eight).
         if (skewed) {
-            const long long budget = ceil_div(mean_steps, in_flight) <= 6 ? 16384 : 8192;
+            const int mean_blocks = ceil_div(mean_steps, in_flight);
+            const int typical = mean_blocks <= 1 ? 1 : next_pow2(mean_blocks);
+            const int base = typical < room ? typical : room;
+            per_wave = typical / base;
+            const long long budget = mean_blocks <= 6 ? 16384 : 8192;
             int cap = 16;
             while (cap > 4 && blocks * cap > budget) cap >>= 1;
-            int for_longest = next_pow2(ceil_div(longest_steps, 16));
+            int for_longest = next_pow2(ceil_div(ceil_div(longest_steps, in_flight), per_wave));
             if (for_longest > cap) for_longest = cap;
-            if (waves < for_longest) waves = for_longest;
+            waves = base > for_longest ? base : for_longest;
         }
     }
     if (waves <= 0) {
