@@ -290,6 +290,37 @@ def test_longest_row_hint_on_heavy_tailed_rows(gpu):
         assert_parity(hinted.cpu().numpy(), ref, "heavy tail, hinted")
 
 
+@pytest.mark.parametrize("V,m_vec", [(8, 1100), (1, 2500)])
+@pytest.mark.parametrize("N", [64, 256])
+def test_skewed_rows_on_a_grid_that_fills_the_chip(gpu, V, m_vec, N):
+    """More workgroups than the chip holds at once: the launches keep a few waves per workgroup for rows far longer
+    than expected and let a wave take several 64-vector blocks of a row (reference-shaped entry: lengths unknown;
+    batched entry: mean and longest known).  Pareto lengths with a dense row, empty rows and rows that end inside
+    a block, every guard setting, identity and sorted order."""
+    rng = np.random.default_rng(90 + V)
+    n = 2304
+    lengths = np.minimum((rng.pareto(1.5, m_vec) + 0.05) * 60, n).astype(np.int64)
+    lengths[3] = n
+    lengths[m_vec // 2] = n - 1
+    lengths[10:14] = 0
+    lengths[20:26] = [1, 63, 64, 65, 127, 129]
+    ro, ci = cv._pattern_from_lengths(rng, m_vec, n, lengths)
+    pat = cv.random_values(cv.ColVecCSR(m_vec, n, V, ro, ci).validate(), seed=91)
+    B = cv.dense_uniform(n, N, seed=92)
+    ref = _oracle(pat, B)
+    Bd = torch.from_numpy(B).cuda()
+    for sort in (False, True):
+        prob = ops.DeviceProblem(pat, sort=sort)
+        for guard in (0, 1, 2, 8):
+            with _lib.thread_options(spmm_guard_waves=guard):
+                plain = prob.spmm(Bd)
+            torch.cuda.synchronize()
+            assert_parity(plain.cpu().numpy(), ref, "full grid, V%d N%d sort %d guard %d" % (V, N, sort, guard))
+        hinted = prob.spmm(Bd, row_length_hint=True)
+        torch.cuda.synchronize()
+        assert_parity(hinted.cpu().numpy(), ref, "full grid, hinted, V%d N%d sort %d" % (V, N, sort))
+
+
 @pytest.mark.parametrize("V", [1, 2, 4, 8])
 def test_lds_dma_gather_variant_keeps_parity(gpu, V):
     """The variant of the MFMA kernel whose gathered rows go global -> LDS directly and reach the MFMA through
