@@ -397,6 +397,7 @@ def main():
 
     # ---- cold caches (how the reference measures: Nsight --cache-control all)
     cold_ms = time_cold(torch, step)
+    cold_floor_ms = time_cold(torch, probe(512))  # what the same method reads for a kernel that does nothing
     cold_dense_ms = time_cold(torch, lambda: torch.matmul(Ad, Bd, out=dense_out))
     cold_large_ms = time_cold(torch, lambda: lprob.spmm(lBd, kernel="wmma", out=lout), samples=10)
     cold_sddmm_ms = time_cold(torch, sddmm_step, samples=10)
@@ -435,8 +436,10 @@ def main():
                         caches="warm: the 3.2 MB working set stays in the Infinity Cache between launches (the L2s "
                                "start every launch cold); see extra.cold_cache",
                         frac_cold=alg_bytes / (cold_ms * 1e-3) * 1e-9 / HBM_PEAK_GBS,
+                        frac_cold_note="from extra.cold_cache.spmm_config2_us, which contains the %.1f us the same "
+                                       "method reads for an empty kernel" % (cold_floor_ms * 1e3),
                         ceiling_frac=alg_bytes / (floor_ms * 1e-3) * 1e-9 / HBM_PEAK_GBS,
-                        ceiling_note="a kernel that does nothing on this launch's grid (256 workgroups of 1024 threads) "
+                        ceiling_note="a kernel that does nothing on this launch's grid (256 workgroups of up to 1024 threads) "
                                      "takes extra.launch_floor.empty_grid_us: the HBM-roofline time of config 2 "
                                      "(0.40 us) is a quarter of it, so frac cannot exceed ceiling_frac on this config"),
         "parity": {"max_rel_err": max_rel, "errors_gt_0.5": errors},
@@ -447,7 +450,11 @@ def main():
             "speedup_vs_dense_gemm": dense_ms / ev_ms,
             "launch_floor": {"empty_grid_us": floor_ms * 1e3, "empty_grid_one_wave_per_workgroup_us": floor_small_ms * 1e3,
                              "frac_of_floor": floor_ms / ev_ms},
-            "cold_cache": {"spmm_config2_us": cold_ms * 1e3, "dense_gemm_config2_us": cold_dense_ms * 1e3,
+            "cold_cache": {"method": "HIP events round one eager launch that follows a 1 GiB fill; the same method reads "
+                                     "empty_kernel_us for a kernel that does nothing on config 2's grid, so only the "
+                                     "differences to it are kernel time",
+                           "empty_kernel_us": cold_floor_ms * 1e3,
+                           "spmm_config2_us": cold_ms * 1e3, "dense_gemm_config2_us": cold_dense_ms * 1e3,
                            "spmm_largest_us": cold_large_ms * 1e3, "sddmm_config4_us": cold_sddmm_ms * 1e3,
                            "attention_config5_us": cold_attn_ms * 1e3},
             "spmm_largest_sweep_point": dict(
