@@ -423,9 +423,12 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
         // grids beyond 2048 workgroups get two.
         int guard = options().spmm_guard_waves;
         if (guard <= 0) guard = blocks <= 2048 ? 4 : 2;
-        if (!hinted && want > room && guard > room) {
+        // A wave takes twice the blocks the estimate gives it before a second one joins (rows at half density
+        // instead of the assumed quarter stay with one wave: two waves and their sum through LDS were 10-14 %
+        // slower there), and matrices too narrow for a row of more than twelve blocks need no guard at all.
+        if (!hinted && want > room && guard > room && ceil_div(ceil_div(n, kStep), in_flight) > 12) {
             const int launched = want < guard ? want : guard;
-            per_wave = want / room;
+            per_wave = 2 * want / room;
             waves = launched;
         }
         // A few rows far longer than the mean (lengths known): the average row keeps to the waves the chip has room
