@@ -219,6 +219,22 @@ int vs_wmma_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n,
                              const void *values, long long stride_values,
                              const void *rhs_matrix, long long stride_rhs,
                              void *output_matrix, long long stride_output, void *stream);
+/*
+ * vs_wmma_spmm_f16_batched for rows ordered by length, longest first (vs_sorted_row_swizzle): `long_rows` is
+ * the number of leading entries of row_indices whose rows hold more than 512 nonzero vectors (negative: not
+ * known, then this is vs_wmma_spmm_f16_batched).  On launches that fill the chip only those rows are shared
+ * by the waves of a workgroup; every other row is served by a single wave, so that no wave is launched
+ * without work - where the unsorted entry points hand every row the waves that only the long ones need.
+ * A pure launch-shape hint like the other two: a wrong count, or an order that is not by length, costs
+ * time (a long row behind the count is served by one wave), never correctness.  No counterpart in the
+ * reference, whose sorted order only reorders the dispatch of whole rows (include/bm_test_utils.h:200-215).
+ */
+int vs_wmma_spmm_f16_batched_sorted(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
+                                    int longest_row_vec, int long_rows, const int *row_indices,
+                                    const int *row_offsets, const int *column_indices, const void *values,
+                                    long long stride_values, const void *rhs_matrix, long long stride_rhs,
+                                    void *output_matrix, long long stride_output, void *stream);
+
 int vs_cuda_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
                              int longest_row_vec, const int *row_indices, const int *row_offsets,
                              const int *column_indices,
@@ -362,7 +378,8 @@ int vs_launch_floor_probe(int blocks, int threads_per_block, void *stream);
  * rows a wave of the MFMA SpMM keeps in flight: 1, 2, 4, 0 = automatic), "spmm_guard_waves"
  * (MFMA SpMM through the entry points that do not know the row lengths, on grids that fill the
  * chip by themselves: waves per workgroup kept for rows far longer than expected, 1 = none,
- * 0 = automatic), "spmm_gather" (how the MFMA SpMM
+ * 0 = automatic), "spmm_teams" (vs_wmma_spmm_f16_batched_sorted: 1 = ignore the long-row count),
+ * "spmm_gather" (how the MFMA SpMM
  * brings the gathered rows of the dense operand to the matrix cores: 1 = through
  * registers and an in-register transpose, 2 = global -> LDS loads and transposing LDS
  * reads, k % 8 == 0 only; 0 = automatic, which is 1: 2 measured 10-18 % slower),

@@ -211,6 +211,7 @@ struct Options {
     int spmm_waves = 0;
     int spmm_cols_per_lane = 0;
     int spmm_steps = 0;         // MFMA SpMM: 32-vector steps a wave keeps in flight (1, 2, 4), 0 = automatic
+    int spmm_teams = 0;         // MFMA SpMM with the long-row count known: 1 = every row gets a team of waves, 0 = automatic
     int spmm_guard_waves = 0;   // MFMA SpMM, row lengths unknown, full grid: waves per workgroup kept for rows longer than expected
     int spmm_gather = 0;        // 1 = gathered rows through registers, 2 = through LDS-DMA loads, 0 = automatic
     int spmm_flat_piece = 0;    // split-row SpMM: nonzero vectors per wave (rounded up to 32), 0 = automatic
@@ -254,6 +255,7 @@ struct Batch {
     long long stride_out = 0;  // SpMM: output_matrix SDDMM: output_values
     int nonzeros_vec = -1;     // SpMM: nonzero vectors of the pattern when the caller knows them (launch-shape hint)
     int longest_row_vec = -1;  // SpMM: nonzero vectors of the longest row when the caller knows them (same)
+    int long_rows = -1;        // SpMM, rows ordered by length: leading entries of row_indices with more than 512 vectors
     int algorithm = 0;         // SDDMM on MFMA: 2 = waves split the nonzero range, else (row, slot) per wave
 };
 

@@ -293,7 +293,7 @@ int vs_cuda_sddmm_f16_f32out(int m_vec, int k, int n, int nonzeros_vec, const in
 }
 
 static vs::Batch make_batch(int batch, long long a, long long b, long long out, int nonzeros_vec = -1,
-                            int longest_row_vec = -1)
+                            int longest_row_vec = -1, int long_rows = -1)
 {
     vs::Batch x;
     x.count = batch;
@@ -302,6 +302,7 @@ static vs::Batch make_batch(int batch, long long a, long long b, long long out, 
     x.stride_out = out;
     x.nonzeros_vec = nonzeros_vec;
     x.longest_row_vec = longest_row_vec;
+    x.long_rows = long_rows;
     return x;
 }
 
@@ -324,6 +325,25 @@ int vs_wmma_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n,
                                         static_cast<const half_t *>(values), static_cast<const half_t *>(rhs_matrix),
                                         static_cast<half_t *>(output_matrix), static_cast<hipStream_t>(stream),
                                         make_batch(batch, stride_values, stride_rhs, stride_output, nonzeros_vec, longest_row_vec));
+}
+
+int vs_wmma_spmm_f16_batched_sorted(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
+                                    int longest_row_vec, int long_rows, const int *row_indices, const int *row_offsets,
+                                    const int *column_indices, const void *values, long long stride_values,
+                                    const void *rhs_matrix, long long stride_rhs, void *output_matrix,
+                                    long long stride_output, void *stream)
+{
+    if (batch < 0) return VS_ERROR_INVALID_VALUE;
+    int st = check_spmm(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices, values, rhs_matrix,
+                        output_matrix, sizeof(half_t));
+    if (st != VS_SUCCESS) return st;
+    if (!stride_ok(stride_values, vec_length) || !stride_ok(stride_rhs, 8) || !stride_ok(stride_output, 8))
+        return VS_ERROR_INVALID_VALUE;
+    return vs::launch_spmm_mfma<half_t>(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices,
+                                        static_cast<const half_t *>(values), static_cast<const half_t *>(rhs_matrix),
+                                        static_cast<half_t *>(output_matrix), static_cast<hipStream_t>(stream),
+                                        make_batch(batch, stride_values, stride_rhs, stride_output, nonzeros_vec,
+                                                   longest_row_vec, long_rows < 0 ? -1 : long_rows));
 }
 
 int vs_cuda_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
@@ -521,6 +541,9 @@ static int set_option_field(vs::Options &o, const char *name, int value)
     } else if (std::strcmp(name, "spmm_cols_per_lane") == 0) {
         if (value != 0 && value != 4 && value != 8) return VS_ERROR_INVALID_VALUE;
         o.spmm_cols_per_lane = value;
+    } else if (std::strcmp(name, "spmm_teams") == 0) {
+        if (value > 1) return VS_ERROR_INVALID_VALUE;
+        o.spmm_teams = value;
     } else if (std::strcmp(name, "spmm_guard_waves") == 0) {
         if (value > 16) return VS_ERROR_INVALID_VALUE;
         o.spmm_guard_waves = value;

@@ -153,17 +153,23 @@ def _stride(t, batch):
 
 
 def spmm_batched(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices, values, rhs_matrix,
-                 output_matrix, kernel="wmma", stream=None, nonzeros_vec=-1, longest_row_vec=-1):
+                 output_matrix, kernel="wmma", stream=None, nonzeros_vec=-1, longest_row_vec=-1, long_rows=-1):
     """`batch` SpMMs sharing one pattern in one launch.
 
     values: [batch, nnz_vec, V] (or [nnz_vec, V] shared), rhs_matrix: [batch, n, k] (or [n, k] shared),
     output_matrix: [batch, m, k], all fp16 and contiguous in their trailing dimensions.
+    long_rows >= 0 (MFMA path): row_indices orders the rows by length, longest first, and its first long_rows
+    entries are the rows of more than LONG_ROW_VECTORS nonzero vectors (vs_wmma_spmm_f16_batched_sorted).
     """
     batch = output_matrix.shape[0]
     for t, nm in ((values, "values"), (rhs_matrix, "rhs_matrix"), (output_matrix, "output_matrix")):
         _expect_batched(t, torch.float16, nm)
     entry = "vs_wmma_spmm_f16_batched" if kernel == "wmma" else "vs_cuda_spmm_f16_batched"
-    st = getattr(_lib.lib(), entry)(batch, m_vec, vec_length, k, n, int(nonzeros_vec), int(longest_row_vec),
+    hints = [int(nonzeros_vec), int(longest_row_vec)]
+    if kernel == "wmma" and long_rows >= 0:
+        entry = "vs_wmma_spmm_f16_batched_sorted"
+        hints.append(int(long_rows))
+    st = getattr(_lib.lib(), entry)(batch, m_vec, vec_length, k, n, *hints,
                                     _ptr(row_indices), _ptr(row_offsets), _ptr(column_indices), _ptr(values), _stride(values, batch), _ptr(rhs_matrix),
                                     _stride(rhs_matrix, batch), _ptr(output_matrix), _stride(output_matrix, batch),
                                     _stream(stream))
@@ -420,6 +426,9 @@ def SortedRowSwizzle(rows, row_offsets):
     return out
 
 
+LONG_ROW_VECTORS = 512  # rows beyond this are "long" for vs_wmma_spmm_f16_batched_sorted (eight 64-vector blocks)
+
+
 def split_rows_pays(m_vec, nonzeros_vec, longest_row_vec):
     """Whether the split-row SpMM schedule is expected to beat the row-per-workgroup one with row-length hints.
     Measured at N = 256, V = 8, rows of up to 4608 vectors, 64 to 2048 vector rows: a row of 25 or more mean lengths
@@ -442,6 +451,8 @@ class DeviceProblem:
         self.nnz_vec = pattern.nnz_vec
         lengths = np.diff(pattern.row_offsets)
         self.longest_row_vec = int(lengths.max()) if lengths.size else 0
+        # with the sorted swizzle the long rows are the first entries of row_indices
+        self.long_rows = int(np.count_nonzero(lengths > LONG_ROW_VECTORS)) if sort else -1
         # a few rows far longer than the rest: schedules that give every row the same number of waves stall on them
         self.skewed = bool(pattern.nnz_vec >= 65536 and lengths.max() >= 8 * max(1.0, lengths.mean()))
         swz = SortedRowSwizzle(pattern.m_vec, pattern.row_offsets) if sort else IdentityRowSwizzle(pattern.m_vec)
@@ -476,7 +487,7 @@ class DeviceProblem:
         if row_length_hint and out.dtype == torch.float16:
             spmm_batched(self.m_vec, self.vec_length, k, self.n, self.row_indices, self.row_offsets,
                          self.column_indices, self.values, rhs_matrix, out.unsqueeze(0), kernel=kernel, stream=stream,
-                         nonzeros_vec=self.nnz_vec, longest_row_vec=self.longest_row_vec)
+                         nonzeros_vec=self.nnz_vec, longest_row_vec=self.longest_row_vec, long_rows=self.long_rows)
             return out
         fn = spmm.wmmaSpmm if kernel == "wmma" else spmm.cudaSpmm
         return fn(self.m_vec, self.vec_length, k, self.n, self.row_indices, self.row_offsets,
