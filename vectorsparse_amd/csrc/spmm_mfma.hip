@@ -30,14 +30,15 @@ namespace vs {
 // boundary, the last chunk of a row is cut): chunks are fetched and stored half by half.
 // S: 32-vector steps a wave keeps in flight at once (1, 2 or 4): its unit of work is a block of S steps whose 8 * S
 // row segments per lane are all requested before the first MFMA.
-template <int V, int CPL, bool SOFTMAX, bool IDX32, typename OutT, bool RAGGED = false, int S = 1>
+// TEAMS: rows ordered by length; only the first team_slots entries of row_indices get the workgroup's waves as a
+// team, behind them every wave takes a row of its own (below).
+template <int V, int CPL, bool SOFTMAX, bool IDX32, typename OutT, bool RAGGED = false, int S = 1, bool TEAMS = false>
 __global__ void __launch_bounds__(S * CPL >= 32 ? 256 : (S * CPL >= 16 ? 512 : 1024))
-spmm_mfma_kernel(int n_cols, int n_tiles, int per_wave_log2, int team_slots, int n_slots,
-                 const int *__restrict__ row_indices,
+spmm_mfma_kernel(int n_cols, int n_tiles, int per_wave_log2, const int *__restrict__ row_indices,
                  const int *__restrict__ row_offsets, const int *__restrict__ column_indices,
                  const half_t *__restrict__ values, const half_t *__restrict__ rhs,
                  OutT *__restrict__ out, long long stride_values, long long stride_rhs, long long stride_out,
-                 float scale)
+                 float scale, int team_slots, int n_slots)  // (the first sixteen dwords arrive preloaded in registers)
 {
     values += blockIdx.y * stride_values;  // batch: shared pattern, per-problem operands
     rhs += blockIdx.y * stride_rhs;
@@ -54,17 +55,19 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int per_wave_log2, int team_slots, int
     // With rows ordered by length (team_slots >= 0) only the first team_slots entries of row_indices - the long
     // rows - get a team; behind them a workgroup takes n_waves consecutive entries, one row per wave, which then
     // needs neither barrier nor LDS for its result and leaves no wave without work.
-    int tile = blockIdx.x % n_tiles;
+    int tile = blockIdx.x % n_tiles;  // (a grid of (tile, slot, batch) without this division measured 1 % slower)
     int slot = blockIdx.x / n_tiles;
     int wave = slot_wave;  // the wave's place in its row's team
     bool solo = false;
-    if (team_slots >= 0 && slot >= team_slots) {
-        const int b = blockIdx.x - team_slots * n_tiles;
-        tile = b % n_tiles;
-        slot = team_slots + (b / n_tiles) * n_waves + slot_wave;
-        wave = 0;
-        solo = true;
-        if (slot >= n_slots) return;
+    if constexpr (TEAMS) {
+        if (slot >= team_slots) {
+            const int b = blockIdx.x - team_slots * n_tiles;
+            tile = b % n_tiles;
+            slot = team_slots + (b / n_tiles) * n_waves + slot_wave;
+            wave = 0;
+            solo = true;
+            if (slot >= n_slots) return;
+        }
     }
     // The row's extent is requested for the identity order together with the swizzle entry itself, and again
     // only if the entry names another row: one dependent load less in the common case.
@@ -286,7 +289,7 @@ static int next_pow2(int x)
     return p;
 }
 
-template <int V, int CPL, bool SOFTMAX, bool IDX32, typename OutT, int S = 1>
+template <int V, int CPL, bool SOFTMAX, bool IDX32, typename OutT, int S = 1, bool TEAMS = false>
 static int launch_idx(int m_vec, int k, int n, int waves, const int *row_indices, const int *row_offsets,
                       const int *column_indices, const half_t *values, const half_t *rhs, OutT *out,
                       hipStream_t stream, const Batch &batch, float scale, int per_wave = 1, int team_slots = -1)
@@ -302,13 +305,13 @@ static int launch_idx(int m_vec, int k, int n, int waves, const int *row_indices
     if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
     const size_t lds = (size_t)waves * S * stage_bytes<V>() +
                        (waves > 1 ? (size_t)waves * V * (TN + 1) * sizeof(float) : 0);
-    auto kernel = spmm_mfma_kernel<V, CPL, SOFTMAX, IDX32, OutT, false, S>;
+    auto kernel = spmm_mfma_kernel<V, CPL, SOFTMAX, IDX32, OutT, false, S, TEAMS>;
     static std::atomic<unsigned long long> lds_allowed{0};
     const hipError_t attr = allow_large_lds(reinterpret_cast<const void *>(kernel), 96 * 1024, lds_allowed);
     if (attr != hipSuccess) return (int)attr;
     hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)batch.count), dim3(64 * waves), lds, stream,
-                       k, n_tiles, per_wave_log2, team_slots, m_vec, row_indices, row_offsets, column_indices, values, rhs, out,
-                       batch.stride_a, batch.stride_b, batch.stride_out, scale);
+                       k, n_tiles, per_wave_log2, row_indices, row_offsets, column_indices, values, rhs, out,
+                       batch.stride_a, batch.stride_b, batch.stride_out, scale, team_slots, m_vec);
     return (int)hipGetLastError();
 }
 
@@ -324,8 +327,8 @@ static int launch_ragged(int m_vec, int k, int waves, const int *row_indices, co
     if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
     const size_t lds = (size_t)waves * stage_bytes<V>() + (waves > 1 ? (size_t)waves * V * (TN + 1) * sizeof(float) : 0);
     hipLaunchKernelGGL((spmm_mfma_kernel<V, 4, false, false, OutT, true>), dim3((unsigned)blocks, (unsigned)batch.count),
-                       dim3(64 * waves), lds, stream, k, n_tiles, 0, -1, m_vec, row_indices, row_offsets, column_indices, values, rhs,
-                       out, batch.stride_a, batch.stride_b, batch.stride_out, 1.f);
+                       dim3(64 * waves), lds, stream, k, n_tiles, 0, row_indices, row_offsets, column_indices, values, rhs,
+                       out, batch.stride_a, batch.stride_b, batch.stride_out, 1.f, -1, m_vec);
     return (int)hipGetLastError();
 }
 
@@ -342,7 +345,12 @@ static int launch_one(int m_vec, int k, int n, int waves, int in_flight, const i
             if (in_flight == 4)
                 return launch_idx<V, CPL, SOFTMAX, true, OutT, 4>(m_vec, k, n, waves, row_indices, row_offsets,
                                                                    column_indices, values, rhs, out, stream, batch, scale,
-                                                                   per_wave, team_slots);
+                                                                   per_wave);
+            if (in_flight >= 2 && team_slots >= 0)
+                return launch_idx<V, CPL, SOFTMAX, true, OutT, 2, true>(m_vec, k, n, waves, row_indices, row_offsets,
+                                                                         column_indices, values, rhs, out, stream, batch,
+                                                                         scale, per_wave, team_slots);
+            team_slots = -1;  // only the two-step variant has the team mapping
             if (in_flight >= 2)
                 return launch_idx<V, CPL, SOFTMAX, true, OutT, 2>(m_vec, k, n, waves, row_indices, row_offsets,
                                                                    column_indices, values, rhs, out, stream, batch, scale,
