@@ -44,11 +44,13 @@ sddmm_mfma_kernel(int m_vec, int K, int slots, const int *__restrict__ row_indic
     out += blockIdx.y * stride_out;
     constexpr int SUPER = 16 * GRP;
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const long long wg = (long long)blockIdx.x * (blockDim.x >> 6) + wave;
-    if (wg >= (long long)m_vec * slots) return;
-    const int slot = (int)(wg / slots);
-    const int s = (int)(wg % slots);
+    // (row slot, slot within the row) from the wave's number in the launch: wave-uniform 32-bit arithmetic (the
+    // launcher keeps m_vec * slots below 2^32)
+    const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const unsigned wg = blockIdx.x * (blockDim.x >> 6) + wave;
+    if (wg >= (unsigned)m_vec * (unsigned)slots) return;
+    const int slot = (int)(wg / (unsigned)slots);
+    const int s = (int)(wg % (unsigned)slots);
     // the row's extent is requested for the identity order together with the swizzle entry, and again only if
     // the entry names another row: one dependent load less in the common case
     const int row = row_indices[slot];
@@ -286,7 +288,7 @@ static int launch_one(int m_vec, int k, int nonzeros_vec, const int *row_indices
     const int slots = sddmm_auto_slots((long long)m_vec * batch.count, (long long)nonzeros_vec * batch.count, 16 * GRP, true);
     const long long waves = (long long)m_vec * slots;
     const long long blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
-    if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
+    if (blocks > 0x7fffffffLL || blocks * kWavesPerBlock > 0xffffffffLL) return hipErrorNotSupported;
     hipLaunchKernelGGL((sddmm_mfma_kernel<V, KS, GRP, OutT>), dim3((unsigned)blocks, (unsigned)batch.count), dim3(64 * kWavesPerBlock), 0, stream,
                        m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out,
                        batch.stride_a, batch.stride_b, batch.stride_out);

@@ -86,14 +86,22 @@ sddmm_valu_kernel(int m_vec, int K, int slots, const int *__restrict__ row_indic
     constexpr int G = 64 / LK;
     constexpr int CHUNK = LK * VEC;
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const long long wg = (long long)blockIdx.x * (blockDim.x >> 6) + wave;
-    if (wg >= (long long)m_vec * slots) return;
-    const int slot = (int)(wg / slots);
-    const int s = (int)(wg % slots);
+    // wave-uniform 32-bit arithmetic (the launcher keeps m_vec * slots below 2^32): a 64-bit division per lane
+    // here cost 0.15 us per launch
+    const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const unsigned wg = blockIdx.x * (blockDim.x >> 6) + wave;
+    if (wg >= (unsigned)m_vec * (unsigned)slots) return;
+    const int slot = (int)(wg / (unsigned)slots);
+    const int s = (int)(wg % (unsigned)slots);
+    // the row's extent is requested for the identity order together with the swizzle entry, and again only if
+    // the entry names another row
     const int row = row_indices[slot];
-    const int beg = row_offsets[row];
-    const int end = row_offsets[row + 1];
+    int beg = row_offsets[slot];
+    int end = row_offsets[slot + 1];
+    if (row != slot) {
+        beg = row_offsets[row];
+        end = row_offsets[row + 1];
+    }
     const int n_groups = (end - beg + G - 1) / G;
     if (s >= n_groups) return;
     const int cl = lane % LK;
@@ -159,7 +167,7 @@ static int launch_one(int m_vec, int k, int nonzeros_vec, const int *row_indices
     const int slots = sddmm_auto_slots((long long)m_vec * batch.count, (long long)nonzeros_vec * batch.count, 64 / LK, false);
     const long long waves = (long long)m_vec * slots;
     const long long blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
-    if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
+    if (blocks > 0x7fffffffLL || blocks * kWavesPerBlock > 0xffffffffLL) return hipErrorNotSupported;
     hipLaunchKernelGGL((sddmm_valu_kernel<V, LK, VEC, SINGLE, OutT>), dim3((unsigned)blocks, (unsigned)batch.count),
                        dim3(64 * kWavesPerBlock), 0, stream, m_vec, k, slots, row_indices, row_offsets,
                        col_indices, lhs, rhs, out,

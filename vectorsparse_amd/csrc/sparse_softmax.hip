@@ -56,7 +56,7 @@ sparse_softmax_kernel(int m_vec, const int *__restrict__ row_indices, const int 
     in += blockIdx.y * stride_in;
     out += blockIdx.y * stride_out;
     const int lane = threadIdx.x & 63;
-    const int slot = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int slot = blockIdx.x * (blockDim.x >> 6) + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform
     if (slot >= m_vec) return;
     const int row = row_indices[slot];
     const int beg = row_offsets[row];
