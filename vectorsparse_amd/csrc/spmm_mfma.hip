@@ -34,15 +34,23 @@ namespace vs {
 // team, behind them every wave takes a row of its own (below).
 template <int V, int CPL, bool SOFTMAX, bool IDX32, typename OutT, bool RAGGED = false, int S = 1, bool TEAMS = false>
 __global__ void __launch_bounds__(S * CPL >= 32 ? 256 : (S * CPL >= 16 ? 512 : 1024))
-spmm_mfma_kernel(int n_cols, int n_tiles, int per_wave_log2, const int *__restrict__ row_indices,
+spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row_indices,
                  const int *__restrict__ row_offsets, const int *__restrict__ column_indices,
                  const half_t *__restrict__ values, const half_t *__restrict__ rhs,
                  OutT *__restrict__ out, long long stride_values, long long stride_rhs, long long stride_out,
                  float scale, int team_slots, int n_slots)  // (the first sixteen dwords arrive preloaded in registers)
 {
-    values += blockIdx.y * stride_values;  // batch: shared pattern, per-problem operands
-    rhs += blockIdx.y * stride_rhs;
-    out += blockIdx.y * stride_out;
+    // `shape` packs what the prologue needs into one of the kernel arguments that arrive in registers: bits 0-7
+    // log2 of the blocks a wave takes of a row, bits 8-15 the waves per workgroup, bit 16 "the grid has 512
+    // workgroups or more" - the workgroup size and the grid size would otherwise be loads from the hidden arguments.
+    const int per_wave_log2 = shape & 255;
+    const int n_waves = (shape >> 8) & 255;
+    const bool full_grid = (shape >> 16) & 1;
+    if (blockIdx.y != 0) {  // batch: shared pattern, per-problem operands (the strides are not loaded for problem 0)
+        values += blockIdx.y * stride_values;
+        rhs += blockIdx.y * stride_rhs;
+        out += blockIdx.y * stride_out;
+    }
     extern __shared__ __align__(16) unsigned char smem[];  // [W] staging slots, then [W][V][TN] partials
     constexpr int TN = 16 * CPL;
     constexpr int kStage = S * stage_bytes<V>();
@@ -50,7 +58,6 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int per_wave_log2, const int *__restri
     constexpr int F = (S + 1) / 2;          // vectors a lane fetches per block (lanes 0..31 only when S = 1)
     const int lane = threadIdx.x & 63;
     const int slot_wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the wave's LDS slot
-    const int n_waves = blockDim.x >> 6;
     // Workgroup -> rows.  A team: the workgroup's waves share one row (team_slots < 0: every workgroup is one).
     // With rows ordered by length (team_slots >= 0) only the first team_slots entries of row_indices - the long
     // rows - get a team; behind them a workgroup takes n_waves consecutive entries, one row per wave, which then
@@ -74,6 +81,9 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int per_wave_log2, const int *__restri
     const int row = row_indices[slot];
     int beg = row_offsets[slot];
     int end = row_offsets[slot + 1];
+    // (the empty statement keeps the two requests above: the compiler otherwise folds them into the dependent
+    // ones below by selecting the index)
+    asm volatile("" : "+s"(beg), "+s"(end));
     if (row != slot) {
         beg = row_offsets[row];
         end = row_offsets[row + 1];
@@ -102,7 +112,7 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int per_wave_log2, const int *__restri
     // other, so that a row of the expected length keeps to the waves the chip has room for and only a row far longer
     // than expected spreads over the rest of its workgroup.
     int active = S == 1 ? (steps + 1) >> 1 : (steps + S - 1) / S;
-    if (S > 1 && active == 2 && gridDim.x * gridDim.y >= 512) active = 1;
+    if (S > 1 && active == 2 && full_grid) active = 1;
     if (S > 1) active = (active + (1 << per_wave_log2) - 1) >> per_wave_log2;
     active = active < 1 ? 1 : (active > n_waves ? n_waves : active);
     if (solo) active = 1;
@@ -310,8 +320,9 @@ static int launch_idx(int m_vec, int k, int n, int waves, const int *row_indices
     const hipError_t attr = allow_large_lds(reinterpret_cast<const void *>(kernel), 96 * 1024, lds_allowed);
     if (attr != hipSuccess) return (int)attr;
     hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)batch.count), dim3(64 * waves), lds, stream,
-                       k, n_tiles, per_wave_log2, row_indices, row_offsets, column_indices, values, rhs, out,
-                       batch.stride_a, batch.stride_b, batch.stride_out, scale, team_slots, m_vec);
+                       k, n_tiles, per_wave_log2 | (waves << 8) | (blocks * batch.count >= 512 ? 1 << 16 : 0), row_indices,
+                       row_offsets, column_indices, values, rhs, out, batch.stride_a, batch.stride_b, batch.stride_out, scale,
+                       team_slots, m_vec);
     return (int)hipGetLastError();
 }
 
@@ -327,7 +338,7 @@ static int launch_ragged(int m_vec, int k, int waves, const int *row_indices, co
     if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
     const size_t lds = (size_t)waves * stage_bytes<V>() + (waves > 1 ? (size_t)waves * V * (TN + 1) * sizeof(float) : 0);
     hipLaunchKernelGGL((spmm_mfma_kernel<V, 4, false, false, OutT, true>), dim3((unsigned)blocks, (unsigned)batch.count),
-                       dim3(64 * waves), lds, stream, k, n_tiles, 0, row_indices, row_offsets, column_indices, values, rhs,
+                       dim3(64 * waves), lds, stream, k, n_tiles, waves << 8, row_indices, row_offsets, column_indices, values, rhs,
                        out, batch.stride_a, batch.stride_b, batch.stride_out, 1.f, -1, m_vec);
     return (int)hipGetLastError();
 }
