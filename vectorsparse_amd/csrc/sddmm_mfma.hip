@@ -34,20 +34,24 @@ __device__ __forceinline__ void store_group(OutT *out, int j, int g, const float
 // KS > 0: K <= 32*KS, lhs slices preloaded; KS == 0: any K % 8 == 0, lhs re-read per super-group.
 template <int V, int KS, int GRP, typename OutT>
 __global__ void __launch_bounds__(1024)
-sddmm_mfma_kernel(int m_vec, int K, int slots, const int *__restrict__ row_indices,
+sddmm_mfma_kernel(int m_vec, int K, int slots, int waves_per_block, const int *__restrict__ row_indices,
                   const int *__restrict__ row_offsets, const int *__restrict__ col_indices,
                   const half_t *__restrict__ lhs, const half_t *__restrict__ rhs, OutT *__restrict__ out,
                   long long stride_lhs, long long stride_rhs, long long stride_out)
 {
-    lhs += blockIdx.y * stride_lhs;  // batch: shared mask, per-problem operands
-    rhs += blockIdx.y * stride_rhs;
-    out += blockIdx.y * stride_out;
+    if (blockIdx.y != 0) {  // batch: shared mask, per-problem operands (the strides are not loaded for problem 0)
+        lhs += blockIdx.y * stride_lhs;
+        rhs += blockIdx.y * stride_rhs;
+        out += blockIdx.y * stride_out;
+    }
     constexpr int SUPER = 16 * GRP;
     const int lane = threadIdx.x & 63;
     // (row slot, slot within the row) from the wave's number in the launch: wave-uniform 32-bit arithmetic (the
-    // launcher keeps m_vec * slots below 2^32)
+    // launcher keeps m_vec * slots below 2^32).  The waves per workgroup come as an argument, which sits in
+    // scalar registers when the wave starts: the workgroup size would be a load from the hidden arguments, in
+    // front of everything else.
     const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const unsigned wg = blockIdx.x * (blockDim.x >> 6) + wave;
+    const unsigned wg = blockIdx.x * (unsigned)waves_per_block + wave;
     if (wg >= (unsigned)m_vec * (unsigned)slots) return;
     const int slot = (int)(wg / (unsigned)slots);
     const int s = (int)(wg % (unsigned)slots);
@@ -56,6 +60,7 @@ sddmm_mfma_kernel(int m_vec, int K, int slots, const int *__restrict__ row_indic
     const int row = row_indices[slot];
     int beg = row_offsets[slot];
     int end = row_offsets[slot + 1];
+    asm volatile("" : "+s"(beg), "+s"(end));  // keeps these two requests apart from the dependent ones below
     if (row != slot) {
         beg = row_offsets[row];
         end = row_offsets[row + 1];
@@ -145,20 +150,24 @@ sddmm_mfma_kernel(int m_vec, int K, int slots, const int *__restrict__ row_indic
 // changes and stay in registers while it lasts, one MFMA pass over the touched 16-vector groups per
 // segment.  The arithmetic of an output is the same as in the row-slot kernel (same operands, same MFMA
 // order): same bits.
+constexpr int kFlatWaves = 8;  // waves per workgroup of the flat kernel
+
 template <int V, int KS, int GRP, typename OutT>
-__global__ void __launch_bounds__(512)
+__global__ void __launch_bounds__(64 * kFlatWaves)
 sddmm_mfma_flat_kernel(int m_vec, int K, int nonzeros_vec, int supers, const int *__restrict__ row_offsets,
                        const int *__restrict__ col_indices, const half_t *__restrict__ lhs,
                        const half_t *__restrict__ rhs, OutT *__restrict__ out, long long stride_lhs,
                        long long stride_rhs, long long stride_out)
 {
-    lhs += blockIdx.y * stride_lhs;
-    rhs += blockIdx.y * stride_rhs;
-    out += blockIdx.y * stride_out;
+    if (blockIdx.y != 0) {
+        lhs += blockIdx.y * stride_lhs;
+        rhs += blockIdx.y * stride_rhs;
+        out += blockIdx.y * stride_out;
+    }
     constexpr int SUPER = 16 * GRP;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const long long first = ((long long)blockIdx.x * (blockDim.x >> 6) + wave) * supers * SUPER;
+    const long long first = ((long long)blockIdx.x * kFlatWaves + wave) * supers * SUPER;
     if (first >= nonzeros_vec) return;
     const int range_begin = (int)first;
     const int range_end = first + (long long)supers * SUPER < nonzeros_vec ? range_begin + supers * SUPER : nonzeros_vec;
@@ -277,10 +286,10 @@ static int launch_one(int m_vec, int k, int nonzeros_vec, const int *row_indices
             if (supers < min_supers) supers = min_supers;
             if (supers > 16) supers = 16;
             const long long flat_waves = (n_supers + supers - 1) / supers;
-            const long long flat_blocks = (flat_waves + 7) / 8;
+            const long long flat_blocks = (flat_waves + kFlatWaves - 1) / kFlatWaves;
             if (flat_blocks > 0x7fffffffLL) return hipErrorNotSupported;
             hipLaunchKernelGGL((sddmm_mfma_flat_kernel<V, KS, GRP, OutT>), dim3((unsigned)flat_blocks, (unsigned)batch.count),
-                               dim3(512), 0, stream, m_vec, k, nonzeros_vec, (int)supers, row_offsets, col_indices, lhs, rhs,
+                               dim3(64 * kFlatWaves), 0, stream, m_vec, k, nonzeros_vec, (int)supers, row_offsets, col_indices, lhs, rhs,
                                out, batch.stride_a, batch.stride_b, batch.stride_out);
             return (int)hipGetLastError();
         }
@@ -290,7 +299,7 @@ static int launch_one(int m_vec, int k, int nonzeros_vec, const int *row_indices
     const long long blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks > 0x7fffffffLL || blocks * kWavesPerBlock > 0xffffffffLL) return hipErrorNotSupported;
     hipLaunchKernelGGL((sddmm_mfma_kernel<V, KS, GRP, OutT>), dim3((unsigned)blocks, (unsigned)batch.count), dim3(64 * kWavesPerBlock), 0, stream,
-                       m_vec, k, slots, row_indices, row_offsets, col_indices, lhs, rhs, out,
+                       m_vec, k, slots, kWavesPerBlock, row_indices, row_offsets, col_indices, lhs, rhs, out,
                        batch.stride_a, batch.stride_b, batch.stride_out);
     return (int)hipGetLastError();
 }

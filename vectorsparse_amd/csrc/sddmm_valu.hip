@@ -75,21 +75,25 @@ __device__ __forceinline__ void slice_dot(float (&acc)[V], const half_t (&a)[V][
 // SINGLE: the whole of K fits one chunk (K <= LK*VEC) and the lhs slices stay in registers.
 template <int V, int LK, int VEC, bool SINGLE, typename OutT>
 __global__ void __launch_bounds__(256)
-sddmm_valu_kernel(int m_vec, int K, int slots, const int *__restrict__ row_indices,
+sddmm_valu_kernel(int m_vec, int K, int slots, int waves_per_block, const int *__restrict__ row_indices,
                   const int *__restrict__ row_offsets, const int *__restrict__ col_indices,
                   const half_t *__restrict__ lhs, const half_t *__restrict__ rhs, OutT *__restrict__ out,
                   long long stride_lhs, long long stride_rhs, long long stride_out)
 {
-    lhs += blockIdx.y * stride_lhs;  // batch: shared mask, per-problem operands
-    rhs += blockIdx.y * stride_rhs;
-    out += blockIdx.y * stride_out;
+    if (blockIdx.y != 0) {  // batch: shared mask, per-problem operands (the strides are not loaded for problem 0)
+        lhs += blockIdx.y * stride_lhs;
+        rhs += blockIdx.y * stride_rhs;
+        out += blockIdx.y * stride_out;
+    }
     constexpr int G = 64 / LK;
     constexpr int CHUNK = LK * VEC;
     const int lane = threadIdx.x & 63;
     // wave-uniform 32-bit arithmetic (the launcher keeps m_vec * slots below 2^32): a 64-bit division per lane
     // here cost 0.15 us per launch
+    // (the waves per workgroup come as an argument, which sits in scalar registers when the wave starts: the
+    // workgroup size would be a load from the hidden arguments)
     const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const unsigned wg = blockIdx.x * (blockDim.x >> 6) + wave;
+    const unsigned wg = blockIdx.x * (unsigned)waves_per_block + wave;
     if (wg >= (unsigned)m_vec * (unsigned)slots) return;
     const int slot = (int)(wg / (unsigned)slots);
     const int s = (int)(wg % (unsigned)slots);
@@ -98,6 +102,7 @@ sddmm_valu_kernel(int m_vec, int K, int slots, const int *__restrict__ row_indic
     const int row = row_indices[slot];
     int beg = row_offsets[slot];
     int end = row_offsets[slot + 1];
+    asm volatile("" : "+s"(beg), "+s"(end));  // keeps these two requests apart from the dependent ones below
     if (row != slot) {
         beg = row_offsets[row];
         end = row_offsets[row + 1];
@@ -169,7 +174,7 @@ static int launch_one(int m_vec, int k, int nonzeros_vec, const int *row_indices
     const long long blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks > 0x7fffffffLL || blocks * kWavesPerBlock > 0xffffffffLL) return hipErrorNotSupported;
     hipLaunchKernelGGL((sddmm_valu_kernel<V, LK, VEC, SINGLE, OutT>), dim3((unsigned)blocks, (unsigned)batch.count),
-                       dim3(64 * kWavesPerBlock), 0, stream, m_vec, k, slots, row_indices, row_offsets,
+                       dim3(64 * kWavesPerBlock), 0, stream, m_vec, k, slots, kWavesPerBlock, row_indices, row_offsets,
                        col_indices, lhs, rhs, out,
                        batch.stride_a, batch.stride_b, batch.stride_out);
     return (int)hipGetLastError();

@@ -37,20 +37,21 @@ __device__ __forceinline__ void load_values(uint32_t (&dst)[V > 1 ? V / 2 : 1], 
 // boundary, the last chunk of a row is cut): chunks are fetched and stored half by half.
 template <int V, int LR, typename OutT, bool RAGGED = false>
 __global__ void __launch_bounds__(1024)
-spmm_valu_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
+spmm_valu_kernel(int n_cols, int n_tiles, int n_waves, const int *__restrict__ row_indices,
                  const int *__restrict__ row_offsets, const int *__restrict__ column_indices,
                  const half_t *__restrict__ values, const half_t *__restrict__ rhs,
                  OutT *__restrict__ out, long long stride_values, long long stride_rhs, long long stride_out)
 {
-    values += blockIdx.y * stride_values;  // batch: shared pattern, per-problem operands
-    rhs += blockIdx.y * stride_rhs;
-    out += blockIdx.y * stride_out;
+    if (blockIdx.y != 0) {  // batch: shared pattern, per-problem operands (the strides are not loaded for problem 0)
+        values += blockIdx.y * stride_values;
+        rhs += blockIdx.y * stride_rhs;
+        out += blockIdx.y * stride_out;
+    }
     extern __shared__ float partial[];  // [W*G][V][TN]
     constexpr int G = 64 / LR;
     constexpr int TN = 8 * LR;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int n_waves = blockDim.x >> 6;
     const int tile = blockIdx.x % n_tiles;
     const int slot = blockIdx.x / n_tiles;
     // the row's extent is requested for the identity order together with the swizzle entry, and again only if
@@ -58,6 +59,7 @@ spmm_valu_kernel(int n_cols, int n_tiles, const int *__restrict__ row_indices,
     const int row = row_indices[slot];
     int beg = row_offsets[slot];
     int end = row_offsets[slot + 1];
+    asm volatile("" : "+s"(beg), "+s"(end));  // keeps these two requests apart from the dependent ones below
     if (row != slot) {
         beg = row_offsets[row];
         end = row_offsets[row + 1];
@@ -211,7 +213,7 @@ static int launch_one(int m_vec, int k, int waves, const int *row_indices, const
     if (waves < 1) waves = 1;
     const size_t lds = (waves * G > 1) ? (size_t)waves * G * V * TN * sizeof(float) : 0;
     hipLaunchKernelGGL((spmm_valu_kernel<V, LR, OutT, RAGGED>), dim3((unsigned)blocks, (unsigned)batch.count),
-                       dim3(64 * waves), lds, stream, k, n_tiles, row_indices, row_offsets, column_indices, values,
+                       dim3(64 * waves), lds, stream, k, n_tiles, waves, row_indices, row_offsets, column_indices, values,
                        rhs, out, batch.stride_a, batch.stride_b, batch.stride_out);
     return (int)hipGetLastError();
 }
