@@ -366,6 +366,19 @@ void vs_sorted_row_swizzle(int rows, const int *row_offsets, int *row_indices);
 int vs_launch_floor_probe(int blocks, int threads_per_block, void *stream);
 
 /*
+ * Reports the launch shape that vs_wmma_spmm_f16 (hints negative) or the batched SpMM entry points (hints as
+ * passed to them) would choose for a problem, under the calling thread's options; touches no device.  shape[0]
+ * dense columns per lane (4 or 8: tiles of 64 or 128 columns), [1] 32-vector steps of gathered rows a wave keeps
+ * in flight (1, 2, 4), [2] waves per workgroup (1..16), [3] blocks of a row a wave takes before another wave joins
+ * in, [4] leading entries of row_indices served by a team of waves (-1: all rows), [5] 1 for the variant for dense
+ * widths that are not a multiple of 4, [6] 1 for the LDS-DMA variant, [7] reserved (0).  Returns
+ * VS_ERROR_INVALID_VALUE for sizes the entry points reject.  No counterpart in the reference, whose launch shape
+ * is fixed (src/wmma_spmm.cu:362-378: one warp per vector row and 64-column tile).
+ */
+int vs_wmma_spmm_launch_shape(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
+                              int longest_row_vec, int long_rows, int shape[8]);
+
+/*
  * Launch-shape tuning knobs.  vs_set_option sets the process-wide default (not
  * synchronised: set it before launching from several threads).
  * vs_set_thread_option sets the value for the calling thread only: from its first

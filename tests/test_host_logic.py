@@ -5,7 +5,7 @@ import pytest
 
 from oracle import c_oracle as co
 from vectorsparse_amd import colvec_csr as cv
-from vectorsparse_amd import ops, sweep
+from vectorsparse_amd import _lib, ops, sweep
 
 
 def _largest_union(mask, rows):
@@ -90,6 +90,77 @@ def test_split_row_choice_follows_the_row_lengths():
     assert not pays(128, 128 * 300, 4500) and not pays(1024, 1024 * 300, 4500)
     # too small to matter, and degenerate shapes
     assert not pays(8, 400, 300) and not pays(0, 0, 0)
+
+
+def test_spmm_launch_shape_choice():
+    """The host-side shape choice of the MFMA SpMM: what it picks on the named configurations, and that every
+    choice respects what the kernel variants assume (their launch bounds and the grid arithmetic)."""
+    shape = ops.spmm_launch_shape
+    # headline shape (512 x 4608 x 256, V = 8): narrow tiles so that 64 rows give 256 workgroups, two steps in
+    # flight, eight waves per row of about fifteen steps
+    headline = shape(64, 8, 256, 4608)
+    assert (headline["cols_per_lane"], headline["steps_in_flight"], headline["waves"]) == (4, 2, 8)
+    assert headline["team_slots"] == -1 and not headline["ragged"] and not headline["dma"]
+    # largest sweep point: wide tiles (128-bit row segments); four steps in flight only with the row lengths known
+    assert shape(256, 8, 256, 4608)["cols_per_lane"] == 8
+    assert shape(256, 8, 256, 4608)["steps_in_flight"] == 2
+    assert shape(256, 8, 256, 4608, nonzeros_vec=256 * 461, longest_row_vec=470)["steps_in_flight"] == 4
+    # one 64-column tile for narrow dense operands, the half-by-half variant for widths off a multiple of 4
+    assert shape(512, 8, 64, 4096)["cols_per_lane"] == 4
+    assert shape(64, 8, 147, 4608)["ragged"] == 1 and shape(64, 8, 148, 4608)["ragged"] == 0
+    # rows of under one step: one wave, one step
+    short = shape(4096, 8, 256, 64, nonzeros_vec=4096 * 6, longest_row_vec=6)
+    assert (short["steps_in_flight"], short["waves"]) == (1, 1)
+    # unhinted launch on a grid that fills the chip keeps guard waves for a row far longer than expected ...
+    guarded = shape(1024, 8, 256, 4608)
+    assert guarded["waves"] >= 2 and guarded["blocks_per_wave"] >= 2
+    # ... and drops them with the lengths known
+    assert shape(1024, 8, 256, 4608, nonzeros_vec=1024 * 461, longest_row_vec=470)["blocks_per_wave"] >= 1
+    # skewed rows, ordered by length, the count of long rows known: teams for those rows only
+    teams = shape(1024, 8, 256, 4608, nonzeros_vec=1024 * 100 + 4508, longest_row_vec=4608, long_rows=1)
+    assert teams["team_slots"] == 1 and teams["steps_in_flight"] == 2 and 4 <= teams["waves"] <= 8
+    with _lib.thread_options(spmm_teams=1):
+        assert shape(1024, 8, 256, 4608, nonzeros_vec=1024 * 100 + 4508, longest_row_vec=4608,
+                     long_rows=1)["team_slots"] == -1
+    # an override is taken as given
+    with _lib.thread_options(spmm_waves=2, spmm_steps=1, spmm_cols_per_lane=8):
+        forced = shape(64, 8, 256, 4608)
+        assert (forced["cols_per_lane"], forced["steps_in_flight"], forced["waves"]) == (8, 1, 2)
+    # invariants over random problems, hinted and not
+    rng = np.random.default_rng(11)
+    for _ in range(3000):
+        m_vec = int(rng.integers(1, 9000))
+        k = int(rng.integers(1, 1100))
+        n = int(rng.integers(1, 9000))
+        batch = int(rng.choice([1, 1, 1, 4, 16]))
+        hints = {}
+        if rng.random() < 0.6:
+            longest = int(rng.integers(0, n + 1))
+            mean = int(rng.integers(0, longest + 1))
+            hints = dict(nonzeros_vec=min(mean * m_vec, 2**31 - 1), longest_row_vec=longest)
+            if rng.random() < 0.5:
+                hints["long_rows"] = int(rng.integers(0, m_vec + 1))
+        got = shape(m_vec, int(rng.choice([1, 2, 4, 8])), k, n, batch=batch, **hints)
+        case = (m_vec, k, n, batch, hints, got)
+        assert got["cols_per_lane"] in (4, 8) and got["steps_in_flight"] in (1, 2, 4), case
+        assert got["waves"] in (1, 2, 4, 8, 16), case
+        # the launch bounds of the variants with 64 / 128 registers of row segments in flight
+        assert got["waves"] * 64 <= (256 if got["steps_in_flight"] * got["cols_per_lane"] >= 32 else
+                                     512 if got["steps_in_flight"] * got["cols_per_lane"] >= 16 else 1024), case
+        assert got["blocks_per_wave"] >= 1 and got["blocks_per_wave"] & (got["blocks_per_wave"] - 1) == 0, case
+        assert -1 <= got["team_slots"] <= m_vec, case
+        if got["team_slots"] >= 0:
+            assert got["steps_in_flight"] == 2 and got["blocks_per_wave"] == 1, case
+        assert bool(got["ragged"]) == (k % 4 != 0), case
+        if got["ragged"]:
+            assert got["cols_per_lane"] == 4 and got["steps_in_flight"] == 1 and got["waves"] <= 8, case
+        if got["cols_per_lane"] == 8:
+            assert k % 8 == 0, case
+    for bad in (dict(m_vec=0), dict(k=0), dict(vec_length=3), dict(batch=0)):
+        args = dict(m_vec=64, vec_length=8, k=256, n=4608)
+        args.update(bad)
+        with pytest.raises(_lib.VSparseError):
+            shape(**args)
 
 
 def test_sweep_benchmark_selection(tmp_path):

@@ -28,6 +28,7 @@ SIGNATURES = {
     "vs_cuda_sddmm_f16_f32out": ([_int] * 4 + [_vp] * 6 + [_int, _vp], _int),
     "vs_wmma_spmm_f16_batched": ([_int] * 7 + [_vp] * 3 + [_vp, _ll, _vp, _ll, _vp, _ll, _vp], _int),
     "vs_wmma_spmm_f16_batched_sorted": ([_int] * 8 + [_vp] * 3 + [_vp, _ll, _vp, _ll, _vp, _ll, _vp], _int),
+    "vs_wmma_spmm_launch_shape": ([_int] * 8 + [_vp], _int),
     "vs_cuda_spmm_f16_batched": ([_int] * 7 + [_vp] * 3 + [_vp, _ll, _vp, _ll, _vp, _ll, _vp], _int),
     "vs_wmma_sddmm_f16_batched": ([_int] * 5 + [_vp] * 3 + [_vp, _ll, _vp, _ll, _vp, _ll, _int, _vp, _int], _int),
     "vs_cuda_sddmm_f16_batched": ([_int] * 5 + [_vp] * 3 + [_vp, _ll, _vp, _ll, _vp, _ll, _int, _vp], _int),

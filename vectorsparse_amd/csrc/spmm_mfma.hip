@@ -389,18 +389,15 @@ static int launch_v(int vec_length, int m_vec, int k, int n, int waves, int in_f
     }
 }
 
-template <bool SOFTMAX, typename OutT>
-static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_indices,
-                      const int *row_offsets, const int *column_indices, const half_t *values,
-                      const half_t *rhs, OutT *out, hipStream_t stream, const Batch &batch, float scale)
+// The launch shape of an MFMA SpMM, chosen on the host from what the entry point knows of the problem (the row
+// lengths only through the hints of the batched entry points) and from the calling thread's options.
+SpmmShape choose_spmm_shape(bool softmax, int m_vec, int k, int n, const Batch &batch)
 {
-    if (m_vec == 0 || k == 0 || batch.count == 0) return hipSuccess;
-    if (batch.count > 65535) return hipErrorNotSupported;
-    if (SOFTMAX && k % 4 != 0) return hipErrorNotSupported;
+    SpmmShape shape;
     constexpr int kTargetBlocks = 256;   // one workgroup per CU at least
     constexpr int kTargetWaves = 4096;
     int cpl = options().spmm_cols_per_lane;
-    const bool use_dma = !SOFTMAX && options().spmm_gather == 2 && k % 8 == 0;
+    const bool use_dma = !softmax && options().spmm_gather == 2 && k % 8 == 0;
     if (use_dma) cpl = 8;
     const bool hinted = batch.nonzeros_vec >= 0;
     const int mean_steps = hinted ? ceil_div(ceil_div(batch.nonzeros_vec, m_vec), kStep) : ceil_div(n, 4 * kStep);
@@ -427,7 +424,7 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
     // of the workgroup beyond four waves), while too few waves for denser rows cost 10-18 %.
     // while the chip has room the workgroup of the longest row ends last, so that row sets the size
     const int row_steps = longest_steps > mean_steps ? longest_steps : mean_steps;
-    const bool blocks_exist = !SOFTMAX && !ragged && !use_dma && (long long)n * k < (1LL << 31);
+    const bool blocks_exist = !softmax && !ragged && !use_dma && (long long)n * k < (1LL << 31);
     int in_flight = options().spmm_steps;
     if (in_flight != 1 && in_flight != 2 && in_flight != 4) {
         in_flight = row_steps >= 2 ? 2 : 1;
@@ -539,9 +536,29 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
     // launch bounds of the variants with 64 / 128 registers of row segments in flight
     if (in_flight * cpl >= 16 && waves > 8) waves = 8;
     if (in_flight * cpl >= 32 && waves > 4) waves = 4;
+    if (ragged && waves > 8) waves = 8;  // 8 x 2.7 KB of LDS stay below the default limit of dynamic LDS
+    shape.cols_per_lane = cpl;
+    shape.steps_in_flight = in_flight;
+    shape.waves = waves;
+    shape.blocks_per_wave = per_wave;
+    shape.team_slots = team_slots;
+    shape.ragged = ragged;
+    shape.dma = use_dma && !ragged;
+    return shape;
+}
+
+template <bool SOFTMAX, typename OutT>
+static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_indices,
+                      const int *row_offsets, const int *column_indices, const half_t *values,
+                      const half_t *rhs, OutT *out, hipStream_t stream, const Batch &batch, float scale)
+{
+    if (m_vec == 0 || k == 0 || batch.count == 0) return hipSuccess;
+    if (batch.count > 65535) return hipErrorNotSupported;
+    if (SOFTMAX && k % 4 != 0) return hipErrorNotSupported;
+    const SpmmShape shape = choose_spmm_shape(SOFTMAX, m_vec, k, n, batch);
+    const int waves = shape.waves;
     if constexpr (!SOFTMAX) {
-        if (ragged) {
-            if (waves > 8) waves = 8;  // 8 x 2.7 KB of LDS stay below the default limit of dynamic LDS
+        if (shape.ragged) {
             switch (vec_length) {
             case 1: return launch_ragged<1, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
             case 2: return launch_ragged<2, OutT>(m_vec, k, waves, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch);
@@ -550,13 +567,14 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
             default: return hipErrorInvalidValue;
             }
         }
-        if (use_dma)
+        if (shape.dma)
             return launch_spmm_mfma_dma<OutT>(m_vec, vec_length, k, n, waves, row_indices, row_offsets, column_indices,
                                               values, rhs, out, stream, batch);
     }
-    if (cpl == 8)
-        return launch_v<8, SOFTMAX, OutT>(vec_length, m_vec, k, n, waves, in_flight | (per_wave << 8), row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale, team_slots);
-    return launch_v<4, SOFTMAX, OutT>(vec_length, m_vec, k, n, waves, in_flight | (per_wave << 8), row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale, team_slots);
+    const int packed = shape.steps_in_flight | (shape.blocks_per_wave << 8);
+    if (shape.cols_per_lane == 8)
+        return launch_v<8, SOFTMAX, OutT>(vec_length, m_vec, k, n, waves, packed, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale, shape.team_slots);
+    return launch_v<4, SOFTMAX, OutT>(vec_length, m_vec, k, n, waves, packed, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale, shape.team_slots);
 }
 
 template <typename OutT>

@@ -259,6 +259,18 @@ struct Batch {
     int algorithm = 0;         // SDDMM on MFMA: 2 = waves split the nonzero range, else (row, slot) per wave
 };
 
+// Launch shape of the MFMA SpMM (spmm_mfma.hip), chosen on the host.
+struct SpmmShape {
+    int cols_per_lane = 4;     // dense columns per lane: tiles of 16 x this many columns, 64- or 128-bit row segments
+    int steps_in_flight = 1;   // 32-vector steps whose gathered rows a wave requests before its first MFMA (1, 2, 4)
+    int waves = 1;             // waves per workgroup
+    int blocks_per_wave = 1;   // blocks of a row a wave takes before another wave of the workgroup joins in
+    int team_slots = -1;       // >= 0: only that many leading entries of row_indices get the workgroup as a team
+    bool ragged = false;       // dense width not a multiple of 4: the half-by-half variant
+    bool dma = false;          // the variant that gathers through LDS-DMA loads (option spmm_gather = 2)
+};
+SpmmShape choose_spmm_shape(bool softmax, int m_vec, int k, int n, const Batch &batch);
+
 // Launchers (one per kernel family); return a hipError_t-valued int.
 template <typename OutT>
 int launch_spmm_mfma(int m_vec, int vec_length, int k, int n, const int *row_indices,

@@ -346,6 +346,24 @@ int vs_wmma_spmm_f16_batched_sorted(int batch, int m_vec, int vec_length, int k,
                                                    longest_row_vec, long_rows < 0 ? -1 : long_rows));
 }
 
+int vs_wmma_spmm_launch_shape(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
+                              int longest_row_vec, int long_rows, int shape[8])
+{
+    if (shape == nullptr || batch < 1 || batch > 65535 || m_vec < 1 || k < 1 || n < 0) return VS_ERROR_INVALID_VALUE;
+    if (vec_length != 1 && vec_length != 2 && vec_length != 4 && vec_length != 8) return VS_ERROR_INVALID_VALUE;
+    const vs::SpmmShape chosen = vs::choose_spmm_shape(
+        false, m_vec, k, n, make_batch(batch, 0, 0, 0, nonzeros_vec, longest_row_vec, long_rows < 0 ? -1 : long_rows));
+    shape[0] = chosen.cols_per_lane;
+    shape[1] = chosen.steps_in_flight;
+    shape[2] = chosen.waves;
+    shape[3] = chosen.blocks_per_wave;
+    shape[4] = chosen.team_slots;
+    shape[5] = chosen.ragged ? 1 : 0;
+    shape[6] = chosen.dma ? 1 : 0;
+    shape[7] = 0;
+    return VS_SUCCESS;
+}
+
 int vs_cuda_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
                              int longest_row_vec, const int *row_indices,
                              const int *row_offsets, const int *column_indices, const void *values,

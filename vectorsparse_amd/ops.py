@@ -100,6 +100,18 @@ class spmm:
                      values, rhs_matrix, output_matrix, stream)
 
 
+def spmm_launch_shape(m_vec, vec_length, k, n, batch=1, nonzeros_vec=-1, longest_row_vec=-1, long_rows=-1):
+    """The launch shape `wmmaSpmm` (hints negative) or `spmm_batched` (hints as passed there) would choose, under the
+    calling thread's options, as a dict; touches no device."""
+    import ctypes
+    shape = (ctypes.c_int * 8)()
+    _lib.check(_lib.lib().vs_wmma_spmm_launch_shape(batch, m_vec, vec_length, k, n, nonzeros_vec, longest_row_vec,
+                                                    long_rows, ctypes.cast(shape, ctypes.c_void_p)),
+               "vs_wmma_spmm_launch_shape")
+    names = ("cols_per_lane", "steps_in_flight", "waves", "blocks_per_wave", "team_slots", "ragged", "dma")
+    return dict(zip(names, (int(x) for x in shape)))
+
+
 def spmm_workspace_bytes(m_vec, vec_length, k, n, nonzeros_vec):
     """Preferred workspace size of `spmm_split_rows` for this problem (0: no row can be split)."""
     return int(_lib.lib().vs_wmma_spmm_workspace_bytes(m_vec, vec_length, k, n, nonzeros_vec))
