@@ -156,9 +156,10 @@ int vs_cuda_spmm_f16_f32out(int m_vec, int vec_length, int k, int n,
  * 3 (the reference's timing-only hardware
  * simulation, whose results are wrong by design) is rejected with
  * hipErrorInvalidValue.
- * Requirements: k % 8 == 0 (the whole of k is contracted — the reference drops
- * k % 64); lhs_matrix / rhs_matrix aligned to 16 bytes, output_values to
- * 2*vec_length bytes.
+ * Any k >= 0; the whole of k is contracted (the reference drops k % 64).  k % 8 != 0
+ * runs on the scalar-load variant of the fine-grained kernel of vs_cuda_sddmm_f16,
+ * whatever the algorithm.  lhs_matrix / rhs_matrix aligned to 16 bytes when
+ * k % 8 == 0 (2 bytes otherwise), output_values to 2*vec_length bytes.
  */
 int vs_wmma_sddmm_f16(int m_vec, int k, int n, int nonzeros_vec,
                       const int *row_indices, const int *row_offsets,

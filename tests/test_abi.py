@@ -70,11 +70,11 @@ def test_argument_validation_without_launch():
     assert L.vs_wmma_sddmm_f16(4, 64, 64, 10, p, p, p, p, p, p, 8, None, 3) == INVALID
     assert L.vs_wmma_sddmm_f16(4, 64, 64, 10, p, p, p, p, p, p, 8, None, -1) == INVALID
     # shapes a path cannot take
-    # (the reference-shaped SpMM entry points take any dense width; the split-row schedule needs k % 4 == 0)
+    # (the reference-shaped entry points take any dense width / contraction length; the split-row schedule needs
+    # k % 4 == 0)
     assert L.vs_wmma_spmm_f16_ws(4, 8, 66, 64, 10, p, p, p, p, p, p, None, 0, None) == 801
     assert L.vs_wmma_spmm_f16_noalloc(4, 8, 66, 64, 10, p, p, p, p, p, p, None) == 801
     assert L.vs_wmma_spmm_f16_noalloc(4, 8, 4224, 64, 10, p, p, p, p, p, p, None) == 801   # beyond the scratch
-    assert L.vs_wmma_sddmm_f16(4, 60, 64, 10, p, p, p, p, p, p, 8, None, 1) == 801
     # empty problems succeed without touching the device
     assert L.vs_wmma_spmm_f16(0, 8, 64, 64, None, None, None, None, None, None, None) == OK
     assert L.vs_cuda_spmm_f16(4, 8, 0, 64, None, None, None, None, None, None, None) == OK

@@ -62,11 +62,17 @@ def test_vec_lengths_and_contraction_sizes(gpu, V, K):
 
 @pytest.mark.parametrize("V", [1, 2, 4, 8])
 @pytest.mark.parametrize("K", [1, 7, 12, 50, 100, 130])
-def test_cuda_path_takes_any_k(gpu, V, K):
+def test_both_paths_take_any_k(gpu, V, K):
+    """Contraction lengths off a multiple of 8 on both entry points and under every algorithm of the MFMA one (the
+    whole of K is contracted; the reference's MMA kernels drop K % 64, src/wmma_sddmm.cu:88-120)."""
     pat = cv.binomial_pattern(48 // V, 100, 0.8, seed=V * 100 + K, vec_length=V)
     A = cv.dense_normal(pat.m, K, seed=3)
     B = cv.dense_normal(100, K, seed=4)
-    assert_parity(_run(pat, A, B, "cuda"), _oracle(pat, A, B), "cuda V%d K%d" % (V, K))
+    ref = _oracle(pat, A, B)
+    assert_parity(_run(pat, A, B, "cuda"), ref, "cuda V%d K%d" % (V, K))
+    for algorithm in (0, 1, 2):
+        assert_parity(_run(pat, A, B, "wmma", algorithm=algorithm), ref, "wmma V%d K%d algorithm %d" % (V, K, algorithm))
+    assert_parity(_run(pat, A, B, "wmma", out_dtype=torch.float32), ref, "wmma f32 out V%d K%d" % (V, K))
 
 
 @pytest.mark.parametrize("V", [1, 2, 4, 8])

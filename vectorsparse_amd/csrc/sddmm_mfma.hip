@@ -381,7 +381,13 @@ int launch_sddmm_mfma(int m_vec, int k, int n, int nonzeros_vec, const int *row_
     (void)n;
     if (m_vec == 0 || nonzeros_vec == 0 || batch.count == 0) return hipSuccess;
     if (batch.count > 65535) return hipErrorNotSupported;
-    if (k <= 0 || k % 8 != 0) return hipErrorNotSupported;
+    if (k <= 0) return hipErrorNotSupported;
+    // Contraction lengths off a multiple of 8 (rows of the dense operands then start at any 2-byte boundary, out of
+    // reach of 128-bit loads) run on the fine-grained kernel's scalar-load variant, whatever the algorithm: the
+    // whole of k is contracted on both paths (the reference's MMA kernels drop k % 64, src/wmma_sddmm.cu:88-120).
+    if (k % 8 != 0)
+        return launch_sddmm_valu<OutT>(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out,
+                                       vec_length, stream, batch);
     // algorithm 0 (automatic): vectors of 1, 2 or 4 rows fill 1/16 to 4/16 of an MFMA tile, and on masks of few
     // nonzeros the fine-grained kernel (dot products on the vector ALU, reduced across lanes with DPP) is ahead:
     // over the M = N = 512..4096, K = 64..256 grid by 5-40 % below these nonzero counts, behind above them.
