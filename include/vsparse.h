@@ -392,7 +392,8 @@ int vs_wmma_spmm_launch_shape(int batch, int m_vec, int vec_length, int k, int n
  * rows a wave of the MFMA SpMM keeps in flight: 1, 2, 4, 0 = automatic), "spmm_guard_waves"
  * (MFMA SpMM through the entry points that do not know the row lengths, on grids that fill the
  * chip by themselves: waves per workgroup kept for rows far longer than expected, 1 = none,
- * 0 = automatic), "spmm_teams" (vs_wmma_spmm_f16_batched_sorted: 1 = ignore the long-row count),
+ * 0 = automatic), "spmm_teams" (vs_wmma_spmm_f16_batched_sorted: 1 = ignore the long-row count, 2 = use it on every
+ * launch, 0 = where it measured faster),
  * "spmm_gather" (how the MFMA SpMM
  * brings the gathered rows of the dense operand to the matrix cores: 1 = through
  * registers and an in-register transpose, 2 = global -> LDS loads and transposing LDS

@@ -321,12 +321,15 @@ def test_skewed_rows_on_a_grid_that_fills_the_chip(gpu, V, m_vec, N):
         assert_parity(hinted.cpu().numpy(), ref, "full grid, hinted, V%d N%d sort %d" % (V, N, sort))
         # the long-row count of the sorted entry point is a hint: any count, in any order of the rows, gives the
         # same result (teams of waves for the first `long_rows` entries, one wave per row behind them)
-        for long_rows in (0, 1, 5, 64, m_vec - 1, m_vec, m_vec + 9):
+        # (spmm_teams = 2: on every launch, not only where the library expects the team mapping to pay)
+        for teams, long_rows in [(2, x) for x in (0, 1, 5, 64, m_vec - 1, m_vec, m_vec + 9)] + [(0, 1), (0, 64)]:
             out = torch.full((1, pat.m, N), 3.0, dtype=torch.float16, device="cuda")
-            ops.spmm_batched(pat.m_vec, V, N, n, prob.row_indices, prob.row_offsets, prob.column_indices, prob.values,
-                             Bd, out, nonzeros_vec=pat.nnz_vec, longest_row_vec=n, long_rows=long_rows)
+            with _lib.thread_options(spmm_teams=teams):
+                ops.spmm_batched(pat.m_vec, V, N, n, prob.row_indices, prob.row_offsets, prob.column_indices,
+                                 prob.values, Bd, out, nonzeros_vec=pat.nnz_vec, longest_row_vec=n, long_rows=long_rows)
             torch.cuda.synchronize()
-            assert_parity(out[0].cpu().numpy(), ref, "full grid, %d long rows said, V%d N%d sort %d" % (long_rows, V, N, sort))
+            assert_parity(out[0].cpu().numpy(), ref,
+                          "full grid, %d long rows said (teams %d), V%d N%d sort %d" % (long_rows, teams, V, N, sort))
         with _lib.thread_options(spmm_teams=1):
             assert_parity(prob.spmm(Bd, row_length_hint=True).cpu().numpy(), ref, "teams for every row")
 

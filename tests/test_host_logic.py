@@ -117,10 +117,13 @@ def test_spmm_launch_shape_choice():
     # ... and drops them with the lengths known
     assert shape(1024, 8, 256, 4608, nonzeros_vec=1024 * 461, longest_row_vec=470)["blocks_per_wave"] >= 1
     # skewed rows, ordered by length, the count of long rows known: teams for those rows only
-    teams = shape(1024, 8, 256, 4608, nonzeros_vec=1024 * 100 + 4508, longest_row_vec=4608, long_rows=1)
+    # (on grids of sixteen workgroups per CU or more whose average row is short)
+    teams = shape(2048, 8, 256, 4608, nonzeros_vec=2048 * 100 + 4508, longest_row_vec=4608, long_rows=1)
     assert teams["team_slots"] == 1 and teams["steps_in_flight"] == 2 and 4 <= teams["waves"] <= 8
+    assert shape(512, 8, 256, 4608, nonzeros_vec=512 * 100 + 4508, longest_row_vec=4608, long_rows=1)["team_slots"] == -1
+    assert shape(2048, 8, 256, 4608, nonzeros_vec=2048 * 300 + 4308, longest_row_vec=4608, long_rows=1)["team_slots"] == -1
     with _lib.thread_options(spmm_teams=1):
-        assert shape(1024, 8, 256, 4608, nonzeros_vec=1024 * 100 + 4508, longest_row_vec=4608,
+        assert shape(2048, 8, 256, 4608, nonzeros_vec=2048 * 100 + 4508, longest_row_vec=4608,
                      long_rows=1)["team_slots"] == -1
     # an override is taken as given
     with _lib.thread_options(spmm_waves=2, spmm_steps=1, spmm_cols_per_lane=8):

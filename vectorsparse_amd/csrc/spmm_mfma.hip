@@ -484,16 +484,26 @@ SpmmShape choose_spmm_shape(bool softmax, int m_vec, int k, int n, const Batch &
             waves = base > for_longest ? base : for_longest;
         }
         // Rows ordered by length and the count of long ones known (batch.long_rows: the leading entries of
-        // row_indices whose rows hold more than 512 vectors), on a grid that fills the chip: only those rows get a
-        // team of waves - the longest at about eight blocks per wave - and every other row one wave of a workgroup
-        // that takes as many rows as it has waves.  No wave is launched without work (the launches above hand
-        // every row the team that only the long ones need, at 0.3 us per thousand waves that end at once).
-        // Measured, N = 256, V = 8: one dense row among 2047 rows of 100 vectors 15.0 -> 13.0 us, 1024 Pareto rows
-        // 14.5 -> 13.8 us; it loses where the average row itself is long (log-normal rows of 470 vectors on
-        // average: 11.2 -> 14.8 us, a wave then walks up to eight blocks alone) or no row is long (uniform rows of
-        // 50: 5.9 -> 6.3 us), so it is kept for skewed rows of at most five blocks on average.
-        if (skewed && batch.long_rows > 0 && room <= 2 && ceil_div(mean_steps, in_flight) <= 5 &&
-            options().spmm_teams != 1) {
+        // row_indices whose rows hold more than 512 vectors), on a grid of sixteen workgroups per CU or more whose
+        // other rows are short: only the long rows get a team of waves - the longest at about eight blocks per
+        // wave - and every other row one wave of a workgroup that takes as many rows as it has waves.  No wave is
+        // launched without work (the launches above hand every row the team that only the long ones need, at
+        // 0.3 us per thousand waves that end at once), but a lone wave walks its row's blocks one after the other.
+        // Measured, N = 256, V = 8, 1 to 5 % of the rows between 1500 and 4608 vectors long among rows of 50 to 400:
+        // 2048 rows of 50 to 150 vectors 4-18 % faster, 4096 rows of 50 to 100 vectors 5-12 % faster while the
+        // long rows are 1 % or fewer; slower where the other rows are longer (200 to 300 vectors: 5-15 %), on
+        // 4096 rows with 5 % long ones (8 %) and on smaller grids (512 rows of 100: 6.2 -> 7.6 us; 1024 rows: the
+        // same within 3 %).  The other rows' mean length is bounded from what the hints say: every long row holds
+        // 513 vectors at least.
+        bool teams_pay = false;
+        if (skewed && batch.long_rows > 0 && batch.long_rows < m_vec && blocks >= 4096) {
+            const long long in_long = 513LL * batch.long_rows + (batch.longest_row_vec > 513 ? batch.longest_row_vec - 513 : 0);
+            const long long others = batch.nonzeros_vec > in_long ? batch.nonzeros_vec - in_long : 0;
+            const int others_mean = (int)(others / (m_vec - batch.long_rows));
+            const int others_blocks = ceil_div(ceil_div(others_mean, kStep), 2);
+            teams_pay = blocks < 8192 ? others_blocks <= 3 : (others_blocks <= 2 && 100LL * batch.long_rows <= m_vec);
+        }
+        if (batch.long_rows > 0 && options().spmm_teams != 1 && (teams_pay || options().spmm_teams == 2)) {
             team_slots = batch.long_rows < m_vec ? batch.long_rows : m_vec;
             per_wave = 1;
             if (in_flight == 4) in_flight = 2;

@@ -560,7 +560,7 @@ static int set_option_field(vs::Options &o, const char *name, int value)
         if (value != 0 && value != 4 && value != 8) return VS_ERROR_INVALID_VALUE;
         o.spmm_cols_per_lane = value;
     } else if (std::strcmp(name, "spmm_teams") == 0) {
-        if (value > 1) return VS_ERROR_INVALID_VALUE;
+        if (value > 2) return VS_ERROR_INVALID_VALUE;
         o.spmm_teams = value;
     } else if (std::strcmp(name, "spmm_guard_waves") == 0) {
         if (value > 16) return VS_ERROR_INVALID_VALUE;
