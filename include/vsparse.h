@@ -372,7 +372,8 @@ int vs_launch_floor_probe(int blocks, int threads_per_block, void *stream);
  * dense columns per lane (4 or 8: tiles of 64 or 128 columns), [1] 32-vector steps of gathered rows a wave keeps
  * in flight (1, 2, 4), [2] waves per workgroup (1..16), [3] blocks of a row a wave takes before another wave joins
  * in, [4] leading entries of row_indices served by a team of waves (-1: all rows), [5] 1 for the variant for dense
- * widths that are not a multiple of 4, [6] 1 for the LDS-DMA variant, [7] reserved (0).  Returns
+ * widths that are not a multiple of 4, [6] 1 for the LDS-DMA variant, [7] 1 when waves pipeline successive blocks of
+ * a row.  Returns
  * VS_ERROR_INVALID_VALUE for sizes the entry points reject.  No counterpart in the reference, whose launch shape
  * is fixed (src/wmma_spmm.cu:362-378: one warp per vector row and 64-column tile).
  */
@@ -393,7 +394,9 @@ int vs_wmma_spmm_launch_shape(int batch, int m_vec, int vec_length, int k, int n
  * (MFMA SpMM through the entry points that do not know the row lengths, on grids that fill the
  * chip by themselves: waves per workgroup kept for rows far longer than expected, 1 = none,
  * 0 = automatic), "spmm_teams" (vs_wmma_spmm_f16_batched_sorted: 1 = ignore the long-row count, 2 = use it on every
- * launch, 0 = where it measured faster),
+ * launch, 0 = where it measured faster), "spmm_pipe" (two steps in flight: 2 = a wave that takes several
+ * blocks of a row requests the next block behind each multiplication, 1 = after both, 0 = automatic; same
+ * bits either way),
  * "spmm_gather" (how the MFMA SpMM
  * brings the gathered rows of the dense operand to the matrix cores: 1 = through
  * registers and an in-register transpose, 2 = global -> LDS loads and transposing LDS

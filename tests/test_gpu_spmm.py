@@ -115,6 +115,16 @@ def test_steps_in_flight_variants_keep_parity(gpu, V, steps, cpl):
             assert_parity(got, ref, "steps=%d cpl=%d waves=%d N=%d" % (steps, cpl, waves, N))
             if got32 is not None:
                 assert_parity(got32, ref, "fp32 out, steps=%d cpl=%d waves=%d N=%d" % (steps, cpl, waves, N))
+            if steps == 2:
+                # the walk that pipelines successive blocks of a row and the plain one multiply and add in the same
+                # order: same bits
+                for pipe in (1, 2):
+                    with _lib.thread_options(spmm_steps=steps, spmm_cols_per_lane=cpl, spmm_waves=waves, spmm_pipe=pipe):
+                        other = _run(pat, B, "wmma")
+                    assert_parity(other, ref, "pipe=%d cpl=%d waves=%d N=%d" % (pipe, cpl, waves, N))
+                    if pipe == 1:
+                        plain = other
+                assert np.array_equal(plain, other), "pipelined and plain walks differ, cpl=%d waves=%d N=%d" % (cpl, waves, N)
 
 
 @pytest.mark.parametrize("kernel", ["wmma", "cuda"])
@@ -311,20 +321,21 @@ def test_skewed_rows_on_a_grid_that_fills_the_chip(gpu, V, m_vec, N):
     Bd = torch.from_numpy(B).cuda()
     for sort in (False, True):
         prob = ops.DeviceProblem(pat, sort=sort)
-        for guard in (0, 1, 2, 8):
-            with _lib.thread_options(spmm_guard_waves=guard):
+        for guard, pipe in [(0, 0), (1, 0), (2, 0), (8, 0), (0, 1), (0, 2), (2, 2), (8, 2)]:
+            with _lib.thread_options(spmm_guard_waves=guard, spmm_pipe=pipe):
                 plain = prob.spmm(Bd)
             torch.cuda.synchronize()
-            assert_parity(plain.cpu().numpy(), ref, "full grid, V%d N%d sort %d guard %d" % (V, N, sort, guard))
+            assert_parity(plain.cpu().numpy(), ref, "full grid, V%d N%d sort %d guard %d pipe %d" % (V, N, sort, guard, pipe))
         hinted = prob.spmm(Bd, row_length_hint=True)
         torch.cuda.synchronize()
         assert_parity(hinted.cpu().numpy(), ref, "full grid, hinted, V%d N%d sort %d" % (V, N, sort))
         # the long-row count of the sorted entry point is a hint: any count, in any order of the rows, gives the
         # same result (teams of waves for the first `long_rows` entries, one wave per row behind them)
         # (spmm_teams = 2: on every launch, not only where the library expects the team mapping to pay)
-        for teams, long_rows in [(2, x) for x in (0, 1, 5, 64, m_vec - 1, m_vec, m_vec + 9)] + [(0, 1), (0, 64)]:
+        for teams, long_rows, pipe in ([(2, x, 0) for x in (0, 1, 5, 64, m_vec - 1, m_vec, m_vec + 9)] +
+                                       [(0, 1, 0), (0, 64, 0), (2, 5, 1), (2, 5, 2), (2, m_vec, 2), (1, 5, 2)]):
             out = torch.full((1, pat.m, N), 3.0, dtype=torch.float16, device="cuda")
-            with _lib.thread_options(spmm_teams=teams):
+            with _lib.thread_options(spmm_teams=teams, spmm_pipe=pipe):
                 ops.spmm_batched(pat.m_vec, V, N, n, prob.row_indices, prob.row_offsets, prob.column_indices,
                                  prob.values, Bd, out, nonzeros_vec=pat.nnz_vec, longest_row_vec=n, long_rows=long_rows)
             torch.cuda.synchronize()

@@ -101,10 +101,18 @@ def test_spmm_launch_shape_choice():
     headline = shape(64, 8, 256, 4608)
     assert (headline["cols_per_lane"], headline["steps_in_flight"], headline["waves"]) == (4, 2, 8)
     assert headline["team_slots"] == -1 and not headline["ragged"] and not headline["dma"]
-    # largest sweep point: wide tiles (128-bit row segments); four steps in flight only with the row lengths known
-    assert shape(256, 8, 256, 4608)["cols_per_lane"] == 8
-    assert shape(256, 8, 256, 4608)["steps_in_flight"] == 2
-    assert shape(256, 8, 256, 4608, nonzeros_vec=256 * 461, longest_row_vec=470)["steps_in_flight"] == 4
+    # largest sweep point: wide tiles (128-bit row segments), two steps in flight and waves that pipeline the blocks
+    # they walk; four steps in flight only where that walk is switched off and the row lengths are known
+    largest = shape(256, 8, 256, 4608)
+    assert (largest["cols_per_lane"], largest["steps_in_flight"], largest["pipelined"]) == (8, 2, 1)
+    hinted = shape(256, 8, 256, 4608, nonzeros_vec=256 * 461, longest_row_vec=470)
+    assert (hinted["steps_in_flight"], hinted["pipelined"]) == (2, 1)
+    with _lib.thread_options(spmm_pipe=1):
+        assert shape(256, 8, 256, 4608, nonzeros_vec=256 * 461, longest_row_vec=470)["steps_in_flight"] == 4
+        assert shape(256, 8, 256, 4608)["pipelined"] == 0
+    # rows of one block, or a grid of 4096 workgroups without hints: the plain walk
+    assert shape(512, 8, 256, 4608, nonzeros_vec=512 * 60, longest_row_vec=64)["pipelined"] == 0
+    assert shape(2048, 8, 256, 4608)["pipelined"] == 0
     # one 64-column tile for narrow dense operands, the half-by-half variant for widths off a multiple of 4
     assert shape(512, 8, 64, 4096)["cols_per_lane"] == 4
     assert shape(64, 8, 147, 4608)["ragged"] == 1 and shape(64, 8, 148, 4608)["ragged"] == 0
@@ -154,6 +162,8 @@ def test_spmm_launch_shape_choice():
         assert -1 <= got["team_slots"] <= m_vec, case
         if got["team_slots"] >= 0:
             assert got["steps_in_flight"] == 2 and got["blocks_per_wave"] == 1, case
+        if got["pipelined"]:
+            assert got["steps_in_flight"] == 2 and not got["ragged"] and not got["dma"], case
         assert bool(got["ragged"]) == (k % 4 != 0), case
         if got["ragged"]:
             assert got["cols_per_lane"] == 4 and got["steps_in_flight"] == 1 and got["waves"] <= 8, case

@@ -67,6 +67,13 @@ def lib():
             raise ImportError(
                 "%s not found: build it with `python -m vectorsparse_amd.build` "
                 "(hipcc --offload-arch=gfx950)" % LIB_PATH)
+        # PyTorch ships a HIP runtime of its own.  Whichever copy a process loads first is the one that sees the
+        # GPU; a second copy loaded later reports "no ROCm-capable device".  The tensors this package works on are
+        # torch's, so torch goes first and the library binds to the runtime that is already there.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         L = ctypes.CDLL(LIB_PATH)
         for name, (argtypes, restype) in SIGNATURES.items():
             fn = getattr(L, name)

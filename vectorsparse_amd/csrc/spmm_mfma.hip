@@ -32,7 +32,12 @@ namespace vs {
 // row segments per lane are all requested before the first MFMA.
 // TEAMS: rows ordered by length; only the first team_slots entries of row_indices get the workgroup's waves as a
 // team, behind them every wave takes a row of its own (below).
-template <int V, int CPL, bool SOFTMAX, bool IDX32, typename OutT, bool RAGGED = false, int S = 1, bool TEAMS = false>
+// PIPE (S = 2): a wave that takes several blocks of a row one after the other requests each step of the next block
+// as soon as the same step of the current one is multiplied, so that it always has one or two steps in flight
+// instead of two while it waits and none while it multiplies; the next block's indices and vectors are requested a
+// block earlier for that, ahead of the current block's row segments (loads return in order).
+template <int V, int CPL, bool SOFTMAX, bool IDX32, typename OutT, bool RAGGED = false, int S = 1, bool TEAMS = false,
+          bool PIPE = false>
 __global__ void __launch_bounds__(S * CPL >= 32 ? 256 : (S * CPL >= 16 ? 512 : 1024))
 spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row_indices,
                  const int *__restrict__ row_offsets, const int *__restrict__ column_indices,
@@ -147,13 +152,12 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row
     const bool has_work = base < end;
     int next_idx[F];
     bool next_valid[F];
-    half_t next_vec[F][V];
+    PackedVector<V> next_vec[F];  // as loaded: the halves are taken apart when the block is staged
 #pragma unroll
     for (int i = 0; i < F; ++i) {
         next_idx[i] = 0;
         next_valid[i] = false;
-#pragma unroll
-        for (int v = 0; v < V; ++v) next_vec[i][v] = (half_t)0.f;
+        next_vec[i].clear();
     }
     auto fetch = [&](int b) {
 #pragma unroll
@@ -165,13 +169,13 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row
                 // in bounds and contributes nothing.
                 const int jc = next_valid[i] ? j : end - 1;
                 next_idx[i] = column_indices[jc];
-                load_vector<V>(next_vec[i], values + (size_t)jc * V);
+                next_vec[i].load(values + (size_t)jc * V);
             }
         }
     };
     if (has_work) fetch(base);
 
-    for (; has_work && base < end; base += stride) {
+    auto stage = [&]() {  // the fetched block into the wave's LDS slot
 #pragma unroll
         for (int i = 0; i < F; ++i) {
             const int at = 64 * i + lane;
@@ -179,10 +183,10 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row
                 idx_s[at] = next_idx[i];
 #pragma unroll
                 for (int v = 0; v < V; ++v) {
-                    half_t staged = next_valid[i] ? next_vec[i][v] : (half_t)0.f;
+                    half_t staged = next_valid[i] ? next_vec[i].at(v) : (half_t)0.f;
                     if constexpr (SOFTMAX) {
                         const float p =
-                            next_valid[i] ? __builtin_amdgcn_exp2f((float)next_vec[i][v] * s2 - row_max[v]) : 0.f;
+                            next_valid[i] ? __builtin_amdgcn_exp2f((float)next_vec[i].at(v) * s2 - row_max[v]) : 0.f;
                         row_sum[v] += p;
                         staged = (half_t)p;
                     }
@@ -191,26 +195,9 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row
             }
         }
         wave_lds_fence();
-        if constexpr (S == 1) {
-            spmm_mfma_step<V, CPL, IDX32, RAGGED>(idx_s, vec_s, rhs, n_cols, col_off, cs, g, acc, [&] {
-                if (base + stride < end) fetch(base + stride);
-            }, valid);
-        } else {
-            // A block that the row fills only in part still requests all its steps (the padding repeats one row
-            // segment, which stays in the L1): asking for fewer steps behind a uniform branch measured 5 % slower
-            // on short rows (the three code paths) and 4 % faster on long ones.
-            spmm_mfma_block<V, CPL, S, IDX32>(idx_s, vec_s, rhs, n_cols, col_off, cs, g, acc, [&] {
-                if (base + stride < end) fetch(base + stride);
-            });
-        }
-    }
-
-    if constexpr (SOFTMAX) {
-#pragma unroll
-        for (int v = 0; v < V; ++v) row_sum[v] = wave_sum(row_sum[v]);
-    }
-
-    if (active == 1) {
+    };
+    // the row's tile straight from the accumulators of the one wave that worked on it
+    auto store_alone = [&]() {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const int v = 4 * g + e;
@@ -231,6 +218,81 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row
                     store_converted<OutT, CPL>(out + ((size_t)row * V + v) * n_cols + col0, tmp);
             }
         }
+    };
+    if constexpr (PIPE) {
+        static_assert(S == 2 && IDX32 && !SOFTMAX && !RAGGED, "the pipelined walk exists for blocks of two steps");
+        // (expected: the compiler then lays the walk's code out behind the epilogue, out of the short row's way -
+        // the instruction cache starts every launch cold)
+        if (__builtin_expect(has_work && base + stride >= end, 1)) {  // a single block: nothing to overlap it with
+            stage();
+            spmm_mfma_block<V, CPL, S, IDX32>(idx_s, vec_s, rhs, n_cols, col_off, cs, g, acc, [] {});
+        } else if (has_work) {
+            StagedStep now[2], then[2];
+            RowChunk<CPL> first[8], second[8];
+            stage();
+            read_staged_step<V, kBlock>(now[0], idx_s, vec_s, 0, cs, g);
+            read_staged_step<V, kBlock>(now[1], idx_s, vec_s, 1, cs, g);
+            wave_lds_fence();
+            // (fetched whether or not the block exists - past the row's end the lanes re-read its last vector - so
+            // that the number of loads in flight is the same on every path and the waits below count exactly)
+            fetch(base + stride);  // ahead of the row segments below
+            __builtin_amdgcn_sched_barrier(0);
+            request_step<CPL>(first, now[0], rhs, n_cols, col_off);
+            request_step<CPL>(second, now[1], rhs, n_cols, col_off);
+            __builtin_amdgcn_sched_barrier(0);
+            for (;;) {
+                base += stride;
+                if (base >= end) break;
+                stage();  // waits for the indices and vectors only: they were requested before the segments
+                read_staged_step<V, kBlock>(then[0], idx_s, vec_s, 0, cs, g);
+                read_staged_step<V, kBlock>(then[1], idx_s, vec_s, 1, cs, g);
+                wave_lds_fence();
+                fetch(base + stride);
+                // (the scheduler otherwise waits for both steps, transposes both and only then requests the next
+                // two: the barriers keep each step's requests right behind its multiplication)
+                __builtin_amdgcn_sched_barrier(0);
+                multiply_step<CPL>(first, now[0].a, acc);
+                __builtin_amdgcn_sched_barrier(0);
+                request_step<CPL>(first, then[0], rhs, n_cols, col_off);
+                __builtin_amdgcn_sched_barrier(0);
+                multiply_step<CPL>(second, now[1].a, acc);
+                __builtin_amdgcn_sched_barrier(0);
+                request_step<CPL>(second, then[1], rhs, n_cols, col_off);
+                __builtin_amdgcn_sched_barrier(0);
+                now[0] = then[0];
+                now[1] = then[1];
+            }
+            multiply_step<CPL>(first, now[0].a, acc);
+            multiply_step<CPL>(second, now[1].a, acc);
+            // (a use of the last fetch on this path too: with uses only inside the loop the compiler moves the first
+            // fetch behind the loop test, i.e. behind the row segments, and every wait for it becomes a wait for them)
+#pragma unroll
+            for (int i = 0; i < F; ++i) asm volatile("" ::"v"(next_idx[i]), "v"(next_vec[i].first()));
+        }
+    }
+    for (; !PIPE && has_work && base < end; base += stride) {
+        stage();
+        if constexpr (S == 1) {
+            spmm_mfma_step<V, CPL, IDX32, RAGGED>(idx_s, vec_s, rhs, n_cols, col_off, cs, g, acc, [&] {
+                if (base + stride < end) fetch(base + stride);
+            }, valid);
+        } else {
+            // A block that the row fills only in part still requests all its steps (the padding repeats one row
+            // segment, which stays in the L1): asking for fewer steps behind a uniform branch measured 5 % slower
+            // on short rows (the three code paths) and 4 % faster on long ones.
+            spmm_mfma_block<V, CPL, S, IDX32>(idx_s, vec_s, rhs, n_cols, col_off, cs, g, acc, [&] {
+                if (base + stride < end) fetch(base + stride);
+            });
+        }
+    }
+
+    if constexpr (SOFTMAX) {
+#pragma unroll
+        for (int v = 0; v < V; ++v) row_sum[v] = wave_sum(row_sum[v]);
+    }
+
+    if (active == 1) {
+        store_alone();
         return;
     }
 
@@ -299,7 +361,7 @@ static int next_pow2(int x)
     return p;
 }
 
-template <int V, int CPL, bool SOFTMAX, bool IDX32, typename OutT, int S = 1, bool TEAMS = false>
+template <int V, int CPL, bool SOFTMAX, bool IDX32, typename OutT, int S = 1, bool TEAMS = false, bool PIPE = false>
 static int launch_idx(int m_vec, int k, int n, int waves, const int *row_indices, const int *row_offsets,
                       const int *column_indices, const half_t *values, const half_t *rhs, OutT *out,
                       hipStream_t stream, const Batch &batch, float scale, int per_wave = 1, int team_slots = -1)
@@ -315,7 +377,7 @@ static int launch_idx(int m_vec, int k, int n, int waves, const int *row_indices
     if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
     const size_t lds = (size_t)waves * S * stage_bytes<V>() +
                        (waves > 1 ? (size_t)waves * V * (TN + 1) * sizeof(float) : 0);
-    auto kernel = spmm_mfma_kernel<V, CPL, SOFTMAX, IDX32, OutT, false, S, TEAMS>;
+    auto kernel = spmm_mfma_kernel<V, CPL, SOFTMAX, IDX32, OutT, false, S, TEAMS, PIPE>;
     static std::atomic<unsigned long long> lds_allowed{0};
     const hipError_t attr = allow_large_lds(reinterpret_cast<const void *>(kernel), 96 * 1024, lds_allowed);
     if (attr != hipSuccess) return (int)attr;
@@ -348,7 +410,8 @@ static int launch_one(int m_vec, int k, int n, int waves, int in_flight, const i
                       const int *row_offsets, const int *column_indices, const half_t *values, const half_t *rhs,
                       OutT *out, hipStream_t stream, const Batch &batch, float scale, int team_slots)
 {
-    const int per_wave = in_flight >> 8;  // blocks a wave takes of one row, packed above the steps in flight
+    const int per_wave = (in_flight >> 8) & 255;  // blocks a wave takes of one row, packed above the steps in flight
+    const bool pipe = (in_flight >> 16) & 1;      // waves walk several blocks each: the pipelined walk
     in_flight &= 255;
     if ((long long)n * k < (1LL << 31)) {
         if constexpr (!SOFTMAX) {
@@ -357,11 +420,19 @@ static int launch_one(int m_vec, int k, int n, int waves, int in_flight, const i
                 return launch_idx<V, CPL, SOFTMAX, true, OutT, 4>(m_vec, k, n, waves, row_indices, row_offsets,
                                                                    column_indices, values, rhs, out, stream, batch, scale,
                                                                    per_wave);
+            if (in_flight >= 2 && team_slots >= 0 && pipe)
+                return launch_idx<V, CPL, SOFTMAX, true, OutT, 2, true, true>(m_vec, k, n, waves, row_indices, row_offsets,
+                                                                               column_indices, values, rhs, out, stream,
+                                                                               batch, scale, per_wave, team_slots);
             if (in_flight >= 2 && team_slots >= 0)
                 return launch_idx<V, CPL, SOFTMAX, true, OutT, 2, true>(m_vec, k, n, waves, row_indices, row_offsets,
                                                                          column_indices, values, rhs, out, stream, batch,
                                                                          scale, per_wave, team_slots);
             team_slots = -1;  // only the two-step variant has the team mapping
+            if (in_flight >= 2 && pipe)
+                return launch_idx<V, CPL, SOFTMAX, true, OutT, 2, false, true>(m_vec, k, n, waves, row_indices, row_offsets,
+                                                                                column_indices, values, rhs, out, stream,
+                                                                                batch, scale, per_wave, team_slots);
             if (in_flight >= 2)
                 return launch_idx<V, CPL, SOFTMAX, true, OutT, 2>(m_vec, k, n, waves, row_indices, row_offsets,
                                                                    column_indices, values, rhs, out, stream, batch, scale,
@@ -430,7 +501,9 @@ SpmmShape choose_spmm_shape(bool softmax, int m_vec, int k, int n, const Batch &
         in_flight = row_steps >= 2 ? 2 : 1;
         // (rows of unequal length end in half-empty blocks of 128: on log-normal and Pareto lengths four steps in
         // flight were 10-25 % behind two)
-        if (hinted && cpl == 8 && blocks >= 512 && mean_steps >= 8 && 2 * longest_steps <= 3 * mean_steps) in_flight = 4;
+        if (options().spmm_pipe == 1 && hinted && cpl == 8 && blocks >= 512 && mean_steps >= 8 &&
+            2 * longest_steps <= 3 * mean_steps)
+            in_flight = 4;  // (only without the pipelined walk, which is 5-15 % ahead of it on the same shapes)
     }
     if (!blocks_exist) in_flight = 1;
     int per_wave = 1;
@@ -552,6 +625,28 @@ SpmmShape choose_spmm_shape(bool softmax, int m_vec, int k, int n, const Batch &
     shape.waves = waves;
     shape.blocks_per_wave = per_wave;
     shape.team_slots = team_slots;
+    // The pipelined walk (two-step blocks): a wave that takes several blocks of a row one after the other requests
+    // the next block's segments step by step behind the multiplications instead of after them - 10-20 % on waves that
+    // walk many blocks where the launch is not at the gather ceiling anyway, at 26 more registers.  Measured over
+    // the ResNet-shaped grid (geometric means by grid size and row length, against the plain walk): with the row
+    // lengths known 2-4 % faster on rows of two to eight blocks and 7-14 % on longer ones from 512 workgroups on,
+    // the same within 1 % on rows of one block, 1-3 % slower only on rows of two blocks across 4096 workgroups;
+    // without hints 1.5-2.5 % faster up to 2048 workgroups (rows of 230 vectors and more on 2048 workgroups 6-12 %)
+    // and 2.5 % slower on 4096, where one guard wave walks each row at the gather ceiling.  1024 to 4096 Pareto
+    // rows: 4-11 % faster hinted, 12-19 % without hints.  It also outruns four steps in flight (5-15 % on the
+    // shapes that used to take them), which the automatic choice therefore no longer takes.
+    bool pipelined = false;
+    if (in_flight == 2 && blocks_exist && options().spmm_pipe != 1) {
+        if (options().spmm_pipe == 2) {
+            pipelined = true;
+        } else if (hinted) {
+            const int longest_blocks = ceil_div(row_steps, in_flight);
+            pipelined = longest_blocks >= 3 || (longest_blocks == 2 && blocks < 4096);
+        } else {
+            pipelined = blocks <= 2048;
+        }
+    }
+    shape.pipelined = pipelined;
     shape.ragged = ragged;
     shape.dma = use_dma && !ragged;
     return shape;
@@ -581,7 +676,7 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
             return launch_spmm_mfma_dma<OutT>(m_vec, vec_length, k, n, waves, row_indices, row_offsets, column_indices,
                                               values, rhs, out, stream, batch);
     }
-    const int packed = shape.steps_in_flight | (shape.blocks_per_wave << 8);
+    const int packed = shape.steps_in_flight | (shape.blocks_per_wave << 8) | (shape.pipelined ? 1 << 16 : 0);
     if (shape.cols_per_lane == 8)
         return launch_v<8, SOFTMAX, OutT>(vec_length, m_vec, k, n, waves, packed, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale, shape.team_slots);
     return launch_v<4, SOFTMAX, OutT>(vec_length, m_vec, k, n, waves, packed, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale, shape.team_slots);

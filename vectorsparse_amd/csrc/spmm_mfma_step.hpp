@@ -35,6 +35,25 @@ __device__ __forceinline__ void load_vector(half_t (&dst)[V], const half_t *p)
     }
 }
 
+// The same vector kept as loaded (one register per two halves) until its halves are needed.
+template <int V>
+struct PackedVector {
+    typedef half_t vec_t __attribute__((ext_vector_type(V)));
+    vec_t d;
+    __device__ __forceinline__ void load(const half_t *p) { d = *reinterpret_cast<const vec_t *>(p); }
+    __device__ __forceinline__ void clear() { d = vec_t(0); }
+    __device__ __forceinline__ half_t at(int v) const { return d[v]; }
+    __device__ __forceinline__ float first() const { return (float)d[0]; }
+};
+template <>
+struct PackedVector<1> {
+    half_t d;
+    __device__ __forceinline__ void load(const half_t *p) { d = p[0]; }
+    __device__ __forceinline__ void clear() { d = (half_t)0.f; }
+    __device__ __forceinline__ half_t at(int) const { return d; }
+    __device__ __forceinline__ float first() const { return (float)d; }
+};
+
 __device__ __forceinline__ void wave_lds_fence()
 {
     // LDS operations of one wave execute in order; this only stops the compiler from moving
@@ -183,6 +202,52 @@ __device__ __forceinline__ void spmm_mfma_block(const int *idx_s, const half_t *
             acc[2 * p] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[s], b_even, acc[2 * p], 0, 0, 0);
             acc[2 * p + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[s], b_odd, acc[2 * p + 1], 0, 0, 0);
         }
+    }
+}
+
+// The two halves of a step for a wave that keeps steps of successive blocks in flight: what a lane reads of a
+// staged step (its eight column indices and its slice of the transposed vectors), the requests for the eight row
+// segments, and - later, when they have returned - the transposition and the MFMAs.
+struct StagedStep {
+    int4_t i_lo, i_hi;
+    half8_t a;
+};
+
+template <int V, int PITCH>
+__device__ __forceinline__ void read_staged_step(StagedStep &st, const int *idx_s, const half_t *vec_s, int s, int cs, int g)
+{
+    st.i_lo = *reinterpret_cast<const int4_t *>(idx_s + s * kStep + 8 * g);
+    st.i_hi = *reinterpret_cast<const int4_t *>(idx_s + s * kStep + 8 * g + 4);
+    st.a = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    if (cs < V) st.a = *reinterpret_cast<const half8_t *>(vec_s + cs * PITCH + s * kStep + 8 * g);
+}
+
+template <int CPL>
+__device__ __forceinline__ void request_step(RowChunk<CPL> (&chunk)[8], const StagedStep &st, const half_t *rhs,
+                                             int n_cols, uint32_t col_off)
+{
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const int col = e < 4 ? st.i_lo[e] : st.i_hi[e - 4];
+        chunk[e].load(rhs + ((uint32_t)col * (uint32_t)n_cols + col_off));  // rhs has fewer than 2^31 elements
+    }
+}
+
+template <int CPL>
+__device__ __forceinline__ void multiply_step(const RowChunk<CPL> (&chunk)[8], const half8_t &a, float4_t (&acc)[CPL])
+{
+#pragma unroll
+    for (int p = 0; p < CPL / 2; ++p) {
+        uint4_t even, odd;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            even[q] = pack_lo(chunk[2 * q].dword(p), chunk[2 * q + 1].dword(p));
+            odd[q] = pack_hi(chunk[2 * q].dword(p), chunk[2 * q + 1].dword(p));
+        }
+        const half8_t b_even = __builtin_bit_cast(half8_t, even);
+        const half8_t b_odd = __builtin_bit_cast(half8_t, odd);
+        acc[2 * p] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b_even, acc[2 * p], 0, 0, 0);
+        acc[2 * p + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b_odd, acc[2 * p + 1], 0, 0, 0);
     }
 }
 

@@ -212,6 +212,7 @@ struct Options {
     int spmm_cols_per_lane = 0;
     int spmm_steps = 0;         // MFMA SpMM: 32-vector steps a wave keeps in flight (1, 2, 4), 0 = automatic
     int spmm_teams = 0;         // MFMA SpMM with the long-row count known: 1 = every row gets a team of waves, 2 = only the long rows do, 0 = automatic
+    int spmm_pipe = 0;          // MFMA SpMM, two steps in flight: 2 = waves pipeline successive blocks, 1 = never, 0 = automatic
     int spmm_guard_waves = 0;   // MFMA SpMM, row lengths unknown, full grid: waves per workgroup kept for rows longer than expected
     int spmm_gather = 0;        // 1 = gathered rows through registers, 2 = through LDS-DMA loads, 0 = automatic
     int spmm_flat_piece = 0;    // split-row SpMM: nonzero vectors per wave (rounded up to 32), 0 = automatic
@@ -266,6 +267,7 @@ struct SpmmShape {
     int waves = 1;             // waves per workgroup
     int blocks_per_wave = 1;   // blocks of a row a wave takes before another wave of the workgroup joins in
     int team_slots = -1;       // >= 0: only that many leading entries of row_indices get the workgroup as a team
+    bool pipelined = false;    // waves keep steps of successive blocks of a row in flight (two-step blocks only)
     bool ragged = false;       // dense width not a multiple of 4: the half-by-half variant
     bool dma = false;          // the variant that gathers through LDS-DMA loads (option spmm_gather = 2)
 };

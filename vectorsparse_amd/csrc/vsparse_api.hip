@@ -360,7 +360,7 @@ int vs_wmma_spmm_launch_shape(int batch, int m_vec, int vec_length, int k, int n
     shape[4] = chosen.team_slots;
     shape[5] = chosen.ragged ? 1 : 0;
     shape[6] = chosen.dma ? 1 : 0;
-    shape[7] = 0;
+    shape[7] = chosen.pipelined ? 1 : 0;
     return VS_SUCCESS;
 }
 
@@ -562,6 +562,9 @@ static int set_option_field(vs::Options &o, const char *name, int value)
     } else if (std::strcmp(name, "spmm_teams") == 0) {
         if (value > 2) return VS_ERROR_INVALID_VALUE;
         o.spmm_teams = value;
+    } else if (std::strcmp(name, "spmm_pipe") == 0) {
+        if (value > 2) return VS_ERROR_INVALID_VALUE;
+        o.spmm_pipe = value;
     } else if (std::strcmp(name, "spmm_guard_waves") == 0) {
         if (value > 16) return VS_ERROR_INVALID_VALUE;
         o.spmm_guard_waves = value;

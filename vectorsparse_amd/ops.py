@@ -108,7 +108,7 @@ def spmm_launch_shape(m_vec, vec_length, k, n, batch=1, nonzeros_vec=-1, longest
     _lib.check(_lib.lib().vs_wmma_spmm_launch_shape(batch, m_vec, vec_length, k, n, nonzeros_vec, longest_row_vec,
                                                     long_rows, ctypes.cast(shape, ctypes.c_void_p)),
                "vs_wmma_spmm_launch_shape")
-    names = ("cols_per_lane", "steps_in_flight", "waves", "blocks_per_wave", "team_slots", "ragged", "dma")
+    names = ("cols_per_lane", "steps_in_flight", "waves", "blocks_per_wave", "team_slots", "ragged", "dma", "pipelined")
     return dict(zip(names, (int(x) for x in shape)))
 
 
