@@ -110,9 +110,9 @@ def test_spmm_launch_shape_choice():
     with _lib.thread_options(spmm_pipe=1):
         assert shape(256, 8, 256, 4608, nonzeros_vec=256 * 461, longest_row_vec=470)["steps_in_flight"] == 4
         assert shape(256, 8, 256, 4608)["pipelined"] == 0
-    # rows of one block, or a grid of 4096 workgroups without hints: the plain walk
+    # rows known to hold one block: the plain walk
     assert shape(512, 8, 256, 4608, nonzeros_vec=512 * 60, longest_row_vec=64)["pipelined"] == 0
-    assert shape(2048, 8, 256, 4608)["pipelined"] == 0
+    assert shape(2048, 8, 256, 4608)["pipelined"] == 1
     # one 64-column tile for narrow dense operands, the half-by-half variant for widths off a multiple of 4
     assert shape(512, 8, 64, 4096)["cols_per_lane"] == 4
     assert shape(64, 8, 147, 4608)["ragged"] == 1 and shape(64, 8, 148, 4608)["ragged"] == 0

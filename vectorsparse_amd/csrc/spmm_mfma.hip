@@ -527,10 +527,12 @@ SpmmShape choose_spmm_shape(bool softmax, int m_vec, int k, int n, const Batch &
         // expected spreads over all of them instead of holding one wave for the whole launch (1024 Pareto rows x
         // 4608, N = 256: 39 -> 15 us with four waves, 23 us with two; one dense row among 1023 short ones 39 -> 14 us).
         // The waves a row does not need end after reading the row's extent, but hold a wave slot until then:
-        // 0.3 us per thousand of them (binomial rows, 1024 x 4608: 14.1 -> 16.0 us with four, 14.6 us with two), so
-        // grids beyond 2048 workgroups get two.
+        // 0.3-0.5 us per thousand of them.  Four waves against two, N = 256, K = 4608: on 2048 workgroups uniform rows
+        // 4-16 % slower and Pareto / log-normal / one dense row 18-43 % faster; on 4096 workgroups uniform rows 0-4 %
+        // slower, the skewed ones 8-39 % faster; on 8192 workgroups uniform rows up to 15 % slower and only the single
+        // dense row faster - so grids beyond 4096 workgroups get two.
         int guard = options().spmm_guard_waves;
-        if (guard <= 0) guard = blocks <= 2048 ? 4 : 2;
+        if (guard <= 0) guard = blocks <= 4096 ? 4 : 2;
         // A wave takes twice the blocks the estimate gives it before a second one joins (rows at half density
         // instead of the assumed quarter stay with one wave: two waves and their sum through LDS were 10-14 %
         // slower there), and matrices too narrow for a row of more than twelve blocks need no guard at all.
@@ -632,8 +634,8 @@ SpmmShape choose_spmm_shape(bool softmax, int m_vec, int k, int n, const Batch &
     // lengths known 2-4 % faster on rows of two to eight blocks and 7-14 % on longer ones from 512 workgroups on,
     // the same within 1 % on rows of one block, 1-3 % slower only on rows of two blocks across 4096 workgroups;
     // without hints 1.5-2.5 % faster up to 2048 workgroups (rows of 230 vectors and more on 2048 workgroups 6-12 %)
-    // and 2.5 % slower on 4096, where one guard wave walks each row at the gather ceiling.  1024 to 4096 Pareto
-    // rows: 4-11 % faster hinted, 12-19 % without hints.  It also outruns four steps in flight (5-15 % on the
+    // and 2.5 % slower on 4096, where one guard wave walks each row at the gather ceiling - taken there too, for the
+    // rows that the guard waves exist for: 1024 to 4096 Pareto rows are 4-11 % faster hinted, 12-19 % without hints.  It also outruns four steps in flight (5-15 % on the
     // shapes that used to take them), which the automatic choice therefore no longer takes.
     bool pipelined = false;
     if (in_flight == 2 && blocks_exist && options().spmm_pipe != 1) {
@@ -643,7 +645,7 @@ SpmmShape choose_spmm_shape(bool softmax, int m_vec, int k, int n, const Batch &
             const int longest_blocks = ceil_div(row_steps, in_flight);
             pipelined = longest_blocks >= 3 || (longest_blocks == 2 && blocks < 4096);
         } else {
-            pipelined = blocks <= 2048;
+            pipelined = true;  // (on 4096 workgroups: uniform rows 2.5 % slower, Pareto rows 12-19 % faster)
         }
     }
     shape.pipelined = pipelined;
