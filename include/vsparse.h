@@ -393,7 +393,8 @@ int vs_wmma_spmm_launch_shape(int batch, int m_vec, int vec_length, int k, int n
  * rows a wave of the MFMA SpMM keeps in flight: 1, 2, 4, 0 = automatic), "spmm_guard_waves"
  * (MFMA SpMM through the entry points that do not know the row lengths, on grids that fill the
  * chip by themselves: waves per workgroup kept for rows far longer than expected, 1 = none,
- * 0 = automatic), "spmm_teams" (vs_wmma_spmm_f16_batched_sorted: 1 = ignore the long-row count, 2 = use it on every
+ * 0 = automatic), "spmm_blocks_per_wave" (same launches: blocks of 64 vectors a wave takes of a row before the
+ * next kept wave joins in, a power of two up to 64, 0 = automatic), "spmm_teams" (vs_wmma_spmm_f16_batched_sorted: 1 = ignore the long-row count, 2 = use it on every
  * launch, 0 = where it measured faster), "spmm_pipe" (two steps in flight: 2 = a wave that takes several
  * blocks of a row requests the next block behind each multiplication, 1 = after both, 0 = automatic; same
  * bits either way),

@@ -533,12 +533,15 @@ SpmmShape choose_spmm_shape(bool softmax, int m_vec, int k, int n, const Batch &
         // dense row faster - so grids beyond 4096 workgroups get two.
         int guard = options().spmm_guard_waves;
         if (guard <= 0) guard = blocks <= 4096 ? 4 : 2;
-        // A wave takes twice the blocks the estimate gives it before a second one joins (rows at half density
-        // instead of the assumed quarter stay with one wave: two waves and their sum through LDS were 10-14 %
-        // slower there), and matrices too narrow for a row of more than twelve blocks need no guard at all.
+        // A wave takes half the blocks the estimate gives a row before a second one joins (four, for the eight the
+        // cap allows on a full chip): with pipelined walks a second wave pays from there, the idle ones cost more
+        // than the sum through LDS (N = 256, K = 4608, 1024 / 2048 rows; 2 / 4 / 8 / 16 blocks per wave: uniform rows at
+        // 90 % 14.2 / 14.6 / 15.4 / 15.4 and 25.9 / 26.4 / 26.4 / 26.2 us, log-normal 13.8 / 13.5 / 13.4 / 15.5 and 26.3 /
+        // 25.7 / 25.0 / 25.2, Pareto 14.9 / 14.8 / 14.5 / 15.1 and 19.1 / 19.0 / 18.5 / 19.8; 98 % and 50 % the same within
+        // 1 %).  Matrices too narrow for a row of more than twelve blocks need no guard at all.
         if (!hinted && want > room && guard > room && ceil_div(ceil_div(n, kStep), in_flight) > 12) {
             const int launched = want < guard ? want : guard;
-            per_wave = 2 * want / room;
+            per_wave = options().spmm_blocks_per_wave > 0 ? options().spmm_blocks_per_wave : (want >= 4 * room ? want / (2 * room) : 1);
             waves = launched;
         }
         // A few rows far longer than the mean (lengths known): the average row keeps to the waves the chip has room

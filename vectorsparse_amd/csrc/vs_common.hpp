@@ -213,6 +213,7 @@ struct Options {
     int spmm_steps = 0;         // MFMA SpMM: 32-vector steps a wave keeps in flight (1, 2, 4), 0 = automatic
     int spmm_teams = 0;         // MFMA SpMM with the long-row count known: 1 = every row gets a team of waves, 2 = only the long rows do, 0 = automatic
     int spmm_pipe = 0;          // MFMA SpMM, two steps in flight: 2 = waves pipeline successive blocks, 1 = never, 0 = automatic
+    int spmm_blocks_per_wave = 0;  // ... blocks of a row a wave takes before another of the kept waves joins in (power of two), 0 = automatic
     int spmm_guard_waves = 0;   // MFMA SpMM, row lengths unknown, full grid: waves per workgroup kept for rows longer than expected
     int spmm_gather = 0;        // 1 = gathered rows through registers, 2 = through LDS-DMA loads, 0 = automatic
     int spmm_flat_piece = 0;    // split-row SpMM: nonzero vectors per wave (rounded up to 32), 0 = automatic

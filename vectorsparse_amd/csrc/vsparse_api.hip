@@ -562,6 +562,9 @@ static int set_option_field(vs::Options &o, const char *name, int value)
     } else if (std::strcmp(name, "spmm_teams") == 0) {
         if (value > 2) return VS_ERROR_INVALID_VALUE;
         o.spmm_teams = value;
+    } else if (std::strcmp(name, "spmm_blocks_per_wave") == 0) {
+        if (value > 64 || (value & (value - 1)) != 0) return VS_ERROR_INVALID_VALUE;
+        o.spmm_blocks_per_wave = value;
     } else if (std::strcmp(name, "spmm_pipe") == 0) {
         if (value > 2) return VS_ERROR_INVALID_VALUE;
         o.spmm_pipe = value;
