@@ -64,17 +64,23 @@ def time_graph(torch, fn, steps, warmup, replays=7):
     graph.replay()  # untimed: first replay uploads the graph
     torch.cuda.synchronize()
     walls, events = [], []
+    # wall clock and device events in replays of their own: the two event records are packets of their own in the
+    # stream and cost a short graph 0.4 us per step of wall time (20 steps: 4.6 against 4.2 us)
+    for _ in range(max(1, replays)):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        graph.replay()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        walls.append((t1 - t0) * 1e3 / steps)
     for _ in range(max(1, replays)):
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
         e0.record()
         graph.replay()
         e1.record()
         torch.cuda.synchronize()
-        t1 = time.perf_counter()
-        walls.append((t1 - t0) * 1e3 / steps)
         events.append(e0.elapsed_time(e1) / steps)
     walls.sort()
     events.sort()
