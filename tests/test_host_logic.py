@@ -110,8 +110,8 @@ def test_spmm_launch_shape_choice():
     with _lib.thread_options(spmm_pipe=1):
         assert shape(256, 8, 256, 4608, nonzeros_vec=256 * 461, longest_row_vec=470)["steps_in_flight"] == 4
         assert shape(256, 8, 256, 4608)["pipelined"] == 0
-    # rows known to hold one block: the plain walk
-    assert shape(512, 8, 256, 4608, nonzeros_vec=512 * 60, longest_row_vec=64)["pipelined"] == 0
+    # rows known to hold one or two blocks on a grid of 4096 workgroups: the plain walk
+    assert shape(2048, 8, 256, 4608, nonzeros_vec=2048 * 60, longest_row_vec=100)["pipelined"] == 0
     assert shape(2048, 8, 256, 4608)["pipelined"] == 1
     # one 64-column tile for narrow dense operands, the half-by-half variant for widths off a multiple of 4
     assert shape(512, 8, 64, 4096)["cols_per_lane"] == 4

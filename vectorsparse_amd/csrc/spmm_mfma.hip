@@ -514,9 +514,11 @@ SpmmShape choose_spmm_shape(bool softmax, int m_vec, int k, int n, const Batch &
         // shorter row leaves without a block end at once.
         const int row_blocks = ceil_div(row_steps, in_flight);
         int want = row_blocks <= 1 ? 1 : next_pow2(row_blocks);
-        // Row lengths unknown: sixteen-wave workgroups cost 3.5 % on rows that fill eight waves or fewer (K = 4608
-        // at 90 % and up) and gain 5 % on rows that fill all sixteen (K = 4608 at 50 %), so eight is the limit.
-        if (!hinted && want > 8) want = 8;
+        // Eight waves at most: with pipelined walks eight waves that take two blocks and more each are ahead of
+        // sixteen with one each also where the rows are known to fill all sixteen (64 rows x 4608, N = 256, rows of
+        // 922 / 2304 vectors: 4.2 against 4.7 and 7.2 against 7.6 us), and sixteen-wave workgroups cost 3.5 % on rows
+        // that fill eight or fewer.  (The skewed launches below size theirs themselves.)
+        if (want > 8) want = 8;
         const int registers = in_flight * cpl;                                 // in flight per lane, of 32 bits / 2
         const int resident = (registers >= 32 ? 2 : registers >= 16 ? 3 : 5) * 1024;   // waves the chip holds at once
         int room = 1;
@@ -646,7 +648,7 @@ SpmmShape choose_spmm_shape(bool softmax, int m_vec, int k, int n, const Batch &
             pipelined = true;
         } else if (hinted) {
             const int longest_blocks = ceil_div(row_steps, in_flight);
-            pipelined = longest_blocks >= 3 || (longest_blocks == 2 && blocks < 4096);
+            pipelined = longest_blocks >= 3 || blocks < 4096;  // (its single-block path is the plain one)
         } else {
             pipelined = true;  // (on 4096 workgroups: uniform rows 2.5 % slower, Pareto rows 12-19 % faster)
         }
