@@ -44,6 +44,41 @@ def test_spmm_random(gpu, seed):
         assert_parity(prob.spmm(Bd, kernel="cuda").cpu().numpy(), ref, "cuda " + what)
 
 
+@pytest.mark.parametrize("seed", range(60))
+def test_spmm_random_launch_shapes(gpu, seed):
+    """Random patterns under random launch-shape overrides (waves, columns per lane, steps in flight, pipelined or
+    plain walk, guard waves, blocks per wave, team mapping) through the reference-shaped entry and through the
+    hinted batched one: every combination the options allow computes the same function."""
+    from vectorsparse_amd import _lib
+    rng = np.random.default_rng(5000 + seed)
+    V = int(rng.choice([1, 2, 4, 8]))
+    pat = _random_pattern(rng, V)
+    if seed % 3 == 0:   # long rows, so that waves walk several blocks
+        n = int(rng.integers(700, 3000))
+        lengths = np.minimum((rng.pareto(1.2, pat.m_vec) + 0.05) * n * 0.2, n).astype(np.int64)
+        ro, ci = cv._pattern_from_lengths(rng, pat.m_vec, n, lengths)
+        pat = cv.ColVecCSR(pat.m_vec, n, V, ro, ci).validate()
+    pat = cv.random_values(pat, seed=seed)
+    N = int(rng.choice([8, 64, 128, 136, 256, 264]))
+    B = cv.dense_uniform(pat.n, N, seed=seed + 1)
+    ref = co.spmm_host_ref_f32(pat.m_vec, V, N, pat.n, pat.row_offsets, pat.column_indices, pat.values, B)
+    Bd = torch.from_numpy(B).cuda()
+    prob = ops.DeviceProblem(pat, sort=bool(seed % 2))
+    for trial in range(4):
+        opts = dict(spmm_waves=int(rng.choice([0, 0, 1, 2, 3, 4, 8, 16])), spmm_cols_per_lane=int(rng.choice([0, 4, 8])),
+                    spmm_steps=int(rng.choice([0, 1, 2, 2, 4])), spmm_pipe=int(rng.choice([0, 1, 2, 2])),
+                    spmm_guard_waves=int(rng.choice([0, 1, 2, 4, 8])),
+                    spmm_blocks_per_wave=int(rng.choice([0, 1, 2, 8, 64])), spmm_teams=int(rng.choice([0, 1, 2])))
+        hint = bool(rng.integers(0, 2))
+        what = "seed %d trial %d V%d m_vec%d n%d N%d nnz_vec%d hint %d %s" % (seed, trial, V, pat.m_vec, pat.n, N,
+                                                                              pat.nnz_vec, hint, opts)
+        print(what, flush=True)
+        with _lib.thread_options(**opts):
+            got = prob.spmm(Bd, kernel="wmma", row_length_hint=hint)
+        torch.cuda.synchronize()
+        assert_parity(got.cpu().numpy(), ref, what)
+
+
 @pytest.mark.parametrize("seed", range(40))
 def test_sddmm_random(gpu, seed):
     rng = np.random.default_rng(2000 + seed)
