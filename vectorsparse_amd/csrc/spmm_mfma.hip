@@ -438,6 +438,12 @@ static int launch_one(int m_vec, int k, int n, int waves, int in_flight, const i
                                                                    column_indices, values, rhs, out, stream, batch, scale,
                                                                    per_wave, team_slots);
         }
+        if constexpr (SOFTMAX) {
+            if (in_flight >= 2)
+                return launch_idx<V, CPL, SOFTMAX, true, OutT, 2>(m_vec, k, n, waves, row_indices, row_offsets,
+                                                                   column_indices, values, rhs, out, stream, batch, scale,
+                                                                   per_wave);
+        }
         return launch_idx<V, CPL, SOFTMAX, true, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices,
                                                         values, rhs, out, stream, batch, scale);
     }
@@ -462,7 +468,7 @@ static int launch_v(int vec_length, int m_vec, int k, int n, int waves, int in_f
 
 // The launch shape of an MFMA SpMM, chosen on the host from what the entry point knows of the problem (the row
 // lengths only through the hints of the batched entry points) and from the calling thread's options.
-SpmmShape choose_spmm_shape(bool softmax, int m_vec, int k, int n, const Batch &batch)
+SpmmShape choose_spmm_shape(bool softmax, int m_vec, int vec_length, int k, int n, const Batch &batch)
 {
     SpmmShape shape;
     constexpr int kTargetBlocks = 256;   // one workgroup per CU at least
@@ -495,10 +501,16 @@ SpmmShape choose_spmm_shape(bool softmax, int m_vec, int k, int n, const Batch &
     // of the workgroup beyond four waves), while too few waves for denser rows cost 10-18 %.
     // while the chip has room the workgroup of the longest row ends last, so that row sets the size
     const int row_steps = longest_steps > mean_steps ? longest_steps : mean_steps;
-    const bool blocks_exist = !softmax && !ragged && !use_dma && (long long)n * k < (1LL << 31);
+    const bool blocks_exist = !ragged && !use_dma && (long long)n * k < (1LL << 31);
     int in_flight = options().spmm_steps;
     if (in_flight != 1 && in_flight != 2 && in_flight != 4) {
         in_flight = row_steps >= 2 ? 2 : 1;
+        // Many heads of a large mask with vectors of one or two rows (16384 workgroups and more, every one a single
+        // wave): such a launch is bound by its gather requests, and a row's last block of 64 is half padding on
+        // average - 16 requested slots per row that a walk in steps of 32 does not issue.  16 heads x 4096 rows, N = 64,
+        // V = 1: rows of 82 / 205 / 410 vectors 62.4 -> 50.0, 120.9 -> 109.8, 208.6 -> 201.1 us; V = 2, 205: 63.2 ->
+        // 58.5; V = 4 and 8 are the other way round (rows of 102, V = 4: 11.8 against 12.8 us).
+        if (hinted && vec_length <= 2 && blocks >= 16384 && mean_steps <= 16) in_flight = 1;
         // (rows of unequal length end in half-empty blocks of 128: on log-normal and Pareto lengths four steps in
         // flight were 10-25 % behind two)
         if (options().spmm_pipe == 1 && hinted && cpl == 8 && blocks >= 512 && mean_steps >= 8 &&
@@ -506,6 +518,11 @@ SpmmShape choose_spmm_shape(bool softmax, int m_vec, int k, int n, const Batch &
             in_flight = 4;  // (only without the pipelined walk, which is 5-15 % ahead of it on the same shapes)
     }
     if (!blocks_exist) in_flight = 1;
+    // The softmax-fused kernel has the two-step blocks only, and gains from them on rows of more than two blocks
+    // of vectors of four or eight (16 heads x 4096, d = 64: band + strided mask 37.2 -> 31.0 us, uniform 90 % 44.5 ->
+    // 39.2 us; rows of 82 vectors 15.8 -> 16.4 us, V = 1 at 95 % 114 -> 125 us).
+    if (softmax && in_flight == 4) in_flight = 2;
+    if (softmax && options().spmm_steps == 0 && (vec_length < 4 || row_steps <= 4)) in_flight = 1;
     int per_wave = 1;
     int team_slots = -1;
     int waves = options().spmm_waves;
@@ -643,7 +660,7 @@ SpmmShape choose_spmm_shape(bool softmax, int m_vec, int k, int n, const Batch &
     // rows that the guard waves exist for: 1024 to 4096 Pareto rows are 4-11 % faster hinted, 12-19 % without hints.  It also outruns four steps in flight (5-15 % on the
     // shapes that used to take them), which the automatic choice therefore no longer takes.
     bool pipelined = false;
-    if (in_flight == 2 && blocks_exist && options().spmm_pipe != 1) {
+    if (in_flight == 2 && blocks_exist && !softmax && options().spmm_pipe != 1) {
         if (options().spmm_pipe == 2) {
             pipelined = true;
         } else if (hinted) {
@@ -667,7 +684,7 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
     if (m_vec == 0 || k == 0 || batch.count == 0) return hipSuccess;
     if (batch.count > 65535) return hipErrorNotSupported;
     if (SOFTMAX && k % 4 != 0) return hipErrorNotSupported;
-    const SpmmShape shape = choose_spmm_shape(SOFTMAX, m_vec, k, n, batch);
+    const SpmmShape shape = choose_spmm_shape(SOFTMAX, m_vec, vec_length, k, n, batch);
     const int waves = shape.waves;
     if constexpr (!SOFTMAX) {
         if (shape.ragged) {

@@ -272,7 +272,7 @@ struct SpmmShape {
     bool ragged = false;       // dense width not a multiple of 4: the half-by-half variant
     bool dma = false;          // the variant that gathers through LDS-DMA loads (option spmm_gather = 2)
 };
-SpmmShape choose_spmm_shape(bool softmax, int m_vec, int k, int n, const Batch &batch);
+SpmmShape choose_spmm_shape(bool softmax, int m_vec, int vec_length, int k, int n, const Batch &batch);
 
 // Launchers (one per kernel family); return a hipError_t-valued int.
 template <typename OutT>

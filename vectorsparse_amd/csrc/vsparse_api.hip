@@ -352,7 +352,7 @@ int vs_wmma_spmm_launch_shape(int batch, int m_vec, int vec_length, int k, int n
     if (shape == nullptr || batch < 1 || batch > 65535 || m_vec < 1 || k < 1 || n < 0) return VS_ERROR_INVALID_VALUE;
     if (vec_length != 1 && vec_length != 2 && vec_length != 4 && vec_length != 8) return VS_ERROR_INVALID_VALUE;
     const vs::SpmmShape chosen = vs::choose_spmm_shape(
-        false, m_vec, k, n, make_batch(batch, 0, 0, 0, nonzeros_vec, longest_row_vec, long_rows < 0 ? -1 : long_rows));
+        false, m_vec, vec_length, k, n, make_batch(batch, 0, 0, 0, nonzeros_vec, longest_row_vec, long_rows < 0 ? -1 : long_rows));
     shape[0] = chosen.cols_per_lane;
     shape[1] = chosen.steps_in_flight;
     shape[2] = chosen.waves;
