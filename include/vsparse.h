@@ -31,6 +31,11 @@
  *     On a non-zero return no kernel was launched.
  *   - `row_indices[m_vec]` is the row swizzle: work item t processes vector
  *     row row_indices[t].  It must be a permutation of 0..m_vec-1.
+ *   - `row_offsets` is ascending from 0 and row_offsets[m_vec] = nnz_vec must not
+ *     exceed 2^31 - 65536: the kernels step past a row's end in 32-bit arithmetic
+ *     before they clamp the position.  Column indices lie in [0, n); they need not
+ *     be sorted within a row.  None of this is checked: the arrays are in device
+ *     memory, which the entry points do not read on the host.
  */
 #ifndef VSPARSE_H
 #define VSPARSE_H
