@@ -34,7 +34,8 @@
  *   - `row_offsets` is ascending from 0 and row_offsets[m_vec] = nnz_vec must not
  *     exceed 2^31 - 65536: the kernels step past a row's end in 32-bit arithmetic
  *     before they clamp the position.  Column indices lie in [0, n); they need not
- *     be sorted within a row.  None of this is checked: the arrays are in device
+ *     be sorted within a row (vs_sparse_attention_f16 takes a row's columns as a set:
+ *     distinct within the row).  None of this is checked: the arrays are in device
  *     memory, which the entry points do not read on the host.
  */
 #ifndef VSPARSE_H
