@@ -75,6 +75,26 @@ def test_both_paths_take_any_k(gpu, V, K):
     assert_parity(_run(pat, A, B, "wmma", out_dtype=torch.float32), ref, "wmma f32 out V%d K%d" % (V, K))
 
 
+@pytest.mark.parametrize("V", [1, 8])
+@pytest.mark.parametrize("kernel", ["wmma", "cuda"])
+def test_columns_in_any_order_within_a_row(gpu, V, kernel):
+    """Mask rows shuffled in place: outputs stay aligned with the CSR positions (include/bm_test_utils.h:171-193
+    takes the columns as they come)."""
+    rng = np.random.default_rng(80 + V)
+    lengths = np.array([0, 5, 64, 65, 300, 33, 17, 128], dtype=np.int64)
+    n = 320
+    ro, ci = cv._pattern_from_lengths(rng, len(lengths), n, lengths)
+    ci = ci.copy()
+    for i in range(len(lengths)):
+        rng.shuffle(ci[ro[i]:ro[i + 1]])
+    pat = cv.ColVecCSR(len(lengths), n, V, ro, ci)
+    A = cv.dense_normal(pat.m, 72, seed=81)
+    B = cv.dense_normal(n, 72, seed=82)
+    ref = _oracle(pat, A, B)
+    for algorithm in ((0, 1, 2) if kernel == "wmma" else (1,)):
+        assert_parity(_run(pat, A, B, kernel, algorithm=algorithm), ref, "shuffled columns V%d %s alg %d" % (V, kernel, algorithm))
+
+
 @pytest.mark.parametrize("V", [1, 2, 4, 8])
 @pytest.mark.parametrize("kernel", ["wmma", "cuda"])
 def test_ragged_and_empty_rows(gpu, V, kernel):

@@ -128,6 +128,23 @@ def test_steps_in_flight_variants_keep_parity(gpu, V, steps, cpl):
 
 
 @pytest.mark.parametrize("kernel", ["wmma", "cuda"])
+@pytest.mark.parametrize("V", [1, 8])
+def test_columns_in_any_order_within_a_row(gpu, kernel, V):
+    """The format does not promise ascending columns within a row (the reference's loops take them as they come,
+    spmm_benchmark.cpp:66-86): rows shuffled in place, long and short ones."""
+    rng = np.random.default_rng(70 + V)
+    lengths = np.array([0, 5, 64, 65, 700, 33, 1500, 128], dtype=np.int64)
+    n = 1600
+    ro, ci = cv._pattern_from_lengths(rng, len(lengths), n, lengths)
+    ci = ci.copy()
+    for i in range(len(lengths)):
+        rng.shuffle(ci[ro[i]:ro[i + 1]])
+    pat = cv.random_values(cv.ColVecCSR(len(lengths), n, V, ro, ci), seed=71)
+    B = cv.dense_uniform(n, 136, seed=72)
+    assert_parity(_run(pat, B, kernel), _oracle(pat, B), "shuffled columns V%d %s" % (V, kernel))
+
+
+@pytest.mark.parametrize("kernel", ["wmma", "cuda"])
 def test_all_rows_empty(gpu, kernel):
     pat = cv.ColVecCSR(8, 64, 8, np.zeros(9, np.int32), np.zeros(0, np.int32), np.zeros((0, 8), np.float16))
     B = cv.dense_uniform(64, 64, seed=1)
