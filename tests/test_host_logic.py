@@ -80,9 +80,10 @@ def test_device_problem_reads_the_row_statistics():
 def test_split_row_choice_follows_the_row_lengths():
     """The rule behind DeviceProblem.spmm(split_rows=None), on the row-length shapes it was measured on."""
     pays = ops.split_rows_pays
-    # one dense row among rows of a hundred vectors: pays at every row count
-    for m_vec in (64, 256, 1024, 2048):
+    # one dense row among rows of a hundred vectors: pays up to 1024 rows
+    for m_vec in (64, 256, 1024):
         assert pays(m_vec, 4608 + 100 * (m_vec - 1), 4608)
+    assert not pays(2048, 4608 + 100 * 2047, 4608)
     # uniform lengths: never
     for m_vec in (64, 1024):
         assert not pays(m_vec, 461 * m_vec, 461)

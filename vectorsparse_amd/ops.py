@@ -444,10 +444,11 @@ LONG_ROW_VECTORS = 512  # rows beyond this are "long" for vs_wmma_spmm_f16_batch
 def split_rows_pays(m_vec, nonzeros_vec, longest_row_vec):
     """Whether the split-row SpMM schedule is expected to beat the row-per-workgroup one with row-length hints.
     Measured at N = 256, V = 8, rows of up to 4608 vectors, 64 to 2048 vector rows: a row of 25 or more mean lengths
-    (one dense row among short ones) holds its workgroups for 11.2-13.4 us where the split schedule needs 9.8-11.8 us;
-    on milder skew (Pareto or log-normal lengths, longest row 6 to 18 mean lengths) the hinted schedule is ahead at
-    every size (1024 Pareto rows: 14.5 against 18.2 us), and on uniform or binomial lengths by 1.5 to 2.5 times."""
-    if m_vec <= 0 or nonzeros_vec < 8192:
+    (one dense row among rows of a hundred) holds its workgroups for 11.1-12.0 us on up to 1024 rows where the split
+    schedule needs 9.8-11.4 us; on 2048 rows the hinted schedule is ahead (12.5 against 14.9 us), as it is on milder
+    skew (Pareto or log-normal lengths, longest row 6 to 18 mean lengths: 1024 Pareto rows 13.4 against 16.9 us) and
+    on uniform or binomial lengths (by 1.6 to 2 times)."""
+    if m_vec <= 0 or m_vec > 1024 or nonzeros_vec < 8192:
         return False
     return longest_row_vec * m_vec >= 25.0 * nonzeros_vec
 
