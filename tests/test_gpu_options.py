@@ -102,9 +102,21 @@ def test_automatic_launch_shapes_are_close_to_the_best_on_the_headline_configs(g
     prob = ops.DeviceProblem(pat, sort=True)
     out = torch.empty((512, 256), dtype=torch.float16, device="cuda")
     auto, best = _best_of(lambda: prob.spmm(Bd, out=out),
-                          [dict(spmm_cols_per_lane=c, spmm_waves=w) for c in (4, 8) for w in (4, 8, 16)])
+                          [dict(spmm_cols_per_lane=c, spmm_waves=w, spmm_pipe=p) for c in (4, 8) for w in (4, 8, 16)
+                           for p in (1, 2)])
     print("config 2 SpMM: automatic %.2f us, best override %.2f us" % (auto, best))
     assert auto <= 1.10 * best
+
+    # the largest point of the sweep at the headline sparsity, reference-shaped and hinted entry
+    big = cv.random_values(cv.uniform_pattern(256, 4608, 0.9, seed=3, vec_length=8), seed=102)
+    bprob = ops.DeviceProblem(big)
+    bout = torch.empty((2048, 256), dtype=torch.float16, device="cuda")
+    for hint in (False, True):
+        auto, best = _best_of(lambda: bprob.spmm(Bd, out=bout, row_length_hint=hint),
+                              [dict(spmm_cols_per_lane=8, spmm_waves=w, spmm_steps=st, spmm_pipe=p)
+                               for w in (2, 4, 8) for st, p in ((2, 1), (2, 2), (4, 1))])
+        print("2048 x 4608 at 90 %%, hints %d: automatic %.2f us, best override %.2f us" % (hint, auto, best))
+        assert auto <= 1.10 * best
 
     for K, s in ((64, 0.9), (128, 0.9), (64, 0.95), (128, 0.95)):
         mask = cv.uniform_pattern(256, 2048, s, seed=4, vec_length=8)
