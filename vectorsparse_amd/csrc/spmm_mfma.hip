@@ -405,63 +405,45 @@ static int launch_ragged(int m_vec, int k, int waves, const int *row_indices, co
     return (int)hipGetLastError();
 }
 
+// The kernel variant a launch shape names (blocks of several steps exist for offsets that fit 32 bits only).
 template <int V, int CPL, bool SOFTMAX, typename OutT>
-static int launch_one(int m_vec, int k, int n, int waves, int in_flight, const int *row_indices,
-                      const int *row_offsets, const int *column_indices, const half_t *values, const half_t *rhs,
-                      OutT *out, hipStream_t stream, const Batch &batch, float scale, int team_slots)
+static int launch_one(const SpmmShape &shape, int m_vec, int k, int n, const int *row_indices, const int *row_offsets,
+                      const int *column_indices, const half_t *values, const half_t *rhs, OutT *out,
+                      hipStream_t stream, const Batch &batch, float scale)
 {
-    const int per_wave = (in_flight >> 8) & 255;  // blocks a wave takes of one row, packed above the steps in flight
-    const bool pipe = (in_flight >> 16) & 1;      // waves walk several blocks each: the pipelined walk
-    in_flight &= 255;
-    if ((long long)n * k < (1LL << 31)) {
-        if constexpr (!SOFTMAX) {
-            // blocks of several steps in flight exist for the common case only: offsets that fit 32 bits
-            if (in_flight == 4)
-                return launch_idx<V, CPL, SOFTMAX, true, OutT, 4>(m_vec, k, n, waves, row_indices, row_offsets,
-                                                                   column_indices, values, rhs, out, stream, batch, scale,
-                                                                   per_wave);
-            if (in_flight >= 2 && team_slots >= 0 && pipe)
-                return launch_idx<V, CPL, SOFTMAX, true, OutT, 2, true, true>(m_vec, k, n, waves, row_indices, row_offsets,
-                                                                               column_indices, values, rhs, out, stream,
-                                                                               batch, scale, per_wave, team_slots);
-            if (in_flight >= 2 && team_slots >= 0)
-                return launch_idx<V, CPL, SOFTMAX, true, OutT, 2, true>(m_vec, k, n, waves, row_indices, row_offsets,
-                                                                         column_indices, values, rhs, out, stream, batch,
-                                                                         scale, per_wave, team_slots);
-            team_slots = -1;  // only the two-step variant has the team mapping
-            if (in_flight >= 2 && pipe)
-                return launch_idx<V, CPL, SOFTMAX, true, OutT, 2, false, true>(m_vec, k, n, waves, row_indices, row_offsets,
-                                                                                column_indices, values, rhs, out, stream,
-                                                                                batch, scale, per_wave, team_slots);
-            if (in_flight >= 2)
-                return launch_idx<V, CPL, SOFTMAX, true, OutT, 2>(m_vec, k, n, waves, row_indices, row_offsets,
-                                                                   column_indices, values, rhs, out, stream, batch, scale,
-                                                                   per_wave, team_slots);
+    const int waves = shape.waves;
+    const int per_wave = shape.blocks_per_wave;
+#define VS_SPMM_VARIANT(...)                                                                                          \
+    launch_idx<V, CPL, SOFTMAX, __VA_ARGS__>(m_vec, k, n, waves, row_indices, row_offsets, column_indices, values, rhs, \
+                                             out, stream, batch, scale,
+    if ((long long)n * k >= (1LL << 31)) return VS_SPMM_VARIANT(false, OutT) 1, -1);
+    if constexpr (SOFTMAX) {
+        if (shape.steps_in_flight >= 2) return VS_SPMM_VARIANT(true, OutT, 2) per_wave, -1);
+    } else {
+        if (shape.steps_in_flight == 4) return VS_SPMM_VARIANT(true, OutT, 4) per_wave, -1);
+        if (shape.steps_in_flight >= 2) {
+            // (only the two-step variants have the team mapping and the pipelined walk)
+            if (shape.team_slots >= 0)
+                return shape.pipelined ? VS_SPMM_VARIANT(true, OutT, 2, true, true) per_wave, shape.team_slots)
+                                       : VS_SPMM_VARIANT(true, OutT, 2, true, false) per_wave, shape.team_slots);
+            return shape.pipelined ? VS_SPMM_VARIANT(true, OutT, 2, false, true) per_wave, -1)
+                                   : VS_SPMM_VARIANT(true, OutT, 2, false, false) per_wave, -1);
         }
-        if constexpr (SOFTMAX) {
-            if (in_flight >= 2)
-                return launch_idx<V, CPL, SOFTMAX, true, OutT, 2>(m_vec, k, n, waves, row_indices, row_offsets,
-                                                                   column_indices, values, rhs, out, stream, batch, scale,
-                                                                   per_wave);
-        }
-        return launch_idx<V, CPL, SOFTMAX, true, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices,
-                                                        values, rhs, out, stream, batch, scale);
     }
-    return launch_idx<V, CPL, SOFTMAX, false, OutT>(m_vec, k, n, waves, row_indices, row_offsets, column_indices,
-                                                     values, rhs, out, stream, batch, scale);
+    return VS_SPMM_VARIANT(true, OutT) 1, -1);
+#undef VS_SPMM_VARIANT
 }
 
 template <int CPL, bool SOFTMAX, typename OutT>
-static int launch_v(int vec_length, int m_vec, int k, int n, int waves, int in_flight, const int *row_indices,
-                    const int *row_offsets, const int *column_indices, const half_t *values,
-                    const half_t *rhs, OutT *out, hipStream_t stream, const Batch &batch,
-                    float scale, int team_slots)
+static int launch_v(const SpmmShape &shape, int vec_length, int m_vec, int k, int n, const int *row_indices,
+                    const int *row_offsets, const int *column_indices, const half_t *values, const half_t *rhs,
+                    OutT *out, hipStream_t stream, const Batch &batch, float scale)
 {
     switch (vec_length) {
-    case 1: return launch_one<1, CPL, SOFTMAX, OutT>(m_vec, k, n, waves, in_flight, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale, team_slots);
-    case 2: return launch_one<2, CPL, SOFTMAX, OutT>(m_vec, k, n, waves, in_flight, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale, team_slots);
-    case 4: return launch_one<4, CPL, SOFTMAX, OutT>(m_vec, k, n, waves, in_flight, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale, team_slots);
-    case 8: return launch_one<8, CPL, SOFTMAX, OutT>(m_vec, k, n, waves, in_flight, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale, team_slots);
+    case 1: return launch_one<1, CPL, SOFTMAX, OutT>(shape, m_vec, k, n, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
+    case 2: return launch_one<2, CPL, SOFTMAX, OutT>(shape, m_vec, k, n, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
+    case 4: return launch_one<4, CPL, SOFTMAX, OutT>(shape, m_vec, k, n, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
+    case 8: return launch_one<8, CPL, SOFTMAX, OutT>(shape, m_vec, k, n, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
     default: return hipErrorInvalidValue;
     }
 }
@@ -700,10 +682,9 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
             return launch_spmm_mfma_dma<OutT>(m_vec, vec_length, k, n, waves, row_indices, row_offsets, column_indices,
                                               values, rhs, out, stream, batch);
     }
-    const int packed = shape.steps_in_flight | (shape.blocks_per_wave << 8) | (shape.pipelined ? 1 << 16 : 0);
     if (shape.cols_per_lane == 8)
-        return launch_v<8, SOFTMAX, OutT>(vec_length, m_vec, k, n, waves, packed, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale, shape.team_slots);
-    return launch_v<4, SOFTMAX, OutT>(vec_length, m_vec, k, n, waves, packed, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale, shape.team_slots);
+        return launch_v<8, SOFTMAX, OutT>(shape, vec_length, m_vec, k, n, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
+    return launch_v<4, SOFTMAX, OutT>(shape, vec_length, m_vec, k, n, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);
 }
 
 template <typename OutT>
