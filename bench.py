@@ -376,6 +376,9 @@ def main():
     _, sddmm_ms = time_graph(torch, sddmm_step, args.steps, args.warmup)
     sddmm_flops = 2.0 * mask.nnz * 64
     sddmm_bytes = sddmm_algorithmic_bytes(mask, 64)
+    # the fine-grained paths (cudaSpmm / cudaSddmm of the reference) on the same two workloads
+    _, valu_spmm_ms = time_graph(torch, lambda: prob.spmm(Bd, kernel="cuda", out=out), args.steps, args.warmup)
+    _, valu_sddmm_ms = time_graph(torch, lambda: sprob.sddmm(lhs, rhs, kernel="cuda", out=sout), args.steps, args.warmup)
     full = torch.empty((2048, 2048), dtype=torch.float16, device="cuda")
     _, sddmm_dense_ms = time_graph(torch, lambda: torch.matmul(lhs, rhs.t(), out=full), args.steps, args.warmup)
 
@@ -477,6 +480,12 @@ def main():
                 hbm(sddmm_bytes, sddmm_ms, sddmm_traffic, traffic_note=sddmm_note, kernel="sddmm_mfma_kernel<V=8>"),
                 ms=sddmm_ms, tflops=sddmm_flops / (sddmm_ms * 1e-3) * 1e-12, dense_product_us=sddmm_dense_ms * 1e3,
                 speedup_vs_dense=sddmm_dense_ms / sddmm_ms),
+            "fine_grained_paths": {
+                "spmm_config2": dict(hbm(alg_bytes, valu_spmm_ms, kernel="spmm_valu_kernel<V=8>"),
+                                     tflops=flops / (valu_spmm_ms * 1e-3) * 1e-12, speedup_vs_dense_gemm=dense_ms / valu_spmm_ms),
+                "sddmm_config4_k64": dict(hbm(sddmm_bytes, valu_sddmm_ms, kernel="sddmm_valu_kernel<V=8>"),
+                                          tflops=sddmm_flops / (valu_sddmm_ms * 1e-3) * 1e-12,
+                                          speedup_vs_dense=sddmm_dense_ms / valu_sddmm_ms)},
             "attention_window513": {"layer_ms": window_ms, "density": 1.0 - wmask.sparsity,
                                     "tflops": 2.0 * wmask.nnz * heads * dim * 2 / (window_ms * 1e-3) * 1e-12},
             "attention_config5": {"layer_ms": attn_ms, "density": 1.0 - amask.sparsity,
