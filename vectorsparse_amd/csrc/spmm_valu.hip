@@ -88,8 +88,10 @@ spmm_valu_kernel(int n_cols, int n_tiles, int n_waves, const int *__restrict__ r
 #pragma unroll
         for (int c = 0; c < 8; ++c) acc[v][c] = 0.f;
 
-    // (fetching the next turn's column indices and values while the gathered rows of the current one are in flight
-    // costs 18 to 40 registers and measured 2-6 % slower over the ResNet-shaped grid)
+    // (fetching the next turn's column indices and values a turn ahead costs 18 to 40 registers and measured 2-6 %
+    // slower over the ResNet-shaped grid when requested behind the gathered rows of the current turn, 3-5 % slower
+    // when requested ahead of them: with up to sixteen waves per workgroup the two round trips of a turn hide behind
+    // other waves)
     for (int j0 = beg + (wave * G + g) * U; j0 < end; j0 += n_waves * G * U) {
         int col[U];
         uint32_t a[U][V > 1 ? V / 2 : 1];  // the vector's halves, two per word (V = 1: one half in the low bits)
