@@ -9,6 +9,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <chrono>
 #include <cstdio>
 #include <cstdlib>
 #include <random>
@@ -161,6 +162,24 @@ int main()
                                           d_rhs_s, d_sd_h, V, stream, 3) != hipSuccess;
     std::printf("%-22s %s\n", "unsupported overloads", rejects ? "rejected: ok" : "FAILED");
     ok &= rejects;
+
+    // how fast a plain C++ loop issues the operator (the reference's benchmark is such a loop, spmm_benchmark.cpp:127):
+    // calls back to back on one stream, no HIP graph; printed for information
+    {
+        const int calls = 2000;
+        for (int i = 0; i < 50; ++i)
+            HIP_OK(spmm::wmmaSpmm(m_vec, V, k_dense, n, d_row_indices, d_row_offsets, d_cols, d_values, d_rhs, d_out_h));
+        HIP_OK(hipDeviceSynchronize());
+        const auto t0 = std::chrono::steady_clock::now();
+        for (int i = 0; i < calls; ++i)
+            HIP_OK(spmm::wmmaSpmm(m_vec, V, k_dense, n, d_row_indices, d_row_offsets, d_cols, d_values, d_rhs, d_out_h));
+        const auto t1 = std::chrono::steady_clock::now();
+        HIP_OK(hipDeviceSynchronize());
+        const auto t2 = std::chrono::steady_clock::now();
+        std::printf("%-22s %.2f us per call to issue, %.2f us per call until the last one has finished (%d calls)\n",
+                    "spmm::wmmaSpmm loop", std::chrono::duration<double, std::micro>(t1 - t0).count() / calls,
+                    std::chrono::duration<double, std::micro>(t2 - t0).count() / calls, calls);
+    }
 
     HIP_OK(hipStreamDestroy(stream));
     for (void *p : {(void *)d_row_indices, (void *)d_row_offsets, (void *)d_cols, (void *)d_values, (void *)d_rhs,
