@@ -79,7 +79,7 @@ def build_cxx_caller(verbose=False):
 
 def build_probes(verbose=False):
     """Compile csrc/probes/machine_probe.hip (launch floor, dependent-load latency, gather ceiling of the GPU) to
-    vectorsparse_amd/probes/machine_probe; run it on a GPU box to get the floors DESIGN.md prices the kernels by."""
+    vectorsparse_amd/probes/machine_probe; run it on an MI355X to get the floors that the kernels' timings are judged against."""
     out_dir = os.path.join(_HERE, "probes")
     os.makedirs(out_dir, exist_ok=True)
     exe = os.path.join(out_dir, "machine_probe")
