@@ -86,7 +86,9 @@ int vs_wmma_spmm_f16_f32out(int m_vec, int vec_length, int k, int n,
  * nonzeros_vec must equal row_offsets[m_vec] (the host cannot read it from device memory).
  * workspace: device memory, 16-byte aligned, workspace_bytes long, owned by the caller, ZERO-FILLED before its
  * first use: it starts with arrival counters that every call finds at zero and leaves at zero (so no call
- * spends a launch on clearing them); the rest is undefined before and after.  Not shared between calls that may
+ * spends a launch on clearing them); the rest is undefined before and after.  The counters' area (1/128 of the
+ * workspace) depends on workspace_bytes alone, so one workspace serves problems of different shapes one after
+ * the other as long as it is always passed with the same size.  Not shared between calls that may
  * overlap.  (Option "spmm_flat_launches" = 2 adds the parts in a second launch instead and uses no counters.)  vs_wmma_spmm_workspace_bytes() returns the
  * size that lets the library pick its preferred run length (0 when one workgroup takes everything); a smaller
  * workspace - even none - is accepted and makes the runs longer (fewer waves, same results up to the
@@ -112,11 +114,11 @@ int vs_wmma_spmm_f16_f32out_ws(int m_vec, int vec_length, int k, int n, int nonz
  * runs on until the process ends.  The call allocates and frees nothing.  It has no counterpart in the
  * reference.  Same results, bit for bit, as vs_wmma_spmm_f16_ws with a workspace of that size.
  * Size limit: vec_length * (k rounded up to a multiple of 128) <= 32768 (the array must hold the partial tiles
- * of 64 pieces); beyond it the call returns 801 (hipErrorNotSupported) and launches nothing.
+ * of some sixty pieces beside its counters); beyond it the call returns 801 (hipErrorNotSupported) and launches nothing.
  * Every call on a GPU shares that GPU's array: calls that may overlap on one GPU (different streams, different
  * threads) race on it and must be serialised by the caller.  Nothing in the array has to be cleared between
- * calls: it starts zeroed, every call leaves its arrival counters at zero, and every partial tile that is read
- * was written by the same call.
+ * calls, whatever their shapes: it starts zeroed, the arrival counters have a fixed area of their own that every
+ * call leaves at zero, and every partial tile that is read was written by the same call.
  */
 long long vs_wmma_spmm_noalloc_scratch_bytes(void);
 int vs_wmma_spmm_f16_noalloc(int m_vec, int vec_length, int k, int n, int nonzeros_vec,

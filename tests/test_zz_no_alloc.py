@@ -1,7 +1,7 @@
 """`vs_wmma_spmm_f16_noalloc`: the split-row SpMM with its workspace in a static device array of the library.
 Through the C ABI, against `vs_wmma_spmm_f16_ws` with a caller workspace of the same size (bit for bit) and
-against the CPU oracle; two calls in a row, the second on a smaller problem, so that whatever the first call left
-in the array must not leak into the second."""
+against the CPU oracle; calls in a row on problems of different shapes - a smaller one, then larger ones with more
+arrival counters than any call before - so that whatever a call left in the array must not leak into the next."""
 import numpy as np
 import pytest
 import torch
@@ -34,8 +34,11 @@ def test_two_calls_in_a_row_match_the_workspace_entry_point(gpu):
     scratch = L.vs_wmma_spmm_noalloc_scratch_bytes()
     assert scratch == 16 << 20
     workspace = torch.zeros(scratch, dtype=torch.uint8, device="cuda")
-    # the first problem splits many rows across pieces; the second is smaller in every dimension
-    for (m_vec, n, V, N, seed, longest) in ((512, 4096, 8, 256, 1, 4096), (96, 1024, 8, 128, 2, 1000)):
+    # the first problem splits many rows across pieces; the second is smaller in every dimension; the third and
+    # fourth have more pieces and other tile shapes than any before them (their arrival counters lie where an
+    # earlier call's would have put partial tiles, if the layout followed the problem instead of the array)
+    for (m_vec, n, V, N, seed, longest) in ((512, 4096, 8, 256, 1, 4096), (96, 1024, 8, 128, 2, 1000),
+                                            (1024, 4608, 8, 256, 5, 4608), (2048, 2048, 2, 64, 6, 2048)):
         pat, B = _problem(m_vec, n, V, N, seed, longest)
         ro, ci, vals, Bd = _device(pat, B)
         assert L.vs_wmma_spmm_workspace_bytes(m_vec, V, N, n, pat.nnz_vec) > 0, "the case must use the scratch"
