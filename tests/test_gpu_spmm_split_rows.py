@@ -19,7 +19,7 @@ def _oracle(pat, B):
                                 pat.column_indices, pat.values, B)
 
 
-def _run(pat, B, out_dtype=torch.float16, workspace="auto", piece=0, waves=0, launches=0, shared=0, pipe=0):
+def _run(pat, B, out_dtype=torch.float16, workspace="auto", piece=0, waves=0, launches=0, shared=0):
     """One call with canaries round the output and round the workspace; returns the host copy of the output."""
     prob = ops.DeviceProblem(pat)
     Bd = torch.from_numpy(B).cuda()
@@ -32,7 +32,6 @@ def _run(pat, B, out_dtype=torch.float16, workspace="auto", piece=0, waves=0, la
         _lib.set_option("spmm_flat_waves", waves)
         _lib.set_option("spmm_flat_launches", launches)
         _lib.set_option("spmm_flat_shared", shared)
-        _lib.set_option("spmm_flat_pipe", pipe)
         need = ops.spmm_workspace_bytes(pat.m_vec, pat.vec_length, k, pat.n, pat.nnz_vec)
         ws_bytes = need if workspace == "auto" else int(workspace)
         guard = 4096
@@ -50,7 +49,6 @@ def _run(pat, B, out_dtype=torch.float16, workspace="auto", piece=0, waves=0, la
         _lib.set_option("spmm_flat_waves", 0)
         _lib.set_option("spmm_flat_launches", 0)
         _lib.set_option("spmm_flat_shared", 0)
-        _lib.set_option("spmm_flat_pipe", 0)
     host = buf.cpu().numpy()
     assert np.all(host[:pad] == 12345.0) and np.all(host[pad + pat.m:] == 12345.0), "wrote outside the output"
     wsh = ws_buf.cpu().numpy()
@@ -71,17 +69,16 @@ def _from_lengths(lengths, n, V, seed):
 @pytest.mark.parametrize("piece", [0, 32, 64, 96, 512])
 @pytest.mark.parametrize("waves", [0, 1, 3])
 @pytest.mark.parametrize("launches", [1, 2])
-@pytest.mark.parametrize("walk", ["one step in flight", "two steps in flight", "rows share steps"])
-def test_ragged_empty_and_long_rows(gpu, V, piece, waves, launches, walk):
+@pytest.mark.parametrize("shared", [1, 2])
+def test_ragged_empty_and_long_rows(gpu, V, piece, waves, launches, shared):
     # empty rows at the start, in the middle and at the end; rows of every tail length; rows that span many runs
     # and pieces; a row that starts exactly on a run boundary (the 64 in front of it ends nonzero 128)
     lengths = [0, 0, 1, 15, 16, 17, 0, 31, 33, 14, 0, 64, 65, 300, 2, 0, 128, 7, 640, 1, 0, 0]
     pat = _from_lengths(lengths, 640, V, seed=5)
     B = cv.dense_uniform(640, 192, seed=7)
-    shared, pipe = {"one step in flight": (1, 1), "two steps in flight": (1, 2), "rows share steps": (2, 0)}[walk]
-    got = _run(pat, B, piece=piece, waves=waves, launches=launches, shared=shared, pipe=pipe)
+    got = _run(pat, B, piece=piece, waves=waves, launches=launches, shared=shared)
     assert_parity(got, _oracle(pat, B),
-                  "split rows V%d run %d waves %d launches %d, %s" % (V, piece, waves, launches, walk))
+                  "split rows V%d run %d waves %d launches %d shared %d" % (V, piece, waves, launches, shared))
     for i in np.nonzero(np.asarray(lengths) == 0)[0]:
         assert not got[i * V:(i + 1) * V].any(), "empty vector row %d must be written as zeros" % i
 
@@ -93,15 +90,13 @@ def test_all_rows_empty_and_single_row(gpu):
     assert got.shape == (64, 64) and not got.any()
     one = _from_lengths([2048], 2048, 8, seed=3)   # one dense row: every piece holds a segment of it
     B = cv.dense_uniform(2048, 128, seed=4)
-    for waves in (1, 4, 16):   # sixteen waves: the walk with two steps in flight has no such variant
-        for pipe in (1, 2):
-            assert_parity(_run(one, B, piece=64, waves=waves, pipe=pipe), _oracle(one, B),
-                          "single dense row, %d waves, pipe %d" % (waves, pipe))
+    for waves in (1, 4, 16):
+        assert_parity(_run(one, B, piece=64, waves=waves), _oracle(one, B), "single dense row, %d waves" % waves)
 
 
 @pytest.mark.parametrize("V", [1, 2, 4, 8])
-@pytest.mark.parametrize("shared,pipe", [(1, 1), (1, 2), (2, 0)])
-def test_many_short_rows_share_steps(gpu, V, shared, pipe):
+@pytest.mark.parametrize("shared", [1, 2])
+def test_many_short_rows_share_steps(gpu, V, shared):
     """Rows of 0 to 40 vectors, more than sixty of them empty in a row (the offsets window of a wave moves on
     several times inside one step), then long rows again: with shared steps up to 16 / V rows meet in one MFMA."""
     rng = np.random.default_rng(70 + V)
@@ -111,8 +106,8 @@ def test_many_short_rows_share_steps(gpu, V, shared, pipe):
     B = cv.dense_uniform(1024, 136, seed=72)
     ref = _oracle(pat, B)
     for piece, waves in ((0, 0), (32, 2), (160, 5)):
-        got = _run(pat, B, piece=piece, waves=waves, shared=shared, pipe=pipe)
-        assert_parity(got, ref, "short rows V%d run %d waves %d shared %d pipe %d" % (V, piece, waves, shared, pipe))
+        got = _run(pat, B, piece=piece, waves=waves, shared=shared)
+        assert_parity(got, ref, "short rows V%d run %d waves %d shared %d" % (V, piece, waves, shared))
         for i in np.nonzero(lengths == 0)[0]:
             assert not got[i * V:(i + 1) * V].any(), "empty vector row %d must be written as zeros" % i
 
@@ -133,9 +128,6 @@ def test_pareto_rows_with_a_dense_row(gpu, V):
     assert np.array_equal(a.view(np.uint16), b.view(np.uint16)), "two runs differ"
     c = _run(pat, B, launches=2)
     assert np.array_equal(a.view(np.uint16), c.view(np.uint16)), "one launch and two launches add in the same order"
-    for piece in (0, 96):   # one and two steps in flight along the walk add in the same order
-        d, e = _run(pat, B, piece=piece, shared=1, pipe=1), _run(pat, B, piece=piece, shared=1, pipe=2)
-        assert np.array_equal(d.view(np.uint16), e.view(np.uint16)), "one and two steps in flight differ"
     assert_parity(_run(pat, B, out_dtype=torch.float32), ref, "pareto rows, fp32 out")
 
 
@@ -153,8 +145,7 @@ def test_dense_width_edges(gpu):
     pat = _from_lengths([5, 700, 0, 40, 333, 64], 768, 8, seed=9)
     for N in (4, 8, 24, 64, 72, 136, 512, 1000):
         B = cv.dense_uniform(768, N, seed=N)
-        for pipe in (1, 2):
-            assert_parity(_run(pat, B, piece=64, waves=2, pipe=pipe), _oracle(pat, B), "N=%d pipe %d" % (N, pipe))
+        assert_parity(_run(pat, B, piece=64, waves=2), _oracle(pat, B), "N=%d" % N)
 
 
 def test_device_problem_switch_and_bad_arguments(gpu):

@@ -157,11 +157,8 @@ __device__ __forceinline__ void tile_to_output(OutT *out, int row, int n_cols, i
 // operand holds every row's values in its own group of rows and zeros elsewhere, and a row's group is written out
 // (or parked, for a row that started before the run) and cleared after the step in which the row ends.  A run
 // then takes sub / 32 steps however short its rows are; without it every row segment starts a step of its own.
-// PIPED: the walk keeps two steps in flight - the rows of the step after the one at hand are requested before its
-// multiplication, whatever rows the two belong to - at twice the registers for gathered rows, so a workgroup has
-// eight waves at most.  Same additions in the same order as the plain walk: same bits.
-template <int V, int CPL, bool IDX32, bool ONE_LAUNCH, typename OutT, bool SHARED = false, bool PIPED = false>
-__global__ void __launch_bounds__(PIPED ? 512 : 1024)
+template <int V, int CPL, bool IDX32, bool ONE_LAUNCH, typename OutT, bool SHARED = false>
+__global__ void __launch_bounds__(1024)
 spmm_mfma_flat_kernel(int m_vec, int n_cols, int n_tiles, int nonzeros_vec, int sub, int main_blocks, int *counters,
                       const int *__restrict__ row_offsets, const int *__restrict__ column_indices,
                       const half_t *__restrict__ values, const half_t *__restrict__ rhs, OutT *__restrict__ out,
@@ -212,170 +209,6 @@ spmm_mfma_flat_kernel(int m_vec, int n_cols, int n_tiles, int nonzeros_vec, int 
     int t_row = 0, t_row_end = 0, f_row = 0, f_row_beg = 0, f_row_end = 0;
     int t_pos = 0;        // SHARED: the group of accumulator rows that holds the row that goes on
 
-    if constexpr (PIPED) {
-        static_assert(IDX32 && !SHARED, "the pipelined walk exists for 32-bit offsets and a step per row segment");
-        if (sb_ll < nonzeros_vec) {
-            const int sb = (int)sb_ll;
-            const int se = sb + sub < nonzeros_vec ? sb + sub : nonzeros_vec;
-            int next_idx = 0;
-            PackedVector<V> next_vec;
-            next_vec.clear();
-            // always made, and clamped: a request that may or may not have been made would make every wait behind
-            // it count for the worse case.  (Only the lanes with a slot take part: the branch round the others
-            // also keeps the request in front of the multiplication, where a branch-free one was moved behind it.)
-            auto fetch = [&](int pos) {
-                if (lane < kStep) {
-                    const int j = pos + lane < nonzeros_vec ? pos + lane : nonzeros_vec - 1;
-                    next_idx = column_indices[j];
-                    next_vec.load(values + (size_t)j * V);
-                }
-            };
-            fetch(sb);
-            int base_row, ri;
-            int offs = find_row_window(row_offsets, m_vec, sb, lane, base_row, ri);
-
-            // The steps of the run in order: a step is up to 32 nonzeros of one row segment; the segments follow
-            // each other without gaps, so the step after one starts where it ends whatever its row is.  `kind`:
-            // what becomes of the accumulators after the step - 0 the segment goes on, 1 a whole row has been
-            // added up (output), 2 the row started in an earlier run (its part goes to F[wave]), 3 the row goes on
-            // past the run (it stays: the run's last step).  A step past the run's end is an empty one (count 0).
-            struct Step {
-                int count, kind, row;
-            };
-            bool rows_left = true;
-            int seg_pos = sb, seg_end = sb, seg_row = 0, seg_kind = 0;
-            auto advance = [&](Step &d) -> bool {
-                d.count = 0;
-                d.kind = 0;
-                d.row = 0;
-                while (seg_pos >= seg_end) {
-                    if (!rows_left) return false;
-                    if (ri == 63) {
-                        base_row += 63;
-                        ri = 0;
-                        offs = row_offsets[base_row + lane <= m_vec ? base_row + lane : m_vec];
-                        // waited for here, once in 63 rows, and not where the two paths meet again, for every row
-                        asm volatile("" : "+v"(offs));
-                    }
-                    const int row = base_row + ri;
-                    const int row_beg = __builtin_amdgcn_readlane(offs, ri);
-                    const int row_end = __builtin_amdgcn_readlane(offs, ri + 1);
-                    // rows that start at or after the run's end belong to later runs; past the last row nothing
-                    // of the pattern is left (also when nonzeros_vec exceeds row_offsets[m_vec])
-                    if (row >= m_vec || row_beg >= se) {
-                        rows_left = false;
-                        return false;
-                    }
-                    ++ri;
-                    if (row_end == row_beg) continue;  // empty: its zeros are written elsewhere
-                    seg_row = row;
-                    seg_pos = row_beg > sb ? row_beg : sb;
-                    seg_end = row_end < se ? row_end : se;
-                    if (row_beg < sb) {  // at most one such row in a run: the first
-                        seg_kind = 2;
-                        has_f = true;
-                        f_row = row;
-                        f_row_beg = row_beg;
-                        f_row_end = row_end;
-                    } else if (row_end <= se) {
-                        seg_kind = 1;
-                    } else {  // at most one: the last
-                        seg_kind = 3;
-                        has_t = true;
-                        t_row = row;
-                        t_row_end = row_end;
-                    }
-                }
-                d.count = seg_end - seg_pos < kStep ? seg_end - seg_pos : kStep;
-                d.row = seg_row;
-                seg_pos += d.count;
-                d.kind = seg_pos < seg_end ? 0 : seg_kind;
-                return true;
-            };
-            // slots >= count repeat the step's last column (in bounds, one the pattern really has) with a zero
-            // value; an empty step is all such slots
-            auto stage = [&](const Step &d) {
-                const int last_idx = __builtin_amdgcn_readlane(next_idx, d.count > 0 ? d.count - 1 : 0);
-                if (lane < kStep) {
-                    const bool valid = lane < d.count;
-                    idx_s[lane] = valid ? next_idx : last_idx;
-#pragma unroll
-                    for (int v = 0; v < V; ++v) vec_s[v * kStep + lane] = valid ? next_vec.at(v) : (half_t)0.f;
-                }
-                wave_lds_fence();
-            };
-            auto retire = [&](const Step &d) {
-                if (d.kind == 1)
-                    tile_to_output<V, CPL, OutT>(out, d.row, n_cols, col0, col_ok, g, acc);
-                else if (d.kind == 2)
-                    tile_store<V, CPL>(f_mine, TN, cs, g, acc);
-                if (d.kind == 1 || d.kind == 2) {
-#pragma unroll
-                    for (int q = 0; q < CPL; ++q) acc[q] = float4_t{0.f, 0.f, 0.f, 0.f};
-                }
-            };
-
-            // Two steps in flight.  Each half of the loop's body stages the step after the next (its LDS round trip
-            // runs under the multiplication), multiplies the step whose rows have arrived and requests the staged
-            // one into the registers that has freed.  The step staged past the run's end is an empty one whose
-            // rows nobody uses; the loop has one way out, at the end of its body.  Both because requests that
-            // may or may not have been made make every wait behind them count for the worse case - and ways out
-            // in the middle of a loop are merged into a common block in front of its back edge.
-            Step cur_a, cur_b, nxt;
-            StagedStep staged;
-            half8_t values_a, values_b;
-            RowChunk<CPL> rows_a[8], rows_b[8];
-            if (advance(cur_a)) {
-                stage(cur_a);
-                read_staged_step<V, kStep>(staged, idx_s, vec_s, 0, cs, g);
-                wave_lds_fence();
-                values_a = staged.a;
-                fetch(seg_pos);
-                __builtin_amdgcn_sched_barrier(0);
-                request_step<CPL>(rows_a, staged, rhs, n_cols, col_off);
-                __builtin_amdgcn_sched_barrier(0);
-                advance(cur_b);
-                stage(cur_b);
-                read_staged_step<V, kStep>(staged, idx_s, vec_s, 0, cs, g);
-                wave_lds_fence();
-                values_b = staged.a;
-                fetch(seg_pos);
-                __builtin_amdgcn_sched_barrier(0);
-                request_step<CPL>(rows_b, staged, rhs, n_cols, col_off);
-                __builtin_amdgcn_sched_barrier(0);
-                bool more = true;
-                while (more) {
-                    more = advance(nxt);
-                    stage(nxt);
-                    read_staged_step<V, kStep>(staged, idx_s, vec_s, 0, cs, g);
-                    wave_lds_fence();
-                    fetch(seg_pos);
-                    __builtin_amdgcn_sched_barrier(0);
-                    multiply_step<CPL>(rows_a, values_a, acc);
-                    __builtin_amdgcn_sched_barrier(0);
-                    retire(cur_a);
-                    request_step<CPL>(rows_a, staged, rhs, n_cols, col_off);
-                    __builtin_amdgcn_sched_barrier(0);
-                    cur_a = nxt;
-                    values_a = staged.a;
-
-                    advance(nxt);
-                    stage(nxt);
-                    read_staged_step<V, kStep>(staged, idx_s, vec_s, 0, cs, g);
-                    wave_lds_fence();
-                    fetch(seg_pos);
-                    __builtin_amdgcn_sched_barrier(0);
-                    multiply_step<CPL>(rows_b, values_b, acc);
-                    __builtin_amdgcn_sched_barrier(0);
-                    retire(cur_b);
-                    request_step<CPL>(rows_b, staged, rhs, n_cols, col_off);
-                    __builtin_amdgcn_sched_barrier(0);
-                    cur_b = nxt;
-                    values_b = staged.a;
-                }
-            }
-        }
-    } else
     if (sb_ll < nonzeros_vec) {
         const int sb = (int)sb_ll;
         const int se = sb + sub < nonzeros_vec ? sb + sub : nonzeros_vec;
@@ -688,7 +521,6 @@ inline long long flat_workspace_for(long long tile_bytes)
 struct FlatShape {
     bool one_launch;  // cross-workgroup parts added inside the launch (arrival counters) instead of by a second one
     bool shared;      // steps shared by consecutive rows
-    bool piped;       // two steps in flight along the walk (a step per row segment, eight waves at most)
     int cpl;       // columns per lane (tile of 16*cpl dense columns)
     int waves;     // runs (= waves) per piece (= workgroup)
     int sub;       // nonzero vectors per run
@@ -717,7 +549,6 @@ bool flat_shape(int vec_length, int k, int nonzeros_vec, long long workspace_byt
     s.waves = o.spmm_flat_waves > 0 ? o.spmm_flat_waves : 8;
     s.one_launch = o.spmm_flat_launches != 2;  // (and the tile area below 2 GiB: 32-bit buffer offsets, see below)
     s.shared = o.spmm_flat_shared == 2;  // the launcher turns it on for short rows, which it knows the count of
-    s.piped = o.spmm_flat_pipe == 2;     // (where the kernel has the variant: see launch_flat_idx)
     long long sub = o.spmm_flat_piece > 0 ? o.spmm_flat_piece : ((long long)nonzeros_vec * n_tiles + 3583) / 3584;
     sub = (sub + kStep - 1) / kStep * kStep;
     if (o.spmm_flat_piece <= 0) {
@@ -745,7 +576,7 @@ bool flat_shape(int vec_length, int k, int nonzeros_vec, long long workspace_byt
     }
 }
 
-template <int V, int CPL, bool IDX32, bool ONE_LAUNCH, typename OutT, bool SHARED = false, bool PIPED = false>
+template <int V, int CPL, bool IDX32, bool ONE_LAUNCH, typename OutT, bool SHARED = false>
 int launch_flat_kernel(int m_vec, int k, int nonzeros_vec, const FlatShape &s, const int *row_offsets,
                        const int *column_indices, const half_t *values, const half_t *rhs, OutT *out, float *workspace,
                        hipStream_t stream)
@@ -758,7 +589,7 @@ int launch_flat_kernel(int m_vec, int k, int nonzeros_vec, const FlatShape &s, c
     float *tiles = reinterpret_cast<float *>(reinterpret_cast<unsigned char *>(workspace) +
                                              (s.n_pieces > 1 ? s.counter_bytes : 0));
     const size_t lds = (size_t)s.waves * (stage_bytes<V>() + (size_t)V * 16 * CPL * sizeof(float));
-    auto kernel = spmm_mfma_flat_kernel<V, CPL, IDX32, ONE_LAUNCH, OutT, SHARED, PIPED>;
+    auto kernel = spmm_mfma_flat_kernel<V, CPL, IDX32, ONE_LAUNCH, OutT, SHARED>;
     static std::atomic<unsigned long long> lds_allowed{0};
     const hipError_t attr = allow_large_lds(reinterpret_cast<const void *>(kernel), 96 * 1024, lds_allowed);
     if (attr != hipSuccess) return (int)attr;
@@ -786,15 +617,6 @@ int launch_flat_idx(int m_vec, int k, int nonzeros_vec, const FlatShape &s, cons
         if (s.shared)
             return launch_flat_kernel<V, CPL, IDX32, false, OutT, true>(m_vec, k, nonzeros_vec, s, row_offsets,
                                                                         column_indices, values, rhs, out, ws, stream);
-    }
-    if constexpr (IDX32) {
-        if (s.piped && s.waves <= 8) {
-            if (s.one_launch)
-                return launch_flat_kernel<V, CPL, IDX32, true, OutT, false, true>(m_vec, k, nonzeros_vec, s, row_offsets,
-                                                                                  column_indices, values, rhs, out, ws, stream);
-            return launch_flat_kernel<V, CPL, IDX32, false, OutT, false, true>(m_vec, k, nonzeros_vec, s, row_offsets,
-                                                                               column_indices, values, rhs, out, ws, stream);
-        }
     }
     if (s.one_launch)
         return launch_flat_kernel<V, CPL, IDX32, true, OutT>(m_vec, k, nonzeros_vec, s, row_offsets, column_indices, values,

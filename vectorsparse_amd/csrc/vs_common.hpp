@@ -219,7 +219,6 @@ struct Options {
     int spmm_flat_piece = 0;    // split-row SpMM: nonzero vectors per wave (rounded up to 32), 0 = automatic
     int spmm_flat_launches = 0; // split-row SpMM: 1 = parts added inside the launch, 2 = by a second launch, 0 = automatic
     int spmm_flat_waves = 0;    // split-row SpMM: waves per workgroup, 0 = automatic
-    int spmm_flat_pipe = 0;     // split-row SpMM: 2 = two steps in flight along the walk where the kernel has the variant, 1 or 0 = one
     int spmm_flat_shared = 0;   // split-row SpMM: 1 = every row segment starts its own step, 2 = rows share steps, 0 = automatic
     int sddmm_slots = 0;
     int sddmm_block_waves = 0;

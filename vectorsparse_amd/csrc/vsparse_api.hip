@@ -582,9 +582,6 @@ static int set_option_field(vs::Options &o, const char *name, int value)
     } else if (std::strcmp(name, "spmm_flat_launches") == 0) {
         if (value > 2) return VS_ERROR_INVALID_VALUE;
         o.spmm_flat_launches = value;
-    } else if (std::strcmp(name, "spmm_flat_pipe") == 0) {
-        if (value > 2) return VS_ERROR_INVALID_VALUE;
-        o.spmm_flat_pipe = value;
     } else if (std::strcmp(name, "spmm_flat_shared") == 0) {
         if (value > 2) return VS_ERROR_INVALID_VALUE;
         o.spmm_flat_shared = value;
