@@ -244,6 +244,40 @@ int vs_wmma_spmm_f16_batched_sorted(int batch, int m_vec, int vec_length, int k,
                                     long long stride_values, const void *rhs_matrix, long long stride_rhs,
                                     void *output_matrix, long long stride_output, void *stream);
 
+/*
+ * Rows in parts: the row swizzle of the reference (SortedRowSwizzle, include/bm_test_utils.h:200-215, which
+ * reorders the dispatch of whole rows) taken one step further - a row far longer than the rest is dispatched as
+ * several parts, each to a workgroup of its own, so that no workgroup is left walking one row when the rest of
+ * the launch has finished.  No counterpart in the reference.
+ *
+ * vs_spmm_row_parts (HOST function on HOST arrays, like the swizzles): the dispatch list of a pattern.  Rows of more
+ * than limit_vec nonzero vectors (0 = the library's default, 512; rounded up to a multiple of 64) are cut into
+ * equal parts of whole 64-vector blocks, at most 255 per row; every other row, the empty ones included, is a
+ * slot of its own; the slots are ordered longest first.  slots: four ints per slot {vector row, first nonzero,
+ * end, part info (0 = a whole row)}, room for max_slots of them.  Returns the number of slots, of split rows, the
+ * most parts any row has and the longest slot through the pointers; VS_ERROR_NOT_SUPPORTED with the counts set
+ * when max_slots is too small (m_vec + nonzeros_vec / 64 + 1 slots always suffice for the default limit) or more
+ * than 32767 rows would be split.
+ *
+ * vs_wmma_spmm_f16_row_parts: the operator of vs_wmma_spmm_f16 (same operands, same contract for the output)
+ * driven by that list, copied to DEVICE memory (16-byte aligned), in place of row_indices and row_offsets.
+ * nonzeros_vec and longest_part_vec size the launch as the hints of vs_wmma_spmm_f16_batched do.  The parts of
+ * a split row leave fp32 partial tiles in `workspace` and the workgroup that brings the last one adds them in
+ * ascending order (deterministic, no atomics on the output, nobody waits).  workspace: device memory, 16-byte
+ * aligned, at least vs_wmma_spmm_row_parts_workspace_bytes(vec_length, k, n_split, parts_max) bytes (0 when no
+ * row is split), ZERO-FILLED before its first use; its arrival counters (an area that depends on
+ * workspace_bytes alone) are left at zero by every call, so it serves any sequence of calls that do not
+ * overlap, whatever their shapes, as long as it is passed with the same size.  Requires k % 4 == 0 and
+ * n * k < 2^31, else 801.
+ */
+int vs_spmm_row_parts(int m_vec, const int *row_offsets, int limit_vec, int *slots, int max_slots, int *n_slots,
+                      int *n_split, int *parts_max, int *longest_part_vec);
+long long vs_wmma_spmm_row_parts_workspace_bytes(int vec_length, int k, int n_split, int parts_max);
+int vs_wmma_spmm_f16_row_parts(int vec_length, int k, int n, int n_slots, const int *slots, int n_split,
+                               int parts_max, int nonzeros_vec, int longest_part_vec,
+                               const int *column_indices, const void *values, const void *rhs_matrix,
+                               void *output_matrix, void *workspace, long long workspace_bytes, void *stream);
+
 int vs_cuda_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
                              int longest_row_vec, const int *row_indices, const int *row_offsets,
                              const int *column_indices,

@@ -1,0 +1,173 @@
+"""SpMM with long rows dispatched in parts (`vs_spmm_row_parts` + `vs_wmma_spmm_f16_row_parts`): the list names
+parts of rows, each served by a workgroup of its own; the parts of a split row meet as fp32 partial tiles in a
+workspace and the workgroup that arrives last adds them up.  Same contract as the reference-shaped entry point
+(tests/util.py), checked against the CPU oracle through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle as co
+from vectorsparse_amd import _lib, ops
+from vectorsparse_amd import colvec_csr as cv
+from util import assert_parity
+
+pytestmark = pytest.mark.gpu
+
+
+def _oracle(pat, B):
+    return co.spmm_host_ref_f32(pat.m_vec, pat.vec_length, B.shape[1], pat.n, pat.row_offsets,
+                                pat.column_indices, pat.values, B)
+
+
+def _from_lengths(lengths, n, V, seed):
+    rng = np.random.default_rng(seed)
+    lengths = np.asarray(lengths, dtype=np.int64)
+    ro, ci = cv._pattern_from_lengths(rng, len(lengths), n, lengths)
+    return cv.random_values(cv.ColVecCSR(len(lengths), n, V, ro, ci).validate(), seed=seed + 1)
+
+
+def _run(pat, B, limit=0, calls=2, options=None):
+    """`calls` calls in a row on one workspace, canaries round the output and the workspace; the host copy of the
+    output and the dispatch list."""
+    parts = ops.RowParts(pat.m_vec, pat.row_offsets, limit)
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    slots, ci, vals, Bd = d(parts.slots), d(pat.column_indices), d(pat.values), d(B)
+    k = B.shape[1]
+    pad = 64
+    buf = torch.full((pat.m + 2 * pad, k), 12345.0, dtype=torch.float16, device="cuda")
+    out = buf[pad:pad + pat.m]
+    need = ops.spmm_row_parts_workspace_bytes(pat.vec_length, k, parts.n_split, parts.parts_max)
+    assert (need > 0) == (parts.n_split > 0)
+    guard = 4096
+    ws_buf = torch.full((need + 2 * guard,), 0x5A, dtype=torch.uint8, device="cuda")
+    ws = ws_buf[guard:guard + need] if need else None
+    if ws is not None:
+        ws.zero_()   # the contract: zero before the first use; every call leaves it ready for the next
+    with _lib.thread_options(**(options or {})):
+        for _ in range(calls):
+            out.fill_(777.0)
+            ops.spmm_row_parts(pat.vec_length, k, pat.n, parts, slots, pat.nnz_vec, ci, vals, Bd, out, ws)
+    torch.cuda.synchronize()
+    host = buf.cpu().numpy()
+    assert np.all(host[:pad] == 12345.0) and np.all(host[pad + pat.m:] == 12345.0), "wrote outside the output"
+    wsh = ws_buf.cpu().numpy()
+    assert np.all(wsh[:guard] == 0x5A) and np.all(wsh[guard + need:] == 0x5A), "wrote outside the workspace"
+    if need:
+        counters = wsh[guard:guard + need // 128 // 256 * 256]
+        assert not counters.any(), "the arrival counters must be back at zero"
+    assert np.array_equal(ci.cpu().numpy(), pat.column_indices)
+    assert np.array_equal(slots.cpu().numpy(), parts.slots)
+    return host[pad:pad + pat.m], parts
+
+
+@pytest.mark.parametrize("V", [1, 2, 4, 8])
+@pytest.mark.parametrize("limit", [64, 128, 320, 0])
+@pytest.mark.parametrize("N", [64, 136, 256])
+def test_ragged_empty_and_long_rows(gpu, V, limit, N):
+    # empty rows at the start, in the middle and at the end; rows of every tail length; rows just under, at and
+    # over the limits; rows of many parts
+    lengths = [0, 0, 1, 15, 16, 17, 0, 31, 33, 63, 64, 65, 127, 128, 129, 300, 2, 0, 320, 321, 640, 1, 1024, 0, 0]
+    pat = _from_lengths(lengths, 1024, V, seed=5)
+    B = cv.dense_uniform(1024, N, seed=7)
+    got, parts = _run(pat, B, limit=limit)
+    assert parts.n_split > 0
+    assert_parity(got, _oracle(pat, B), "row parts V%d limit %d N%d" % (V, limit, N))
+    for i in np.nonzero(np.asarray(lengths) == 0)[0]:
+        assert not got[i * V:(i + 1) * V].any(), "empty vector row %d must be written as zeros" % i
+
+
+@pytest.mark.parametrize("V", [2, 8])
+def test_pareto_rows_with_dense_rows_on_every_launch_shape(gpu, V):
+    rng = np.random.default_rng(5)
+    m_vec, n = 300, 4608
+    lengths = np.minimum((rng.pareto(1.5, m_vec) + 0.3) * 80, n).astype(np.int64)
+    lengths[7] = n
+    lengths[150] = n
+    lengths[100] = 0
+    pat = _from_lengths(lengths, n, V, seed=6)
+    B = cv.dense_uniform(n, 256, seed=7)
+    ref = _oracle(pat, B)
+    a, parts = _run(pat, B)
+    assert parts.parts_max == 9 and parts.longest_part_vec == 512
+    assert_parity(a, ref, "pareto rows, default limit")
+    b, _ = _run(pat, B)
+    assert np.array_equal(a.view(np.uint16), b.view(np.uint16)), "two runs differ"
+    # one block per wave, several blocks per wave one after the other and pipelined, both tile widths, one wave
+    for opts in ({"spmm_pipe": 1}, {"spmm_pipe": 2}, {"spmm_waves": 1, "spmm_pipe": 2}, {"spmm_waves": 2},
+                 {"spmm_cols_per_lane": 4}, {"spmm_cols_per_lane": 8, "spmm_waves": 3},
+                 {"spmm_blocks_per_wave": 2, "spmm_pipe": 2}, {"spmm_steps": 1}, {"spmm_steps": 4}):
+        for limit in (0, 1152):
+            got, _ = _run(pat, B, limit=limit, calls=1, options=opts)
+            assert_parity(got, ref, "pareto rows, limit %d, %s" % (limit, opts))
+
+
+def test_no_row_split_and_all_rows_empty(gpu):
+    pat = cv.random_values(cv.uniform_pattern(64, 512, 0.9, seed=3, vec_length=8), 4)
+    B = cv.dense_uniform(512, 128, seed=5)
+    got, parts = _run(pat, B)
+    assert parts.n_split == 0 and parts.parts_max == 0 and parts.n_slots == 64
+    assert_parity(got, _oracle(pat, B), "no row over the limit")
+    empty = cv.ColVecCSR(8, 64, 8, np.zeros(9, np.int32), np.zeros(0, np.int32), np.zeros((0, 8), np.float16))
+    got, parts = _run(empty, cv.dense_uniform(64, 64, seed=1))
+    assert parts.n_slots == 8 and not got.any()
+
+
+def test_dense_width_edges_and_rejections(gpu):
+    pat = _from_lengths([5, 700, 0, 40, 333, 64], 768, 8, seed=9)
+    for N in (4, 8, 24, 72, 512, 1000):
+        B = cv.dense_uniform(768, N, seed=N)
+        got, _ = _run(pat, B, limit=128)
+        assert_parity(got, _oracle(pat, B), "N=%d" % N)
+    L = _lib.lib()
+    parts = ops.RowParts(pat.m_vec, pat.row_offsets, 128)
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    slots, ci, vals = d(parts.slots), d(pat.column_indices), d(pat.values)
+    B = d(cv.dense_uniform(768, 64, seed=1))
+    out = torch.full((pat.m, 64), 9.0, dtype=torch.float16, device="cuda")
+    need = ops.spmm_row_parts_workspace_bytes(8, 64, parts.n_split, parts.parts_max)
+    ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
+    args = lambda k, ws_bytes: (8, k, 768, parts.n_slots, slots.data_ptr(), parts.n_split, parts.parts_max, pat.nnz_vec,
+                                parts.longest_part_vec, ci.data_ptr(), vals.data_ptr(), B.data_ptr(), out.data_ptr(),
+                                ws.data_ptr(), ws_bytes, 0)
+    assert L.vs_wmma_spmm_f16_row_parts(*args(62, need)) == 801       # dense width not a multiple of 4
+    assert L.vs_wmma_spmm_f16_row_parts(*args(64, need - 16)) == 801  # workspace too small
+    assert L.vs_wmma_spmm_f16_row_parts(*args(64, -1)) == 1
+    bad = list(args(64, need))
+    bad[4] = slots.data_ptr() + 4
+    assert L.vs_wmma_spmm_f16_row_parts(*bad) == 1                    # misaligned list
+    torch.cuda.synchronize()
+    assert bool((out == 9.0).all()), "a rejected call must not launch anything"
+
+
+def test_one_workspace_for_problems_of_different_shapes(gpu):
+    L = _lib.lib()
+    shapes = ((64, 1024, 8, 128, 30, 1000), (512, 4608, 8, 256, 31, 4608), (32, 512, 4, 64, 32, 500),
+              (700, 2048, 1, 192, 33, 2048), (512, 4608, 8, 256, 34, 3000))
+    ws_bytes = 24 << 20
+    ws = torch.zeros(ws_bytes, dtype=torch.uint8, device="cuda")   # zeroed once, before the first use
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    for (m_vec, n, V, N, seed, longest) in shapes:
+        rng = np.random.default_rng(seed)
+        lengths = np.minimum((rng.pareto(1.5, m_vec) + 0.3) * 60, n).astype(np.int64)
+        lengths[m_vec // 3] = longest
+        pat = _from_lengths(lengths, n, V, seed=seed)
+        B = cv.dense_uniform(n, N, seed=seed + 1)
+        parts = ops.RowParts(m_vec, pat.row_offsets, 256)
+        assert ops.spmm_row_parts_workspace_bytes(V, N, parts.n_split, parts.parts_max) <= ws_bytes
+        out = torch.full((pat.m, N), 55.0, dtype=torch.float16, device="cuda")
+        ops.spmm_row_parts(V, N, n, parts, d(parts.slots), pat.nnz_vec, d(pat.column_indices), d(pat.values), d(B), out, ws)
+        torch.cuda.synchronize()
+        assert_parity(out.cpu().numpy(), _oracle(pat, B), "shared workspace, %d rows V%d N%d" % (m_vec, V, N))
+
+
+def test_device_problem_entry(gpu):
+    pat = _from_lengths([2048] + [40] * 255, 2048, 8, seed=13)
+    B = cv.dense_uniform(2048, 128, seed=14)
+    prob = ops.DeviceProblem(pat)
+    Bd = torch.from_numpy(B).cuda()
+    out = prob.spmm_row_parts(Bd)
+    out2 = prob.spmm_row_parts(Bd, limit_vec=1024)
+    torch.cuda.synchronize()
+    ref = _oracle(pat, B)
+    assert_parity(out.cpu().numpy(), ref, "DeviceProblem.spmm_row_parts")
+    assert_parity(out2.cpu().numpy(), ref, "DeviceProblem.spmm_row_parts(limit_vec=1024)")

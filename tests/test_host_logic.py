@@ -258,3 +258,57 @@ def test_the_sweep_check_catches_a_wrong_result():
     worse = good.astype(np.float16).copy()
     worse[3] = -worse[3] + np.float16(2.0)
     assert not sweep.verify_sddmm(pat, A, R, worse)[0]
+
+
+def test_row_parts_dispatch_list():
+    """vs_spmm_row_parts (host): every nonzero in exactly one slot, the parts of a split row in ascending order and
+    whole 64-vector blocks except the last, the list longest first, the counts as promised."""
+    import ctypes
+    rng = np.random.default_rng(12)
+    for trial in range(40):
+        m_vec = int(rng.integers(0, 200))
+        lengths = np.minimum((rng.pareto(1.2, m_vec) + 0.1) * rng.integers(1, 300), 5000).astype(np.int64)
+        lengths[rng.random(m_vec) < 0.1] = 0
+        ro = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+        limit = int(rng.choice([0, 1, 64, 100, 512, 1000, 4096]))
+        parts = ops.RowParts(m_vec, ro, limit)
+        step = 512 if limit == 0 else (limit + 63) // 64 * 64
+        s = parts.slots
+        assert s.shape == (parts.n_slots, 4)
+        seg = s[:, 2] - s[:, 1]
+        assert (seg >= 0).all() and (seg <= step).all()
+        assert (np.diff(seg) <= 0).all(), "longest first"
+        assert parts.longest_part_vec == (int(seg.max()) if len(seg) else 0)
+        covered = np.zeros(int(ro[-1]), dtype=np.int32)
+        seen_rows = set()
+        split_ids = set()
+        for row in range(m_vec):
+            mine = s[s[:, 0] == row]
+            assert len(mine) >= 1, "every row, the empty ones included, has a slot"
+            seen_rows.add(row)
+            if len(mine) == 1:
+                assert mine[0, 3] == 0 and mine[0, 1] == ro[row] and mine[0, 2] == ro[row + 1]
+                assert ro[row + 1] - ro[row] <= step
+            else:
+                info = mine[:, 3]
+                assert ((info & 255) == len(mine)).all() and len(mine) <= parts.parts_max
+                assert np.array_equal((info >> 8) & 255, np.arange(len(mine))), "parts in ascending order in the list"
+                assert len(set(info >> 16)) == 1
+                split_ids.add(int(info[0] >> 16))
+                assert mine[0, 1] == ro[row] and mine[-1, 2] == ro[row + 1]
+                assert np.array_equal(mine[1:, 1], mine[:-1, 2]), "parts follow each other without gaps"
+                assert ((mine[:-1, 2] - mine[:-1, 1]) % 64 == 0).all()
+            for b, e in mine[:, 1:3]:
+                covered[b:e] += 1
+        assert (covered == 1).all()
+        assert split_ids == set(range(parts.n_split))
+        assert parts.parts_max == (max((s[:, 3] & 255)) if parts.n_split else 0)
+    # too little room: the counts say what the list needs
+    ro = np.array([0, 2000, 2010], dtype=np.int32)
+    slots = np.zeros((2, 4), dtype=np.int32)
+    c = [ctypes.c_int(0) for _ in range(4)]
+    st = _lib.lib().vs_spmm_row_parts(2, ro.ctypes.data, 512, slots.ctypes.data, 2, *[ctypes.addressof(x) for x in c])
+    assert st == 801 and c[0].value == 5 and c[1].value == 1 and c[2].value == 4
+    assert _lib.lib().vs_spmm_row_parts(2, ro.ctypes.data, -1, slots.ctypes.data, 2, *[ctypes.addressof(x) for x in c]) == 1
+    assert _lib.lib().vs_wmma_spmm_row_parts_workspace_bytes(8, 256, 0, 0) == 0
+    assert _lib.lib().vs_wmma_spmm_row_parts_workspace_bytes(8, 256, 3, 4) > 3 * 4 * 8 * 256 * 4

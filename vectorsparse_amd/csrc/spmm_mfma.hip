@@ -36,15 +36,26 @@ namespace vs {
 // as soon as the same step of the current one is multiplied, so that it always has one or two steps in flight
 // instead of two while it waits and none while it multiplies; the next block's indices and vectors are requested a
 // block earlier for that, ahead of the current block's row segments (loads return in order).
+// PARTS: the dispatch list names parts of rows instead of rows - `row_indices` holds four ints per workgroup slot,
+// {vector row, first nonzero, end, part info} (vs_spmm_row_parts makes the list; row_offsets is not read) - so that
+// a row far longer than the rest is served by several workgroups, each taking a run of its nonzeros.  Part info 0:
+// the slot is a whole row and everything is as without the list.  Otherwise (parts | part << 8 | split row << 16)
+// the workgroup's fp32 tile goes to the workspace (`part_tiles`, tile of (split row, part, column tile)) and the
+// workgroup counts itself in on the row's arrival counter; the one that arrives last adds the parts in ascending
+// order - same bits whoever it is - writes the row and puts the counter back to zero.  Nobody waits for anybody.
+// The eight L2s of the chip do not see each other's lines within a launch, so the parts are written and read
+// with the device-coherence bits of the cache policy set (spmm_mfma_step.hpp).
 template <int V, int CPL, bool SOFTMAX, bool IDX32, typename OutT, bool RAGGED = false, int S = 1, bool TEAMS = false,
-          bool PIPE = false>
+          bool PIPE = false, bool PARTS = false>
 __global__ void __launch_bounds__(S * CPL >= 32 ? 256 : (S * CPL >= 16 ? 512 : 1024))
 spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row_indices,
                  const int *__restrict__ row_offsets, const int *__restrict__ column_indices,
                  const half_t *__restrict__ values, const half_t *__restrict__ rhs,
                  OutT *__restrict__ out, long long stride_values, long long stride_rhs, long long stride_out,
-                 float scale, int team_slots, int n_slots)  // (the first sixteen dwords arrive preloaded in registers)
+                 float scale, int team_slots, int n_slots,  // (the first sixteen dwords arrive preloaded in registers)
+                 int *part_counters, float *part_tiles, int parts_max)
 {
+    static_assert(!PARTS || (!SOFTMAX && !RAGGED && !TEAMS), "row parts exist for the plain operator on whole chunks");
     // `shape` packs what the prologue needs into one of the kernel arguments that arrive in registers: bits 0-7
     // log2 of the blocks a wave takes of a row, bits 8-15 the waves per workgroup, bit 16 "the grid has 512
     // workgroups or more" - the workgroup size and the grid size would otherwise be loads from the hidden arguments.
@@ -83,15 +94,24 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row
     }
     // The row's extent is requested for the identity order together with the swizzle entry itself, and again
     // only if the entry names another row: one dependent load less in the common case.
-    const int row = row_indices[slot];
-    int beg = row_offsets[slot];
-    int end = row_offsets[slot + 1];
-    // (the empty statement keeps the two requests above: the compiler otherwise folds them into the dependent
-    // ones below by selecting the index)
-    asm volatile("" : "+s"(beg), "+s"(end));
-    if (row != slot) {
-        beg = row_offsets[row];
-        end = row_offsets[row + 1];
+    int row, beg, end, part_info = 0;
+    if constexpr (PARTS) {
+        const int4_t d = reinterpret_cast<const int4_t *>(row_indices)[slot];  // one request for everything
+        row = d[0];
+        beg = d[1];
+        end = d[2];
+        part_info = d[3];
+    } else {
+        row = row_indices[slot];
+        beg = row_offsets[slot];
+        end = row_offsets[slot + 1];
+        // (the empty statement keeps the two requests above: the compiler otherwise folds them into the dependent
+        // ones below by selecting the index)
+        asm volatile("" : "+s"(beg), "+s"(end));
+        if (row != slot) {
+            beg = row_offsets[row];
+            end = row_offsets[row + 1];
+        }
     }
     const int cs = lane & 15;
     const int g = lane >> 4;
@@ -219,6 +239,54 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row
             }
         }
     };
+    // PARTS, a slot that is a part of a row: where its tile lies in the workspace (byte offset), how a thread puts
+    // its CPL sums of scalar row v there, and what the wave that has counted the workgroup in does when it is the
+    // last of the row's parts.
+    const int part_count = part_info & 255;
+    const uint32_t part_tile_bytes = (uint32_t)V * TN * (uint32_t)sizeof(float);
+    const uint32_t part_row_base =
+        (uint32_t)(((part_info >> 16) * parts_max) * n_tiles + tile) * part_tile_bytes;  // part 0 of the row, this tile
+    auto park = [&](int v, int cs_at, const float (&vals)[CPL]) {
+        const uint32_t at = part_row_base + (uint32_t)(((part_info >> 8) & 255) * n_tiles) * part_tile_bytes +
+                            4u * (uint32_t)(v * TN + cs_at * CPL);
+#pragma unroll
+        for (int c4 = 0; c4 < CPL / 4; ++c4) {
+            const float4_t t = {vals[4 * c4], vals[4 * c4 + 1], vals[4 * c4 + 2], vals[4 * c4 + 3]};
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, t), tile_area(part_tiles), at + 16u * c4, 0,
+                                                   kCoherent);
+        }
+    };
+    auto arrive_and_finish = [&]() {  // one wave, all of its lanes; the workgroup's stores have completed
+        int *counter = part_counters + (size_t)(part_info >> 16) * n_tiles + tile;
+        int arrived = 0;
+        if (lane == 0) arrived = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        arrived = __builtin_amdgcn_readfirstlane(arrived);
+        if (arrived != part_count - 1) return;  // parts are still to come: whoever brings the last adds up
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // the parts are read after the count was seen
+        for (int item = lane; item < V * 16; item += 64) {
+            const int v = item >> 4;
+            const int cs_at = item & 15;
+            const int col = tile * TN + cs_at * CPL;
+            float total[CPL];
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) total[c] = 0.f;
+            for (int p = 0; p < part_count; ++p) {
+                const uint32_t at = part_row_base + (uint32_t)(p * n_tiles) * part_tile_bytes +
+                                    4u * (uint32_t)(v * TN + cs_at * CPL);
+#pragma unroll
+                for (int c4 = 0; c4 < CPL / 4; ++c4) {
+                    const float4_t x = __builtin_bit_cast(
+                        float4_t, __builtin_amdgcn_raw_buffer_load_b128(tile_area(part_tiles), at + 16u * c4, 0, kCoherent));
+                    total[4 * c4] += x[0];
+                    total[4 * c4 + 1] += x[1];
+                    total[4 * c4 + 2] += x[2];
+                    total[4 * c4 + 3] += x[3];
+                }
+            }
+            if (col < n_cols) store_converted<OutT, CPL>(out + ((size_t)row * V + v) * n_cols + col, total);
+        }
+        if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+    };
     if constexpr (PIPE) {
         static_assert(S == 2 && IDX32 && !SOFTMAX && !RAGGED, "the pipelined walk exists for blocks of two steps");
         // (expected: the compiler then lays the walk's code out behind the epilogue, out of the short row's way -
@@ -292,6 +360,25 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row
     }
 
     if (active == 1) {
+        if constexpr (PARTS) {
+            if (part_info != 0) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int v = 4 * g + e;
+                    if (v < V) {
+                        float tmp[CPL];
+#pragma unroll
+                        for (int c = 0; c < CPL; ++c) tmp[c] = acc[c][e];
+                        park(v, cs, tmp);
+                    }
+                }
+                // the part's stores have completed (they go through to memory) before the count says so
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                __builtin_amdgcn_s_waitcnt(0);
+                arrive_and_finish();
+                return;
+            }
+        }
         store_alone();
         return;
     }
@@ -346,10 +433,23 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row
 #pragma unroll
                 for (int c = 0; c < CPL; ++c) sum[c] *= norm;
             }
-            if constexpr (RAGGED)
+            if constexpr (PARTS) {
+                if (part_info != 0)
+                    park(v, cs2, sum);
+                else
+                    store_converted<OutT, CPL>(out + ((size_t)row * V + v) * n_cols + col, sum);
+            } else if constexpr (RAGGED)
                 store_ragged<OutT, CPL>(out + ((size_t)row * V + v) * n_cols + col, sum, n_cols - col);
             else
                 store_converted<OutT, CPL>(out + ((size_t)row * V + v) * n_cols + col, sum);
+        }
+    }
+    if constexpr (PARTS) {
+        if (part_info != 0) {  // (uniform over the workgroup; the waves that had no block of the part have left)
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            __builtin_amdgcn_s_waitcnt(0);
+            if (V * 16 > 64) __syncthreads();  // the adding threads span two waves: both have stored
+            if (wave == 0) arrive_and_finish();
         }
     }
 }
@@ -384,7 +484,7 @@ static int launch_idx(int m_vec, int k, int n, int waves, const int *row_indices
     hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)batch.count), dim3(64 * waves), lds, stream,
                        k, n_tiles, per_wave_log2 | (waves << 8) | (blocks * batch.count >= 512 ? 1 << 16 : 0), row_indices,
                        row_offsets, column_indices, values, rhs, out, batch.stride_a, batch.stride_b, batch.stride_out, scale,
-                       team_slots, m_vec);
+                       team_slots, m_vec, static_cast<int *>(nullptr), static_cast<float *>(nullptr), 0);
     return (int)hipGetLastError();
 }
 
@@ -401,7 +501,8 @@ static int launch_ragged(int m_vec, int k, int waves, const int *row_indices, co
     const size_t lds = (size_t)waves * stage_bytes<V>() + (waves > 1 ? (size_t)waves * V * (TN + 1) * sizeof(float) : 0);
     hipLaunchKernelGGL((spmm_mfma_kernel<V, 4, false, false, OutT, true>), dim3((unsigned)blocks, (unsigned)batch.count),
                        dim3(64 * waves), lds, stream, k, n_tiles, waves << 8, row_indices, row_offsets, column_indices, values, rhs,
-                       out, batch.stride_a, batch.stride_b, batch.stride_out, 1.f, -1, m_vec);
+                       out, batch.stride_a, batch.stride_b, batch.stride_out, 1.f, -1, m_vec, static_cast<int *>(nullptr),
+                       static_cast<float *>(nullptr), 0);
     return (int)hipGetLastError();
 }
 
@@ -702,6 +803,86 @@ int launch_spmm_softmax_mfma(int m_vec, int vec_length, int k, int n, const int 
 {
     return launch_any<true, half_t>(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices, scores, rhs,
                                     out, stream, batch, scale);
+}
+
+// Rows in parts (the kernel's PARTS variant): `slots` is the dispatch list of vs_spmm_row_parts in device memory,
+// the workspace holds the arrival counters of the split rows and their fp32 partial tiles.
+namespace {
+
+template <int V, int CPL, bool PIPE>
+int launch_parts_kernel(int k, int n_slots, int waves, int per_wave, const int *slots, int parts_max,
+                        const int *column_indices, const half_t *values, const half_t *rhs, half_t *out, int *counters,
+                        float *tiles, hipStream_t stream)
+{
+    int per_wave_log2 = 0;
+    while ((2 << per_wave_log2) <= per_wave) ++per_wave_log2;
+    constexpr int TN = 16 * CPL;
+    const int n_tiles = ceil_div(k, TN);
+    const long long blocks = (long long)n_slots * n_tiles;
+    if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
+    const size_t lds = (size_t)waves * 2 * stage_bytes<V>() + (waves > 1 ? (size_t)waves * V * (TN + 1) * sizeof(float) : 0);
+    auto kernel = spmm_mfma_kernel<V, CPL, false, true, half_t, false, 2, false, PIPE, true>;
+    static std::atomic<unsigned long long> lds_allowed{0};
+    const hipError_t attr = allow_large_lds(reinterpret_cast<const void *>(kernel), 96 * 1024, lds_allowed);
+    if (attr != hipSuccess) return (int)attr;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, 1u), dim3(64 * waves), lds, stream, k, n_tiles,
+                       per_wave_log2 | (waves << 8) | (blocks >= 512 ? 1 << 16 : 0), slots, static_cast<const int *>(nullptr),
+                       column_indices, values, rhs, out, 0LL, 0LL, 0LL, 1.f, -1, n_slots, counters, tiles, parts_max);
+    return (int)hipGetLastError();
+}
+
+template <int V>
+int launch_parts_v(const SpmmShape &shape, int k, int n_slots, const int *slots, int parts_max, const int *column_indices,
+                   const half_t *values, const half_t *rhs, half_t *out, int *counters, float *tiles, hipStream_t stream)
+{
+#define VS_PARTS_VARIANT(CPL, PIPE)                                                                                   \
+    launch_parts_kernel<V, CPL, PIPE>(k, n_slots, shape.waves, shape.blocks_per_wave, slots, parts_max, column_indices, \
+                                      values, rhs, out, counters, tiles, stream)
+    if (shape.cols_per_lane == 8) return shape.pipelined ? VS_PARTS_VARIANT(8, true) : VS_PARTS_VARIANT(8, false);
+    return shape.pipelined ? VS_PARTS_VARIANT(4, true) : VS_PARTS_VARIANT(4, false);
+#undef VS_PARTS_VARIANT
+}
+
+}  // namespace
+
+long long spmm_row_parts_workspace_bytes(int vec_length, int k, int n_split, int parts_max)
+{
+    if (n_split <= 0 || parts_max <= 0 || k <= 0) return 0;
+    const long long k_pad = (long long)ceil_div(k, 128) * 128;  // whole tiles of either width
+    return partial_tile_workspace_for((long long)n_split * parts_max * vec_length * k_pad * (long long)sizeof(float));
+}
+
+int launch_spmm_mfma_row_parts(int vec_length, int k, int n, int n_slots, const int *slots, int n_split, int parts_max,
+                               int nonzeros_vec, int longest_part_vec, const int *column_indices, const half_t *values,
+                               const half_t *rhs, half_t *out, void *workspace, long long workspace_bytes,
+                               hipStream_t stream)
+{
+    if (n_slots == 0 || k == 0) return hipSuccess;
+    if (k % 4 != 0 || (long long)n * k >= (1LL << 31)) return hipErrorNotSupported;  // whole chunks, 32-bit offsets
+    if (n_split > 32767 || parts_max > 255 || (n_split > 0 && parts_max < 2)) return hipErrorInvalidValue;
+    const long long need = spmm_row_parts_workspace_bytes(vec_length, k, n_split, parts_max);
+    if (need > workspace_bytes || need - partial_tile_counter_bytes(need) >= (1LL << 31)) return hipErrorNotSupported;
+    Batch hints;
+    hints.nonzeros_vec = nonzeros_vec;
+    hints.longest_row_vec = longest_part_vec;
+    SpmmShape shape = choose_spmm_shape(false, n_slots, vec_length, k, n, hints);
+    if (shape.ragged || shape.dma) return hipErrorNotSupported;
+    if (k % 8 != 0) shape.cols_per_lane = 4;
+    if (shape.steps_in_flight != 2) {  // the variant exists for blocks of two steps
+        shape.steps_in_flight = 2;
+        shape.pipelined = false;
+        shape.blocks_per_wave = 1;
+    }
+    int *counters = static_cast<int *>(workspace);
+    float *tiles = reinterpret_cast<float *>(static_cast<unsigned char *>(workspace) +
+                                             (n_split > 0 ? partial_tile_counter_bytes(workspace_bytes) : 0));
+    switch (vec_length) {
+    case 1: return launch_parts_v<1>(shape, k, n_slots, slots, parts_max, column_indices, values, rhs, out, counters, tiles, stream);
+    case 2: return launch_parts_v<2>(shape, k, n_slots, slots, parts_max, column_indices, values, rhs, out, counters, tiles, stream);
+    case 4: return launch_parts_v<4>(shape, k, n_slots, slots, parts_max, column_indices, values, rhs, out, counters, tiles, stream);
+    case 8: return launch_parts_v<8>(shape, k, n_slots, slots, parts_max, column_indices, values, rhs, out, counters, tiles, stream);
+    default: return hipErrorInvalidValue;
+    }
 }
 
 template int launch_spmm_mfma<half_t>(int, int, int, int, const int *, const int *, const int *, const half_t *,

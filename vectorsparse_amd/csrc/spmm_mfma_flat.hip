@@ -77,14 +77,6 @@ __device__ __forceinline__ void tile_add(const float *tile_base, int pitch, int 
 // set (sc0 sc1: written through to memory, read past the caches), so that no cache-wide write-back or invalidate
 // is needed around the arrival counter.  `tiles` is a buffer descriptor over the tile area of the workspace
 // (below 2^31 bytes), offsets are in bytes.
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-constexpr int kCoherent = 1 | 16;  // cache policy bits: sc0, sc1
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_area(float *base)
-{
-    return __builtin_amdgcn_make_buffer_rsrc(base, 0, 0x7fffffff, 0x00020000);
-}
-
 template <int V, int CPL>
 __device__ __forceinline__ void tile_store_coherent(__amdgpu_buffer_rsrc_t tiles, uint32_t tile_bytes, int pitch, int cs,
                                                     int g, const float4_t (&acc)[CPL], int p = 0)
@@ -502,22 +494,7 @@ spmm_flat_fixup_kernel(int m_vec, int n_cols, long long piece, int n_pieces, con
 namespace {
 
 // The workspace starts with the arrival counters, one per (piece, column tile), followed by the tiles F and T of
-// every piece.  The counters' area depends on the size of the workspace alone, not on the problem: a caller may
-// use one workspace for problems of different shapes, every call leaves the counters it has used at zero, and
-// no call may find another shape's tiles where it looks for its counters.  A (piece, tile) takes 4 bytes of
-// counter and at least 512 bytes of partial tiles (two tiles of 64 floats for V = 1), so 1/128 of the workspace
-// holds the counters of whatever fits the rest.
-inline long long flat_counter_bytes(long long workspace_bytes)
-{
-    return (workspace_bytes / 128 + 255) / 256 * 256;
-}
-
-// Workspace that holds `tile_bytes` of partial tiles and the counters' area that goes with its size.
-inline long long flat_workspace_for(long long tile_bytes)
-{
-    return tile_bytes + (tile_bytes / 127 + 255) / 256 * 256 + 512;
-}
-
+// every piece (partial_tile_counter_bytes: the counters' area follows the workspace's size, not the problem's shape).
 struct FlatShape {
     bool one_launch;  // cross-workgroup parts added inside the launch (arrival counters) instead of by a second one
     bool shared;      // steps shared by consecutive rows
@@ -558,7 +535,7 @@ bool flat_shape(int vec_length, int k, int nonzeros_vec, long long workspace_byt
     const long long slot_bytes = 2LL * vec_length * s.ws_pitch * (long long)sizeof(float);  // T and F of one piece
     // (a size query passes "no limit": the counters' area then follows from the tiles, see flat_workspace_for)
     const bool unlimited = workspace_bytes == 0x7fffffffffffffffLL;
-    s.counter_bytes = unlimited || workspace_bytes <= 0 ? 0 : flat_counter_bytes(workspace_bytes);
+    s.counter_bytes = unlimited || workspace_bytes <= 0 ? 0 : partial_tile_counter_bytes(workspace_bytes);
     for (;;) {
         const long long piece = sub * s.waves;
         const long long n_pieces = ((long long)nonzeros_vec + piece - 1) / piece;
@@ -647,7 +624,7 @@ long long spmm_flat_workspace_bytes(int vec_length, int k, int nonzeros_vec)
     FlatShape s;
     if (!flat_shape(vec_length, k, nonzeros_vec, 0x7fffffffffffffffLL, s)) return 0;
     if (s.n_pieces <= 1) return 0;
-    return flat_workspace_for(2LL * s.n_pieces * vec_length * s.ws_pitch * (long long)sizeof(float));
+    return partial_tile_workspace_for(2LL * s.n_pieces * vec_length * s.ws_pitch * (long long)sizeof(float));
 }
 
 template <typename OutT>

@@ -251,6 +251,17 @@ __device__ __forceinline__ void multiply_step(const RowChunk<CPL> (&chunk)[8], c
     }
 }
 
+// Partial tiles that waves on other CUs - and other XCDs, whose L2 is a different one - read within the same
+// launch go through a buffer descriptor over the tile area of a workspace (below 2^31 bytes, offsets in bytes)
+// with the device-coherence bits of the cache policy set: written through to memory, read past the caches.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+constexpr int kCoherent = 1 | 16;  // cache policy bits: sc0, sc1
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_area(float *base)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(base, 0, 0x7fffffff, 0x00020000);
+}
+
 // Last index i in [0, rows] with offsets[i] <= pos (of equal offsets, i.e. empty rows, the last one): the row
 // that holds nonzero `pos` when pos < offsets[rows].  64-ary search, one probe per lane and round (two dependent
 // loads for up to 4095 rows); every lane of the wave must be active and gets the same answer.

@@ -302,6 +302,30 @@ int launch_sddmm_valu(int m_vec, int k, int n, int nonzeros_vec, const int *row_
 // callers may capture the call into a HIP graph).
 int launch_zero_fill(void *out, long long bytes, long long stride_bytes, int batch, hipStream_t stream);
 
+// Workspaces of fp32 partial tiles with arrival counters in front (split-row SpMM, rows in parts).  The counters'
+// area depends on the size of the workspace alone, not on the problem: a caller may use one workspace for
+// problems of different shapes, every call leaves the counters it has used at zero, and no call may find another
+// shape's tiles where it looks for its counters.  A counter takes 4 bytes and stands for at least 512 bytes of
+// partial tiles (two tiles of 64 floats for V = 1), so 1/128 of the workspace holds the counters of whatever
+// fits the rest.
+inline long long partial_tile_counter_bytes(long long workspace_bytes)
+{
+    return (workspace_bytes / 128 + 255) / 256 * 256;
+}
+// Workspace that holds `tile_bytes` of partial tiles and the counters' area that goes with its size.
+inline long long partial_tile_workspace_for(long long tile_bytes)
+{
+    return tile_bytes + (tile_bytes / 127 + 255) / 256 * 256 + 512;
+}
+
+// Rows in parts (csrc/spmm_mfma.hip, the kernel's PARTS variant): `slots` = the dispatch list of
+// vs_spmm_row_parts in device memory, four ints per workgroup slot.
+int launch_spmm_mfma_row_parts(int vec_length, int k, int n, int n_slots, const int *slots, int n_split, int parts_max,
+                               int nonzeros_vec, int longest_part_vec, const int *column_indices, const half_t *values,
+                               const half_t *rhs, half_t *out, void *workspace, long long workspace_bytes,
+                               hipStream_t stream);
+long long spmm_row_parts_workspace_bytes(int vec_length, int k, int n_split, int parts_max);
+
 // Split-row SpMM (csrc/spmm_mfma_flat.hip): `workspace` holds the fp32 partial tiles of rows longer than a piece.
 template <typename OutT>
 int launch_spmm_mfma_flat(int m_vec, int vec_length, int k, int n, int nonzeros_vec, const int *row_offsets,

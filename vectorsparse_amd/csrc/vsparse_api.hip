@@ -542,6 +542,93 @@ void vs_sorted_row_swizzle(int rows, const int *row_offsets, int *row_indices)
     });
 }
 
+int vs_spmm_row_parts(int m_vec, const int *row_offsets, int limit_vec, int *slots, int max_slots, int *n_slots,
+                      int *n_split, int *parts_max, int *longest_part_vec)
+{
+    if (m_vec < 0 || !row_offsets || !n_slots || !n_split || !parts_max || !longest_part_vec || max_slots < 0 ||
+        (max_slots > 0 && !slots) || limit_vec < 0)
+        return VS_ERROR_INVALID_VALUE;
+    long long limit = limit_vec > 0 ? limit_vec : 512;
+    limit = (limit + 63) / 64 * 64;  // whole blocks of two 32-vector steps
+    struct Part {
+        int row, beg, end, info;
+    };
+    std::vector<Part> parts;
+    parts.reserve((size_t)m_vec + 64);
+    int split = 0, most = 0, longest = 0;
+    for (int row = 0; row < m_vec; ++row) {
+        const int beg = row_offsets[row], end = row_offsets[row + 1];
+        if (end < beg) return VS_ERROR_INVALID_VALUE;
+        const long long len = (long long)end - beg;
+        if (len <= limit) {
+            parts.push_back({row, beg, end, 0});
+            longest = len > longest ? (int)len : longest;
+            continue;
+        }
+        // equal parts, each a whole number of blocks, no more of them than the limit asks for
+        long long count = (len + limit - 1) / limit;
+        if (count > 255) count = 255;
+        const long long per = ((len + count - 1) / count + 63) / 64 * 64;
+        count = (len + per - 1) / per;
+        if (count < 2) {  // (rounding the part up to whole blocks took the whole row)
+            parts.push_back({row, beg, end, 0});
+            longest = len > longest ? (int)len : longest;
+            continue;
+        }
+        if (split >= 32767) return VS_ERROR_NOT_SUPPORTED;
+        for (long long p = 0; p < count; ++p) {
+            const long long from = beg + p * per;
+            const long long to = from + per < end ? from + per : end;
+            parts.push_back({row, (int)from, (int)to, (int)count | (int)(p << 8) | (split << 16)});
+        }
+        longest = per > longest ? (int)per : longest;
+        most = count > most ? (int)count : most;
+        ++split;
+    }
+    // Longest first, as the sorted swizzle dispatches whole rows (include/bm_test_utils.h:200-215 of the
+    // reference); a stable sort keeps the list reproducible and the parts of a row in ascending order.
+    std::stable_sort(parts.begin(), parts.end(),
+                     [](const Part &a, const Part &b) { return a.end - a.beg > b.end - b.beg; });
+    *n_slots = (int)parts.size();
+    *n_split = split;
+    *parts_max = most;
+    *longest_part_vec = longest;
+    if ((long long)parts.size() > max_slots) return VS_ERROR_NOT_SUPPORTED;  // the counts say what the list needs
+    for (size_t i = 0; i < parts.size(); ++i) {
+        slots[4 * i] = parts[i].row;
+        slots[4 * i + 1] = parts[i].beg;
+        slots[4 * i + 2] = parts[i].end;
+        slots[4 * i + 3] = parts[i].info;
+    }
+    return VS_SUCCESS;
+}
+
+long long vs_wmma_spmm_row_parts_workspace_bytes(int vec_length, int k, int n_split, int parts_max)
+{
+    if (!vec_ok(vec_length)) return 0;
+    return vs::spmm_row_parts_workspace_bytes(vec_length, k, n_split, parts_max);
+}
+
+int vs_wmma_spmm_f16_row_parts(int vec_length, int k, int n, int n_slots, const int *slots, int n_split, int parts_max,
+                               int nonzeros_vec, int longest_part_vec, const int *column_indices, const void *values,
+                               const void *rhs_matrix, void *output_matrix, void *workspace, long long workspace_bytes,
+                               void *stream)
+{
+    if (!vec_ok(vec_length) || k < 0 || n < 0 || n_slots < 0 || n_split < 0 || parts_max < 0 ||
+        nonzeros_vec < 0 || longest_part_vec < 0 || workspace_bytes < 0)
+        return VS_ERROR_INVALID_VALUE;
+    if (n_slots > 0 && (!slots || !aligned(slots, 16))) return VS_ERROR_INVALID_VALUE;
+    if (n_slots > 0 && k > 0 && (!rhs_matrix || !output_matrix)) return VS_ERROR_INVALID_VALUE;
+    if (nonzeros_vec > 0 && (!column_indices || !values)) return VS_ERROR_INVALID_VALUE;
+    if (!aligned(values, 2 * vec_length) || !aligned(rhs_matrix, 16) || !aligned(output_matrix, 16))
+        return VS_ERROR_INVALID_VALUE;
+    if (workspace_bytes > 0 && (!workspace || !aligned(workspace, 16))) return VS_ERROR_INVALID_VALUE;
+    return vs::launch_spmm_mfma_row_parts(vec_length, k, n, n_slots, slots, n_split, parts_max, nonzeros_vec,
+                                          longest_part_vec, column_indices, static_cast<const half_t *>(values),
+                                          static_cast<const half_t *>(rhs_matrix), static_cast<half_t *>(output_matrix),
+                                          workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
 int vs_launch_floor_probe(int blocks, int threads_per_block, void *stream)
 {
     if (blocks < 1 || threads_per_block < 1 || threads_per_block > 1024) return VS_ERROR_INVALID_VALUE;

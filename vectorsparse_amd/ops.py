@@ -438,6 +438,47 @@ def SortedRowSwizzle(rows, row_offsets):
     return out
 
 
+class RowParts:
+    """The dispatch list of `vs_spmm_row_parts` for a pattern: rows of more than `limit_vec` nonzero vectors (0 =
+    the library's default) cut into parts that get a workgroup each, everything ordered longest first.  Host arrays in,
+    host array out (`slots`, int32 [n_slots][4]); `n_split`, `parts_max`, `longest_part_vec` as the C function
+    returns them."""
+
+    def __init__(self, m_vec, row_offsets, limit_vec=0):
+        import ctypes
+        ro = np.ascontiguousarray(row_offsets, dtype=np.int32)
+        step = 512 if limit_vec <= 0 else (limit_vec + 63) // 64 * 64
+        room = m_vec + int(ro[m_vec] if m_vec > 0 else 0) // min(step, 512) + 64
+        slots = np.empty((room, 4), dtype=np.int32)
+        counts = [ctypes.c_int(0) for _ in range(4)]
+        st = _lib.lib().vs_spmm_row_parts(m_vec, ro.ctypes.data, limit_vec, slots.ctypes.data, room,
+                                          *[ctypes.addressof(c) for c in counts])
+        if st:
+            _lib.check(st, "vs_spmm_row_parts")
+        self.n_slots, self.n_split, self.parts_max, self.longest_part_vec = (c.value for c in counts)
+        self.slots = np.ascontiguousarray(slots[:self.n_slots])
+
+
+def spmm_row_parts_workspace_bytes(vec_length, k, n_split, parts_max):
+    return int(_lib.lib().vs_wmma_spmm_row_parts_workspace_bytes(vec_length, k, n_split, parts_max))
+
+
+def spmm_row_parts(vec_length, k, n, parts, slots, nonzeros_vec, column_indices, values, rhs_matrix, output_matrix,
+                   workspace=None, stream=None):
+    """wmmaSpmm driven by a dispatch list of row parts (`parts`: a RowParts, `slots`: its list as a device int32
+    tensor).  workspace: a device tensor of at least spmm_row_parts_workspace_bytes(...) bytes, zero-filled before
+    its first use, or None when no row is split.  Returns output_matrix."""
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    st = _lib.lib().vs_wmma_spmm_f16_row_parts(
+        vec_length, k, n, parts.n_slots, _expect(slots, torch.int32, "slots"), parts.n_split, parts.parts_max,
+        nonzeros_vec, parts.longest_part_vec, _expect(column_indices, torch.int32, "column_indices"),
+        _expect(values, torch.float16, "values"), _expect(rhs_matrix, torch.float16, "rhs_matrix"),
+        _expect(output_matrix, torch.float16, "output_matrix"), _ptr(workspace), ws_bytes, _stream(stream))
+    if st:
+        _lib.check(st, "vs_wmma_spmm_f16_row_parts")
+    return output_matrix
+
+
 LONG_ROW_VECTORS = 512  # rows beyond this are "long" for vs_wmma_spmm_f16_batched_sorted (eight 64-vector blocks)
 
 
@@ -473,9 +514,32 @@ class DeviceProblem:
         self.row_offsets = torch.from_numpy(np.ascontiguousarray(pattern.row_offsets)).to(device)
         self.column_indices = torch.from_numpy(np.ascontiguousarray(pattern.column_indices)).to(device)
         self._workspace = None  # partial tiles of the split-row SpMM, allocated on first use
+        self._parts = {}        # limit -> (RowParts, its list on the device, workspace), made on first use
         self.values = None
         if pattern.values is not None:
             self.values = torch.from_numpy(np.ascontiguousarray(pattern.values)).to(device)
+
+    def row_parts(self, limit_vec=0):
+        """The pattern's dispatch list of row parts (see RowParts) on the device, made once per limit."""
+        if limit_vec not in self._parts:
+            parts = RowParts(self.m_vec, self.pattern.row_offsets, limit_vec)
+            slots = torch.from_numpy(parts.slots).to(self.column_indices.device)
+            self._parts[limit_vec] = [parts, slots, None]
+        return self._parts[limit_vec]
+
+    def spmm_row_parts(self, rhs_matrix, out=None, stream=None, limit_vec=0):
+        """SpMM (MFMA path, fp16 output) with long rows dispatched as several parts; the list and the workspace
+        for the parts' partial tiles belong to this object."""
+        k = rhs_matrix.shape[1]
+        if out is None:
+            out = torch.empty((self.m_vec * self.vec_length, k), dtype=torch.float16, device=rhs_matrix.device)
+        entry = self.row_parts(limit_vec)
+        parts, slots = entry[0], entry[1]
+        need = spmm_row_parts_workspace_bytes(self.vec_length, k, parts.n_split, parts.parts_max)
+        if need and (entry[2] is None or entry[2].numel() < need):
+            entry[2] = torch.zeros(need, dtype=torch.uint8, device=rhs_matrix.device)
+        return spmm_row_parts(self.vec_length, k, self.n, parts, slots, self.nnz_vec, self.column_indices, self.values,
+                              rhs_matrix, out, entry[2] if need else None, stream)
 
     def spmm(self, rhs_matrix, kernel="wmma", out_dtype=torch.float16, out=None, stream=None, row_length_hint=False,
              split_rows=False):
