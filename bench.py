@@ -366,7 +366,7 @@ def main():
     lA = torch.randn((lpat.m, 4608), dtype=torch.float16, device="cuda")
     _, large_dense_ms = time_graph(torch, lambda: torch.matmul(lA, lBd, out=lout), dev_steps, args.warmup)
 
-    # ---- skewed rows: reference-shaped entry, batched entry with the row-length hints, split-row schedule
+    # ---- skewed rows: reference-shaped entry, batched entry with the row-length hints, split-row schedule, rows in parts
     kpat, kB = skewed_point(cv, np)
     kprob = ops.DeviceProblem(kpat, sort=True)
     kBd = torch.from_numpy(kB).cuda()
@@ -375,9 +375,19 @@ def main():
     _, skew_plain_ms = time_graph(torch, lambda: kprob.spmm(kBd, out=kout), skew_steps, 3)
     _, skew_hint_ms = time_graph(torch, lambda: kprob.spmm(kBd, out=kout, row_length_hint=True), skew_steps, 3)
     _, skew_split_ms = time_graph(torch, lambda: kprob.spmm(kBd, out=kout, split_rows=True), skew_steps, 3)
+    kref = kout.clone()
+    _, skew_parts_ms = time_graph(torch, lambda: kprob.spmm_row_parts(kBd, out=kout), skew_steps, 3)
+    torch.cuda.synchronize()
+    # (rows in parts add a split row's nonzeros in another order than the split-row schedule: equal up to fp32 rounding
+    # of sums of a few thousand terms, then both rounded to fp16)
+    skew_parts_diff = float((kout.float() - kref.float()).abs().max() / kref.float().abs().max())
+    if not skew_parts_diff < 2e-3:
+        raise SystemExit("rows in parts and split rows disagree on the skewed point: %g" % skew_parts_diff)
+    kparts = kprob.row_parts(0)[0]
     upat = cv.random_values(cv.uniform_pattern(kpat.m_vec, kpat.n, 1 - kpat.nnz_vec / (kpat.m_vec * kpat.n), 1, 8), 1)
     uprob = ops.DeviceProblem(upat, sort=True)
     _, skew_uniform_ms = time_graph(torch, lambda: uprob.spmm(kBd, out=kout), skew_steps, 3)
+    _, skew_uniform_hint_ms = time_graph(torch, lambda: uprob.spmm(kBd, out=kout, row_length_hint=True), skew_steps, 3)
 
     # ---- SDDMM config 4
     _, sddmm_ms = time_graph(torch, sddmm_step, dev_steps, args.warmup)
@@ -483,7 +493,11 @@ def main():
                                              % (kpat.nnz_vec / kpat.m_vec, int(np.diff(kpat.row_offsets).max())),
                                  "reference_entry_us": skew_plain_ms * 1e3, "hinted_batched_entry_us": skew_hint_ms * 1e3,
                                  "split_rows_entry_us": skew_split_ms * 1e3,
-                                 "uniform_rows_same_nonzeros_us": skew_uniform_ms * 1e3},
+                                 "row_parts_entry_us": skew_parts_ms * 1e3,
+                                 "row_parts": "%d rows in up to %d parts" % (kparts.n_split, kparts.parts_max),
+                                 "uniform_rows_same_nonzeros_us": skew_uniform_ms * 1e3,
+                                 "uniform_rows_same_nonzeros_hinted_us": skew_uniform_hint_ms * 1e3,
+                                 "row_parts_over_uniform_hinted": skew_parts_ms / skew_uniform_hint_ms},
             "sddmm_config4_k64": dict(
                 hbm(sddmm_bytes, sddmm_ms, sddmm_traffic, traffic_note=sddmm_note, kernel="sddmm_mfma_kernel<V=8>"),
                 ms=sddmm_ms, tflops=sddmm_flops / (sddmm_ms * 1e-3) * 1e-12, dense_product_us=sddmm_dense_ms * 1e3,

@@ -251,16 +251,20 @@ int vs_wmma_spmm_f16_batched_sorted(int batch, int m_vec, int vec_length, int k,
  * the launch has finished.  No counterpart in the reference.
  *
  * vs_spmm_row_parts (HOST function on HOST arrays, like the swizzles): the dispatch list of a pattern.  Rows of more
- * than limit_vec nonzero vectors (0 = the library's default, 512; rounded up to a multiple of 64) are cut into
+ * than limit_vec nonzero vectors (0 = the library's default: 1152 or four mean row lengths, whichever is more;
+ * rounded up to a multiple of 64) are cut into
  * equal parts of whole 64-vector blocks, at most 255 per row; every other row, the empty ones included, is a
  * slot of its own; the slots are ordered longest first.  slots: four ints per slot {vector row, first nonzero,
  * end, part info (0 = a whole row)}, room for max_slots of them.  Returns the number of slots, of split rows, the
  * most parts any row has and the longest slot through the pointers; VS_ERROR_NOT_SUPPORTED with the counts set
- * when max_slots is too small (m_vec + nonzeros_vec / 64 + 1 slots always suffice for the default limit) or more
- * than 32767 rows would be split.
+ * when max_slots is too small or more than 32767 rows would be split.  Behind the n_slots entries the list holds
+ * one more entry per split row ({vector row, parts, 0, 0}, for the launch that adds the parts when option
+ * "spmm_parts_launches" is 2): n_slots + n_split entries in all, m_vec + 2 * (nonzeros_vec / limit) + 1 always
+ * suffice.
  *
  * vs_wmma_spmm_f16_row_parts: the operator of vs_wmma_spmm_f16 (same operands, same contract for the output)
- * driven by that list, copied to DEVICE memory (16-byte aligned), in place of row_indices and row_offsets.
+ * driven by that list (all n_slots + n_split entries), copied to DEVICE memory (16-byte aligned), in place of
+ * row_indices and row_offsets.
  * nonzeros_vec and longest_part_vec size the launch as the hints of vs_wmma_spmm_f16_batched do.  The parts of
  * a split row leave fp32 partial tiles in `workspace` and the workgroup that brings the last one adds them in
  * ascending order (deterministic, no atomics on the output, nobody waits).  workspace: device memory, 16-byte
@@ -447,7 +451,9 @@ int vs_wmma_spmm_launch_shape(int batch, int m_vec, int vec_length, int k, int n
  * "spmm_flat_piece" (nonzero vectors
  * per wave of the split-row SpMM, rounded up to 32, 0 = automatic), "spmm_flat_waves"
  * (its waves per workgroup, 1..16, 0 = automatic), "spmm_flat_launches" (1 = partial tiles
- * added inside the launch, 2 = by a second launch, 0 = automatic), "spmm_flat_shared" (1 = every
+ * added inside the launch, 2 = by a second launch, 0 = automatic), "spmm_parts_launches" (rows in
+ * parts: 1 = the parts of a split row meet inside the launch, 2 = a second launch adds them, 0 = automatic,
+ * which is 1; same bits either way), "spmm_flat_shared" (1 = every
  * row segment of the split-row SpMM starts a 32-vector step of its own, 2 = consecutive rows share
  * steps, 0 = automatic), "sddmm_slots" (waves per
  * vector row, 0 = automatic), "sddmm_group" (16-vector groups per wave step of the

@@ -133,7 +133,7 @@ def test_options():
         _lib.set_option("spmm_cols_per_lane", 3)
     # every documented name is known, takes 0 (automatic) and rejects a value outside its range
     ranges = {"spmm_waves": 17, "spmm_cols_per_lane": 5, "spmm_steps": 3, "spmm_guard_waves": 17, "spmm_teams": 3, "spmm_pipe": 3, "spmm_blocks_per_wave": 3, "spmm_gather": 3,
-              "spmm_flat_launches": 3, "spmm_flat_waves": 17, "spmm_flat_shared": 3, "sddmm_group": 3,
+              "spmm_flat_launches": 3, "spmm_flat_waves": 17, "spmm_flat_shared": 3, "spmm_parts_launches": 3, "sddmm_group": 3,
               "sddmm_block_waves": 17, "sddmm_flat_supers": 17, "attention_waves": 9}
     for name, bad in ranges.items():
         _lib.set_option(name, 0)

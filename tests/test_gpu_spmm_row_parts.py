@@ -63,15 +63,16 @@ def _run(pat, B, limit=0, calls=2, options=None):
 @pytest.mark.parametrize("V", [1, 2, 4, 8])
 @pytest.mark.parametrize("limit", [64, 128, 320, 0])
 @pytest.mark.parametrize("N", [64, 136, 256])
-def test_ragged_empty_and_long_rows(gpu, V, limit, N):
+@pytest.mark.parametrize("launches", [1, 2])
+def test_ragged_empty_and_long_rows(gpu, V, limit, N, launches):
     # empty rows at the start, in the middle and at the end; rows of every tail length; rows just under, at and
     # over the limits; rows of many parts
     lengths = [0, 0, 1, 15, 16, 17, 0, 31, 33, 63, 64, 65, 127, 128, 129, 300, 2, 0, 320, 321, 640, 1, 1024, 0, 0]
     pat = _from_lengths(lengths, 1024, V, seed=5)
     B = cv.dense_uniform(1024, N, seed=7)
-    got, parts = _run(pat, B, limit=limit)
-    assert parts.n_split > 0
-    assert_parity(got, _oracle(pat, B), "row parts V%d limit %d N%d" % (V, limit, N))
+    got, parts = _run(pat, B, limit=limit, options={"spmm_parts_launches": launches})
+    assert parts.n_split > 0 or limit == 0   # (the default limit is beyond these rows)
+    assert_parity(got, _oracle(pat, B), "row parts V%d limit %d N%d, %d launches" % (V, limit, N, launches))
     for i in np.nonzero(np.asarray(lengths) == 0)[0]:
         assert not got[i * V:(i + 1) * V].any(), "empty vector row %d must be written as zeros" % i
 
@@ -88,15 +89,19 @@ def test_pareto_rows_with_dense_rows_on_every_launch_shape(gpu, V):
     B = cv.dense_uniform(n, 256, seed=7)
     ref = _oracle(pat, B)
     a, parts = _run(pat, B)
-    assert parts.parts_max == 9 and parts.longest_part_vec == 512
+    assert parts.parts_max == 4 and parts.longest_part_vec == 1152
     assert_parity(a, ref, "pareto rows, default limit")
     b, _ = _run(pat, B)
     assert np.array_equal(a.view(np.uint16), b.view(np.uint16)), "two runs differ"
+    one, _ = _run(pat, B, options={"spmm_parts_launches": 1})
+    two, _ = _run(pat, B, options={"spmm_parts_launches": 2})
+    assert np.array_equal(one.view(np.uint16), two.view(np.uint16)), "one launch and two launches add in the same order"
     # one block per wave, several blocks per wave one after the other and pipelined, both tile widths, one wave
     for opts in ({"spmm_pipe": 1}, {"spmm_pipe": 2}, {"spmm_waves": 1, "spmm_pipe": 2}, {"spmm_waves": 2},
                  {"spmm_cols_per_lane": 4}, {"spmm_cols_per_lane": 8, "spmm_waves": 3},
-                 {"spmm_blocks_per_wave": 2, "spmm_pipe": 2}, {"spmm_steps": 1}, {"spmm_steps": 4}):
-        for limit in (0, 1152):
+                 {"spmm_blocks_per_wave": 2, "spmm_pipe": 2}, {"spmm_steps": 1}, {"spmm_steps": 4},
+                 {"spmm_parts_launches": 1, "spmm_waves": 1}, {"spmm_parts_launches": 2, "spmm_waves": 1}):
+        for limit in (0, 512):
             got, _ = _run(pat, B, limit=limit, calls=1, options=opts)
             assert_parity(got, ref, "pareto rows, limit %d, %s" % (limit, opts))
 

@@ -272,9 +272,14 @@ def test_row_parts_dispatch_list():
         ro = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
         limit = int(rng.choice([0, 1, 64, 100, 512, 1000, 4096]))
         parts = ops.RowParts(m_vec, ro, limit)
-        step = 512 if limit == 0 else (limit + 63) // 64 * 64
-        s = parts.slots
-        assert s.shape == (parts.n_slots, 4)
+        default = max(1152, 4 * (int(ro[-1]) // m_vec)) if m_vec else 1152
+        step = ((default if limit == 0 else limit) + 63) // 64 * 64
+        assert parts.slots.shape == (parts.n_slots + parts.n_split, 4)
+        s = parts.slots[:parts.n_slots]
+        tail = parts.slots[parts.n_slots:]   # behind the list: {row, parts} of every split row, by its number
+        for number, (row, count, _, _) in enumerate(tail):
+            mine = s[(s[:, 3] != 0) & ((s[:, 3] >> 16) == number)]
+            assert len(mine) == count and (mine[:, 0] == row).all()
         seg = s[:, 2] - s[:, 1]
         assert (seg >= 0).all() and (seg <= step).all()
         assert (np.diff(seg) <= 0).all(), "longest first"

@@ -62,6 +62,7 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row
     const int per_wave_log2 = shape & 255;
     const int n_waves = (shape >> 8) & 255;
     const bool full_grid = (shape >> 16) & 1;
+    const bool parts_meet_later = (shape >> 17) & 1;  // PARTS: a second launch adds the parts of split rows
     if (blockIdx.y != 0) {  // batch: shared pattern, per-problem operands (the strides are not loaded for problem 0)
         values += blockIdx.y * stride_values;
         rhs += blockIdx.y * stride_rhs;
@@ -252,12 +253,16 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row
 #pragma unroll
         for (int c4 = 0; c4 < CPL / 4; ++c4) {
             const float4_t t = {vals[4 * c4], vals[4 * c4 + 1], vals[4 * c4 + 2], vals[4 * c4 + 3]};
-            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, t), tile_area(part_tiles), at + 16u * c4, 0,
-                                                   kCoherent);
+            if (parts_meet_later)  // read by the next launch: an ordinary store
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, t), tile_area(part_tiles),
+                                                       at + 16u * c4, 0, 0);
+            else
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, t), tile_area(part_tiles),
+                                                       at + 16u * c4, 0, kCoherent);
         }
     };
     auto arrive_and_finish = [&]() {  // one wave, all of its lanes; the workgroup's stores have completed
-        int *counter = part_counters + (size_t)(part_info >> 16) * n_tiles + tile;
+        int *counter = part_counters + ((size_t)(part_info >> 16) * n_tiles + tile) * kPartCounterStride;
         int arrived = 0;
         if (lane == 0) arrived = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         arrived = __builtin_amdgcn_readfirstlane(arrived);
@@ -372,6 +377,7 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row
                         park(v, cs, tmp);
                     }
                 }
+                if (parts_meet_later) return;
                 // the part's stores have completed (they go through to memory) before the count says so
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
                 __builtin_amdgcn_s_waitcnt(0);
@@ -445,13 +451,49 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row
         }
     }
     if constexpr (PARTS) {
-        if (part_info != 0) {  // (uniform over the workgroup; the waves that had no block of the part have left)
+        if (part_info != 0 && !parts_meet_later) {  // (uniform over the workgroup; idle waves have left)
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
             __builtin_amdgcn_s_waitcnt(0);
             if (V * 16 > 64) __syncthreads();  // the adding threads span two waves: both have stored
             if (wave == 0) arrive_and_finish();
         }
     }
+}
+
+// Second launch of the rows in parts (when the parts do not meet inside the first): one workgroup per (split row,
+// column tile) adds the row's partial tiles in ascending order - the same sum as the workgroup that arrives last
+// computes in the one-launch form - and writes the row.  `split_rows`: four ints per split row, {vector row, parts}.
+template <int V, int CPL>
+__global__ void __launch_bounds__(V * 16 < 64 ? 64 : V * 16)
+spmm_row_parts_sum_kernel(int n_cols, int n_tiles, const int *__restrict__ split_rows, int parts_max,
+                          const float *__restrict__ tiles, half_t *__restrict__ out)
+{
+    constexpr int TN = 16 * CPL;
+    const int tile = blockIdx.x % n_tiles;
+    const int split = blockIdx.x / n_tiles;
+    const int row = split_rows[4 * split];
+    const int parts = split_rows[4 * split + 1];
+    const int item = threadIdx.x;
+    if (item >= V * 16) return;
+    const int v = item >> 4;
+    const int cs = item & 15;
+    const int col = tile * TN + cs * CPL;
+    if (col >= n_cols) return;
+    float total[CPL];
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) total[c] = 0.f;
+    const float *src = tiles + ((size_t)split * parts_max * n_tiles + tile) * V * TN + v * TN + cs * CPL;
+    for (int p = 0; p < parts; ++p) {
+#pragma unroll
+        for (int c4 = 0; c4 < CPL / 4; ++c4) {
+            const float4_t x = *reinterpret_cast<const float4_t *>(src + (size_t)p * n_tiles * V * TN + 4 * c4);
+            total[4 * c4] += x[0];
+            total[4 * c4 + 1] += x[1];
+            total[4 * c4 + 2] += x[2];
+            total[4 * c4 + 3] += x[3];
+        }
+    }
+    store_converted<half_t, CPL>(out + ((size_t)row * V + v) * n_cols + col, total);
 }
 
 static int next_pow2(int x)
@@ -810,9 +852,9 @@ int launch_spmm_softmax_mfma(int m_vec, int vec_length, int k, int n, const int 
 namespace {
 
 template <int V, int CPL, bool PIPE>
-int launch_parts_kernel(int k, int n_slots, int waves, int per_wave, const int *slots, int parts_max,
-                        const int *column_indices, const half_t *values, const half_t *rhs, half_t *out, int *counters,
-                        float *tiles, hipStream_t stream)
+int launch_parts_kernel(int k, int n_slots, int n_split, bool two_launches, int waves, int per_wave, const int *slots,
+                        int parts_max, const int *column_indices, const half_t *values, const half_t *rhs, half_t *out,
+                        int *counters, float *tiles, hipStream_t stream)
 {
     int per_wave_log2 = 0;
     while ((2 << per_wave_log2) <= per_wave) ++per_wave_log2;
@@ -826,18 +868,25 @@ int launch_parts_kernel(int k, int n_slots, int waves, int per_wave, const int *
     const hipError_t attr = allow_large_lds(reinterpret_cast<const void *>(kernel), 96 * 1024, lds_allowed);
     if (attr != hipSuccess) return (int)attr;
     hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, 1u), dim3(64 * waves), lds, stream, k, n_tiles,
-                       per_wave_log2 | (waves << 8) | (blocks >= 512 ? 1 << 16 : 0), slots, static_cast<const int *>(nullptr),
-                       column_indices, values, rhs, out, 0LL, 0LL, 0LL, 1.f, -1, n_slots, counters, tiles, parts_max);
+                       per_wave_log2 | (waves << 8) | (blocks >= 512 ? 1 << 16 : 0) | (two_launches ? 1 << 17 : 0), slots,
+                       static_cast<const int *>(nullptr), column_indices, values, rhs, out, 0LL, 0LL, 0LL, 1.f, -1, n_slots,
+                       counters, tiles, parts_max);
+    const hipError_t st = hipGetLastError();
+    if (st != hipSuccess || !two_launches || n_split == 0) return (int)st;
+    hipLaunchKernelGGL((spmm_row_parts_sum_kernel<V, CPL>), dim3((unsigned)(n_split * n_tiles)),
+                       dim3(V * 16 < 64 ? 64 : V * 16), 0, stream, k, n_tiles, slots + 4 * (size_t)n_slots, parts_max, tiles,
+                       out);
     return (int)hipGetLastError();
 }
 
 template <int V>
-int launch_parts_v(const SpmmShape &shape, int k, int n_slots, const int *slots, int parts_max, const int *column_indices,
-                   const half_t *values, const half_t *rhs, half_t *out, int *counters, float *tiles, hipStream_t stream)
+int launch_parts_v(const SpmmShape &shape, int k, int n_slots, int n_split, bool two_launches, const int *slots,
+                   int parts_max, const int *column_indices, const half_t *values, const half_t *rhs, half_t *out,
+                   int *counters, float *tiles, hipStream_t stream)
 {
-#define VS_PARTS_VARIANT(CPL, PIPE)                                                                                   \
-    launch_parts_kernel<V, CPL, PIPE>(k, n_slots, shape.waves, shape.blocks_per_wave, slots, parts_max, column_indices, \
-                                      values, rhs, out, counters, tiles, stream)
+#define VS_PARTS_VARIANT(CPL, PIPE)                                                                                \
+    launch_parts_kernel<V, CPL, PIPE>(k, n_slots, n_split, two_launches, shape.waves, shape.blocks_per_wave, slots, \
+                                      parts_max, column_indices, values, rhs, out, counters, tiles, stream)
     if (shape.cols_per_lane == 8) return shape.pipelined ? VS_PARTS_VARIANT(8, true) : VS_PARTS_VARIANT(8, false);
     return shape.pipelined ? VS_PARTS_VARIANT(4, true) : VS_PARTS_VARIANT(4, false);
 #undef VS_PARTS_VARIANT
@@ -849,7 +898,7 @@ long long spmm_row_parts_workspace_bytes(int vec_length, int k, int n_split, int
 {
     if (n_split <= 0 || parts_max <= 0 || k <= 0) return 0;
     const long long k_pad = (long long)ceil_div(k, 128) * 128;  // whole tiles of either width
-    return partial_tile_workspace_for((long long)n_split * parts_max * vec_length * k_pad * (long long)sizeof(float));
+    return row_parts_workspace_for((long long)n_split * parts_max * vec_length * k_pad * (long long)sizeof(float));
 }
 
 int launch_spmm_mfma_row_parts(int vec_length, int k, int n, int n_slots, const int *slots, int n_split, int parts_max,
@@ -861,7 +910,7 @@ int launch_spmm_mfma_row_parts(int vec_length, int k, int n, int n_slots, const 
     if (k % 4 != 0 || (long long)n * k >= (1LL << 31)) return hipErrorNotSupported;  // whole chunks, 32-bit offsets
     if (n_split > 32767 || parts_max > 255 || (n_split > 0 && parts_max < 2)) return hipErrorInvalidValue;
     const long long need = spmm_row_parts_workspace_bytes(vec_length, k, n_split, parts_max);
-    if (need > workspace_bytes || need - partial_tile_counter_bytes(need) >= (1LL << 31)) return hipErrorNotSupported;
+    if (need > workspace_bytes || need - row_parts_counter_bytes(need) >= (1LL << 31)) return hipErrorNotSupported;
     Batch hints;
     hints.nonzeros_vec = nonzeros_vec;
     hints.longest_row_vec = longest_part_vec;
@@ -873,14 +922,27 @@ int launch_spmm_mfma_row_parts(int vec_length, int k, int n, int n_slots, const 
         shape.pipelined = false;
         shape.blocks_per_wave = 1;
     }
+    // A list with split rows is cut off at the limit, which the rules for whole rows misread (they size the
+    // workgroups by the mean row or by how far the longest row stands out).  Measured at N = 256, V = 8, K = 4608,
+    // limits of 768-1536 vectors, 64 to 2048 rows of Pareto or log-normal lengths or with one dense row (2 / 4 / 8
+    // waves, us): 39 K-214 K block steps of work 9.4-12.0 / 8.2-9.6 / 7.8-8.8; 418 K-933 K 12.6-15.1 / 10.2-14.8 /
+    // 14.4-21.3; 1.18 M 17.7 / 19.9 / 29.6 - the waves that short slots leave idle cost what the long ones gain
+    // once the launch holds enough work.
+    if (n_split > 0 && options().spmm_waves == 0) {
+        const long long work = (long long)nonzeros_vec * ceil_div(k, 128);
+        shape.waves = work <= (256LL << 10) ? 8 : work <= (1LL << 20) ? 4 : 2;
+        shape.blocks_per_wave = options().spmm_blocks_per_wave > 0 ? options().spmm_blocks_per_wave : 1;
+        shape.pipelined = options().spmm_pipe != 1;
+    }
+    const bool two_launches = options().spmm_parts_launches == 2;
     int *counters = static_cast<int *>(workspace);
     float *tiles = reinterpret_cast<float *>(static_cast<unsigned char *>(workspace) +
-                                             (n_split > 0 ? partial_tile_counter_bytes(workspace_bytes) : 0));
+                                             (n_split > 0 ? row_parts_counter_bytes(workspace_bytes) : 0));
     switch (vec_length) {
-    case 1: return launch_parts_v<1>(shape, k, n_slots, slots, parts_max, column_indices, values, rhs, out, counters, tiles, stream);
-    case 2: return launch_parts_v<2>(shape, k, n_slots, slots, parts_max, column_indices, values, rhs, out, counters, tiles, stream);
-    case 4: return launch_parts_v<4>(shape, k, n_slots, slots, parts_max, column_indices, values, rhs, out, counters, tiles, stream);
-    case 8: return launch_parts_v<8>(shape, k, n_slots, slots, parts_max, column_indices, values, rhs, out, counters, tiles, stream);
+    case 1: return launch_parts_v<1>(shape, k, n_slots, n_split, two_launches, slots, parts_max, column_indices, values, rhs, out, counters, tiles, stream);
+    case 2: return launch_parts_v<2>(shape, k, n_slots, n_split, two_launches, slots, parts_max, column_indices, values, rhs, out, counters, tiles, stream);
+    case 4: return launch_parts_v<4>(shape, k, n_slots, n_split, two_launches, slots, parts_max, column_indices, values, rhs, out, counters, tiles, stream);
+    case 8: return launch_parts_v<8>(shape, k, n_slots, n_split, two_launches, slots, parts_max, column_indices, values, rhs, out, counters, tiles, stream);
     default: return hipErrorInvalidValue;
     }
 }

@@ -219,6 +219,7 @@ struct Options {
     int spmm_flat_piece = 0;    // split-row SpMM: nonzero vectors per wave (rounded up to 32), 0 = automatic
     int spmm_flat_launches = 0; // split-row SpMM: 1 = parts added inside the launch, 2 = by a second launch, 0 = automatic
     int spmm_flat_waves = 0;    // split-row SpMM: waves per workgroup, 0 = automatic
+    int spmm_parts_launches = 0;  // rows in parts: 1 = the parts of a split row meet inside the launch, 2 = a second launch adds them, 0 = automatic
     int spmm_flat_shared = 0;   // split-row SpMM: 1 = every row segment starts its own step, 2 = rows share steps, 0 = automatic
     int sddmm_slots = 0;
     int sddmm_block_waves = 0;
@@ -316,6 +317,20 @@ inline long long partial_tile_counter_bytes(long long workspace_bytes)
 inline long long partial_tile_workspace_for(long long tile_bytes)
 {
     return tile_bytes + (tile_bytes / 127 + 255) / 256 * 256 + 512;
+}
+
+// Rows in parts keep every arrival counter in a cache line of its own: counters that share a line queue up
+// behind each other at the memory side, where device-scope atomics are carried out.  A counter then takes 128
+// bytes and stands for at least 512 bytes of partial tiles, so a fifth of the workspace holds the counters of
+// whatever fits the rest.
+constexpr int kPartCounterStride = 32;  // ints
+inline long long row_parts_counter_bytes(long long workspace_bytes)
+{
+    return (workspace_bytes / 5 + 255) / 256 * 256;
+}
+inline long long row_parts_workspace_for(long long tile_bytes)
+{
+    return tile_bytes + (tile_bytes / 4 + 255) / 256 * 256 + 512;
 }
 
 // Rows in parts (csrc/spmm_mfma.hip, the kernel's PARTS variant): `slots` = the dispatch list of

@@ -447,8 +447,8 @@ class RowParts:
     def __init__(self, m_vec, row_offsets, limit_vec=0):
         import ctypes
         ro = np.ascontiguousarray(row_offsets, dtype=np.int32)
-        step = 512 if limit_vec <= 0 else (limit_vec + 63) // 64 * 64
-        room = m_vec + int(ro[m_vec] if m_vec > 0 else 0) // min(step, 512) + 64
+        step = 1152 if limit_vec <= 0 else (limit_vec + 63) // 64 * 64   # (the default limit is 1152 at least)
+        room = m_vec + 2 * (int(ro[m_vec] if m_vec > 0 else 0) // step) + 64
         slots = np.empty((room, 4), dtype=np.int32)
         counts = [ctypes.c_int(0) for _ in range(4)]
         st = _lib.lib().vs_spmm_row_parts(m_vec, ro.ctypes.data, limit_vec, slots.ctypes.data, room,
@@ -456,7 +456,7 @@ class RowParts:
         if st:
             _lib.check(st, "vs_spmm_row_parts")
         self.n_slots, self.n_split, self.parts_max, self.longest_part_vec = (c.value for c in counts)
-        self.slots = np.ascontiguousarray(slots[:self.n_slots])
+        self.slots = np.ascontiguousarray(slots[:self.n_slots + self.n_split])  # (one entry per split row behind the list)
 
 
 def spmm_row_parts_workspace_bytes(vec_length, k, n_split, parts_max):
