@@ -189,7 +189,8 @@ def cpu_baseline(pat, B, n_dense, flops, budget_s=12.0):
     }
 
 
-PMC_MODES = ["spmm", "spmm_largest", "spmm_dma", "spmm_split_rows", "sddmm", "attention", "attention_window"]
+PMC_MODES = ["spmm", "spmm_largest", "spmm_dma", "spmm_split_rows", "spmm_row_parts", "sddmm", "attention",
+             "attention_window"]
 
 
 def largest_sweep_point(cv):
@@ -218,7 +219,7 @@ def main():
                     help="counter-collection mode for `rocprofv3 --pmc`: a 64 MiB device copy of known size "
                          "(calibration), then ten eager launches of one kernel and nothing else: the headline SpMM "
                          "(config 2), the largest sweep point (2048 x 4608 at 90 %%), config 2 on the LDS-DMA gather "
-                         "variant, the split-row SpMM on Pareto-distributed rows, the config-4 SDDMM, the config-5 "
+                         "variant, the split-row SpMM and the SpMM with rows in parts on Pareto-distributed rows, the config-4 SDDMM, the config-5 "
                          "attention layer with its plan, or that layer with a plain 513-wide window mask")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -294,6 +295,16 @@ def main():
                 kprob.spmm(kBd, kernel="wmma", out=kout, split_rows=True)
             info["algorithmic_bytes"] = spmm_algorithmic_bytes(kpat, 256)
             info["nonzero_vectors"] = int(kpat.nnz_vec)
+        elif args.pmc == "spmm_row_parts":
+            kpat, kB = skewed_point(cv, np)
+            kprob = ops.DeviceProblem(kpat, sort=True)
+            kBd = torch.from_numpy(kB).cuda()
+            kout = torch.empty((kpat.m, 256), dtype=torch.float16, device="cuda")
+            for _ in range(10):
+                kprob.spmm_row_parts(kBd, out=kout)
+            info["algorithmic_bytes"] = spmm_algorithmic_bytes(kpat, 256)
+            info["nonzero_vectors"] = int(kpat.nnz_vec)
+            info["kernel_source_tag"] = kernel_source_tag(*SPMM_SOURCES)
         elif args.pmc == "sddmm":
             for _ in range(10):
                 sddmm_step()

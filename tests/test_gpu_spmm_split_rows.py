@@ -155,21 +155,20 @@ def test_device_problem_switch_and_bad_arguments(gpu):
     out = prob.spmm(torch.from_numpy(B).cuda(), split_rows=True)
     torch.cuda.synchronize()
     assert_parity(out.cpu().numpy(), _oracle(pat, B), "DeviceProblem(split_rows=True)")
-    # split_rows=None: a dense row among short ones goes to the split schedule (its workspace appears), uniform
-    # rows do not; both give the oracle's result
+    # split_rows=None: a dense row among short ones is dispatched in parts (its list and their workspace appear),
+    # uniform rows are not; both give the oracle's result
     lone = _from_lengths([2048] + [40] * 255, 2048, 8, seed=13)
     Bl = cv.dense_uniform(2048, 128, seed=14)
     p_lone = ops.DeviceProblem(lone)
-    assert ops.split_rows_pays(lone.m_vec, lone.nnz_vec, 2048)
     got = p_lone.spmm(torch.from_numpy(Bl).cuda(), split_rows=None)
     torch.cuda.synchronize()
-    assert p_lone._workspace is not None
+    assert p_lone.row_parts(0)[0].n_split == 1 and p_lone.row_parts(0)[2] is not None
     assert_parity(got.cpu().numpy(), _oracle(lone, Bl), "split_rows=None, one dense row")
     even = cv.random_values(cv.uniform_pattern(256, 2048, 0.9, seed=15, vec_length=8), 16)
     p_even = ops.DeviceProblem(even)
     got = p_even.spmm(torch.from_numpy(Bl).cuda(), split_rows=None)
     torch.cuda.synchronize()
-    assert p_even._workspace is None
+    assert p_even.row_parts(0)[0].n_split == 0 and p_even.row_parts(0)[2] is None and p_even._workspace is None
     assert_parity(got.cpu().numpy(), _oracle(even, Bl), "split_rows=None, uniform rows")
     L = _lib.lib()
     args = [pat.m_vec, 4, 64, 1024, pat.nnz_vec, 0, prob.row_offsets.data_ptr(), prob.column_indices.data_ptr(),

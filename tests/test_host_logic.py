@@ -78,7 +78,7 @@ def test_device_problem_reads_the_row_statistics():
 
 
 def test_split_row_choice_follows_the_row_lengths():
-    """The rule behind DeviceProblem.spmm(split_rows=None), on the row-length shapes it was measured on."""
+    """Where the split-row schedule is ahead of the row-length hints, on the row-length shapes it was measured on."""
     pays = ops.split_rows_pays
     # one dense row among rows of a hundred vectors: pays up to 1024 rows
     for m_vec in (64, 256, 1024):

@@ -488,7 +488,8 @@ def split_rows_pays(m_vec, nonzeros_vec, longest_row_vec):
     (one dense row among rows of a hundred) holds its workgroups for 11.1-12.0 us on up to 1024 rows where the split
     schedule needs 9.8-11.4 us; on 2048 rows the hinted schedule is ahead (12.5 against 14.9 us), as it is on milder
     skew (Pareto or log-normal lengths, longest row 6 to 18 mean lengths: 1024 Pareto rows 13.4 against 16.9 us) and
-    on uniform or binomial lengths (by 1.6 to 2 times)."""
+    on uniform or binomial lengths (by 1.6 to 2 times).  (Rows in parts, DeviceProblem.spmm_row_parts, are ahead
+    of both on all of these; the rule is for callers that have a workspace but no dispatch list.)"""
     if m_vec <= 0 or m_vec > 1024 or nonzeros_vec < 8192:
         return False
     return longest_row_vec * m_vec >= 25.0 * nonzeros_vec
@@ -547,13 +548,19 @@ class DeviceProblem:
         batched entry point with batch = 1, which also takes the pattern's nonzero count and longest row and
         sizes its workgroups by the real row lengths instead of by n; with split_rows (MFMA path) on the
         schedule that cuts the nonzero range into equal pieces, with a workspace this object owns.
-        split_rows=None chooses between those two from the row lengths (see split_rows_pays)."""
+        split_rows=None chooses from the row lengths: rows in parts (spmm_row_parts) where the pattern has rows
+        long enough to be split, else the row-length hints."""
         k = rhs_matrix.shape[1]
         if out is None:
             out = torch.empty((self.m_vec * self.vec_length, k), dtype=out_dtype, device=rhs_matrix.device)
         if split_rows is None:
-            split_rows = kernel == "wmma" and k % 4 == 0 and split_rows_pays(self.m_vec, self.nnz_vec,
-                                                                            self.longest_row_vec)
+            # rows in parts wherever the dispatch list splits a row (measured ahead of both other schedules on
+            # Pareto lengths and on a dense row among short ones, 64 to 2048 rows; within 4 % on log-normal lengths),
+            # else the row-length hints
+            if kernel == "wmma" and k % 4 == 0 and out.dtype == torch.float16 and self.n * k < 2 ** 31 \
+                    and self.row_parts(0)[0].n_split > 0:
+                return self.spmm_row_parts(rhs_matrix, out=out, stream=stream)
+            split_rows = False
             row_length_hint = True
         if split_rows and kernel == "wmma":
             need = spmm_workspace_bytes(self.m_vec, self.vec_length, k, self.n, self.nnz_vec)
