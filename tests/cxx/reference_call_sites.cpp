@@ -181,6 +181,33 @@ int main()
                     std::chrono::duration<double, std::micro>(t2 - t0).count() / calls, calls);
     }
 
+    // the same operator with long rows dispatched in parts: the host makes the dispatch list (limit 64 here, so
+    // that several of these short rows are split), the entry point takes it in place of the swizzle and the offsets
+    {
+        int n_slots = 0, n_split = 0, parts_max = 0, longest = 0;
+        std::vector<int> slots(4 * (size_t)(m_vec + 2 * (nnz_vec / 64) + 1));
+        ok &= vs_spmm_row_parts(m_vec, row_offsets.data(), 64, slots.data(), (int)(slots.size() / 4), &n_slots, &n_split,
+                                &parts_max, &longest) == 0;
+        slots.resize(4 * (size_t)(n_slots + n_split));
+        int *d_slots = to_device(slots);
+        const long long bytes = vs_wmma_spmm_row_parts_workspace_bytes(V, k_dense, n_split, parts_max);
+        void *workspace = nullptr;
+        HIP_OK(hipMalloc(&workspace, (size_t)bytes));
+        HIP_OK(hipMemset(workspace, 0, (size_t)bytes));  // zeroed once, before the first use
+        for (int call = 0; call < 2; ++call) {
+            HIP_OK(hipMemset(d_out_h, 0x7f, (size_t)m_vec * V * k_dense * sizeof(half)));
+            HIP_OK((hipError_t)vs_wmma_spmm_f16_row_parts(V, k_dense, n, n_slots, d_slots, n_split, parts_max, nnz_vec, longest,
+                                                          d_cols, d_values, d_rhs, d_out_h, workspace, bytes, nullptr));
+            HIP_OK(hipDeviceSynchronize());
+            fetch_h(d_out_h, want_spmm.size());
+            ok &= close_enough(call == 0 ? "vs_wmma_spmm_f16_row_parts" : "vs_wmma_spmm_f16_row_parts again", got_f, want_spmm);
+        }
+        std::printf("%-22s %d slots, %d rows in up to %d parts\n", "", n_slots, n_split, parts_max);
+        ok &= n_split > 0;
+        HIP_OK(hipFree(workspace));
+        HIP_OK(hipFree(d_slots));
+    }
+
     HIP_OK(hipStreamDestroy(stream));
     for (void *p : {(void *)d_row_indices, (void *)d_row_offsets, (void *)d_cols, (void *)d_values, (void *)d_rhs,
                     (void *)d_lhs_s, (void *)d_rhs_s, (void *)d_out_h, (void *)d_out_f, (void *)d_sd_h, (void *)d_sd_f})
