@@ -54,6 +54,15 @@ def test_cli_end_to_end(gpu, tmp_path):
         assert spmm_benchmark.main([path, "128", "8", str(kernel), "1", "1", "1", "1"]) == 0
         assert sddmm_benchmark.main([path, "64", "4", str(kernel), "1", "0", "1", "1", "1"]) == 0
     assert spmm_benchmark.main(["synthetic:256,512,0.9,1", "64", "4", "0", "0", "1", "1", "1"]) == 0
+    assert spmm_benchmark.main([path, "128", "8", "0", "2", "1", "1", "1"]) == 0       # rows in parts (nothing to split)
+    lengths = np.array([1500] + [20] * 63)                                             # a row that is split
+    ro = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    ci = np.concatenate([np.sort(np.random.default_rng(i).choice(2048, n, replace=False)) for i, n in enumerate(lengths)])
+    skew = str(tmp_path / "skew.smtx")
+    cv.write_smtx(skew, 64, 2048, ro, ci.astype(np.int32))
+    assert spmm_benchmark.main([skew, "128", "8", "0", "2", "1", "1", "1"]) == 0
+    assert spmm_benchmark.main([skew, "128", "8", "1", "2", "1", "1", "1"]) == 1       # only on the MFMA path
+    assert spmm_benchmark.main([skew, "128", "8", "0", "3", "1", "1", "1"]) == 1
     assert spmm_benchmark.main([path, "128", "8", "0", "0", "1", "0", "1"]) == 0       # dense baseline
     assert sddmm_benchmark.main([path, "64", "8", "0", "0", "0", "1", "0", "1"]) == 0   # dense baseline
     assert spmm_benchmark.main([path, "128", "8", "2", "0", "0", "1", "1"]) == 1       # Sputnik: unsupported

@@ -7,7 +7,8 @@
     k        dense width (columns of B and C)
     v        vector length, 1 / 2 / 4 / 8
     kernel   0 = MFMA path (wmmaSpmm), 1 = fine-grained path (cudaSpmm); 2, 3 (Sputnik, cuSPARSE) unsupported
-    sort     1 = rows dispatched longest first (SortedRowSwizzle), 0 = in order
+    sort     1 = rows dispatched longest first (SortedRowSwizzle), 0 = in order; 2 (MFMA path; not in the
+             reference) = longest first with rows far longer than the rest dispatched in parts (vs_spmm_row_parts)
     function 1 = verify the result, 0 = skip
     sparse   1 = SpMM, 0 = dense fp16 GEMM baseline (hipBLASLt through torch); 2 (Blocked-ELL) unsupported
     mixed    1 = fp16 operands; 0 (fp32) unsupported, as in the reference's stubs
@@ -65,14 +66,23 @@ def main(argv=None):
     rhs = refgen.make_dense_matrix(n, k)
     values = refgen.make_dense_matrix(1, pat.nnz).reshape(pat.nnz_vec, v)
     pat = pat.with_values(values)
+    if sort not in (0, 1, 2) or (sort == 2 and (kernel != 0 or k % 4 != 0)):
+        print("Unsupported Sort")
+        return 1
     prob = ops.DeviceProblem(pat, sort=bool(sort))
     b = torch.from_numpy(rhs).cuda()
     out = torch.empty((m, k), dtype=torch.float16, device="cuda")
     name = "wmma" if kernel == 0 else "cuda"
     print("Using MFMA" if kernel == 0 else "Using fine-grained VALU")
-    prob.spmm(b, kernel=name, out=out)
+    if sort == 2:
+        parts = prob.row_parts(0)[0]
+        print("Rows in parts: %d slots, %d rows in up to %d parts" % (parts.n_slots, parts.n_split, parts.parts_max))
+        step = lambda: prob.spmm_row_parts(b, out=out)
+    else:
+        step = lambda: prob.spmm(b, kernel=name, out=out)
+    step()
     torch.cuda.synchronize()
-    us = time_launches(torch, lambda: prob.spmm(b, kernel=name, out=out))
+    us = time_launches(torch, step)
     print("SpMM %s V=%d: %.2f us, %.2f effective TFLOP/s (2*nnz*k)" % (name, v, us, 2.0 * pat.nnz * k / us * 1e-6))
     if func:
         ref = np.zeros((m, k), dtype=np.float64)
