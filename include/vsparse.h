@@ -452,8 +452,8 @@ int vs_wmma_spmm_launch_shape(int batch, int m_vec, int vec_length, int k, int n
  * per wave of the split-row SpMM, rounded up to 32, 0 = automatic), "spmm_flat_waves"
  * (its waves per workgroup, 1..16, 0 = automatic), "spmm_flat_launches" (1 = partial tiles
  * added inside the launch, 2 = by a second launch, 0 = automatic), "spmm_parts_launches" (rows in
- * parts: 1 = the parts of a split row meet inside the launch, 2 = a second launch adds them, 0 = automatic,
- * which is 1; same bits either way), "spmm_flat_shared" (1 = every
+ * parts: 1 = the parts of a split row meet inside the launch, 2 = a second launch adds them, 0 = automatic -
+ * the second launch on small problems; same bits either way), "spmm_flat_shared" (1 = every
  * row segment of the split-row SpMM starts a 32-vector step of its own, 2 = consecutive rows share
  * steps, 0 = automatic), "sddmm_slots" (waves per
  * vector row, 0 = automatic), "sddmm_group" (16-vector groups per wave step of the

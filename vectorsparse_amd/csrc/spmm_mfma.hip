@@ -934,7 +934,13 @@ int launch_spmm_mfma_row_parts(int vec_length, int k, int n, int n_slots, const 
         shape.blocks_per_wave = options().spmm_blocks_per_wave > 0 ? options().spmm_blocks_per_wave : 1;
         shape.pipelined = options().spmm_pipe != 1;
     }
-    const bool two_launches = options().spmm_parts_launches == 2;
+    // The meeting inside the launch costs the last part of a row three memory round trips, a second launch costs a
+    // launch: small problems are ahead with the second launch (64 / 256 Pareto rows 6.8 / 7.9 against 7.7 / 8.6 us, a
+    // dense row among 63 / 255 short ones 6.8 / 7.0 against 7.8 / 7.8), from about 200 K block steps on the one launch
+    // is (a dense row among 1023: 8.8 against 10.7 us; 1024 Pareto rows 11.0 against 13.1).
+    const bool two_launches =
+        options().spmm_parts_launches == 2 ||
+        (options().spmm_parts_launches == 0 && n_split > 0 && (long long)nonzeros_vec * ceil_div(k, 128) <= 160 * 1024);
     int *counters = static_cast<int *>(workspace);
     float *tiles = reinterpret_cast<float *>(static_cast<unsigned char *>(workspace) +
                                              (n_split > 0 ? row_parts_counter_bytes(workspace_bytes) : 0));
