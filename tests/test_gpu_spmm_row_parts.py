@@ -176,3 +176,77 @@ def test_device_problem_entry(gpu):
     ref = _oracle(pat, B)
     assert_parity(out.cpu().numpy(), ref, "DeviceProblem.spmm_row_parts")
     assert_parity(out2.cpu().numpy(), ref, "DeviceProblem.spmm_row_parts(limit_vec=1024)")
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_patterns_limits_and_options(gpu, seed):
+    """Random row-length distributions, vector lengths, dense widths, limits and launch shapes against the oracle."""
+    rng = np.random.default_rng(7000 + seed)
+    V = int(rng.choice([1, 2, 4, 8]))
+    m_vec = int(rng.integers(1, 120))
+    n = int(rng.integers(64, 3000))
+    kind = seed % 4
+    if kind == 0:      # heavy tail
+        lengths = np.minimum((rng.pareto(1.1, m_vec) + 0.05) * n * 0.1, n)
+    elif kind == 1:    # a few dense rows among short and empty ones
+        lengths = np.where(rng.random(m_vec) < 0.1, n, rng.integers(0, 20, m_vec))
+    elif kind == 2:    # uniform density
+        lengths = rng.binomial(n, rng.uniform(0.05, 0.9), size=m_vec)
+    else:              # every row dense
+        lengths = np.full(m_vec, n)
+    pat = _from_lengths(lengths.astype(np.int64), n, V, seed=seed)
+    N = int(rng.choice([4, 8, 12, 40, 64, 100, 128, 200, 256, 264, 388]))
+    B = cv.dense_uniform(n, N, seed=seed + 1)
+    limit = int(rng.choice([0, 1, 64, 65, 200, 512, 1000]))
+    opts = {"spmm_parts_launches": int(rng.integers(0, 3))}
+    if rng.random() < 0.5:
+        opts["spmm_waves"] = int(rng.choice([1, 2, 3, 4, 8]))
+    if rng.random() < 0.5:
+        opts["spmm_pipe"] = int(rng.integers(1, 3))
+    if rng.random() < 0.3:
+        opts["spmm_cols_per_lane"] = int(rng.choice([4, 8]))
+    if rng.random() < 0.3:
+        opts["spmm_blocks_per_wave"] = int(rng.choice([1, 2, 4]))
+    what = "seed %d V%d m_vec%d n%d N%d nnz_vec%d limit %d %s" % (seed, V, m_vec, n, N, pat.nnz_vec, limit, opts)
+    print(what, flush=True)
+    got, parts = _run(pat, B, limit=limit, options=opts)
+    assert_parity(got, _oracle(pat, B), what)
+    for i in np.nonzero(np.diff(pat.row_offsets) == 0)[0]:
+        assert not got[i * V:(i + 1) * V].any(), "empty vector row %d must be written as zeros" % i
+
+
+def test_hip_graph_replays_equal_eager(gpu):
+    """The entry point is capturable (no allocation, no memset, no synchronisation inside) and every replay finds the
+    arrival counters as the one before left them: replays with fresh operands in between equal the eager result."""
+    rng = np.random.default_rng(3)
+    lengths = np.minimum((rng.pareto(1.5, 400) + 0.3) * 100, 3000).astype(np.int64)
+    pat = _from_lengths(lengths, 3000, 8, seed=4)
+    prob = ops.DeviceProblem(pat)
+    assert prob.row_parts(0)[0].n_split > 0
+    g = torch.Generator(device="cuda").manual_seed(5)
+    Bd = torch.randn((3000, 128), device="cuda", generator=g).half()
+    out = torch.empty((pat.m, 128), dtype=torch.float16, device="cuda")
+    for launches in (1, 2):
+        with _lib.thread_options(spmm_parts_launches=launches):
+            prob.spmm_row_parts(Bd, out=out)
+            torch.cuda.synchronize()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                prob.spmm_row_parts(Bd, out=out)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                prob.spmm_row_parts(Bd, out=out)
+            for rep in range(4):
+                Bd.copy_(torch.randn(Bd.shape, device="cuda", generator=g).half())   # new operand, same buffer
+                prob.spmm_row_parts(Bd, out=out)
+                torch.cuda.synchronize()
+                want = out.clone()
+                out.zero_()
+                torch.cuda.synchronize()
+                graph.replay()
+                torch.cuda.synchronize()
+                assert torch.equal(out, want), "replay %d, %d launch(es)" % (rep, launches)
+    assert_parity(out.cpu().numpy(), _oracle(pat, Bd.cpu().numpy()), "rows in parts under a HIP graph")
