@@ -282,6 +282,18 @@ int vs_wmma_spmm_f16_row_parts(int vec_length, int k, int n, int n_slots, const 
                                const int *column_indices, const void *values, const void *rhs_matrix,
                                void *output_matrix, void *workspace, long long workspace_bytes, void *stream);
 
+/*
+ * The SDDMM of vs_wmma_sddmm_f16 (sddmm::wmmaSddmm, include/wmma_sddmm.cuh:17-24; same operands, same contract for
+ * the output values) driven by the dispatch list of vs_spmm_row_parts in place of row_indices and row_offsets: rows
+ * far longer than the rest are served as several slots, each by waves of its own - the outputs of a part are the
+ * part's nonzeros, so there is nothing to add up and no workspace.  The list needs only its n_slots entries, in
+ * device memory, 16-byte aligned.  Requires k % 8 == 0 (else 801).  No counterpart in the reference, whose sorted
+ * order only reorders the dispatch of whole rows (include/bm_test_utils.h:200-215).
+ */
+int vs_wmma_sddmm_f16_row_parts(int k, int n, int n_slots, const int *slots, int nonzeros_vec,
+                                const int *col_indices, const void *lhs_matrix, const void *rhs_matrix,
+                                void *output_values, int vec_length, void *stream);
+
 int vs_cuda_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
                              int longest_row_vec, const int *row_indices, const int *row_offsets,
                              const int *column_indices,

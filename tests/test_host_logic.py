@@ -67,7 +67,7 @@ def test_device_problem_reads_the_row_statistics():
     ro, ci = cv._pattern_from_lengths(rng, 1024, 4608, lengths)
     heavy = ops.DeviceProblem(cv.ColVecCSR(1024, 4608, 8, ro, ci), sort=True, device="cpu")
     assert heavy.longest_row_vec == 4608 and heavy.nnz_vec == int(lengths.sum())
-    assert heavy.skewed                                    # SDDMM takes the nonzero-range schedule by default
+    assert heavy.skewed                                    # SDDMM takes rows in parts by default (the nonzero-range schedule where that entry does not apply)
     swz = heavy.row_indices.numpy()
     assert sorted(swz.tolist()) == list(range(1024)) and np.all(np.diff(lengths[swz]) <= 0)
     even = ops.DeviceProblem(cv.uniform_pattern(1024, 4608, 0.9, seed=1, vec_length=8), device="cpu")

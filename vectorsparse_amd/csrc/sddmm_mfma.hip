@@ -14,6 +14,8 @@
 // storage, no barrier).  A wave owns (vector row, slot s) and walks super-groups of GRP*16 vectors
 // s, s + slots, ... with all GRP*KS loads of a super-group in flight together; the lhs slices of the
 // vector row stay in registers across super-groups when K <= 256.
+#include <type_traits>
+
 #include "vs_common.hpp"
 
 namespace vs {
@@ -32,7 +34,10 @@ __device__ __forceinline__ void store_group(OutT *out, int j, int g, const float
 }
 
 // KS > 0: K <= 32*KS, lhs slices preloaded; KS == 0: any K % 8 == 0, lhs re-read per super-group.
-template <int V, int KS, int GRP, typename OutT>
+// PARTS: `row_indices` is a dispatch list of row parts (vs_spmm_row_parts: four ints per slot, {vector row, first
+// nonzero, end, part info}; row_offsets is not read, m_vec counts the slots): rows far longer than the rest are
+// served as several slots, each by its own waves.  The outputs of a part are the part's nonzeros - nothing to add up.
+template <int V, int KS, int GRP, typename OutT, bool PARTS = false>
 __global__ void __launch_bounds__(1024)
 sddmm_mfma_kernel(int m_vec, int K, int slots, int waves_per_block, const int *__restrict__ row_indices,
                   const int *__restrict__ row_offsets, const int *__restrict__ col_indices,
@@ -57,13 +62,21 @@ sddmm_mfma_kernel(int m_vec, int K, int slots, int waves_per_block, const int *_
     const int s = (int)(wg % (unsigned)slots);
     // the row's extent is requested for the identity order together with the swizzle entry, and again only if
     // the entry names another row: one dependent load less in the common case
-    const int row = row_indices[slot];
-    int beg = row_offsets[slot];
-    int end = row_offsets[slot + 1];
-    asm volatile("" : "+s"(beg), "+s"(end));  // keeps these two requests apart from the dependent ones below
-    if (row != slot) {
-        beg = row_offsets[row];
-        end = row_offsets[row + 1];
+    int row, beg, end;
+    if constexpr (PARTS) {
+        const int4_t d = reinterpret_cast<const int4_t *>(row_indices)[slot];  // one request for everything
+        row = d[0];
+        beg = d[1];
+        end = d[2];
+    } else {
+        row = row_indices[slot];
+        beg = row_offsets[slot];
+        end = row_offsets[slot + 1];
+        asm volatile("" : "+s"(beg), "+s"(end));  // keeps these two requests apart from the dependent ones below
+        if (row != slot) {
+            beg = row_offsets[row];
+            end = row_offsets[row + 1];
+        }
     }
     const int n_super = (end - beg + SUPER - 1) / SUPER;
     if (s >= n_super) return;
@@ -277,7 +290,7 @@ static int launch_one(int m_vec, int k, int nonzeros_vec, const int *row_indices
 {
     const int kWavesPerBlock = options().sddmm_block_waves > 0 ? options().sddmm_block_waves : 8;
     if constexpr (KS > 0) {
-        if (batch.algorithm == 2) {
+        if (batch.algorithm == 2 && !batch.row_parts) {
             // super-groups per wave: enough waves to fill the chip (~8192), at least `min_supers` of them per
             // wave so that the lhs slices and the row search are amortised, at most 16
             const long long n_supers = ((long long)nonzeros_vec + 16 * GRP - 1) / (16 * GRP);
@@ -298,6 +311,16 @@ static int launch_one(int m_vec, int k, int nonzeros_vec, const int *row_indices
     const long long waves = (long long)m_vec * slots;
     const long long blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks > 0x7fffffffLL || blocks * kWavesPerBlock > 0xffffffffLL) return hipErrorNotSupported;
+    if (batch.row_parts) {  // m_vec counts the slots of the dispatch list that row_indices points to
+        if constexpr (std::is_same<OutT, half_t>::value) {
+            hipLaunchKernelGGL((sddmm_mfma_kernel<V, KS, GRP, OutT, true>), dim3((unsigned)blocks, (unsigned)batch.count),
+                               dim3(64 * kWavesPerBlock), 0, stream, m_vec, k, slots, kWavesPerBlock, row_indices, row_offsets,
+                               col_indices, lhs, rhs, out, batch.stride_a, batch.stride_b, batch.stride_out);
+            return (int)hipGetLastError();
+        } else {
+            return hipErrorNotSupported;
+        }
+    }
     hipLaunchKernelGGL((sddmm_mfma_kernel<V, KS, GRP, OutT>), dim3((unsigned)blocks, (unsigned)batch.count), dim3(64 * kWavesPerBlock), 0, stream,
                        m_vec, k, slots, kWavesPerBlock, row_indices, row_offsets, col_indices, lhs, rhs, out,
                        batch.stride_a, batch.stride_b, batch.stride_out);
@@ -385,13 +408,15 @@ int launch_sddmm_mfma(int m_vec, int k, int n, int nonzeros_vec, const int *row_
     // Contraction lengths off a multiple of 8 (rows of the dense operands then start at any 2-byte boundary, out of
     // reach of 128-bit loads) run on the fine-grained kernel's scalar-load variant, whatever the algorithm: the
     // whole of k is contracted on both paths (the reference's MMA kernels drop k % 64, src/wmma_sddmm.cu:88-120).
-    if (k % 8 != 0)
+    if (k % 8 != 0) {
+        if (batch.row_parts) return hipErrorNotSupported;  // (the fine-grained kernel takes no dispatch list)
         return launch_sddmm_valu<OutT>(m_vec, k, n, nonzeros_vec, row_indices, row_offsets, col_indices, lhs, rhs, out,
                                        vec_length, stream, batch);
+    }
     // algorithm 0 (automatic): vectors of 1, 2 or 4 rows fill 1/16 to 4/16 of an MFMA tile, and on masks of few
     // nonzeros the fine-grained kernel (dot products on the vector ALU, reduced across lanes with DPP) is ahead:
     // over the M = N = 512..4096, K = 64..256 grid by 5-40 % below these nonzero counts, behind above them.
-    if (batch.algorithm == 0 && vec_length <= 4) {
+    if (batch.algorithm == 0 && vec_length <= 4 && !batch.row_parts) {
         const long long total = (long long)nonzeros_vec * batch.count;
         long long limit = 0;
         if (vec_length == 1) limit = 800000;

@@ -260,6 +260,7 @@ struct Batch {
     int longest_row_vec = -1;  // SpMM: nonzero vectors of the longest row when the caller knows them (same)
     int long_rows = -1;        // SpMM, rows ordered by length: leading entries of row_indices with more than 512 vectors
     int algorithm = 0;         // SDDMM on MFMA: 2 = waves split the nonzero range, else (row, slot) per wave
+    bool row_parts = false;    // SDDMM on MFMA: row_indices is a dispatch list of row parts, m_vec counts its slots
 };
 
 // Launch shape of the MFMA SpMM (spmm_mfma.hip), chosen on the host.

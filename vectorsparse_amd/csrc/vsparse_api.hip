@@ -641,6 +641,29 @@ int vs_wmma_spmm_f16_row_parts(int vec_length, int k, int n, int n_slots, const 
                                           workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
+int vs_wmma_sddmm_f16_row_parts(int k, int n, int n_slots, const int *slots, int nonzeros_vec, const int *col_indices,
+                                const void *lhs_matrix, const void *rhs_matrix, void *output_values, int vec_length,
+                                void *stream)
+{
+    if (!vec_ok(vec_length) || k < 0 || n < 0 || n_slots < 0 || nonzeros_vec < 0) return VS_ERROR_INVALID_VALUE;
+    if (n_slots == 0 || nonzeros_vec == 0) return VS_SUCCESS;
+    if (!slots || !aligned(slots, 16) || !col_indices || !output_values) return VS_ERROR_INVALID_VALUE;
+    if (k > 0 && (!lhs_matrix || !rhs_matrix)) return VS_ERROR_INVALID_VALUE;
+    if (!aligned(output_values, sizeof(half_t) * (size_t)vec_length)) return VS_ERROR_INVALID_VALUE;
+    if (k == 0)
+        return sddmm_zero_outputs(output_values, nonzeros_vec, vec_length, sizeof(half_t), 1, 0,
+                                  static_cast<hipStream_t>(stream));
+    if (k % 8 != 0) return VS_ERROR_NOT_SUPPORTED;
+    if (!aligned(lhs_matrix, 16) || !aligned(rhs_matrix, 16)) return VS_ERROR_INVALID_VALUE;
+    vs::Batch batch;
+    batch.algorithm = 1;
+    batch.row_parts = true;
+    return vs::launch_sddmm_mfma<half_t>(n_slots, k, n, nonzeros_vec, slots, nullptr, col_indices,
+                                         static_cast<const half_t *>(lhs_matrix), static_cast<const half_t *>(rhs_matrix),
+                                         static_cast<half_t *>(output_values), vec_length,
+                                         static_cast<hipStream_t>(stream), batch);
+}
+
 int vs_launch_floor_probe(int blocks, int threads_per_block, void *stream)
 {
     if (blocks < 1 || threads_per_block < 1 || threads_per_block > 1024) return VS_ERROR_INVALID_VALUE;

@@ -479,6 +479,20 @@ def spmm_row_parts(vec_length, k, n, parts, slots, nonzeros_vec, column_indices,
     return output_matrix
 
 
+def sddmm_row_parts(k, n, parts, slots, nonzeros_vec, col_indices, lhs_matrix, rhs_matrix, output_values, vec_length,
+                    stream=None):
+    """wmmaSddmm driven by a dispatch list of row parts (`parts`: a RowParts, `slots`: its list as a device int32
+    tensor).  Returns output_values."""
+    st = _lib.lib().vs_wmma_sddmm_f16_row_parts(
+        k, n, parts.n_slots, _expect(slots, torch.int32, "slots"), nonzeros_vec,
+        _expect(col_indices, torch.int32, "col_indices"), _expect(lhs_matrix, torch.float16, "lhs_matrix"),
+        _expect(rhs_matrix, torch.float16, "rhs_matrix"), _expect(output_values, torch.float16, "output_values"),
+        vec_length, _stream(stream))
+    if st:
+        _lib.check(st, "vs_wmma_sddmm_f16_row_parts")
+    return output_values
+
+
 LONG_ROW_VECTORS = 512  # rows beyond this are "long" for vs_wmma_spmm_f16_batched_sorted (eight 64-vector blocks)
 
 
@@ -577,6 +591,17 @@ class DeviceProblem:
         return fn(self.m_vec, self.vec_length, k, self.n, self.row_indices, self.row_offsets,
                   self.column_indices, self.values, rhs_matrix, out, stream)
 
+    def sddmm_row_parts(self, lhs_matrix, rhs_matrix, out=None, stream=None, limit_vec=256):
+        """SDDMM (MFMA path, fp16 output, k % 8 == 0) with long rows of the mask dispatched as several parts.  The
+        parts have nothing to add up, so the limit is low (measured at K = 64..256 on 256 to 2048 rows of Pareto
+        lengths and on a dense row among short ones: 128 to 512 vectors within 5 % of each other, 1152 20-70 % behind)."""
+        k = lhs_matrix.shape[1]
+        if out is None:
+            out = torch.empty((self.nnz_vec, self.vec_length), dtype=torch.float16, device=lhs_matrix.device)
+        parts, slots = self.row_parts(limit_vec)[:2]
+        return sddmm_row_parts(k, self.n, parts, slots, self.nnz_vec, self.column_indices, lhs_matrix, rhs_matrix, out,
+                               self.vec_length, stream)
+
     def sddmm(self, lhs_matrix, rhs_matrix, kernel="wmma", out_dtype=torch.float16, out=None, stream=None,
               algorithm=None):
         """SDDMM on the mask.  algorithm (MFMA path): 1 = a wave per (row, slot), 2 = waves split the nonzero
@@ -586,6 +611,10 @@ class DeviceProblem:
         if out is None:
             out = torch.empty((self.nnz_vec, self.vec_length), dtype=out_dtype, device=lhs_matrix.device)
         if algorithm is None:
+            # skewed masks: rows in parts (ahead of the nonzero-range schedule by 25-30 % at K = 64..256, and of the
+            # row kernel by 2.7-3.4 times, on Pareto lengths), where the entry point takes the shape
+            if self.skewed and kernel == "wmma" and k % 8 == 0 and k > 0 and out.dtype == torch.float16:
+                return self.sddmm_row_parts(lhs_matrix, rhs_matrix, out=out, stream=stream)
             algorithm = 2 if (self.skewed and k <= 256) else 0
         if kernel == "wmma":
             return sddmm.wmmaSddmm(self.m_vec, k, self.n, self.nnz_vec, self.row_indices, self.row_offsets,
