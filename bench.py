@@ -400,6 +400,21 @@ def main():
     _, skew_uniform_ms = time_graph(torch, lambda: uprob.spmm(kBd, out=kout), skew_steps, 3)
     _, skew_uniform_hint_ms = time_graph(torch, lambda: uprob.spmm(kBd, out=kout, row_length_hint=True), skew_steps, 3)
 
+    # ---- SDDMM on the same skewed pattern as a mask (K = 64): row kernel, nonzero-range schedule, rows in parts
+    kg = torch.Generator(device="cuda").manual_seed(11)
+    klhs = torch.randn((kpat.m, 64), device="cuda", generator=kg).half()
+    krhs = torch.randn((kpat.n, 64), device="cuda", generator=kg).half()
+    ksout = torch.empty((kpat.nnz_vec, 8), dtype=torch.float16, device="cuda")
+    _, sk_sd_row_ms = time_graph(torch, lambda: kprob.sddmm(klhs, krhs, out=ksout, algorithm=1), skew_steps, 3)
+    _, sk_sd_flat_ms = time_graph(torch, lambda: kprob.sddmm(klhs, krhs, out=ksout, algorithm=2), skew_steps, 3)
+    ksref = ksout.clone()
+    _, sk_sd_parts_ms = time_graph(torch, lambda: kprob.sddmm_row_parts(klhs, krhs, out=ksout), skew_steps, 3)
+    torch.cuda.synchronize()
+    if not torch.equal(ksout, ksref):   # (the same arithmetic per output on every schedule)
+        raise SystemExit("SDDMM with rows in parts and on the nonzero-range schedule disagree on the skewed point")
+    _, sk_sd_uniform_ms = time_graph(torch, lambda: uprob.sddmm(klhs, krhs, out=ksout[:upat.nnz_vec], algorithm=1),
+                                     skew_steps, 3)
+
     # ---- SDDMM config 4
     _, sddmm_ms = time_graph(torch, sddmm_step, dev_steps, args.warmup)
     sddmm_flops = 2.0 * mask.nnz * 64
@@ -509,6 +524,10 @@ def main():
                                  "uniform_rows_same_nonzeros_us": skew_uniform_ms * 1e3,
                                  "uniform_rows_same_nonzeros_hinted_us": skew_uniform_hint_ms * 1e3,
                                  "row_parts_over_uniform_hinted": skew_parts_ms / skew_uniform_hint_ms},
+            "sddmm_skewed_rows": {"workload": "the same pattern as a mask, K=64", "row_kernel_us": sk_sd_row_ms * 1e3,
+                                  "nonzero_range_schedule_us": sk_sd_flat_ms * 1e3, "row_parts_entry_us": sk_sd_parts_ms * 1e3,
+                                  "uniform_rows_same_nonzeros_us": sk_sd_uniform_ms * 1e3,
+                                  "row_parts_over_uniform": sk_sd_parts_ms / sk_sd_uniform_ms},
             "sddmm_config4_k64": dict(
                 hbm(sddmm_bytes, sddmm_ms, sddmm_traffic, traffic_note=sddmm_note, kernel="sddmm_mfma_kernel<V=8>"),
                 ms=sddmm_ms, tflops=sddmm_flops / (sddmm_ms * 1e-3) * 1e-12, dense_product_us=sddmm_dense_ms * 1e3,

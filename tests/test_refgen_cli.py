@@ -62,6 +62,8 @@ def test_cli_end_to_end(gpu, tmp_path):
     cv.write_smtx(skew, 64, 2048, ro, ci.astype(np.int32))
     assert spmm_benchmark.main([skew, "128", "8", "0", "2", "1", "1", "1"]) == 0
     assert spmm_benchmark.main([skew, "128", "8", "1", "2", "1", "1", "1"]) == 1       # only on the MFMA path
+    assert sddmm_benchmark.main([skew, "64", "8", "0", "1", "2", "1", "1", "1"]) == 0   # SDDMM, rows in parts
+    assert sddmm_benchmark.main([skew, "60", "8", "0", "1", "2", "1", "1", "1"]) == 1   # needs k % 8 == 0
     assert spmm_benchmark.main([skew, "128", "8", "0", "3", "1", "1", "1"]) == 1
     assert spmm_benchmark.main([path, "128", "8", "0", "0", "1", "0", "1"]) == 0       # dense baseline
     assert sddmm_benchmark.main([path, "64", "8", "0", "0", "0", "1", "0", "1"]) == 0   # dense baseline

@@ -8,7 +8,8 @@
     v        vector length, 1 / 2 / 4 / 8
     kernel   0 = MFMA path (wmmaSddmm), 1 = cross-lane path (cudaSddmm); 2, 3 unsupported
     alg      0..2 accepted (one MFMA kernel serves the reference's three schedules), 3 rejected
-    sort     1 = rows dispatched longest first, 0 = in order
+    sort     1 = rows dispatched longest first, 0 = in order; 2 (MFMA path, k % 8 == 0; not in the reference) =
+             longest first with long rows dispatched in parts (vs_spmm_row_parts, vs_wmma_sddmm_f16_row_parts)
     function 1 = verify the result, 0 = skip
     sparse   1 = SDDMM, 0 = dense fp16 A*B^T baseline (hipBLASLt through torch)
     mixed    1 = fp16 operands; 0 unsupported
@@ -62,9 +63,18 @@ def main(argv=None):
     out = torch.empty((pat.nnz_vec, v), dtype=torch.float16, device="cuda")
     name = "wmma" if kernel == 0 else "cuda"
     print("Using MFMA" if kernel == 0 else "Using cross-lane VALU")
-    prob.sddmm(a, b, kernel=name, out=out, algorithm=alg)
+    if sort not in (0, 1, 2) or (sort == 2 and (kernel != 0 or k % 8 != 0)):
+        print("unsupported sort")
+        return 1
+    if sort == 2:
+        parts = prob.row_parts(256)[0]
+        print("Rows in parts: %d slots, %d rows in up to %d parts" % (parts.n_slots, parts.n_split, parts.parts_max))
+        step = lambda: prob.sddmm_row_parts(a, b, out=out)
+    else:
+        step = lambda: prob.sddmm(a, b, kernel=name, out=out, algorithm=alg)
+    step()
     torch.cuda.synchronize()
-    us = time_launches(torch, lambda: prob.sddmm(a, b, kernel=name, out=out, algorithm=alg))
+    us = time_launches(torch, step)
     print("SDDMM %s V=%d: %.2f us, %.2f effective TFLOP/s (2*nnz*k)" % (name, v, us, 2.0 * pat.nnz * k / us * 1e-6))
     if func:
         rows = np.repeat(np.arange(pat.m_vec), pat.row_lengths())
