@@ -202,6 +202,13 @@ int main()
             fetch_h(d_out_h, want_spmm.size());
             ok &= close_enough(call == 0 ? "vs_wmma_spmm_f16_row_parts" : "vs_wmma_spmm_f16_row_parts again", got_f, want_spmm);
         }
+        // the SDDMM on the same list: nothing to add up across parts, no workspace
+        HIP_OK(hipMemset(d_sd_h, 0x7f, (size_t)nnz_vec * V * sizeof(half)));
+        HIP_OK((hipError_t)vs_wmma_sddmm_f16_row_parts(k_contract, n, n_slots, d_slots, nnz_vec, d_cols, d_lhs_s, d_rhs_s,
+                                                       d_sd_h, V, nullptr));
+        HIP_OK(hipDeviceSynchronize());
+        fetch_h(d_sd_h, want_sddmm.size());
+        ok &= close_enough("vs_wmma_sddmm_f16_row_parts", got_f, want_sddmm);
         std::printf("%-22s %d slots, %d rows in up to %d parts\n", "", n_slots, n_split, parts_max);
         ok &= n_split > 0;
         HIP_OK(hipFree(workspace));
