@@ -268,31 +268,41 @@ int vs_wmma_spmm_f16_batched_sorted(int batch, int m_vec, int vec_length, int k,
  * nonzeros_vec and longest_part_vec size the launch as the hints of vs_wmma_spmm_f16_batched do.  The parts of
  * a split row leave fp32 partial tiles in `workspace` and the workgroup that brings the last one adds them in
  * ascending order (deterministic, no atomics on the output, nobody waits).  workspace: device memory, 16-byte
- * aligned, at least vs_wmma_spmm_row_parts_workspace_bytes(vec_length, k, n_split, parts_max) bytes (0 when no
+ * aligned, at least vs_wmma_spmm_row_parts_workspace_bytes(batch, vec_length, k, n_split, parts_max) bytes (0 when no
  * row is split), ZERO-FILLED before its first use; its arrival counters (an area that depends on
  * workspace_bytes alone) are left at zero by every call, so it serves any sequence of calls that do not
  * overlap, whatever their shapes, as long as it is passed with the same size.  Requires k % 4 == 0 and
- * n * k < 2^31, else 801.
+ * n * k < 2^31, else 801.  batch, stride_*: as in vs_wmma_spmm_f16_batched - `batch` problems share the pattern (and
+ * the list), problem b reads values + b * stride_values and rhs_matrix + b * stride_rhs and writes output_matrix +
+ * b * stride_output (strides in elements, 0 = shared operand; multiples of vec_length / 8 / 8); batch = 1 with
+ * strides 0 is the single operator.
  */
 int vs_spmm_row_parts(int m_vec, const int *row_offsets, int limit_vec, int *slots, int max_slots, int *n_slots,
                       int *n_split, int *parts_max, int *longest_part_vec);
-long long vs_wmma_spmm_row_parts_workspace_bytes(int vec_length, int k, int n_split, int parts_max);
-int vs_wmma_spmm_f16_row_parts(int vec_length, int k, int n, int n_slots, const int *slots, int n_split,
+long long vs_wmma_spmm_row_parts_workspace_bytes(int batch, int vec_length, int k, int n_split, int parts_max);
+int vs_wmma_spmm_f16_row_parts(int batch, int vec_length, int k, int n, int n_slots, const int *slots, int n_split,
                                int parts_max, int nonzeros_vec, int longest_part_vec,
-                               const int *column_indices, const void *values, const void *rhs_matrix,
-                               void *output_matrix, void *workspace, long long workspace_bytes, void *stream);
+                               const int *column_indices,
+                               const void *values, long long stride_values,
+                               const void *rhs_matrix, long long stride_rhs,
+                               void *output_matrix, long long stride_output,
+                               void *workspace, long long workspace_bytes, void *stream);
 
 /*
  * The SDDMM of vs_wmma_sddmm_f16 (sddmm::wmmaSddmm, include/wmma_sddmm.cuh:17-24; same operands, same contract for
  * the output values) driven by the dispatch list of vs_spmm_row_parts in place of row_indices and row_offsets: rows
  * far longer than the rest are served as several slots, each by waves of its own - the outputs of a part are the
  * part's nonzeros, so there is nothing to add up and no workspace.  The list needs only its n_slots entries, in
- * device memory, 16-byte aligned.  Requires k % 8 == 0 (else 801).  No counterpart in the reference, whose sorted
+ * device memory, 16-byte aligned.  Requires k % 8 == 0 (else 801).  batch, stride_*: as in vs_wmma_sddmm_f16_batched
+ * (the mask and its list shared, strides in elements, multiples of 8 / 8 / vec_length).  No counterpart in the reference, whose sorted
  * order only reorders the dispatch of whole rows (include/bm_test_utils.h:200-215).
  */
-int vs_wmma_sddmm_f16_row_parts(int k, int n, int n_slots, const int *slots, int nonzeros_vec,
-                                const int *col_indices, const void *lhs_matrix, const void *rhs_matrix,
-                                void *output_values, int vec_length, void *stream);
+int vs_wmma_sddmm_f16_row_parts(int batch, int k, int n, int n_slots, const int *slots, int nonzeros_vec,
+                                const int *col_indices,
+                                const void *lhs_matrix, long long stride_lhs,
+                                const void *rhs_matrix, long long stride_rhs,
+                                void *output_values, long long stride_output,
+                                int vec_length, void *stream);
 
 int vs_cuda_spmm_f16_batched(int batch, int m_vec, int vec_length, int k, int n, int nonzeros_vec,
                              int longest_row_vec, const int *row_indices, const int *row_offsets,

@@ -190,22 +190,23 @@ int main()
                                 &parts_max, &longest) == 0;
         slots.resize(4 * (size_t)(n_slots + n_split));
         int *d_slots = to_device(slots);
-        const long long bytes = vs_wmma_spmm_row_parts_workspace_bytes(V, k_dense, n_split, parts_max);
+        const long long bytes = vs_wmma_spmm_row_parts_workspace_bytes(1, V, k_dense, n_split, parts_max);
         void *workspace = nullptr;
         HIP_OK(hipMalloc(&workspace, (size_t)bytes));
         HIP_OK(hipMemset(workspace, 0, (size_t)bytes));  // zeroed once, before the first use
         for (int call = 0; call < 2; ++call) {
             HIP_OK(hipMemset(d_out_h, 0x7f, (size_t)m_vec * V * k_dense * sizeof(half)));
-            HIP_OK((hipError_t)vs_wmma_spmm_f16_row_parts(V, k_dense, n, n_slots, d_slots, n_split, parts_max, nnz_vec, longest,
-                                                          d_cols, d_values, d_rhs, d_out_h, workspace, bytes, nullptr));
+            HIP_OK((hipError_t)vs_wmma_spmm_f16_row_parts(1, V, k_dense, n, n_slots, d_slots, n_split, parts_max, nnz_vec,
+                                                          longest, d_cols, d_values, 0, d_rhs, 0, d_out_h, 0, workspace, bytes,
+                                                          nullptr));
             HIP_OK(hipDeviceSynchronize());
             fetch_h(d_out_h, want_spmm.size());
             ok &= close_enough(call == 0 ? "vs_wmma_spmm_f16_row_parts" : "vs_wmma_spmm_f16_row_parts again", got_f, want_spmm);
         }
         // the SDDMM on the same list: nothing to add up across parts, no workspace
         HIP_OK(hipMemset(d_sd_h, 0x7f, (size_t)nnz_vec * V * sizeof(half)));
-        HIP_OK((hipError_t)vs_wmma_sddmm_f16_row_parts(k_contract, n, n_slots, d_slots, nnz_vec, d_cols, d_lhs_s, d_rhs_s,
-                                                       d_sd_h, V, nullptr));
+        HIP_OK((hipError_t)vs_wmma_sddmm_f16_row_parts(1, k_contract, n, n_slots, d_slots, nnz_vec, d_cols, d_lhs_s, 0,
+                                                       d_rhs_s, 0, d_sd_h, 0, V, nullptr));
         HIP_OK(hipDeviceSynchronize());
         fetch_h(d_sd_h, want_sddmm.size());
         ok &= close_enough("vs_wmma_sddmm_f16_row_parts", got_f, want_sddmm);

@@ -92,10 +92,30 @@ def test_device_problem_entry_and_rejections(gpu):
     L = _lib.lib()
     parts, slots = prob.row_parts(512)[:2]
     out.fill_(9.0)
-    args = lambda k, sl: (k, 2048, parts.n_slots, sl, mask.nnz_vec, prob.column_indices.data_ptr(), Ad.data_ptr(),
-                          Bd.data_ptr(), out.data_ptr(), 8, 0)
+    args = lambda k, sl: (1, k, 2048, parts.n_slots, sl, mask.nnz_vec, prob.column_indices.data_ptr(), Ad.data_ptr(), 0,
+                          Bd.data_ptr(), 0, out.data_ptr(), 0, 8, 0)
     assert L.vs_wmma_sddmm_f16_row_parts(*args(60, slots.data_ptr())) == 801      # k not a multiple of 8
     assert L.vs_wmma_sddmm_f16_row_parts(*args(64, slots.data_ptr() + 4)) == 1    # misaligned list
     assert L.vs_wmma_sddmm_f16_row_parts(*args(64, 0)) == 1
     torch.cuda.synchronize()
     assert bool((out == 9.0).all()), "a rejected call must not launch anything"
+
+
+def test_batch_on_a_shared_mask(gpu):
+    rng = np.random.default_rng(31)
+    lengths = np.minimum((rng.pareto(1.4, 120) + 0.2) * 60, 2000).astype(np.int64)
+    lengths[5] = 2000
+    mask = _mask(lengths, 2000, 4, seed=32)
+    batch, K = 6, 64
+    As = np.stack([cv.dense_normal(mask.m, K, seed=50 + b) for b in range(batch)])
+    Bs = np.stack([cv.dense_normal(2000, K, seed=60 + b) for b in range(batch)])
+    parts = ops.RowParts(mask.m_vec, mask.row_offsets, 256)
+    assert parts.n_split > 0
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    slots, ci, Ad, Bd = d(parts.slots), d(mask.column_indices), d(As), d(Bs)
+    out = torch.full((batch, mask.nnz_vec, 4), 3.0, dtype=torch.float16, device="cuda")
+    ops.sddmm_row_parts(K, 2000, parts, slots, mask.nnz_vec, ci, Ad, Bd, out, 4)
+    torch.cuda.synchronize()
+    for b in range(batch):
+        assert_parity(out[b].cpu().numpy().reshape(-1), np.asarray(_oracle(mask, As[b], Bs[b])).reshape(-1),
+                      "batched SDDMM, problem %d" % b)

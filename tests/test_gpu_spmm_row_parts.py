@@ -131,14 +131,14 @@ def test_dense_width_edges_and_rejections(gpu):
     out = torch.full((pat.m, 64), 9.0, dtype=torch.float16, device="cuda")
     need = ops.spmm_row_parts_workspace_bytes(8, 64, parts.n_split, parts.parts_max)
     ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
-    args = lambda k, ws_bytes: (8, k, 768, parts.n_slots, slots.data_ptr(), parts.n_split, parts.parts_max, pat.nnz_vec,
-                                parts.longest_part_vec, ci.data_ptr(), vals.data_ptr(), B.data_ptr(), out.data_ptr(),
+    args = lambda k, ws_bytes: (1, 8, k, 768, parts.n_slots, slots.data_ptr(), parts.n_split, parts.parts_max, pat.nnz_vec,
+                                parts.longest_part_vec, ci.data_ptr(), vals.data_ptr(), 0, B.data_ptr(), 0, out.data_ptr(), 0,
                                 ws.data_ptr(), ws_bytes, 0)
     assert L.vs_wmma_spmm_f16_row_parts(*args(62, need)) == 801       # dense width not a multiple of 4
     assert L.vs_wmma_spmm_f16_row_parts(*args(64, need - 16)) == 801  # workspace too small
     assert L.vs_wmma_spmm_f16_row_parts(*args(64, -1)) == 1
     bad = list(args(64, need))
-    bad[4] = slots.data_ptr() + 4
+    bad[5] = slots.data_ptr() + 4
     assert L.vs_wmma_spmm_f16_row_parts(*bad) == 1                    # misaligned list
     torch.cuda.synchronize()
     assert bool((out == 9.0).all()), "a rejected call must not launch anything"
@@ -250,3 +250,41 @@ def test_hip_graph_replays_equal_eager(gpu):
                 torch.cuda.synchronize()
                 assert torch.equal(out, want), "replay %d, %d launch(es)" % (rep, launches)
     assert_parity(out.cpu().numpy(), _oracle(pat, Bd.cpu().numpy()), "rows in parts under a HIP graph")
+
+
+@pytest.mark.parametrize("V", [2, 8])
+@pytest.mark.parametrize("launches", [1, 2])
+def test_batch_on_a_shared_pattern(gpu, V, launches):
+    """Five problems on one pattern and one list: per-problem values and dense operands, then a shared dense
+    operand; each agrees with the oracle and with the single call on its operands."""
+    rng = np.random.default_rng(21)
+    lengths = np.minimum((rng.pareto(1.4, 90) + 0.2) * 60, 1500).astype(np.int64)
+    lengths[3] = 1500
+    base = _from_lengths(lengths, 1500, V, seed=22)
+    batch, N = 5, 136
+    vals = np.stack([cv.random_values(base, seed=30 + b).values for b in range(batch)])
+    Bs = np.stack([cv.dense_uniform(1500, N, seed=40 + b) for b in range(batch)])
+    parts = ops.RowParts(base.m_vec, base.row_offsets, 128)
+    assert parts.n_split > 0
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    slots, ci, vd, Bd = d(parts.slots), d(base.column_indices), d(vals), d(Bs)
+    need = ops.spmm_row_parts_workspace_bytes(V, N, parts.n_split, parts.parts_max, batch=batch)
+    ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
+    with _lib.thread_options(spmm_parts_launches=launches):
+        out = torch.full((batch, base.m, N), 3.0, dtype=torch.float16, device="cuda")
+        for _ in range(2):
+            ops.spmm_row_parts(V, N, 1500, parts, slots, base.nnz_vec, ci, vd, Bd, out, ws)
+        shared = torch.full((batch, base.m, N), 3.0, dtype=torch.float16, device="cuda")
+        ops.spmm_row_parts(V, N, 1500, parts, slots, base.nnz_vec, ci, vd, Bd[0], shared, ws)
+        torch.cuda.synchronize()
+        for b in range(batch):
+            pat = base.with_values(vals[b])
+            assert_parity(out[b].cpu().numpy(), _oracle(pat, Bs[b]), "batched, problem %d" % b)
+            assert_parity(shared[b].cpu().numpy(), _oracle(pat, Bs[0]), "batched, shared dense operand, problem %d" % b)
+            single = torch.empty((base.m, N), dtype=torch.float16, device="cuda")
+            ws1 = torch.zeros(need, dtype=torch.uint8, device="cuda")
+            ops.spmm_row_parts(V, N, 1500, parts, slots, base.nnz_vec, ci, vd[b], Bd[b], single, ws1)
+            torch.cuda.synchronize()
+            # (not bit for bit: how a row's blocks are shared among waves follows the size of the launch)
+            assert_parity(out[b].cpu().numpy(), single.float().cpu().numpy(), "batched against single, problem %d" % b)
+    assert not ws.cpu().numpy()[:need // 5 // 256 * 256].any(), "the arrival counters must be back at zero"

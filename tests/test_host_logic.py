@@ -315,5 +315,6 @@ def test_row_parts_dispatch_list():
     st = _lib.lib().vs_spmm_row_parts(2, ro.ctypes.data, 512, slots.ctypes.data, 2, *[ctypes.addressof(x) for x in c])
     assert st == 801 and c[0].value == 5 and c[1].value == 1 and c[2].value == 4
     assert _lib.lib().vs_spmm_row_parts(2, ro.ctypes.data, -1, slots.ctypes.data, 2, *[ctypes.addressof(x) for x in c]) == 1
-    assert _lib.lib().vs_wmma_spmm_row_parts_workspace_bytes(8, 256, 0, 0) == 0
-    assert _lib.lib().vs_wmma_spmm_row_parts_workspace_bytes(8, 256, 3, 4) > 3 * 4 * 8 * 256 * 4
+    assert _lib.lib().vs_wmma_spmm_row_parts_workspace_bytes(1, 8, 256, 0, 0) == 0
+    assert _lib.lib().vs_wmma_spmm_row_parts_workspace_bytes(1, 8, 256, 3, 4) > 3 * 4 * 8 * 256 * 4
+    assert _lib.lib().vs_wmma_spmm_row_parts_workspace_bytes(5, 8, 256, 3, 4) > 5 * 3 * 4 * 8 * 256 * 4

@@ -44,9 +44,10 @@ SIGNATURES = {
     "vs_identity_row_swizzle": ([_int, _vp], None),
     "vs_sorted_row_swizzle": ([_int, _vp, _vp], None),
     "vs_spmm_row_parts": ([_int, _vp, _int, _vp, _int, _vp, _vp, _vp, _vp], _int),
-    "vs_wmma_spmm_row_parts_workspace_bytes": ([_int] * 4, _ll),
-    "vs_wmma_spmm_f16_row_parts": ([_int] * 4 + [_vp] + [_int] * 4 + [_vp] * 5 + [_ll, _vp], _int),
-    "vs_wmma_sddmm_f16_row_parts": ([_int] * 3 + [_vp, _int] + [_vp] * 4 + [_int, _vp], _int),
+    "vs_wmma_spmm_row_parts_workspace_bytes": ([_int] * 5, _ll),
+    "vs_wmma_spmm_f16_row_parts": ([_int] * 5 + [_vp] + [_int] * 4 + [_vp] + [_vp, _ll, _vp, _ll, _vp, _ll] + [_vp, _ll, _vp],
+                                   _int),
+    "vs_wmma_sddmm_f16_row_parts": ([_int] * 4 + [_vp, _int, _vp] + [_vp, _ll, _vp, _ll, _vp, _ll] + [_int, _vp], _int),
     "vs_launch_floor_probe": ([_int, _int, _vp], _int),
     "vs_set_option": ([ctypes.c_char_p, _int], _int),
     "vs_set_thread_option": ([ctypes.c_char_p, _int], _int),

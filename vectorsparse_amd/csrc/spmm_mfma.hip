@@ -245,8 +245,11 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row
     // last of the row's parts.
     const int part_count = part_info & 255;
     const uint32_t part_tile_bytes = (uint32_t)V * TN * (uint32_t)sizeof(float);
+    // (the launcher passes the number of split rows where the team mapping has its count: problem b of a batch has
+    // its tiles and counters behind those of problems 0 .. b - 1)
+    const int part_split = (int)blockIdx.y * team_slots + (part_info >> 16);
     const uint32_t part_row_base =
-        (uint32_t)(((part_info >> 16) * parts_max) * n_tiles + tile) * part_tile_bytes;  // part 0 of the row, this tile
+        (uint32_t)((part_split * parts_max) * n_tiles + tile) * part_tile_bytes;  // part 0 of the row, this tile
     auto park = [&](int v, int cs_at, const float (&vals)[CPL]) {
         const uint32_t at = part_row_base + (uint32_t)(((part_info >> 8) & 255) * n_tiles) * part_tile_bytes +
                             4u * (uint32_t)(v * TN + cs_at * CPL);
@@ -262,7 +265,7 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row
         }
     };
     auto arrive_and_finish = [&]() {  // one wave, all of its lanes; the workgroup's stores have completed
-        int *counter = part_counters + ((size_t)(part_info >> 16) * n_tiles + tile) * kPartCounterStride;
+        int *counter = part_counters + ((size_t)part_split * n_tiles + tile) * kPartCounterStride;
         int arrived = 0;
         if (lane == 0) arrived = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         arrived = __builtin_amdgcn_readfirstlane(arrived);
@@ -465,14 +468,16 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row
 // computes in the one-launch form - and writes the row.  `split_rows`: four ints per split row, {vector row, parts}.
 template <int V, int CPL>
 __global__ void __launch_bounds__(V * 16 < 64 ? 64 : V * 16)
-spmm_row_parts_sum_kernel(int n_cols, int n_tiles, const int *__restrict__ split_rows, int parts_max,
-                          const float *__restrict__ tiles, half_t *__restrict__ out)
+spmm_row_parts_sum_kernel(int n_cols, int n_tiles, const int *__restrict__ split_rows, int n_split, int parts_max,
+                          const float *__restrict__ tiles, half_t *__restrict__ out, long long stride_out)
 {
     constexpr int TN = 16 * CPL;
     const int tile = blockIdx.x % n_tiles;
-    const int split = blockIdx.x / n_tiles;
-    const int row = split_rows[4 * split];
-    const int parts = split_rows[4 * split + 1];
+    const int split_in_problem = blockIdx.x / n_tiles;
+    const int row = split_rows[4 * split_in_problem];
+    const int parts = split_rows[4 * split_in_problem + 1];
+    const int split = (int)blockIdx.y * n_split + split_in_problem;  // batch: problem b's tiles behind those before it
+    out += blockIdx.y * stride_out;
     const int item = threadIdx.x;
     if (item >= V * 16) return;
     const int v = item >> 4;
@@ -854,7 +859,7 @@ namespace {
 template <int V, int CPL, bool PIPE>
 int launch_parts_kernel(int k, int n_slots, int n_split, bool two_launches, int waves, int per_wave, const int *slots,
                         int parts_max, const int *column_indices, const half_t *values, const half_t *rhs, half_t *out,
-                        int *counters, float *tiles, hipStream_t stream)
+                        int *counters, float *tiles, hipStream_t stream, const Batch &batch)
 {
     int per_wave_log2 = 0;
     while ((2 << per_wave_log2) <= per_wave) ++per_wave_log2;
@@ -867,26 +872,26 @@ int launch_parts_kernel(int k, int n_slots, int n_split, bool two_launches, int 
     static std::atomic<unsigned long long> lds_allowed{0};
     const hipError_t attr = allow_large_lds(reinterpret_cast<const void *>(kernel), 96 * 1024, lds_allowed);
     if (attr != hipSuccess) return (int)attr;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, 1u), dim3(64 * waves), lds, stream, k, n_tiles,
-                       per_wave_log2 | (waves << 8) | (blocks >= 512 ? 1 << 16 : 0) | (two_launches ? 1 << 17 : 0), slots,
-                       static_cast<const int *>(nullptr), column_indices, values, rhs, out, 0LL, 0LL, 0LL, 1.f, -1, n_slots,
-                       counters, tiles, parts_max);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)batch.count), dim3(64 * waves), lds, stream, k, n_tiles,
+                       per_wave_log2 | (waves << 8) | (blocks * batch.count >= 512 ? 1 << 16 : 0) | (two_launches ? 1 << 17 : 0),
+                       slots, static_cast<const int *>(nullptr), column_indices, values, rhs, out, batch.stride_a, batch.stride_b,
+                       batch.stride_out, 1.f, n_split, n_slots, counters, tiles, parts_max);
     const hipError_t st = hipGetLastError();
     if (st != hipSuccess || !two_launches || n_split == 0) return (int)st;
-    hipLaunchKernelGGL((spmm_row_parts_sum_kernel<V, CPL>), dim3((unsigned)(n_split * n_tiles)),
-                       dim3(V * 16 < 64 ? 64 : V * 16), 0, stream, k, n_tiles, slots + 4 * (size_t)n_slots, parts_max, tiles,
-                       out);
+    hipLaunchKernelGGL((spmm_row_parts_sum_kernel<V, CPL>), dim3((unsigned)(n_split * n_tiles), (unsigned)batch.count),
+                       dim3(V * 16 < 64 ? 64 : V * 16), 0, stream, k, n_tiles, slots + 4 * (size_t)n_slots, n_split, parts_max,
+                       tiles, out, batch.stride_out);
     return (int)hipGetLastError();
 }
 
 template <int V>
 int launch_parts_v(const SpmmShape &shape, int k, int n_slots, int n_split, bool two_launches, const int *slots,
                    int parts_max, const int *column_indices, const half_t *values, const half_t *rhs, half_t *out,
-                   int *counters, float *tiles, hipStream_t stream)
+                   int *counters, float *tiles, hipStream_t stream, const Batch &batch)
 {
 #define VS_PARTS_VARIANT(CPL, PIPE)                                                                                \
     launch_parts_kernel<V, CPL, PIPE>(k, n_slots, n_split, two_launches, shape.waves, shape.blocks_per_wave, slots, \
-                                      parts_max, column_indices, values, rhs, out, counters, tiles, stream)
+                                      parts_max, column_indices, values, rhs, out, counters, tiles, stream, batch)
     if (shape.cols_per_lane == 8) return shape.pipelined ? VS_PARTS_VARIANT(8, true) : VS_PARTS_VARIANT(8, false);
     return shape.pipelined ? VS_PARTS_VARIANT(4, true) : VS_PARTS_VARIANT(4, false);
 #undef VS_PARTS_VARIANT
@@ -894,26 +899,28 @@ int launch_parts_v(const SpmmShape &shape, int k, int n_slots, int n_split, bool
 
 }  // namespace
 
-long long spmm_row_parts_workspace_bytes(int vec_length, int k, int n_split, int parts_max)
+long long spmm_row_parts_workspace_bytes(int batch, int vec_length, int k, int n_split, int parts_max)
 {
-    if (n_split <= 0 || parts_max <= 0 || k <= 0) return 0;
+    if (batch <= 0 || n_split <= 0 || parts_max <= 0 || k <= 0) return 0;
     const long long k_pad = (long long)ceil_div(k, 128) * 128;  // whole tiles of either width
-    return row_parts_workspace_for((long long)n_split * parts_max * vec_length * k_pad * (long long)sizeof(float));
+    return row_parts_workspace_for((long long)batch * n_split * parts_max * vec_length * k_pad * (long long)sizeof(float));
 }
 
 int launch_spmm_mfma_row_parts(int vec_length, int k, int n, int n_slots, const int *slots, int n_split, int parts_max,
                                int nonzeros_vec, int longest_part_vec, const int *column_indices, const half_t *values,
                                const half_t *rhs, half_t *out, void *workspace, long long workspace_bytes,
-                               hipStream_t stream)
+                               hipStream_t stream, const Batch &batch)
 {
-    if (n_slots == 0 || k == 0) return hipSuccess;
+    if (n_slots == 0 || k == 0 || batch.count == 0) return hipSuccess;
+    if (batch.count > 65535 || (long long)batch.count * n_split > 0x7fffffffLL / 256) return hipErrorNotSupported;
     if (k % 4 != 0 || (long long)n * k >= (1LL << 31)) return hipErrorNotSupported;  // whole chunks, 32-bit offsets
     if (n_split > 32767 || parts_max > 255 || (n_split > 0 && parts_max < 2)) return hipErrorInvalidValue;
-    const long long need = spmm_row_parts_workspace_bytes(vec_length, k, n_split, parts_max);
+    const long long need = spmm_row_parts_workspace_bytes(batch.count, vec_length, k, n_split, parts_max);
     if (need > workspace_bytes || need - row_parts_counter_bytes(need) >= (1LL << 31)) return hipErrorNotSupported;
-    Batch hints;
+    Batch hints = batch;
     hints.nonzeros_vec = nonzeros_vec;
     hints.longest_row_vec = longest_part_vec;
+    hints.long_rows = -1;
     SpmmShape shape = choose_spmm_shape(false, n_slots, vec_length, k, n, hints);
     if (shape.ragged || shape.dma) return hipErrorNotSupported;
     if (k % 8 != 0) shape.cols_per_lane = 4;
@@ -929,7 +936,7 @@ int launch_spmm_mfma_row_parts(int vec_length, int k, int n, int n_slots, const 
     // 14.4-21.3; 1.18 M 17.7 / 19.9 / 29.6 - the waves that short slots leave idle cost what the long ones gain
     // once the launch holds enough work.
     if (n_split > 0 && options().spmm_waves == 0) {
-        const long long work = (long long)nonzeros_vec * ceil_div(k, 128);
+        const long long work = (long long)nonzeros_vec * ceil_div(k, 128) * batch.count;
         shape.waves = work <= (256LL << 10) ? 8 : work <= (1LL << 20) ? 4 : 2;
         shape.blocks_per_wave = options().spmm_blocks_per_wave > 0 ? options().spmm_blocks_per_wave : 1;
         shape.pipelined = options().spmm_pipe != 1;
@@ -940,15 +947,16 @@ int launch_spmm_mfma_row_parts(int vec_length, int k, int n, int n_slots, const 
     // is (a dense row among 1023: 8.8 against 10.7 us; 1024 Pareto rows 11.0 against 13.1).
     const bool two_launches =
         options().spmm_parts_launches == 2 ||
-        (options().spmm_parts_launches == 0 && n_split > 0 && (long long)nonzeros_vec * ceil_div(k, 128) <= 160 * 1024);
+        (options().spmm_parts_launches == 0 && n_split > 0 &&
+         (long long)nonzeros_vec * ceil_div(k, 128) * batch.count <= 160 * 1024);
     int *counters = static_cast<int *>(workspace);
     float *tiles = reinterpret_cast<float *>(static_cast<unsigned char *>(workspace) +
                                              (n_split > 0 ? row_parts_counter_bytes(workspace_bytes) : 0));
     switch (vec_length) {
-    case 1: return launch_parts_v<1>(shape, k, n_slots, n_split, two_launches, slots, parts_max, column_indices, values, rhs, out, counters, tiles, stream);
-    case 2: return launch_parts_v<2>(shape, k, n_slots, n_split, two_launches, slots, parts_max, column_indices, values, rhs, out, counters, tiles, stream);
-    case 4: return launch_parts_v<4>(shape, k, n_slots, n_split, two_launches, slots, parts_max, column_indices, values, rhs, out, counters, tiles, stream);
-    case 8: return launch_parts_v<8>(shape, k, n_slots, n_split, two_launches, slots, parts_max, column_indices, values, rhs, out, counters, tiles, stream);
+    case 1: return launch_parts_v<1>(shape, k, n_slots, n_split, two_launches, slots, parts_max, column_indices, values, rhs, out, counters, tiles, stream, batch);
+    case 2: return launch_parts_v<2>(shape, k, n_slots, n_split, two_launches, slots, parts_max, column_indices, values, rhs, out, counters, tiles, stream, batch);
+    case 4: return launch_parts_v<4>(shape, k, n_slots, n_split, two_launches, slots, parts_max, column_indices, values, rhs, out, counters, tiles, stream, batch);
+    case 8: return launch_parts_v<8>(shape, k, n_slots, n_split, two_launches, slots, parts_max, column_indices, values, rhs, out, counters, tiles, stream, batch);
     default: return hipErrorInvalidValue;
     }
 }

@@ -339,8 +339,8 @@ inline long long row_parts_workspace_for(long long tile_bytes)
 int launch_spmm_mfma_row_parts(int vec_length, int k, int n, int n_slots, const int *slots, int n_split, int parts_max,
                                int nonzeros_vec, int longest_part_vec, const int *column_indices, const half_t *values,
                                const half_t *rhs, half_t *out, void *workspace, long long workspace_bytes,
-                               hipStream_t stream);
-long long spmm_row_parts_workspace_bytes(int vec_length, int k, int n_split, int parts_max);
+                               hipStream_t stream, const Batch &batch);
+long long spmm_row_parts_workspace_bytes(int batch, int vec_length, int k, int n_split, int parts_max);
 
 // Split-row SpMM (csrc/spmm_mfma_flat.hip): `workspace` holds the fp32 partial tiles of rows longer than a piece.
 template <typename OutT>

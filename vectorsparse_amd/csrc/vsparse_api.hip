@@ -615,18 +615,19 @@ int vs_spmm_row_parts(int m_vec, const int *row_offsets, int limit_vec, int *slo
     return VS_SUCCESS;
 }
 
-long long vs_wmma_spmm_row_parts_workspace_bytes(int vec_length, int k, int n_split, int parts_max)
+long long vs_wmma_spmm_row_parts_workspace_bytes(int batch, int vec_length, int k, int n_split, int parts_max)
 {
     if (!vec_ok(vec_length)) return 0;
-    return vs::spmm_row_parts_workspace_bytes(vec_length, k, n_split, parts_max);
+    return vs::spmm_row_parts_workspace_bytes(batch, vec_length, k, n_split, parts_max);
 }
 
-int vs_wmma_spmm_f16_row_parts(int vec_length, int k, int n, int n_slots, const int *slots, int n_split, int parts_max,
-                               int nonzeros_vec, int longest_part_vec, const int *column_indices, const void *values,
-                               const void *rhs_matrix, void *output_matrix, void *workspace, long long workspace_bytes,
+int vs_wmma_spmm_f16_row_parts(int batch, int vec_length, int k, int n, int n_slots, const int *slots, int n_split,
+                               int parts_max, int nonzeros_vec, int longest_part_vec, const int *column_indices,
+                               const void *values, long long stride_values, const void *rhs_matrix, long long stride_rhs,
+                               void *output_matrix, long long stride_output, void *workspace, long long workspace_bytes,
                                void *stream)
 {
-    if (!vec_ok(vec_length) || k < 0 || n < 0 || n_slots < 0 || n_split < 0 || parts_max < 0 ||
+    if (!vec_ok(vec_length) || batch < 0 || k < 0 || n < 0 || n_slots < 0 || n_split < 0 || parts_max < 0 ||
         nonzeros_vec < 0 || longest_part_vec < 0 || workspace_bytes < 0)
         return VS_ERROR_INVALID_VALUE;
     if (n_slots > 0 && (!slots || !aligned(slots, 16))) return VS_ERROR_INVALID_VALUE;
@@ -634,34 +635,42 @@ int vs_wmma_spmm_f16_row_parts(int vec_length, int k, int n, int n_slots, const 
     if (nonzeros_vec > 0 && (!column_indices || !values)) return VS_ERROR_INVALID_VALUE;
     if (!aligned(values, 2 * vec_length) || !aligned(rhs_matrix, 16) || !aligned(output_matrix, 16))
         return VS_ERROR_INVALID_VALUE;
+    // every problem of the batch keeps the alignment of the first (as the other batched entry points ask)
+    if (!stride_ok(stride_values, vec_length) || !stride_ok(stride_rhs, 8) || !stride_ok(stride_output, 8))
+        return VS_ERROR_INVALID_VALUE;
     if (workspace_bytes > 0 && (!workspace || !aligned(workspace, 16))) return VS_ERROR_INVALID_VALUE;
     return vs::launch_spmm_mfma_row_parts(vec_length, k, n, n_slots, slots, n_split, parts_max, nonzeros_vec,
                                           longest_part_vec, column_indices, static_cast<const half_t *>(values),
                                           static_cast<const half_t *>(rhs_matrix), static_cast<half_t *>(output_matrix),
-                                          workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+                                          workspace, workspace_bytes, static_cast<hipStream_t>(stream),
+                                          make_batch(batch, stride_values, stride_rhs, stride_output));
 }
 
-int vs_wmma_sddmm_f16_row_parts(int k, int n, int n_slots, const int *slots, int nonzeros_vec, const int *col_indices,
-                                const void *lhs_matrix, const void *rhs_matrix, void *output_values, int vec_length,
-                                void *stream)
+int vs_wmma_sddmm_f16_row_parts(int batch, int k, int n, int n_slots, const int *slots, int nonzeros_vec,
+                                const int *col_indices, const void *lhs_matrix, long long stride_lhs,
+                                const void *rhs_matrix, long long stride_rhs, void *output_values, long long stride_output,
+                                int vec_length, void *stream)
 {
-    if (!vec_ok(vec_length) || k < 0 || n < 0 || n_slots < 0 || nonzeros_vec < 0) return VS_ERROR_INVALID_VALUE;
-    if (n_slots == 0 || nonzeros_vec == 0) return VS_SUCCESS;
+    if (!vec_ok(vec_length) || batch < 0 || k < 0 || n < 0 || n_slots < 0 || nonzeros_vec < 0)
+        return VS_ERROR_INVALID_VALUE;
+    if (batch == 0 || n_slots == 0 || nonzeros_vec == 0) return VS_SUCCESS;
     if (!slots || !aligned(slots, 16) || !col_indices || !output_values) return VS_ERROR_INVALID_VALUE;
     if (k > 0 && (!lhs_matrix || !rhs_matrix)) return VS_ERROR_INVALID_VALUE;
     if (!aligned(output_values, sizeof(half_t) * (size_t)vec_length)) return VS_ERROR_INVALID_VALUE;
+    if (!stride_ok(stride_lhs, 8) || !stride_ok(stride_rhs, 8) || !stride_ok(stride_output, vec_length))
+        return VS_ERROR_INVALID_VALUE;
     if (k == 0)
-        return sddmm_zero_outputs(output_values, nonzeros_vec, vec_length, sizeof(half_t), 1, 0,
+        return sddmm_zero_outputs(output_values, nonzeros_vec, vec_length, sizeof(half_t), batch, stride_output,
                                   static_cast<hipStream_t>(stream));
     if (k % 8 != 0) return VS_ERROR_NOT_SUPPORTED;
     if (!aligned(lhs_matrix, 16) || !aligned(rhs_matrix, 16)) return VS_ERROR_INVALID_VALUE;
-    vs::Batch batch;
-    batch.algorithm = 1;
-    batch.row_parts = true;
+    vs::Batch b = make_batch(batch, stride_lhs, stride_rhs, stride_output);
+    b.algorithm = 1;
+    b.row_parts = true;
     return vs::launch_sddmm_mfma<half_t>(n_slots, k, n, nonzeros_vec, slots, nullptr, col_indices,
                                          static_cast<const half_t *>(lhs_matrix), static_cast<const half_t *>(rhs_matrix),
                                          static_cast<half_t *>(output_values), vec_length,
-                                         static_cast<hipStream_t>(stream), batch);
+                                         static_cast<hipStream_t>(stream), b);
 }
 
 int vs_launch_floor_probe(int blocks, int threads_per_block, void *stream)

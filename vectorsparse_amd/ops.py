@@ -459,21 +459,27 @@ class RowParts:
         self.slots = np.ascontiguousarray(slots[:self.n_slots + self.n_split])  # (one entry per split row behind the list)
 
 
-def spmm_row_parts_workspace_bytes(vec_length, k, n_split, parts_max):
-    return int(_lib.lib().vs_wmma_spmm_row_parts_workspace_bytes(vec_length, k, n_split, parts_max))
+def spmm_row_parts_workspace_bytes(vec_length, k, n_split, parts_max, batch=1):
+    return int(_lib.lib().vs_wmma_spmm_row_parts_workspace_bytes(batch, vec_length, k, n_split, parts_max))
 
 
 def spmm_row_parts(vec_length, k, n, parts, slots, nonzeros_vec, column_indices, values, rhs_matrix, output_matrix,
                    workspace=None, stream=None):
     """wmmaSpmm driven by a dispatch list of row parts (`parts`: a RowParts, `slots`: its list as a device int32
     tensor).  workspace: a device tensor of at least spmm_row_parts_workspace_bytes(...) bytes, zero-filled before
-    its first use, or None when no row is split.  Returns output_matrix."""
+    its first use, or None when no row is split.  A leading batch dimension on output_matrix ([batch, m, k]) runs
+    that many problems on the shared pattern; values / rhs_matrix with the same leading dimension are per problem,
+    without it shared.  Returns output_matrix."""
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    batch = output_matrix.shape[0] if output_matrix.dim() == 3 else 1
+    per_problem = lambda t, dims: (t.stride(0) if t.dim() == dims + 1 else 0)
     st = _lib.lib().vs_wmma_spmm_f16_row_parts(
-        vec_length, k, n, parts.n_slots, _expect(slots, torch.int32, "slots"), parts.n_split, parts.parts_max,
+        batch, vec_length, k, n, parts.n_slots, _expect(slots, torch.int32, "slots"), parts.n_split, parts.parts_max,
         nonzeros_vec, parts.longest_part_vec, _expect(column_indices, torch.int32, "column_indices"),
-        _expect(values, torch.float16, "values"), _expect(rhs_matrix, torch.float16, "rhs_matrix"),
-        _expect(output_matrix, torch.float16, "output_matrix"), _ptr(workspace), ws_bytes, _stream(stream))
+        _expect(values, torch.float16, "values"), per_problem(values, 2),
+        _expect(rhs_matrix, torch.float16, "rhs_matrix"), per_problem(rhs_matrix, 2),
+        _expect(output_matrix, torch.float16, "output_matrix"), per_problem(output_matrix, 2), _ptr(workspace), ws_bytes,
+        _stream(stream))
     if st:
         _lib.check(st, "vs_wmma_spmm_f16_row_parts")
     return output_matrix
@@ -482,12 +488,16 @@ def spmm_row_parts(vec_length, k, n, parts, slots, nonzeros_vec, column_indices,
 def sddmm_row_parts(k, n, parts, slots, nonzeros_vec, col_indices, lhs_matrix, rhs_matrix, output_values, vec_length,
                     stream=None):
     """wmmaSddmm driven by a dispatch list of row parts (`parts`: a RowParts, `slots`: its list as a device int32
-    tensor).  Returns output_values."""
+    tensor).  A leading batch dimension on output_values ([batch, nnz_vec, V]) runs that many problems on the shared
+    mask; lhs_matrix / rhs_matrix with the same leading dimension are per problem, without it shared.  Returns
+    output_values."""
+    batch = output_values.shape[0] if output_values.dim() == 3 else 1
+    per_problem = lambda t, dims: (t.stride(0) if t.dim() == dims + 1 else 0)
     st = _lib.lib().vs_wmma_sddmm_f16_row_parts(
-        k, n, parts.n_slots, _expect(slots, torch.int32, "slots"), nonzeros_vec,
+        batch, k, n, parts.n_slots, _expect(slots, torch.int32, "slots"), nonzeros_vec,
         _expect(col_indices, torch.int32, "col_indices"), _expect(lhs_matrix, torch.float16, "lhs_matrix"),
-        _expect(rhs_matrix, torch.float16, "rhs_matrix"), _expect(output_values, torch.float16, "output_values"),
-        vec_length, _stream(stream))
+        per_problem(lhs_matrix, 2), _expect(rhs_matrix, torch.float16, "rhs_matrix"), per_problem(rhs_matrix, 2),
+        _expect(output_values, torch.float16, "output_values"), per_problem(output_values, 2), vec_length, _stream(stream))
     if st:
         _lib.check(st, "vs_wmma_sddmm_f16_row_parts")
     return output_values
