@@ -7,7 +7,7 @@
 // One wave per vector row: lane t owns the nonzero vectors t, t + 64, ... (one V-wide load each, the
 // row's block of values is contiguous), keeps V running maxima / sums in fp32 and combines them across
 // the 64 lanes with DPP / ds_swizzle / ds_bpermute butterflies.  Rows of up to 512 vectors are held in
-// registers between the passes; longer rows are re-read (from L1/L2) for each of the three passes.
+// registers between the passes; longer rows are read twice (running maximum and sum, then the normalisation).
 // in == out is allowed.
 #include "vs_common.hpp"
 
@@ -111,28 +111,68 @@ sparse_softmax_kernel(int m_vec, const int *__restrict__ row_indices, const int 
         return;
     }
 
-    for (int j = beg + lane; j < end; j += 64) {
-        float x[V];
-        load_scaled<V>(x, in + (size_t)j * V, s2);
+    // Longer rows: two passes over the row, each in chunks of kCached vectors per lane whose loads are all requested
+    // before the first is used - a lane that asks for one vector at a time pays a memory round trip per 64 vectors
+    // of the row (a dense row of 4096 vectors: 192 of them one after the other).  The first pass keeps a running
+    // maximum and a sum relative to it per lane (rescaled once per chunk when the maximum moves), combined across
+    // the lanes at the end; the second normalises.  The loads are made whether or not the vector exists (past the
+    // row's end a lane re-reads the row's last vector): a load behind a branch makes every wait after it count for
+    // the path without it.
+    constexpr int kChunk = 64 * kCached;
+    const int last = end - 1;
+    for (int j0 = beg + lane; j0 < end; j0 += kChunk) {
+        float x[kCached][V];
 #pragma unroll
-        for (int v = 0; v < V; ++v) mx[v] = fmaxf(mx[v], x[v]);
+        for (int c = 0; c < kCached; ++c) {
+            const int j = j0 + 64 * c;
+            load_scaled<V>(x[c], in + (size_t)(j < end ? j : last) * V, s2);
+        }
+        float top[V];
+#pragma unroll
+        for (int v = 0; v < V; ++v) top[v] = mx[v];
+#pragma unroll
+        for (int c = 0; c < kCached; ++c) {
+#pragma unroll
+            for (int v = 0; v < V; ++v) top[v] = fmaxf(top[v], x[c][v]);  // (a repeated vector changes no maximum)
+        }
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            sum[v] *= __builtin_amdgcn_exp2f(mx[v] - top[v]);  // (0 on the first chunk: its maximum was -inf)
+            mx[v] = top[v];
+        }
+#pragma unroll
+        for (int c = 0; c < kCached; ++c) {
+            const bool exists = j0 + 64 * c < end;
+#pragma unroll
+            for (int v = 0; v < V; ++v) sum[v] += exists ? __builtin_amdgcn_exp2f(x[c][v] - mx[v]) : 0.f;
+        }
     }
 #pragma unroll
-    for (int v = 0; v < V; ++v) mx[v] = wave_max(mx[v]);
-    for (int j = beg + lane; j < end; j += 64) {
-        float x[V];
-        load_scaled<V>(x, in + (size_t)j * V, s2);
-#pragma unroll
-        for (int v = 0; v < V; ++v) sum[v] += __builtin_amdgcn_exp2f(x[v] - mx[v]);
+    for (int v = 0; v < V; ++v) {
+        const float all = wave_max(mx[v]);  // every lane has seen at least one vector of a row this long
+        sum[v] = 1.0f / wave_sum(sum[v] * __builtin_amdgcn_exp2f(mx[v] - all));
+        mx[v] = all;
     }
+    for (int j0 = beg + lane; j0 < end; j0 += kChunk) {
+        float x[kCached][V];
 #pragma unroll
-    for (int v = 0; v < V; ++v) sum[v] = 1.0f / wave_sum(sum[v]);
-    for (int j = beg + lane; j < end; j += 64) {
-        float x[V], y[V];
-        load_scaled<V>(x, in + (size_t)j * V, s2);
+        for (int c = 0; c < kCached; ++c) {
+            const int j = j0 + 64 * c;
+            load_scaled<V>(x[c], in + (size_t)(j < end ? j : last) * V, s2);
+        }
+        // (in == out: every load of the chunk is in registers before its first store; the vector that lanes past
+        // the row's end re-read is not used)
+        asm volatile("" ::: "memory");
 #pragma unroll
-        for (int v = 0; v < V; ++v) y[v] = __builtin_amdgcn_exp2f(x[v] - mx[v]) * sum[v];
-        store_vec<V>(out + (size_t)j * V, y);
+        for (int c = 0; c < kCached; ++c) {
+            const int j = j0 + 64 * c;
+            if (j < end) {
+                float y[V];
+#pragma unroll
+                for (int v = 0; v < V; ++v) y[v] = __builtin_amdgcn_exp2f(x[c][v] - mx[v]) * sum[v];
+                store_vec<V>(out + (size_t)j * V, y);
+            }
+        }
     }
 }
 
