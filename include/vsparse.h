@@ -341,6 +341,20 @@ int vs_sparse_softmax_f16(int batch, int m_vec, int vec_length,
                           float scale, void *stream);
 
 /*
+ * vs_sparse_softmax_f16 driven by the dispatch list of vs_spmm_row_parts in place of row_indices and row_offsets
+ * (its n_slots entries, in device memory, 16-byte aligned): a row far longer than the rest - a global token of an
+ * attention mask - is normalised by as many waves as it has parts instead of by one.  The parts of a split row
+ * leave a (maximum, sum) pair per scalar row in `workspace` (8-byte aligned, at least
+ * vs_sparse_softmax_row_parts_workspace_bytes(...) bytes, 0 when no row is split; no need to clear it), a second
+ * launch combines them in ascending order and normalises.  in == out is allowed.  No counterpart in the reference.
+ */
+long long vs_sparse_softmax_row_parts_workspace_bytes(int batch, int vec_length, int n_split, int parts_max);
+int vs_sparse_softmax_f16_row_parts(int batch, int vec_length, int n_slots, const int *slots, int n_split,
+                                    int parts_max, const void *values_in, long long stride_in,
+                                    void *values_out, long long stride_out, float scale,
+                                    void *workspace, long long workspace_bytes, void *stream);
+
+/*
  * Softmax fused into SpMM:  out = softmax_row(scale * scores) * rhs_matrix, where `scores` has the
  * layout of `values` (for example the raw output of SDDMM).  Equivalent to vs_sparse_softmax_f16
  * followed by vs_wmma_spmm_f16_batched without writing the probabilities to memory: the kernel finds

@@ -627,3 +627,39 @@ def test_streamed_kernel_falls_back_on_oversized_unions(gpu):
                                    qd, kd, vd, scale=0.125, rows_per_workgroup=16, plan=plan)
         torch.cuda.synchronize()
         _check_layer(out.cpu().numpy(), _dense_attention(mask, q, k, v, 0.125), name, kind="single")
+
+
+@pytest.mark.parametrize("V", [1, 2, 4, 8])
+@pytest.mark.parametrize("limit", [64, 200, 0])
+def test_sparse_softmax_over_rows_in_parts(gpu, V, limit):
+    """The softmax driven by a dispatch list of row parts: rows of every length incl. empty ones and rows of many
+    parts, a batch of three, in place and out of place, against the float64 definition and the row kernel."""
+    rng = np.random.default_rng(40 + V)
+    lengths = np.array([0, 1, 63, 64, 65, 200, 0, 513, 1500, 31, 3000, 2, 0, 640], dtype=np.int64)
+    ro, ci = cv._pattern_from_lengths(rng, len(lengths), 3000, lengths)
+    pat = cv.ColVecCSR(len(lengths), 3000, V, ro, ci)
+    batch = 3
+    scores = (rng.standard_normal((batch, pat.nnz_vec, V)) * 3).astype(np.float16)
+    scale = 0.37
+    parts = ops.RowParts(pat.m_vec, pat.row_offsets, limit)
+    assert parts.n_split > 0
+    slots = torch.from_numpy(parts.slots).cuda()
+    need = ops.sparse_softmax_row_parts_workspace_bytes(V, parts.n_split, parts.parts_max, batch=batch)
+    ws = torch.full((need + 64,), 0x5A, dtype=torch.uint8, device="cuda")   # (no need to clear it)
+    x = torch.from_numpy(scores).cuda()
+    out = torch.full_like(x, 7.0)
+    ops.sparse_softmax_row_parts(V, parts, slots, x, out, scale=scale, workspace=ws[:need])
+    inplace = x.clone()
+    ops.sparse_softmax_row_parts(V, parts, slots, inplace, scale=scale, workspace=ws[:need])
+    prob = ops.DeviceProblem(pat)
+    plain = ops.sparse_softmax(pat.m_vec, V, prob.row_indices, prob.row_offsets, x.clone(), scale=scale)
+    torch.cuda.synchronize()
+    assert torch.equal(out, inplace), "in place and out of place differ"
+    assert bool((ws[need:] == 0x5A).all()), "wrote outside the workspace"
+    for b in range(batch):
+        ref = no.sparse_softmax_ref(pat.m_vec, V, pat.row_offsets, scores[b], scale)
+        assert_parity(out[b].cpu().numpy(), ref, "softmax over rows in parts V%d limit %d problem %d" % (V, limit, b))
+        assert_parity(out[b].cpu().numpy(), plain[b].float().cpu().numpy(), "against the row kernel")
+    # one vector row of the whole: every scalar row sums to one
+    sums = out[0].float().cpu().numpy()[ro[10]:ro[11]].sum(axis=0)
+    assert np.allclose(sums, 1.0, atol=2e-2)

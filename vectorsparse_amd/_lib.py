@@ -41,6 +41,9 @@ SIGNATURES = {
     "vs_sparse_attention_plan_bytes": ([_int] * 6, _ll),
     "vs_sparse_attention_plan": ([_int] * 6 + [_vp] * 3 + [_ll, _vp], _int),
     "vs_sparse_softmax_f16": ([_int] * 3 + [_vp] * 2 + [_vp, _ll, _vp, _ll, ctypes.c_float, _vp], _int),
+    "vs_sparse_softmax_row_parts_workspace_bytes": ([_int] * 4, _ll),
+    "vs_sparse_softmax_f16_row_parts": ([_int] * 3 + [_vp, _int, _int] + [_vp, _ll, _vp, _ll, ctypes.c_float, _vp, _ll, _vp],
+                                        _int),
     "vs_identity_row_swizzle": ([_int, _vp], None),
     "vs_sorted_row_swizzle": ([_int, _vp, _vp], None),
     "vs_spmm_row_parts": ([_int, _vp, _int, _vp, _int, _vp, _vp, _vp, _vp], _int),

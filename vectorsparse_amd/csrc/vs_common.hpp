@@ -12,6 +12,7 @@ typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
 typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
 typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
 typedef int32_t int4_t __attribute__((ext_vector_type(4)));
@@ -373,5 +374,10 @@ int sparse_attention_union_capacity(int vec_length, int n, int d_qk, int d_v, in
 int launch_sparse_softmax(int m_vec, int vec_length, const int *row_indices, const int *row_offsets,
                           const half_t *values_in, half_t *values_out, float scale, hipStream_t stream,
                           const Batch &batch = Batch());
+// The softmax driven by a dispatch list of row parts: `workspace` takes a (maximum, sum) pair per part and scalar row.
+int launch_sparse_softmax_row_parts(int vec_length, int n_slots, const int *slots, int n_split, int parts_max,
+                                    const half_t *values_in, half_t *values_out, float scale, void *workspace,
+                                    long long workspace_bytes, hipStream_t stream, const Batch &batch);
+long long sparse_softmax_row_parts_workspace_bytes(int batch, int vec_length, int n_split, int parts_max);
 
 }  // namespace vs

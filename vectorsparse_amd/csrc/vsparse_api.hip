@@ -525,6 +525,30 @@ int vs_sparse_softmax_f16(int batch, int m_vec, int vec_length, const int *row_i
                                      make_batch(batch, stride_in, 0, stride_out));
 }
 
+long long vs_sparse_softmax_row_parts_workspace_bytes(int batch, int vec_length, int n_split, int parts_max)
+{
+    if (!vec_ok(vec_length)) return 0;
+    return vs::sparse_softmax_row_parts_workspace_bytes(batch, vec_length, n_split, parts_max);
+}
+
+int vs_sparse_softmax_f16_row_parts(int batch, int vec_length, int n_slots, const int *slots, int n_split, int parts_max,
+                                    const void *values_in, long long stride_in, void *values_out, long long stride_out,
+                                    float scale, void *workspace, long long workspace_bytes, void *stream)
+{
+    if (batch < 0 || n_slots < 0 || n_split < 0 || parts_max < 0 || workspace_bytes < 0 || !vec_ok(vec_length))
+        return VS_ERROR_INVALID_VALUE;
+    if (batch == 0 || n_slots == 0) return VS_SUCCESS;
+    if (!slots || !aligned(slots, 16)) return VS_ERROR_INVALID_VALUE;
+    if (!aligned(values_in, 2 * (size_t)vec_length) || !aligned(values_out, 2 * (size_t)vec_length))
+        return VS_ERROR_INVALID_VALUE;
+    if (!stride_ok(stride_in, vec_length) || !stride_ok(stride_out, vec_length)) return VS_ERROR_INVALID_VALUE;
+    if (workspace_bytes > 0 && (!workspace || !aligned(workspace, 8))) return VS_ERROR_INVALID_VALUE;
+    return vs::launch_sparse_softmax_row_parts(vec_length, n_slots, slots, n_split, parts_max,
+                                               static_cast<const half_t *>(values_in), static_cast<half_t *>(values_out),
+                                               scale, workspace, workspace_bytes, static_cast<hipStream_t>(stream),
+                                               make_batch(batch, stride_in, 0, stride_out));
+}
+
 void vs_identity_row_swizzle(int rows, int *row_indices)
 {
     if (rows <= 0 || !row_indices) return;

@@ -503,6 +503,31 @@ def sddmm_row_parts(k, n, parts, slots, nonzeros_vec, col_indices, lhs_matrix, r
     return output_values
 
 
+def sparse_softmax_row_parts(vec_length, parts, slots, values_in, values_out=None, scale=1.0, workspace=None,
+                             stream=None):
+    """Row-wise softmax of scale * values driven by a dispatch list of row parts (`parts`: a RowParts, `slots`: its
+    list as a device int32 tensor); values [nnz_vec, V] or [batch, nnz_vec, V].  workspace: a device tensor of at
+    least sparse_softmax_row_parts_workspace_bytes(...) bytes (None when no row is split).  Returns values_out
+    (values_in when None: in place)."""
+    if values_out is None:
+        values_out = values_in
+    batch = values_in.shape[0] if values_in.dim() == 3 else 1
+    stride = lambda t: t.stride(0) if t.dim() == 3 else 0
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    st = _lib.lib().vs_sparse_softmax_f16_row_parts(
+        batch, vec_length, parts.n_slots, _expect(slots, torch.int32, "slots"), parts.n_split, parts.parts_max,
+        _expect(values_in, torch.float16, "values_in"), stride(values_in),
+        _expect(values_out, torch.float16, "values_out"), stride(values_out), float(scale), _ptr(workspace), ws_bytes,
+        _stream(stream))
+    if st:
+        _lib.check(st, "vs_sparse_softmax_f16_row_parts")
+    return values_out
+
+
+def sparse_softmax_row_parts_workspace_bytes(vec_length, n_split, parts_max, batch=1):
+    return int(_lib.lib().vs_sparse_softmax_row_parts_workspace_bytes(batch, vec_length, n_split, parts_max))
+
+
 LONG_ROW_VECTORS = 512  # rows beyond this are "long" for vs_wmma_spmm_f16_batched_sorted (eight 64-vector blocks)
 
 
