@@ -663,3 +663,30 @@ def test_sparse_softmax_over_rows_in_parts(gpu, V, limit):
     # one vector row of the whole: every scalar row sums to one
     sums = out[0].float().cpu().numpy()[ro[10]:ro[11]].sum(axis=0)
     assert np.allclose(sums, 1.0, atol=2e-2)
+
+
+def test_attention_with_global_tokens_takes_rows_in_parts(gpu):
+    """A band mask with global tokens (a few rows that attend to everything, a few columns everybody attends to): the
+    layer picks the three operators on the dispatch list of row parts; same contract as the other routes."""
+    seq, V, heads, d = 2048, 8, 3, 64
+    rows = []
+    for i in range(seq // V):
+        c = i * V + V // 2
+        rows.append(np.arange(seq) if i < 2 else np.union1d(np.arange(max(0, c - 24), min(seq, c + 24)), np.arange(16)))
+    ro = np.concatenate([[0], np.cumsum([len(r) for r in rows])]).astype(np.int32)
+    mask = cv.ColVecCSR(seq // V, seq, V, ro, np.concatenate(rows).astype(np.int32))
+    layer = ops.SparseAttention(mask)
+    assert layer.prob.row_parts(0)[0].n_split == 2
+    g = torch.Generator(device="cuda").manual_seed(8)
+    q, k, v = (torch.randn((heads, seq, d), device="cuda", generator=g).half() for _ in range(3))
+    got = layer.forward(q, k, v)                       # automatic: the parts chain
+    forced = layer.forward(q, k, v, fused="parts")
+    chain = layer.forward(q, k, v, fused=False)        # the three operators on whole rows
+    torch.cuda.synchronize()
+    assert torch.equal(got, forced)
+    ref = _dense_attention(mask, q.cpu().numpy(), k.cpu().numpy(), v.cpu().numpy(), 1.0 / 8.0)
+    _check_layer(got.cpu().numpy(), ref, "rows in parts, global tokens")
+    _check_layer(chain.cpu().numpy(), ref, "whole rows, global tokens")
+    # against the chain on whole rows: the same arithmetic up to the order of the fp32 sums
+    diff = (got.float() - chain.float()).abs().max().item()
+    assert diff < 2e-2 * max(1.0, chain.float().abs().max().item()), diff

@@ -384,7 +384,8 @@ class SparseAttention:
     def forward(self, q, k, v, scale=None, kernel="wmma", stream=None, scores=None, out=None, fused=None):
         """q, k, v: fp16 [heads, seq, d] on the device.  Returns fp16 [heads, seq, d].
 
-        fused: "layer" runs the whole layer in one launch with scores and probabilities kept in LDS; True
+        fused: "parts" runs the three operators on the dispatch list of row parts (masks with rows far longer than
+        the rest, e.g. global tokens); "layer" runs the whole layer in one launch with scores and probabilities kept in LDS; True
         folds only the softmax into the SpMM launch (two launches, raw scores go through memory); False runs
         the three operators one after the other.  Default on the MFMA path: "layer" when the cost model of
         `_union_rows` puts the streamed union kernel ahead (banded, blocky, strided and very sparse masks: 1.5-15x
@@ -403,8 +404,17 @@ class SparseAttention:
         if fused is None:
             if kernel != "wmma":
                 fused = False
+            elif d % 8 == 0 and v.shape[2] % 4 == 0 and p.n * v.shape[2] < 2 ** 31 and p.row_parts(0)[0].n_split > 0:
+                # rows far longer than the rest - global tokens: the three operators on the dispatch list of row
+                # parts (16 heads x 4096, d = 64, a +-32..128 band with 64-256 global tokens: 72-119 us against
+                # 145-160 us in one launch and 280-295 us for SDDMM + softmax-fused SpMM on whole rows)
+                fused = "parts"
             else:
                 fused = "layer" if self.union_rows(q.shape[2], v.shape[2], heads) >= 2 else True
+        if fused == "parts":
+            p.sddmm_row_parts(q, k, out=scores, stream=stream)
+            p.softmax_row_parts(scores, scale=scale, stream=stream)
+            return p.spmm_row_parts(v, out=out, stream=stream, limit_vec=512, values=scores)
         if fused == "layer":
             return sparse_attention(p.m_vec, p.vec_length, p.n, p.row_indices, p.row_offsets, p.column_indices,
                                     q, k, v, out=out, scale=scale, stream=stream,
@@ -574,22 +584,38 @@ class DeviceProblem:
         if limit_vec not in self._parts:
             parts = RowParts(self.m_vec, self.pattern.row_offsets, limit_vec)
             slots = torch.from_numpy(parts.slots).to(self.column_indices.device)
-            self._parts[limit_vec] = [parts, slots, None]
+            self._parts[limit_vec] = [parts, slots, None, None]   # (+ SpMM workspace, softmax workspace: on first use)
         return self._parts[limit_vec]
 
-    def spmm_row_parts(self, rhs_matrix, out=None, stream=None, limit_vec=0):
+    def spmm_row_parts(self, rhs_matrix, out=None, stream=None, limit_vec=0, values=None):
         """SpMM (MFMA path, fp16 output) with long rows dispatched as several parts; the list and the workspace
-        for the parts' partial tiles belong to this object."""
-        k = rhs_matrix.shape[1]
+        for the parts' partial tiles belong to this object.  values: the pattern's own by default; [batch, nnz_vec, V]
+        (with rhs_matrix [batch, n, k] or [n, k]) runs a batch on the shared pattern."""
+        values = self.values if values is None else values
+        k = rhs_matrix.shape[-1]
+        batch = values.shape[0] if values.dim() == 3 else 1
         if out is None:
-            out = torch.empty((self.m_vec * self.vec_length, k), dtype=torch.float16, device=rhs_matrix.device)
+            shape = (self.m_vec * self.vec_length, k) if values.dim() == 2 else (batch, self.m_vec * self.vec_length, k)
+            out = torch.empty(shape, dtype=torch.float16, device=rhs_matrix.device)
         entry = self.row_parts(limit_vec)
         parts, slots = entry[0], entry[1]
-        need = spmm_row_parts_workspace_bytes(self.vec_length, k, parts.n_split, parts.parts_max)
+        need = spmm_row_parts_workspace_bytes(self.vec_length, k, parts.n_split, parts.parts_max, batch=batch)
         if need and (entry[2] is None or entry[2].numel() < need):
             entry[2] = torch.zeros(need, dtype=torch.uint8, device=rhs_matrix.device)
-        return spmm_row_parts(self.vec_length, k, self.n, parts, slots, self.nnz_vec, self.column_indices, self.values,
+        return spmm_row_parts(self.vec_length, k, self.n, parts, slots, self.nnz_vec, self.column_indices, values,
                               rhs_matrix, out, entry[2] if need else None, stream)
+
+    def softmax_row_parts(self, values_in, values_out=None, scale=1.0, stream=None, limit_vec=512):
+        """Row-wise softmax of scale * values ([nnz_vec, V] or [batch, nnz_vec, V]) with long rows normalised by
+        several waves (in place by default)."""
+        entry = self.row_parts(limit_vec)
+        parts, slots = entry[0], entry[1]
+        batch = values_in.shape[0] if values_in.dim() == 3 else 1
+        need = sparse_softmax_row_parts_workspace_bytes(self.vec_length, parts.n_split, parts.parts_max, batch=batch)
+        if need and (entry[3] is None or entry[3].numel() < need):
+            entry[3] = torch.empty(need, dtype=torch.uint8, device=values_in.device)
+        return sparse_softmax_row_parts(self.vec_length, parts, slots, values_in, values_out, scale,
+                                        entry[3] if need else None, stream)
 
     def spmm(self, rhs_matrix, kernel="wmma", out_dtype=torch.float16, out=None, stream=None, row_length_hint=False,
              split_rows=False):
@@ -630,9 +656,10 @@ class DeviceProblem:
         """SDDMM (MFMA path, fp16 output, k % 8 == 0) with long rows of the mask dispatched as several parts.  The
         parts have nothing to add up, so the limit is low (measured at K = 64..256 on 256 to 2048 rows of Pareto
         lengths and on a dense row among short ones: 128 to 512 vectors within 5 % of each other, 1152 20-70 % behind)."""
-        k = lhs_matrix.shape[1]
+        k = lhs_matrix.shape[-1]   # (operands [rows, k], or [batch, rows, k] for a batch on the shared mask)
         if out is None:
-            out = torch.empty((self.nnz_vec, self.vec_length), dtype=torch.float16, device=lhs_matrix.device)
+            lead = (lhs_matrix.shape[0],) if lhs_matrix.dim() == 3 else ()
+            out = torch.empty(lead + (self.nnz_vec, self.vec_length), dtype=torch.float16, device=lhs_matrix.device)
         parts, slots = self.row_parts(limit_vec)[:2]
         return sddmm_row_parts(k, self.n, parts, slots, self.nnz_vec, self.column_indices, lhs_matrix, rhs_matrix, out,
                                self.vec_length, stream)
