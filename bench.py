@@ -447,6 +447,25 @@ def main():
     wlayer = ops.SparseAttention(wmask)
     _, window_ms = time_graph(torch, lambda: wlayer.forward(q, kk_, vv, out=ctx), attn_steps, 3)
 
+    # a +-64 band with 64 global tokens (eight vector rows that attend to everything, 64 columns everybody attends
+    # to): rows far longer than the rest, which the layer runs as three operators on a dispatch list of row parts
+    grows = []
+    for i in range(seq // 8):
+        c = 8 * i + 4
+        grows.append(np.arange(seq) if i < 8 else np.union1d(np.arange(max(0, c - 64), min(seq, c + 64)), np.arange(64)))
+    gmask = cv.ColVecCSR(seq // 8, seq, 8, np.concatenate([[0], np.cumsum([len(r) for r in grows])]).astype(np.int32),
+                         np.concatenate(grows).astype(np.int32))
+    glayer = ops.SparseAttention(gmask)
+    gscores = torch.empty((heads, gmask.nnz_vec, 8), dtype=torch.float16, device="cuda")
+    _, global_ms = time_graph(torch, lambda: glayer.forward(q, kk_, vv, scores=gscores, out=ctx), attn_steps, 3)
+    gref = ctx.clone()
+    _, global_whole_rows_ms = time_graph(torch, lambda: glayer.forward(q, kk_, vv, scores=gscores, out=ctx, fused=True),
+                                         attn_steps, 3)
+    torch.cuda.synchronize()
+    global_diff = float((ctx.float() - gref.float()).abs().max())
+    if not global_diff < 2e-2:
+        raise SystemExit("attention with global tokens: rows in parts and whole rows disagree: %g" % global_diff)
+
     # ---- cold caches (how the reference measures: Nsight --cache-control all)
     cold_ms = time_cold(torch, step)
     cold_floor_ms = time_cold(torch, probe(512))  # what the same method reads for a kernel that does nothing
@@ -540,6 +559,10 @@ def main():
                                           speedup_vs_dense=sddmm_dense_ms / valu_sddmm_ms)},
             "attention_window513": {"layer_ms": window_ms, "density": 1.0 - wmask.sparsity,
                                     "tflops": 2.0 * wmask.nnz * heads * dim * 2 / (window_ms * 1e-3) * 1e-12},
+            "attention_global_tokens": {"workload": "16 heads x 4096 x 64, +-64 band with 64 global tokens",
+                                        "density": 1.0 - gmask.sparsity, "layer_ms": global_ms,
+                                        "whole_rows_sddmm_softmax_spmm_ms": global_whole_rows_ms,
+                                        "speedup": global_whole_rows_ms / global_ms},
             "attention_config5": {"layer_ms": attn_ms, "density": 1.0 - amask.sparsity,
                                   "tflops": attn_flops / (attn_ms * 1e-3) * 1e-12,
                                   "dense_masked_attention_ms": dense_attn_ms,
