@@ -459,10 +459,15 @@ class RowParts:
         ro = np.ascontiguousarray(row_offsets, dtype=np.int32)
         step = 1152 if limit_vec <= 0 else (limit_vec + 63) // 64 * 64   # (the default limit is 1152 at least)
         room = m_vec + 2 * (int(ro[m_vec] if m_vec > 0 else 0) // step) + 64
-        slots = np.empty((room, 4), dtype=np.int32)
         counts = [ctypes.c_int(0) for _ in range(4)]
-        st = _lib.lib().vs_spmm_row_parts(m_vec, ro.ctypes.data, limit_vec, slots.ctypes.data, room,
-                                          *[ctypes.addressof(c) for c in counts])
+        for attempt in range(2):
+            slots = np.empty((room, 4), dtype=np.int32)
+            st = _lib.lib().vs_spmm_row_parts(m_vec, ro.ctypes.data, limit_vec, slots.ctypes.data, room,
+                                              *[ctypes.addressof(c) for c in counts])
+            if st == 801 and attempt == 0 and counts[0].value + counts[1].value > room:
+                room = counts[0].value + counts[1].value   # (the counts say what the list needs)
+                continue
+            break
         if st:
             _lib.check(st, "vs_spmm_row_parts")
         self.n_slots, self.n_split, self.parts_max, self.longest_part_vec = (c.value for c in counts)
