@@ -288,3 +288,31 @@ def test_batch_on_a_shared_pattern(gpu, V, launches):
             # (not bit for bit: how a row's blocks are shared among waves follows the size of the launch)
             assert_parity(out[b].cpu().numpy(), single.float().cpu().numpy(), "batched against single, problem %d" % b)
     assert not ws.cpu().numpy()[:need // 5 // 256 * 256].any(), "the arrival counters must be back at zero"
+
+
+def test_batch_of_one_ignores_the_leading_stride(gpu):
+    """[1, ...] operands whose leading stride is no multiple of 16 bytes (n * k odd multiples of 4 halves): a batch of
+    one passes no per-problem stride, so the alignment rule for strides does not apply; all three operators."""
+    V, n, N = 4, 333, 12
+    lengths = [333, 5, 0, 200, 17, 333, 1]
+    pat = _from_lengths(lengths, n, V, seed=61)
+    B = cv.dense_uniform(n, N, seed=62)
+    parts = ops.RowParts(pat.m_vec, pat.row_offsets, 64)
+    assert parts.n_split > 0 and (n * N) % 8 != 0
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    slots, ci = d(parts.slots), d(pat.column_indices)
+    ws = torch.zeros(ops.spmm_row_parts_workspace_bytes(V, N, parts.n_split, parts.parts_max), dtype=torch.uint8,
+                     device="cuda")
+    out = torch.empty((1, pat.m, N), dtype=torch.float16, device="cuda")
+    ops.spmm_row_parts(V, N, n, parts, slots, pat.nnz_vec, ci, d(pat.values[None]), d(B[None]), out, ws)
+    torch.cuda.synchronize()
+    assert_parity(out[0].cpu().numpy(), _oracle(pat, B), "batch of one, [1, n, k] operands")
+
+    scores = d(pat.values[None]).clone()
+    sm_ws = torch.empty(max(8, ops.sparse_softmax_row_parts_workspace_bytes(V, parts.n_split, parts.parts_max)),
+                        dtype=torch.uint8, device="cuda")
+    ops.sparse_softmax_row_parts(V, parts, slots, scores, scale=0.5, workspace=sm_ws)
+    torch.cuda.synchronize()
+    from oracle import numpy_oracle as no
+    assert_parity(scores[0].cpu().numpy(), no.sparse_softmax_ref(pat.m_vec, V, pat.row_offsets, pat.values, 0.5),
+                  "softmax, batch of one")

@@ -487,7 +487,7 @@ def spmm_row_parts(vec_length, k, n, parts, slots, nonzeros_vec, column_indices,
     without it shared.  Returns output_matrix."""
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     batch = output_matrix.shape[0] if output_matrix.dim() == 3 else 1
-    per_problem = lambda t, dims: (t.stride(0) if t.dim() == dims + 1 else 0)
+    per_problem = lambda t, dims: _stride(t, batch)
     st = _lib.lib().vs_wmma_spmm_f16_row_parts(
         batch, vec_length, k, n, parts.n_slots, _expect(slots, torch.int32, "slots"), parts.n_split, parts.parts_max,
         nonzeros_vec, parts.longest_part_vec, _expect(column_indices, torch.int32, "column_indices"),
@@ -507,7 +507,7 @@ def sddmm_row_parts(k, n, parts, slots, nonzeros_vec, col_indices, lhs_matrix, r
     mask; lhs_matrix / rhs_matrix with the same leading dimension are per problem, without it shared.  Returns
     output_values."""
     batch = output_values.shape[0] if output_values.dim() == 3 else 1
-    per_problem = lambda t, dims: (t.stride(0) if t.dim() == dims + 1 else 0)
+    per_problem = lambda t, dims: _stride(t, batch)
     st = _lib.lib().vs_wmma_sddmm_f16_row_parts(
         batch, k, n, parts.n_slots, _expect(slots, torch.int32, "slots"), nonzeros_vec,
         _expect(col_indices, torch.int32, "col_indices"), _expect(lhs_matrix, torch.float16, "lhs_matrix"),
@@ -527,7 +527,7 @@ def sparse_softmax_row_parts(vec_length, parts, slots, values_in, values_out=Non
     if values_out is None:
         values_out = values_in
     batch = values_in.shape[0] if values_in.dim() == 3 else 1
-    stride = lambda t: t.stride(0) if t.dim() == 3 else 0
+    stride = lambda t: _stride(t, batch)
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     st = _lib.lib().vs_sparse_softmax_f16_row_parts(
         batch, vec_length, parts.n_slots, _expect(slots, torch.int32, "slots"), parts.n_split, parts.parts_max,
