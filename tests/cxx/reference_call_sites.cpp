@@ -210,6 +210,30 @@ int main()
         HIP_OK(hipDeviceSynchronize());
         fetch_h(d_sd_h, want_sddmm.size());
         ok &= close_enough("vs_wmma_sddmm_f16_row_parts", got_f, want_sddmm);
+        // the row-wise softmax on the same list, in place on the SDDMM's outputs (layout [nonzero vector][V]: scalar
+        // row v of a vector row owns every V-th value); expected values from the fp16 scores just fetched
+        {
+            const float scale = 0.125f;
+            std::vector<float> want_softmax(got_f.size());
+            for (int r = 0; r < m_vec; ++r)
+                for (int v = 0; v < V; ++v) {
+                    float top = -INFINITY;
+                    double sum = 0;
+                    for (int j = row_offsets[r]; j < row_offsets[r + 1]; ++j) top = std::max(top, scale * got_f[(size_t)j * V + v]);
+                    for (int j = row_offsets[r]; j < row_offsets[r + 1]; ++j) sum += std::exp(scale * got_f[(size_t)j * V + v] - top);
+                    for (int j = row_offsets[r]; j < row_offsets[r + 1]; ++j)
+                        want_softmax[(size_t)j * V + v] = (float)(std::exp(scale * got_f[(size_t)j * V + v] - top) / sum);
+                }
+            const long long sm_bytes = vs_sparse_softmax_row_parts_workspace_bytes(1, V, n_split, parts_max);
+            void *sm_workspace = nullptr;
+            HIP_OK(hipMalloc(&sm_workspace, (size_t)std::max<long long>(sm_bytes, 8)));  // no need to clear it
+            HIP_OK((hipError_t)vs_sparse_softmax_f16_row_parts(1, V, n_slots, d_slots, n_split, parts_max, d_sd_h, 0, d_sd_h, 0,
+                                                               scale, sm_workspace, sm_bytes, nullptr));
+            HIP_OK(hipDeviceSynchronize());
+            fetch_h(d_sd_h, want_softmax.size());
+            ok &= close_enough("vs_sparse_softmax_f16_row_parts", got_f, want_softmax);
+            HIP_OK(hipFree(sm_workspace));
+        }
         std::printf("%-22s %d slots, %d rows in up to %d parts\n", "", n_slots, n_split, parts_max);
         ok &= n_split > 0;
         HIP_OK(hipFree(workspace));
