@@ -257,7 +257,8 @@ int vs_wmma_spmm_f16_batched_sorted(int batch, int m_vec, int vec_length, int k,
  * slot of its own; the slots are ordered longest first.  slots: four ints per slot {vector row, first nonzero,
  * end, part info (0 = a whole row)}, room for max_slots of them.  Returns the number of slots, of split rows, the
  * most parts any row has and the longest slot through the pointers; VS_ERROR_NOT_SUPPORTED with the counts set
- * when max_slots is too small or more than 32767 rows would be split.  Behind the n_slots entries the list holds
+ * when max_slots is too small.  At most 32767 rows are split (the first ones in row order; longer rows past
+ * that number stay whole, which costs balance, not correctness).  Behind the n_slots entries the list holds
  * one more entry per split row ({vector row, parts, 0, 0}, for the launch that adds the parts when option
  * "spmm_parts_launches" is 2): n_slots + n_split entries in all, m_vec + 2 * (nonzeros_vec / limit) + 1 always
  * suffice.

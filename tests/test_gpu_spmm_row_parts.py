@@ -316,3 +316,17 @@ def test_batch_of_one_ignores_the_leading_stride(gpu):
     from oracle import numpy_oracle as no
     assert_parity(scores[0].cpu().numpy(), no.sparse_softmax_ref(pat.m_vec, V, pat.row_offsets, pat.values, 0.5),
                   "softmax, batch of one")
+
+
+def test_more_long_rows_than_split_rows_can_be_numbered(gpu):
+    """33000 rows of 128 vectors at a limit of 64: 32767 rows run as two halves, the others whole, in one list and
+    one launch; one and two launches agree bit for bit and with the oracle."""
+    V, m_vec, n, N = 1, 33000, 256, 8
+    pat = _from_lengths(np.full(m_vec, 128), n, V, seed=71)
+    B = cv.dense_uniform(n, N, seed=72)
+    ref = _oracle(pat, B)
+    one, parts = _run(pat, B, limit=64, options={"spmm_parts_launches": 1})
+    assert parts.n_split == 32767 and parts.n_slots == m_vec + 32767
+    assert_parity(one, ref, "32767 split rows and 233 whole ones")
+    two, _ = _run(pat, B, limit=64, options={"spmm_parts_launches": 2})
+    assert np.array_equal(one, two)

@@ -308,6 +308,22 @@ def test_row_parts_dispatch_list():
         assert (covered == 1).all()
         assert split_ids == set(range(parts.n_split))
         assert parts.parts_max == (max((s[:, 3] & 255)) if parts.n_split else 0)
+    # more rows beyond the limit than a split row's number can count: the first 32767 are split, the others whole
+    m_vec = 33000
+    ro = (np.arange(m_vec + 1, dtype=np.int64) * 128).astype(np.int32)
+    parts = ops.RowParts(m_vec, ro, 64)
+    assert parts.n_split == 32767 and parts.parts_max == 2 and parts.n_slots == m_vec + 32767
+    assert parts.longest_part_vec == 128
+    s = parts.slots[:parts.n_slots]
+    whole = s[s[:, 3] == 0]
+    assert np.array_equal(np.sort(whole[:, 0]), np.arange(32767, m_vec)) and (whole[:, 2] - whole[:, 1] == 128).all()
+    halves = s[s[:, 3] != 0]
+    assert (halves[:, 2] - halves[:, 1] == 64).all() and np.array_equal(np.sort(halves[:, 3] >> 16),
+                                                                        np.repeat(np.arange(32767), 2))
+    covered = np.zeros(int(ro[-1]), dtype=np.int32)
+    np.add.at(covered, (s[:, 1][:, None] + np.arange(64)[None, :]).reshape(-1), 1)
+    np.add.at(covered, (whole[:, 1][:, None] + 64 + np.arange(64)[None, :]).reshape(-1), 1)
+    assert (covered == 1).all()
     # too little room: the counts say what the list needs
     ro = np.array([0, 2000, 2010], dtype=np.int32)
     slots = np.zeros((2, 4), dtype=np.int32)

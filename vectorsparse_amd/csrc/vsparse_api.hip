@@ -600,12 +600,13 @@ int vs_spmm_row_parts(int m_vec, const int *row_offsets, int limit_vec, int *slo
         if (count > 255) count = 255;
         const long long per = ((len + count - 1) / count + 63) / 64 * 64;
         count = (len + per - 1) / per;
-        if (count < 2) {  // (rounding the part up to whole blocks took the whole row)
+        // (rounding the part up to whole blocks may take the whole row; a split row's number has 15 bits in the
+        // part info: past 32767 split rows the others stay whole - slower to finish, the same result)
+        if (count < 2 || split >= 32767) {
             parts.push_back({row, beg, end, 0});
             longest = len > longest ? (int)len : longest;
             continue;
         }
-        if (split >= 32767) return VS_ERROR_NOT_SUPPORTED;
         for (long long p = 0; p < count; ++p) {
             const long long from = beg + p * per;
             const long long to = from + per < end ? from + per : end;
