@@ -272,8 +272,9 @@ int vs_wmma_spmm_f16_batched_sorted(int batch, int m_vec, int vec_length, int k,
  * aligned, at least vs_wmma_spmm_row_parts_workspace_bytes(batch, vec_length, k, n_split, parts_max) bytes (0 when no
  * row is split), ZERO-FILLED before its first use; its arrival counters (an area that depends on
  * workspace_bytes alone) are left at zero by every call, so it serves any sequence of calls that do not
- * overlap, whatever their shapes, as long as it is passed with the same size.  Requires k % 4 == 0 and
- * n * k < 2^31, else 801.  batch, stride_*: as in vs_wmma_spmm_f16_batched - `batch` problems share the pattern (and
+ * overlap, whatever their shapes, as long as it is passed with the same size.  Requires k % 4 == 0,
+ * n * k < 2^31 and partial tiles (batch * n_split * parts_max * vec_length * k rounded up to 128, 4 bytes each) of
+ * less than 2 GiB, else 801 - raise limit_vec in that case.  batch, stride_*: as in vs_wmma_spmm_f16_batched - `batch` problems share the pattern (and
  * the list), problem b reads values + b * stride_values and rhs_matrix + b * stride_rhs and writes output_matrix +
  * b * stride_output (strides in elements, 0 = shared operand; multiples of vec_length / 8 / 8); batch = 1 with
  * strides 0 is the single operator.
