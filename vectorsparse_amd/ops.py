@@ -637,9 +637,12 @@ class DeviceProblem:
             # rows in parts wherever the dispatch list splits a row (measured ahead of both other schedules on
             # Pareto lengths and on a dense row among short ones, 64 to 2048 rows; within 4 % on log-normal lengths),
             # else the row-length hints
-            if kernel == "wmma" and k % 4 == 0 and out.dtype == torch.float16 and self.n * k < 2 ** 31 \
-                    and self.row_parts(0)[0].n_split > 0:
-                return self.spmm_row_parts(rhs_matrix, out=out, stream=stream)
+            if kernel == "wmma" and k % 4 == 0 and out.dtype == torch.float16 and self.n * k < 2 ** 31:
+                parts = self.row_parts(0)[0]
+                # (the entry point addresses the partial tiles with 32-bit offsets: less than 2 GiB of them)
+                if parts.n_split > 0 and spmm_row_parts_workspace_bytes(self.vec_length, k, parts.n_split,
+                                                                        parts.parts_max) < 2 ** 31:
+                    return self.spmm_row_parts(rhs_matrix, out=out, stream=stream)
             split_rows = False
             row_length_hint = True
         if split_rows and kernel == "wmma":
