@@ -40,8 +40,8 @@ def _run(cmd, verbose):
 def _stale(src, obj):
     if not os.path.exists(obj):
         return True
-    newest = max(os.path.getmtime(p) for p in [src, os.path.join(CSRC, "vs_common.hpp"),
-                                               os.path.join(os.path.dirname(_HERE), "include", "vsparse.h")])
+    headers = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp")]
+    newest = max(os.path.getmtime(p) for p in [src, os.path.join(os.path.dirname(_HERE), "include", "vsparse.h")] + headers)
     return os.path.getmtime(obj) < newest
 
 
@@ -77,19 +77,7 @@ def build_cxx_caller(verbose=False):
     return exe
 
 
-def build_probes(verbose=False):
-    """Compile csrc/probes/machine_probe.hip (launch floor, dependent-load latency, gather ceiling of the GPU) to
-    vectorsparse_amd/probes/machine_probe; run it on an MI355X to get the floors that the kernels' timings are judged against."""
-    out_dir = os.path.join(_HERE, "probes")
-    os.makedirs(out_dir, exist_ok=True)
-    exe = os.path.join(out_dir, "machine_probe")
-    _run([HIPCC, "-O3", "--offload-arch=gfx950", "-std=c++17", "-Wno-unused-value",
-          os.path.join(CSRC, "probes", "machine_probe.hip"), "-o", exe], verbose)
-    return exe
-
-
 if __name__ == "__main__":
     print(build(verbose=True, incremental="--incremental" in sys.argv))
     print(build_cxx_caller(verbose=True))
-    print(build_probes(verbose=True))
     sys.exit(0)
