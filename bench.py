@@ -189,7 +189,7 @@ def cpu_baseline(pat, B, n_dense, flops, budget_s=12.0):
     }
 
 
-PMC_MODES = ["spmm", "spmm_largest", "spmm_dma", "spmm_split_rows", "spmm_row_parts", "sddmm", "attention",
+PMC_MODES = ["spmm", "spmm_largest", "spmm_slab_50", "spmm_slab_90", "spmm_dma", "spmm_split_rows", "spmm_row_parts", "sddmm", "attention",
              "attention_window"]
 
 
@@ -218,7 +218,7 @@ def main():
     ap.add_argument("--pmc", nargs="?", const="spmm", default=None, choices=PMC_MODES,
                     help="counter-collection mode for `rocprofv3 --pmc`: a 64 MiB device copy of known size "
                          "(calibration), then ten eager launches of one kernel and nothing else: the headline SpMM "
-                         "(config 2), the largest sweep point (2048 x 4608 at 90 %%), config 2 on the LDS-DMA gather "
+                         "(config 2), the largest sweep point (2048 x 4608 at 90 %%), the LDS-staged schedule on that shape at 50 %% and 90 %%, config 2 on the LDS-DMA gather "
                          "variant, the split-row SpMM and the SpMM with rows in parts on Pareto-distributed rows, the config-4 SDDMM, the config-5 "
                          "attention layer with its plan, or that layer with a plain 513-wide window mask")
     args = ap.parse_args()
@@ -286,6 +286,20 @@ def main():
             info["algorithmic_bytes"] = spmm_algorithmic_bytes(lpat, 256)
             info["nonzero_vectors"] = int(lpat.nnz_vec)
             info["kernel_source_tag"] = kernel_source_tag(*SPMM_SOURCES)
+        elif args.pmc in ("spmm_slab_50", "spmm_slab_90"):
+            # the LDS-staged schedule (vs_wmma_spmm_f16_slab) on 2048 x 4608 x 256 at 50 % / 90 %, ten launches
+            lpat = cv.random_values(cv.uniform_pattern(2048 // 8, 4608, 0.5 if args.pmc.endswith("50") else 0.9,
+                                                       seed=3, vec_length=8), seed=4)
+            lprob = ops.DeviceProblem(lpat, sort=True)
+            lBd = torch.from_numpy(cv.dense_uniform(4608, 256, seed=5)).cuda()
+            lout = torch.empty((lpat.m, 256), dtype=torch.float16, device="cuda")
+            ws = torch.empty(max(16, ops.spmm_slab_workspace_bytes(lpat.m_vec, 8, 256, 4608)), dtype=torch.uint8, device="cuda")
+            for _ in range(10):
+                ops.spmm_slab(lpat.m_vec, 8, 256, 4608, lprob.row_indices, lprob.row_offsets, lprob.column_indices,
+                              lprob.values, lBd, lout, ws)
+            info["algorithmic_bytes"] = spmm_algorithmic_bytes(lpat, 256)
+            info["nonzero_vectors"] = int(lpat.nnz_vec)
+            info["kernel_source_tag"] = kernel_source_tag("spmm_mfma_slab.hip", "spmm_mfma_step.hpp", "vs_common.hpp")
         elif args.pmc == "spmm_split_rows":
             kpat, kB = skewed_point(cv, np)
             kprob = ops.DeviceProblem(kpat, sort=True)

@@ -127,6 +127,28 @@ int vs_wmma_spmm_f16_noalloc(int m_vec, int vec_length, int k, int n, int nonzer
                              const void *rhs_matrix, void *output_matrix, void *stream);
 
 /*
+ * The same operator (spmm::wmmaSpmm, include/wmma_spmm.cuh:15-21; the tile loop of src/wmma_spmm.cu:77-90, whose
+ * dense tile loader src/spmm_utils/dense_tile.h:255-259 fetches every nonzero's rhs row from memory) on a schedule that
+ * stages the dense operand in LDS once per block of eight vector rows: a workgroup walks its part of the contraction in
+ * windows of 128 rhs rows, loaded dense and coalesced, and every wave picks its own row's nonzeros out of the resident
+ * windows.  A block of rows is spread over several parts of the contraction (so that the launch fills the chip); the
+ * parts leave fp32 tiles in `workspace` and a second launch adds them in ascending order (deterministic).
+ * workspace: device memory, 16-byte aligned, at least vs_wmma_spmm_slab_workspace_bytes(...) bytes (0 when the
+ * rows alone fill the chip); its contents are undefined before and after, nothing has to be cleared.  Requires
+ * k % 8 == 0 and n * k < 2^31, else 801.  Columns need not be sorted (sorted columns are what it is fast on).
+ * Measured slower than vs_wmma_spmm_f16 on every shape of the ResNet-shaped sweep (2048 x 4608 x 256, V = 8: 31 us
+ * against 15.6 us at 50 % sparsity, 28 against 5.3 us at 90 %), so no other entry point chooses it; it exists as the
+ * measured form of the LDS-staged tile loop.  Option "spmm_slab_parts" (1..64, 0 = automatic) sets the number of parts
+ * for the calls that follow - pass the same value to both functions.
+ */
+long long vs_wmma_spmm_slab_workspace_bytes(int m_vec, int vec_length, int k, int n);
+int vs_wmma_spmm_f16_slab(int m_vec, int vec_length, int k, int n,
+                          const int *row_indices, const int *row_offsets,
+                          const int *column_indices, const void *values,
+                          const void *rhs_matrix, void *output_matrix,
+                          void *workspace, long long workspace_bytes, void *stream);
+
+/*
  * Replaces spmm::cudaSpmm(half in, half out) — include/cuda_spmm.cuh:15-21,
  * src/cuda_spmm.cu:316-325.  Fine-grained path on the fp16 vector ALU
  * (mixed-precision FMA: exact fp16 x fp16 products, fp32 accumulate).  The
@@ -486,6 +508,7 @@ int vs_wmma_spmm_launch_shape(int batch, int m_vec, int vec_length, int k, int n
  * brings the gathered rows of the dense operand to the matrix cores: 1 = through
  * registers and an in-register transpose, 2 = global -> LDS loads and transposing LDS
  * reads, k % 8 == 0 only; 0 = automatic, which is 1: 2 measured 10-18 % slower),
+ * "spmm_slab_parts" (vs_wmma_spmm_f16_slab: parts of the contraction, 1..64, 0 = automatic),
  * "spmm_flat_piece" (nonzero vectors
  * per wave of the split-row SpMM, rounded up to 32, 0 = automatic), "spmm_flat_waves"
  * (its waves per workgroup, 1..16, 0 = automatic), "spmm_flat_launches" (1 = partial tiles

@@ -20,6 +20,8 @@ SIGNATURES = {
     "vs_wmma_spmm_f16_f32out_ws": ([_int] * 5 + [_vp] * 7 + [_ll, _vp], _int),
     "vs_wmma_spmm_noalloc_scratch_bytes": ([], _ll),
     "vs_wmma_spmm_f16_noalloc": ([_int] * 5 + [_vp] * 6 + [_vp], _int),
+    "vs_wmma_spmm_slab_workspace_bytes": ([_int] * 4, _ll),
+    "vs_wmma_spmm_f16_slab": ([_int] * 4 + [_vp] * 7 + [_ll, _vp], _int),
     "vs_cuda_spmm_f16": ([_int] * 4 + [_vp] * 7, _int),
     "vs_cuda_spmm_f16_f32out": ([_int] * 4 + [_vp] * 7, _int),
     "vs_wmma_sddmm_f16": ([_int] * 4 + [_vp] * 6 + [_int, _vp, _int], _int),

@@ -10,7 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_HERE, "libvsparse.so")
 OBJ_DIR = os.path.join(_HERE, "build")
-SOURCES = ["vsparse_api.hip", "spmm_mfma.hip", "spmm_mfma_flat.hip", "spmm_mfma_dma.hip", "spmm_valu.hip", "sddmm_mfma.hip", "sddmm_valu.hip",
+SOURCES = ["vsparse_api.hip", "spmm_mfma.hip", "spmm_mfma_flat.hip", "spmm_mfma_dma.hip", "spmm_mfma_slab.hip", "spmm_valu.hip", "sddmm_mfma.hip", "sddmm_valu.hip",
            "sparse_softmax.hip", "sparse_attention.hip",
            "sparse_attention_union.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

@@ -41,6 +41,7 @@ struct PackedVector {
     typedef half_t vec_t __attribute__((ext_vector_type(V)));
     vec_t d;
     __device__ __forceinline__ void load(const half_t *p) { d = *reinterpret_cast<const vec_t *>(p); }
+    __device__ __forceinline__ void store(half_t *p) const { *reinterpret_cast<vec_t *>(p) = d; }
     __device__ __forceinline__ void clear() { d = vec_t(0); }
     __device__ __forceinline__ half_t at(int v) const { return d[v]; }
     __device__ __forceinline__ float first() const { return (float)d[0]; }
@@ -49,6 +50,7 @@ template <>
 struct PackedVector<1> {
     half_t d;
     __device__ __forceinline__ void load(const half_t *p) { d = p[0]; }
+    __device__ __forceinline__ void store(half_t *p) const { p[0] = d; }
     __device__ __forceinline__ void clear() { d = (half_t)0.f; }
     __device__ __forceinline__ half_t at(int) const { return d; }
     __device__ __forceinline__ float first() const { return (float)d; }

@@ -217,6 +217,7 @@ struct Options {
     int spmm_blocks_per_wave = 0;  // ... blocks of a row a wave takes before another of the kept waves joins in (power of two), 0 = automatic
     int spmm_guard_waves = 0;   // MFMA SpMM, row lengths unknown, full grid: waves per workgroup kept for rows longer than expected
     int spmm_gather = 0;        // 1 = gathered rows through registers, 2 = through LDS-DMA loads, 0 = automatic
+    int spmm_slab_parts = 0;    // SpMM with the dense operand staged in LDS (vs_wmma_spmm_f16_slab): parts of the contraction a block of rows is spread over (1..64), 0 = automatic
     int spmm_flat_piece = 0;    // split-row SpMM: nonzero vectors per wave (rounded up to 32), 0 = automatic
     int spmm_flat_launches = 0; // split-row SpMM: 1 = parts added inside the launch, 2 = by a second launch, 0 = automatic
     int spmm_flat_waves = 0;    // split-row SpMM: waves per workgroup, 0 = automatic
@@ -342,6 +343,14 @@ int launch_spmm_mfma_row_parts(int vec_length, int k, int n, int n_slots, const 
                                const half_t *rhs, half_t *out, void *workspace, long long workspace_bytes,
                                hipStream_t stream, const Batch &batch);
 long long spmm_row_parts_workspace_bytes(int batch, int vec_length, int k, int n_split, int parts_max);
+
+// SpMM with the dense operand staged in LDS once per block of sixteen vector rows (csrc/spmm_mfma_slab.hip):
+// k % 8 == 0, n * k < 2^31, fp16 output; `workspace` holds the fp32 tiles of the parts.
+int launch_spmm_mfma_slab(int m_vec, int vec_length, int k, int n, int ksplit, const int *row_indices,
+                          const int *row_offsets, const int *column_indices, const half_t *values, const half_t *rhs,
+                          half_t *out, void *workspace, long long workspace_bytes, hipStream_t stream);
+long long spmm_slab_workspace_bytes(int m_vec, int vec_length, int k, int ksplit);
+int choose_spmm_slab_parts(int m_vec, int k, int n);
 
 // Split-row SpMM (csrc/spmm_mfma_flat.hip): `workspace` holds the fp32 partial tiles of rows longer than a piece.
 template <typename OutT>

@@ -199,6 +199,26 @@ int vs_wmma_spmm_f16_f32out_ws(int m_vec, int vec_length, int k, int n, int nonz
                                             static_cast<hipStream_t>(stream));
 }
 
+long long vs_wmma_spmm_slab_workspace_bytes(int m_vec, int vec_length, int k, int n)
+{
+    if (m_vec < 0 || k < 0 || n < 0 || !vec_ok(vec_length)) return 0;
+    return vs::spmm_slab_workspace_bytes(m_vec, vec_length, k, vs::choose_spmm_slab_parts(m_vec, k, n));
+}
+
+int vs_wmma_spmm_f16_slab(int m_vec, int vec_length, int k, int n, const int *row_indices, const int *row_offsets,
+                          const int *column_indices, const void *values, const void *rhs_matrix, void *output_matrix,
+                          void *workspace, long long workspace_bytes, void *stream)
+{
+    int st = check_spmm(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices, values, rhs_matrix,
+                        output_matrix, sizeof(half_t));
+    if (st != VS_SUCCESS) return st;
+    if (workspace_bytes < 0 || (workspace_bytes > 0 && (!workspace || !aligned(workspace, 16)))) return VS_ERROR_INVALID_VALUE;
+    return vs::launch_spmm_mfma_slab(m_vec, vec_length, k, n, vs::choose_spmm_slab_parts(m_vec, k, n), row_indices,
+                                     row_offsets, column_indices, static_cast<const half_t *>(values),
+                                     static_cast<const half_t *>(rhs_matrix), static_cast<half_t *>(output_matrix),
+                                     workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
 int vs_cuda_spmm_f16(int m_vec, int vec_length, int k, int n, const int *row_indices, const int *row_offsets,
                      const int *column_indices, const void *values, const void *rhs_matrix, void *output_matrix,
                      void *stream)
@@ -733,6 +753,9 @@ static int set_option_field(vs::Options &o, const char *name, int value)
     } else if (std::strcmp(name, "spmm_gather") == 0) {
         if (value > 2) return VS_ERROR_INVALID_VALUE;
         o.spmm_gather = value;
+    } else if (std::strcmp(name, "spmm_slab_parts") == 0) {
+        if (value > 64) return VS_ERROR_INVALID_VALUE;
+        o.spmm_slab_parts = value;
     } else if (std::strcmp(name, "spmm_flat_piece") == 0) {
         o.spmm_flat_piece = value;
     } else if (std::strcmp(name, "spmm_flat_launches") == 0) {

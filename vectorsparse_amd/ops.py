@@ -139,6 +139,30 @@ def spmm_split_rows(m_vec, vec_length, k, n, nonzeros_vec, row_offsets, column_i
     return output_matrix
 
 
+def spmm_slab_workspace_bytes(m_vec, vec_length, k, n):
+    """Workspace `spmm_slab` needs for this shape under the current "spmm_slab_parts" option (0: none)."""
+    return int(_lib.lib().vs_wmma_spmm_slab_workspace_bytes(m_vec, vec_length, k, n))
+
+
+def spmm_slab(m_vec, vec_length, k, n, row_indices, row_offsets, column_indices, values, rhs_matrix, output_matrix,
+              workspace=None, stream=None):
+    """wmmaSpmm on the schedule that stages the dense operand in LDS once per block of eight vector rows
+    (`vs_wmma_spmm_f16_slab`; k % 8 == 0, fp16 output).  workspace: a device tensor of at least
+    `spmm_slab_workspace_bytes(...)` bytes, or None to allocate one for the call.  Returns output_matrix."""
+    need = spmm_slab_workspace_bytes(m_vec, vec_length, k, n)
+    if workspace is None and need > 0:
+        workspace = torch.empty(need, dtype=torch.uint8, device=output_matrix.device)
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    st = _lib.lib().vs_wmma_spmm_f16_slab(
+        m_vec, vec_length, k, n, _expect(row_indices, torch.int32, "row_indices"),
+        _expect(row_offsets, torch.int32, "row_offsets"), _expect(column_indices, torch.int32, "column_indices"),
+        _expect(values, torch.float16, "values"), _expect(rhs_matrix, torch.float16, "rhs_matrix"),
+        _expect(output_matrix, torch.float16, "output_matrix"), _ptr(workspace), ws_bytes, _stream(stream))
+    if st:
+        _lib.check(st, "vs_wmma_spmm_f16_slab")
+    return output_matrix
+
+
 class sddmm:
     """Namespace ``sddmm`` of the reference: D = (A[m x k] * B[n x k]^T) sampled on a column-vector CSR mask."""
 
