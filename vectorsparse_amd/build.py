@@ -16,6 +16,10 @@ SOURCES = ["vsparse_api.hip", "spmm_mfma.hip", "spmm_mfma_flat.hip", "spmm_mfma_
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared",
+    # only the C ABI of include/vsparse.h leaves the library (csrc/vsparse_api.hip exports it explicitly)
+    "-fvisibility=hidden",
+    # the device code objects are stored compressed (the HIP runtime unpacks them when the library is loaded)
+    "--offload-compress",
     # packed-fp32 VALU forms are kept out of the generated code on purpose
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     # the first sixteen dwords of kernel arguments arrive in registers with the wave instead of through a load
@@ -57,7 +61,8 @@ def build(verbose=False, jobs=None, incremental=False):
     jobs = jobs or max(1, min(len(cmds), os.cpu_count() or 1, 16))
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         list(pool.map(lambda c: _run(c, verbose), cmds))
-    _run([HIPCC, "--offload-arch=gfx950", "-fPIC", "-shared", "-o", LIB_PATH] + objects, verbose)
+    _run([HIPCC, "--offload-arch=gfx950", "-fPIC", "-shared", "-Wl,--version-script=" + os.path.join(CSRC, "exports.map"),
+          "-o", LIB_PATH] + objects, verbose)
     return LIB_PATH
 
 

@@ -94,6 +94,8 @@ int check_sddmm(int m_vec, int k, int n, int nonzeros_vec, const int *row_indice
 
 }  // namespace
 
+// the library is compiled with hidden visibility: what follows is its whole exported surface
+#pragma GCC visibility push(default)
 extern "C" {
 
 int vs_version(void) { return 100; }
@@ -806,3 +808,4 @@ int vs_set_thread_option(const char *name, int value)
 void vs_clear_thread_options(void) { vs::t_options_active = false; }
 
 }  // extern "C"
+#pragma GCC visibility pop
