@@ -367,11 +367,15 @@ def main():
 
     # ---- the dispatch floor of the headline launch: a kernel that does nothing on the same grid.  No kernel of
     # that shape finishes sooner, so algorithmic bytes / this time is the ceiling of `roofline.frac` on config 2.
-    floor_lib = _lib.lib()
-
+    import ctypes
+    probe_path = os.path.join(ROOT, "vectorsparse_amd", "libvsprobe.so")
+    if not os.path.exists(probe_path):
+        raise SystemExit("%s not found: build it with `python -m vectorsparse_amd.build`" % probe_path)
+    floor_lib = ctypes.CDLL(probe_path)
+    floor_lib.vsprobe_empty_launch.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
 
     def probe(threads):  # on whatever stream is current at the call (the capture stream inside time_graph)
-        return lambda: floor_lib.vs_launch_floor_probe(256, threads, torch.cuda.current_stream().cuda_stream)
+        return lambda: floor_lib.vsprobe_empty_launch(256, threads, torch.cuda.current_stream().cuda_stream)
 
     _, floor_ms = time_graph(torch, probe(1024), dev_steps, args.warmup)
     _, floor_small_ms = time_graph(torch, probe(64), dev_steps, args.warmup)

@@ -79,7 +79,7 @@ int vs_wmma_spmm_f16_f32out(int m_vec, int vec_length, int k, int n,
  * The same operator (spmm::wmmaSpmm, include/wmma_spmm.cuh:15-21 and :7-13) on a schedule that balances
  * skewed row lengths across the whole chip, which the reference's SortedRowSwizzle
  * (include/bm_test_utils.h:200-215) only approximates by reordering whole rows: the nonzero range is cut
- * into equal runs, one wave per (run, column tile) and sixteen runs per workgroup; a row that crosses run
+ * into equal runs, one wave per (run, column tile) and eight runs per workgroup; a row that crosses run
  * boundaries is computed in segments whose fp32 partial tiles are added in ascending order - inside a
  * workgroup through LDS, across workgroups through `workspace` by whichever wave brings a row's last part (one
  * launch, nobody waits, no atomics on the output; deterministic; the result does not depend on row_indices, which may be null and is ignored).
@@ -92,7 +92,7 @@ int vs_wmma_spmm_f16_f32out(int m_vec, int vec_length, int k, int n,
  * overlap.  (Option "spmm_flat_launches" = 2 adds the parts in a second launch instead and uses no counters.)  vs_wmma_spmm_workspace_bytes() returns the
  * size that lets the library pick its preferred run length (0 when one workgroup takes everything); a smaller
  * workspace - even none - is accepted and makes the runs longer (fewer waves, same results up to the
- * order of the fp32 summation).  Other requirements as vs_wmma_spmm_f16.  Faster than vs_wmma_spmm_f16 when
+ * order of the fp32 summation).  Requires k % 4 == 0 (else 801); alignment as vs_wmma_spmm_f16.  Faster than vs_wmma_spmm_f16 when
  * a few rows hold a large share of the nonzeros; slower on uniform rows.
  */
 long long vs_wmma_spmm_workspace_bytes(int m_vec, int vec_length, int k, int n, int nonzeros_vec);
@@ -118,9 +118,16 @@ int vs_wmma_spmm_f16_f32out_ws(int m_vec, int vec_length, int k, int n, int nonz
  * Every call on a GPU shares that GPU's array: calls that may overlap on one GPU (different streams, different
  * threads) race on it and must be serialised by the caller.  Nothing in the array has to be cleared between
  * calls, whatever their shapes: it starts zeroed, the arrival counters have a fixed area of their own that every
- * call leaves at zero, and every partial tile that is read was written by the same call.
+ * call leaves at zero (also a call whose nonzeros_vec is smaller than row_offsets[m_vec]: parts past nonzeros_vec are
+ * neither computed nor counted), and every partial tile that is read was written by the same call.  Only calls that
+ * overlapped on one GPU, or a launch that was aborted, can leave a counter behind; vs_wmma_spmm_noalloc_reset puts
+ * the counters back to zero (a small kernel on `stream`, no allocation; not needed otherwise).
+ * Under HIP graph capture: the address of the current GPU's array is looked up once per device, on the first call of
+ * vs_wmma_spmm_noalloc_scratch_bytes() or of the entry point on that device - make that call before the capture
+ * begins (the lookup is a runtime call, not a stream operation).
  */
 long long vs_wmma_spmm_noalloc_scratch_bytes(void);
+int vs_wmma_spmm_noalloc_reset(void *stream);
 int vs_wmma_spmm_f16_noalloc(int m_vec, int vec_length, int k, int n, int nonzeros_vec,
                              const int *row_indices, const int *row_offsets,
                              const int *column_indices, const void *values,
@@ -465,14 +472,6 @@ void vs_identity_row_swizzle(int rows, int *row_indices);
 void vs_sorted_row_swizzle(int rows, const int *row_offsets, int *row_indices);
 
 /*
- * Measurement aid: launches a kernel that does nothing on a grid of `blocks` workgroups of
- * `threads_per_block` threads (1..1024), asynchronously on `stream`.  Timing it prices the dispatch
- * floor of a launch shape, below which no kernel of that shape can finish.  No counterpart in the
- * reference.
- */
-int vs_launch_floor_probe(int blocks, int threads_per_block, void *stream);
-
-/*
  * Reports the launch shape that vs_wmma_spmm_f16 (hints negative) or the batched SpMM entry points (hints as
  * passed to them) would choose for a problem, under the calling thread's options; touches no device.  shape[0]
  * dense columns per lane (4 or 8: tiles of 64 or 128 columns), [1] 32-vector steps of gathered rows a wave keeps
@@ -494,7 +493,9 @@ int vs_wmma_spmm_launch_shape(int batch, int m_vec, int vec_length, int k, int n
  * from the process-wide values at that moment) until vs_clear_thread_options().
  * Launch shapes are decided on the host inside each call, so a thread can also
  * change its options between two calls on different streams - every call sees
- * exactly what its thread last set, whatever other threads do.  Names: "spmm_waves" (waves per workgroup, 0 = automatic),
+ * exactly what its thread last set, whatever other threads do.  Two variants that measured slower on every
+ * shape - four 32-vector steps in flight ("spmm_steps" = 4) and the LDS-DMA gather ("spmm_gather" = 2) - are
+ * compiled only when the library is built with VS_RETIRED_VARIANTS=1; otherwise those two values return 801.  Names: "spmm_waves" (waves per workgroup, 0 = automatic),
  * "spmm_cols_per_lane" (4, 8, 0 = automatic), "spmm_steps" (32-vector steps of gathered
  * rows a wave of the MFMA SpMM keeps in flight: 1, 2, 4, 0 = automatic), "spmm_guard_waves"
  * (MFMA SpMM through the entry points that do not know the row lengths, on grids that fill the

@@ -141,8 +141,12 @@ def test_options():
             _lib.set_option(name, bad)
     for name in ("spmm_flat_piece", "sddmm_slots", "attention_chunk"):
         _lib.set_option(name, 0)
-    with _lib.thread_options(spmm_steps=4, spmm_guard_waves=2):
+    with _lib.thread_options(spmm_steps=2, spmm_guard_waves=2):
         pass
+    # the two retired variants: accepted by a library built with them, 801 (not 1) otherwise
+    for name, value in (("spmm_steps", 4), ("spmm_gather", 2)):
+        assert _lib.lib().vs_set_option(name.encode(), value) in (0, 801)
+        _lib.set_option(name, 0)
 
 
 def test_header_is_plain_c_and_cxx(tmp_path):

@@ -6,7 +6,7 @@ import torch
 from oracle import c_oracle as co
 from vectorsparse_amd import ops
 from vectorsparse_amd import colvec_csr as cv
-from util import assert_parity
+from util import assert_parity, retired_variants_built
 
 pytestmark = pytest.mark.gpu
 
@@ -64,9 +64,12 @@ def test_spmm_random_launch_shapes(gpu, seed):
     ref = co.spmm_host_ref_f32(pat.m_vec, V, N, pat.n, pat.row_offsets, pat.column_indices, pat.values, B)
     Bd = torch.from_numpy(B).cuda()
     prob = ops.DeviceProblem(pat, sort=bool(seed % 2))
+    # (four steps in flight exist only in a library built with VS_RETIRED_VARIANTS=1; the draw is made either way,
+    # so that the other options of a seed do not depend on the build)
+    step_choice = (lambda x: x) if retired_variants_built() else (lambda x: 2 if x == 4 else x)
     for trial in range(4):
         opts = dict(spmm_waves=int(rng.choice([0, 0, 1, 2, 3, 4, 8, 16])), spmm_cols_per_lane=int(rng.choice([0, 4, 8])),
-                    spmm_steps=int(rng.choice([0, 1, 2, 2, 4])), spmm_pipe=int(rng.choice([0, 1, 2, 2])),
+                    spmm_steps=step_choice(int(rng.choice([0, 1, 2, 2, 4]))), spmm_pipe=int(rng.choice([0, 1, 2, 2])),
                     spmm_guard_waves=int(rng.choice([0, 1, 2, 4, 8])),
                     spmm_blocks_per_wave=int(rng.choice([0, 1, 2, 8, 64])), spmm_teams=int(rng.choice([0, 1, 2])))
         hint = bool(rng.integers(0, 2))

@@ -11,7 +11,7 @@ import torch
 from oracle import c_oracle as co
 from vectorsparse_amd import _lib, ops
 from vectorsparse_amd import colvec_csr as cv
-from util import assert_parity
+from util import assert_parity, retired_variants_built
 
 pytestmark = pytest.mark.gpu
 
@@ -100,6 +100,8 @@ def test_steps_in_flight_variants_keep_parity(gpu, V, steps, cpl):
     """The MFMA kernel with one, two or four 32-vector steps of gathered rows in flight per wave: rows that end
     inside a block (1, 33, 65, 127, 129 vectors), empty rows, rows of many blocks, and every wave count - including
     more waves than a row has blocks."""
+    if steps == 4 and not retired_variants_built():
+        pytest.skip("four steps in flight are compiled only with VS_RETIRED_VARIANTS=1")
     lengths = np.array([0, 1, 33, 64, 65, 0, 127, 128, 129, 300, 2, 0, 700, 7, 96, 0], dtype=np.int64)
     n = 768
     rng = np.random.default_rng(50 + V)
@@ -367,6 +369,8 @@ def test_lds_dma_gather_variant_keeps_parity(gpu, V):
     """The variant of the MFMA kernel whose gathered rows go global -> LDS directly and reach the MFMA through
     transposing LDS reads (option spmm_gather = 2): same contract, every wave count, ragged rows, dense-width
     edges, and the same bits for any row swizzle."""
+    if not retired_variants_built():
+        pytest.skip("the LDS-DMA gather is compiled only with VS_RETIRED_VARIANTS=1")
     lengths = np.array([0, 1, 15, 16, 17, 0, 31, 33, 64, 65, 300, 2, 0, 128, 7, 0], dtype=np.int64)
     rng = np.random.default_rng(5)
     ro, ci = cv._pattern_from_lengths(rng, len(lengths), 320, lengths)

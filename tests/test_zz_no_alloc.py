@@ -82,3 +82,65 @@ def test_sizes_beyond_the_scratch_are_rejected(gpu):
     torch.cuda.synchronize()
     ref = co.spmm_host_ref_f32(16, 8, 4096, 256, pat.row_offsets, pat.column_indices, pat.values, B)
     assert_parity(out.cpu().numpy(), ref, "no-alloc entry point at its size limit")
+
+
+def test_captured_into_a_graph_and_replayed(gpu):
+    """The call under HIP graph capture (the callers it exists for): the symbol lookup is made before the capture
+    by asking for the scratch size; every replay - with eager calls of the same entry point on other shapes and
+    synchronisations in between - gives the bits of the eager call."""
+    L = _lib.lib()
+    assert L.vs_wmma_spmm_noalloc_scratch_bytes() == 16 << 20   # resolves this device's array outside the capture
+    pat, B = _problem(256, 2048, 8, 128, 11, 2048)
+    ro, ci, vals, Bd = _device(pat, B)
+    other, oB = _problem(64, 1024, 4, 64, 12, 1024)
+    oro, oci, ovals, oBd = _device(other, oB)
+    oout = torch.empty((other.m, 64), dtype=torch.float16, device="cuda")
+    eager = torch.empty((pat.m, 128), dtype=torch.float16, device="cuda")
+    st = L.vs_wmma_spmm_f16_noalloc(256, 8, 128, 2048, pat.nnz_vec, 0, ro.data_ptr(), ci.data_ptr(), vals.data_ptr(),
+                                    Bd.data_ptr(), eager.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    assert st == 0
+    torch.cuda.synchronize()
+    want = eager.cpu().numpy().view(np.uint16)
+    out = torch.empty_like(eager)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        st = L.vs_wmma_spmm_f16_noalloc(256, 8, 128, 2048, pat.nnz_vec, 0, ro.data_ptr(), ci.data_ptr(), vals.data_ptr(),
+                                        Bd.data_ptr(), out.data_ptr(), side.cuda_stream)
+    assert st == 0
+    for replay in range(6):
+        out.fill_(-3.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy().view(np.uint16), want), "replay %d differs from the eager call" % replay
+        st = L.vs_wmma_spmm_f16_noalloc(64, 4, 64, 1024, other.nnz_vec, 0, oro.data_ptr(), oci.data_ptr(),
+                                        ovals.data_ptr(), oBd.data_ptr(), oout.data_ptr(),
+                                        torch.cuda.current_stream().cuda_stream)
+        assert st == 0
+        torch.cuda.synchronize()
+    ref = co.spmm_host_ref_f32(256, 8, 128, 2048, pat.row_offsets, pat.column_indices, pat.values, B)
+    assert_parity(out.cpu().numpy(), ref, "no-alloc entry point, replayed")
+
+
+def test_counters_recover_from_an_inconsistent_call_and_reset(gpu):
+    """A call whose nonzeros_vec is smaller than row_offsets[m_vec] computes (and counts) only the parts that exist,
+    so the arrival counters are back at zero for the next call; vs_wmma_spmm_noalloc_reset clears them in any case."""
+    L = _lib.lib()
+    pat, B = _problem(256, 4096, 8, 256, 21, 4096)
+    ro, ci, vals, Bd = _device(pat, B)
+    out = torch.empty((pat.m, 256), dtype=torch.float16, device="cuda")
+    args = (ro.data_ptr(), ci.data_ptr(), vals.data_ptr(), Bd.data_ptr(), out.data_ptr(), 0)
+    ref = co.spmm_host_ref_f32(256, 8, 256, 4096, pat.row_offsets, pat.column_indices, pat.values, B)
+    # cut inside the long row that spans many pieces (results of this call are undefined; only its side effects count)
+    cut = int(pat.row_offsets[256 // 3] + 1500)
+    assert cut < pat.nnz_vec
+    assert L.vs_wmma_spmm_f16_noalloc(256, 8, 256, 4096, cut, 0, *args) == 0
+    torch.cuda.synchronize()
+    assert L.vs_wmma_spmm_f16_noalloc(256, 8, 256, 4096, pat.nnz_vec, 0, *args) == 0
+    torch.cuda.synchronize()
+    assert_parity(out.cpu().numpy(), ref, "the call after an inconsistent one")
+    assert L.vs_wmma_spmm_noalloc_reset(0) == 0
+    out.fill_(0)
+    assert L.vs_wmma_spmm_f16_noalloc(256, 8, 256, 4096, pat.nnz_vec, 0, *args) == 0
+    torch.cuda.synchronize()
+    assert_parity(out.cpu().numpy(), ref, "the call after a reset")

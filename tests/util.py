@@ -29,3 +29,13 @@ def assert_parity(got, ref, what=""):
     err = max_rel_err(got, ref)
     assert err <= REL_TOL, "%s: max relative error %.3e > %.0e" % (what, err, REL_TOL)
     return err
+
+
+def retired_variants_built():
+    """True when the library was built with VS_RETIRED_VARIANTS=1 (the LDS-DMA gather and four steps in flight of the
+    MFMA SpMM, which the default build leaves out): the option values that select them are then accepted."""
+    from vectorsparse_amd import _lib
+    L = _lib.lib()
+    ok = L.vs_set_option(b"spmm_steps", 4) == 0
+    L.vs_set_option(b"spmm_steps", 0)
+    return ok

@@ -19,6 +19,7 @@ SIGNATURES = {
     "vs_wmma_spmm_f16_ws": ([_int] * 5 + [_vp] * 7 + [_ll, _vp], _int),
     "vs_wmma_spmm_f16_f32out_ws": ([_int] * 5 + [_vp] * 7 + [_ll, _vp], _int),
     "vs_wmma_spmm_noalloc_scratch_bytes": ([], _ll),
+    "vs_wmma_spmm_noalloc_reset": ([_vp], _int),
     "vs_wmma_spmm_f16_noalloc": ([_int] * 5 + [_vp] * 6 + [_vp], _int),
     "vs_wmma_spmm_slab_workspace_bytes": ([_int] * 4, _ll),
     "vs_wmma_spmm_f16_slab": ([_int] * 4 + [_vp] * 7 + [_ll, _vp], _int),
@@ -53,7 +54,6 @@ SIGNATURES = {
     "vs_wmma_spmm_f16_row_parts": ([_int] * 5 + [_vp] + [_int] * 4 + [_vp] + [_vp, _ll, _vp, _ll, _vp, _ll] + [_vp, _ll, _vp],
                                    _int),
     "vs_wmma_sddmm_f16_row_parts": ([_int] * 4 + [_vp, _int, _vp] + [_vp, _ll, _vp, _ll, _vp, _ll] + [_int, _vp], _int),
-    "vs_launch_floor_probe": ([_int, _int, _vp], _int),
     "vs_set_option": ([ctypes.c_char_p, _int], _int),
     "vs_set_thread_option": ([ctypes.c_char_p, _int], _int),
     "vs_clear_thread_options": ([], None),

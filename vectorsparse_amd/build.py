@@ -10,9 +10,16 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_HERE, "libvsparse.so")
 OBJ_DIR = os.path.join(_HERE, "build")
-SOURCES = ["vsparse_api.hip", "spmm_mfma.hip", "spmm_mfma_flat.hip", "spmm_mfma_dma.hip", "spmm_mfma_slab.hip", "spmm_valu.hip", "sddmm_mfma.hip", "sddmm_valu.hip",
+SOURCES = ["vsparse_api.hip", "spmm_mfma.hip", "spmm_mfma_flat.hip", "spmm_mfma_slab.hip", "spmm_valu.hip", "sddmm_mfma.hip", "sddmm_valu.hip",
            "sparse_softmax.hip", "sparse_attention.hip",
            "sparse_attention_union.hip"]
+# VS_RETIRED_VARIANTS=1 in the environment also compiles the two SpMM variants that measured slower on every shape
+# and are therefore not part of the default library: the LDS-DMA gather (spmm_mfma_dma.hip, option spmm_gather = 2)
+# and four 32-vector steps in flight (option spmm_steps = 4)
+RETIRED = os.environ.get("VS_RETIRED_VARIANTS") == "1"
+if RETIRED:
+    SOURCES.append("spmm_mfma_dma.hip")
+PROBE_PATH = os.path.join(_HERE, "libvsprobe.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared",
@@ -54,7 +61,7 @@ def build(verbose=False, jobs=None, incremental=False):
     incremental: recompile only the sources that are newer than their objects (or whose shared headers are)."""
     from concurrent.futures import ThreadPoolExecutor
     os.makedirs(OBJ_DIR, exist_ok=True)
-    compile_flags = [f for f in FLAGS if f != "-shared"]
+    compile_flags = [f for f in FLAGS if f != "-shared"] + (["-DVS_RETIRED_VARIANTS"] if RETIRED else [])
     objects = [os.path.join(OBJ_DIR, s.replace(".hip", ".o")) for s in SOURCES]
     cmds = [[HIPCC] + compile_flags + ["-c", os.path.join(CSRC, s), "-o", o] for s, o in zip(SOURCES, objects)
             if not incremental or _stale(os.path.join(CSRC, s), o)]
@@ -64,6 +71,14 @@ def build(verbose=False, jobs=None, incremental=False):
     _run([HIPCC, "--offload-arch=gfx950", "-fPIC", "-shared", "-Wl,--version-script=" + os.path.join(CSRC, "exports.map"),
           "-o", LIB_PATH] + objects, verbose)
     return LIB_PATH
+
+
+def build_probe(verbose=False):
+    """Compile csrc/launch_probe.hip (an empty kernel on a grid of the caller's choice) to libvsprobe.so, the
+    measurement aid bench.py prices the dispatch floor with; not part of libvsparse.so."""
+    _run([HIPCC, "-O2", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
+          os.path.join(CSRC, "launch_probe.hip"), "-o", PROBE_PATH], verbose)
+    return PROBE_PATH
 
 
 def build_cxx_caller(verbose=False):
@@ -84,5 +99,6 @@ def build_cxx_caller(verbose=False):
 
 if __name__ == "__main__":
     print(build(verbose=True, incremental="--incremental" in sys.argv))
+    print(build_probe(verbose=True))
     print(build_cxx_caller(verbose=True))
     sys.exit(0)

@@ -568,7 +568,9 @@ static int launch_one(const SpmmShape &shape, int m_vec, int k, int n, const int
     if constexpr (SOFTMAX) {
         if (shape.steps_in_flight >= 2) return VS_SPMM_VARIANT(true, OutT, 2) per_wave, -1);
     } else {
+#ifdef VS_RETIRED_VARIANTS
         if (shape.steps_in_flight == 4) return VS_SPMM_VARIANT(true, OutT, 4) per_wave, -1);
+#endif
         if (shape.steps_in_flight >= 2) {
             // (only the two-step variants have the team mapping and the pipelined walk)
             if (shape.team_slots >= 0)
@@ -604,7 +606,11 @@ SpmmShape choose_spmm_shape(bool softmax, int m_vec, int vec_length, int k, int 
     constexpr int kTargetBlocks = 256;   // one workgroup per CU at least
     constexpr int kTargetWaves = 4096;
     int cpl = options().spmm_cols_per_lane;
+#ifdef VS_RETIRED_VARIANTS
     const bool use_dma = !softmax && options().spmm_gather == 2 && k % 8 == 0;
+#else
+    const bool use_dma = false;  // (the LDS-DMA gather and four steps in flight are compiled only with VS_RETIRED_VARIANTS)
+#endif
     if (use_dma) cpl = 8;
     const bool hinted = batch.nonzeros_vec >= 0;
     const int mean_steps = hinted ? ceil_div(ceil_div(batch.nonzeros_vec, m_vec), kStep) : ceil_div(n, 4 * kStep);
@@ -633,6 +639,9 @@ SpmmShape choose_spmm_shape(bool softmax, int m_vec, int vec_length, int k, int 
     const int row_steps = longest_steps > mean_steps ? longest_steps : mean_steps;
     const bool blocks_exist = !ragged && !use_dma && (long long)n * k < (1LL << 31);
     int in_flight = options().spmm_steps;
+#ifndef VS_RETIRED_VARIANTS
+    if (in_flight == 4) in_flight = 0;
+#endif
     if (in_flight != 1 && in_flight != 2 && in_flight != 4) {
         in_flight = row_steps >= 2 ? 2 : 1;
         // Many heads of a large mask with vectors of one or two rows (16384 workgroups and more, every one a single
@@ -643,9 +652,11 @@ SpmmShape choose_spmm_shape(bool softmax, int m_vec, int vec_length, int k, int 
         if (hinted && vec_length <= 2 && blocks >= 16384 && mean_steps <= 16) in_flight = 1;
         // (rows of unequal length end in half-empty blocks of 128: on log-normal and Pareto lengths four steps in
         // flight were 10-25 % behind two)
+#ifdef VS_RETIRED_VARIANTS
         if (options().spmm_pipe == 1 && hinted && cpl == 8 && blocks >= 512 && mean_steps >= 8 &&
             2 * longest_steps <= 3 * mean_steps)
             in_flight = 4;  // (only without the pipelined walk, which is 5-15 % ahead of it on the same shapes)
+#endif
     }
     if (!blocks_exist) in_flight = 1;
     // The softmax-fused kernel has the two-step blocks only, and gains from them on rows of more than two blocks
@@ -826,9 +837,11 @@ static int launch_any(int m_vec, int vec_length, int k, int n, const int *row_in
             default: return hipErrorInvalidValue;
             }
         }
+#ifdef VS_RETIRED_VARIANTS
         if (shape.dma)
             return launch_spmm_mfma_dma<OutT>(m_vec, vec_length, k, n, waves, row_indices, row_offsets, column_indices,
                                               values, rhs, out, stream, batch);
+#endif
     }
     if (shape.cols_per_lane == 8)
         return launch_v<8, SOFTMAX, OutT>(shape, vec_length, m_vec, k, n, row_indices, row_offsets, column_indices, values, rhs, out, stream, batch, scale);

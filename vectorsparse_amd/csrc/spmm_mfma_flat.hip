@@ -387,7 +387,9 @@ spmm_mfma_flat_kernel(int m_vec, int n_cols, int n_tiles, int nonzeros_vec, int 
             pending = true;
             p_row = t_row;
             p_first = c;
-            p_last = (int)((t_row_end - 1) / piece);
+            // (a row that row_offsets lets end past nonzeros_vec - an inconsistent call - has no parts beyond the last
+            // launched piece: counting only those that exist leaves the counter at zero whatever the caller passed)
+            p_last = (int)(((t_row_end < nonzeros_vec ? t_row_end : (long long)nonzeros_vec) - 1) / piece);
         } else {
             tile_store<V, CPL>(ws + ((size_t)2 * c + 1) * ws_tile, ws_pitch, cs, g, acc, t_pos);
         }
@@ -409,7 +411,7 @@ spmm_mfma_flat_kernel(int m_vec, int n_cols, int n_tiles, int nonzeros_vec, int 
                     pending = true;
                     p_row = f_row;
                     p_first = (int)(f_row_beg / piece);
-                    p_last = (int)((f_row_end - 1) / piece);
+                    p_last = (int)(((f_row_end < nonzeros_vec ? f_row_end : (long long)nonzeros_vec) - 1) / piece);
                 } else {
                     tile_store<V, CPL>(ws + (size_t)2 * c * ws_tile, ws_pitch, cs, g, sum);
                 }
@@ -657,8 +659,6 @@ constexpr long long kScratchBytes = 16LL << 20;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 static std::atomic<void *> scratch_of_device[64];
 
-long long spmm_flat_scratch_bytes() { return kScratchBytes; }
-
 // The current device's copy of `scratch` (resolved on the first call on that device, with it current).
 static int scratch_address(float **address)
 {
@@ -675,6 +675,24 @@ static int scratch_address(float **address)
     }
     *address = static_cast<float *>(p);
     return hipSuccess;
+}
+
+// Also resolves the current device's copy of the array, so that a caller who asks for the size before capturing a HIP
+// graph has the symbol lookup outside the capture.
+long long spmm_flat_scratch_bytes()
+{
+    float *unused = nullptr;
+    (void)scratch_address(&unused);
+    return kScratchBytes;
+}
+
+// Zeros for the arrival counters of the static array (a kernel, not a memset node: the call may be captured).
+int spmm_flat_scratch_reset(hipStream_t stream)
+{
+    float *ws = nullptr;
+    const int st = scratch_address(&ws);
+    if (st != hipSuccess) return st;
+    return launch_zero_fill(ws, partial_tile_counter_bytes(kScratchBytes), 0, 1, stream);
 }
 
 int launch_spmm_mfma_flat_static(int m_vec, int vec_length, int k, int n, int nonzeros_vec, const int *row_offsets,

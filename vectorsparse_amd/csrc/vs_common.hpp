@@ -363,6 +363,7 @@ int launch_spmm_mfma_flat_static(int m_vec, int vec_length, int k, int n, int no
                                  const int *column_indices, const half_t *values, const half_t *rhs, half_t *out,
                                  hipStream_t stream);
 long long spmm_flat_scratch_bytes();
+int spmm_flat_scratch_reset(hipStream_t stream);
 
 int launch_spmm_softmax_mfma(int m_vec, int vec_length, int k, int n, const int *row_indices,
                              const int *row_offsets, const int *column_indices, const half_t *scores,

@@ -31,9 +31,6 @@ __global__ void zero_fill_kernel(unsigned char *out, long long bytes, long long 
     if (blockIdx.x == 0 && threadIdx.x < (bytes & 3)) dst[(words << 2) + threadIdx.x] = 0;
 }
 
-// A kernel that does nothing: what a launch of a given shape costs before any work.
-__global__ void floor_probe_kernel() {}
-
 int launch_zero_fill(void *out, long long bytes, long long stride_bytes, int batch, hipStream_t stream)
 {
     if (batch > 65535) return hipErrorNotSupported;
@@ -183,6 +180,8 @@ int vs_wmma_spmm_f16_noalloc(int m_vec, int vec_length, int k, int n, int nonzer
 }
 
 long long vs_wmma_spmm_noalloc_scratch_bytes(void) { return vs::spmm_flat_scratch_bytes(); }
+
+int vs_wmma_spmm_noalloc_reset(void *stream) { return vs::spmm_flat_scratch_reset(static_cast<hipStream_t>(stream)); }
 
 int vs_wmma_spmm_f16_f32out_ws(int m_vec, int vec_length, int k, int n, int nonzeros_vec, const int *row_indices,
                                const int *row_offsets, const int *column_indices, const void *values,
@@ -720,14 +719,6 @@ int vs_wmma_sddmm_f16_row_parts(int batch, int k, int n, int n_slots, const int 
                                          static_cast<hipStream_t>(stream), b);
 }
 
-int vs_launch_floor_probe(int blocks, int threads_per_block, void *stream)
-{
-    if (blocks < 1 || threads_per_block < 1 || threads_per_block > 1024) return VS_ERROR_INVALID_VALUE;
-    hipLaunchKernelGGL(vs::floor_probe_kernel, dim3((unsigned)blocks), dim3((unsigned)threads_per_block), 0,
-                       static_cast<hipStream_t>(stream));
-    return (int)hipGetLastError();
-}
-
 static int set_option_field(vs::Options &o, const char *name, int value)
 {
     if (!name || value < 0) return VS_ERROR_INVALID_VALUE;
@@ -751,9 +742,15 @@ static int set_option_field(vs::Options &o, const char *name, int value)
         o.spmm_guard_waves = value;
     } else if (std::strcmp(name, "spmm_steps") == 0) {
         if (value != 0 && value != 1 && value != 2 && value != 4) return VS_ERROR_INVALID_VALUE;
+#ifndef VS_RETIRED_VARIANTS
+        if (value == 4) return VS_ERROR_NOT_SUPPORTED;  // four steps in flight: compiled only with VS_RETIRED_VARIANTS
+#endif
         o.spmm_steps = value;
     } else if (std::strcmp(name, "spmm_gather") == 0) {
         if (value > 2) return VS_ERROR_INVALID_VALUE;
+#ifndef VS_RETIRED_VARIANTS
+        if (value == 2) return VS_ERROR_NOT_SUPPORTED;  // the LDS-DMA gather: compiled only with VS_RETIRED_VARIANTS
+#endif
         o.spmm_gather = value;
     } else if (std::strcmp(name, "spmm_slab_parts") == 0) {
         if (value > 64) return VS_ERROR_INVALID_VALUE;
