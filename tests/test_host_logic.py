@@ -180,6 +180,40 @@ def test_spmm_launch_shape_choice():
             shape(**args)
 
 
+def test_attention_parts_route_respects_the_workspace_limit():
+    """The automatic three-operator route on row parts is taken only while the SpMM's partial tiles stay below the
+    2 GiB the entry point accepts; beyond that the layer falls back to its other routes instead of failing."""
+    import types
+    layer = ops.SparseAttention.__new__(ops.SparseAttention)
+    few = types.SimpleNamespace(n_split=8, parts_max=9)
+    many = types.SimpleNamespace(n_split=4000, parts_max=200)
+    layer.prob = types.SimpleNamespace(vec_length=8, row_parts=lambda limit: [few])
+    assert layer._parts_route_fits(64, 16)
+    layer.prob = types.SimpleNamespace(vec_length=8, row_parts=lambda limit: [many])
+    assert ops.spmm_row_parts_workspace_bytes(8, 64, many.n_split, many.parts_max, batch=16) >= 2 ** 31
+    assert not layer._parts_route_fits(64, 16)
+    assert layer._parts_route_fits(64, 1)
+
+
+def test_thread_option_blocks_nest():
+    """Leaving an inner `thread_options` block restores the enclosing block's overrides (not the process-wide ones),
+    and a rejected value leaves them untouched."""
+    shape = ops.spmm_launch_shape
+    auto = shape(64, 8, 256, 4608)
+    with _lib.thread_options(spmm_waves=2):
+        assert shape(64, 8, 256, 4608)["waves"] == 2
+        with _lib.thread_options(spmm_cols_per_lane=8):
+            inner = shape(64, 8, 256, 4608)
+            assert (inner["waves"], inner["cols_per_lane"]) == (2, 8)
+        after = shape(64, 8, 256, 4608)
+        assert (after["waves"], after["cols_per_lane"]) == (2, auto["cols_per_lane"])
+        with pytest.raises(_lib.VSparseError):
+            with _lib.thread_options(spmm_waves=99):
+                pass
+        assert shape(64, 8, 256, 4608)["waves"] == 2
+    assert shape(64, 8, 256, 4608) == auto
+
+
 def test_sweep_benchmark_selection(tmp_path):
     """The sweep driver's file handling (job_launcher.py:25-50): list files, ranges, layer widths, buckets."""
     from vectorsparse_amd import sweep

@@ -105,16 +105,37 @@ def set_option(name, value):
 
 class thread_options:
     """Launch-shape overrides for the calls the current thread makes inside the `with` block, e.g.
-    `with thread_options(spmm_waves=4): prob.spmm(...)`.  Other threads are not affected."""
+    `with thread_options(spmm_waves=4): prob.spmm(...)`.  Other threads are not affected.  Blocks nest: leaving an
+    inner block puts back what the enclosing block had set."""
+
+    _stack = __import__("threading").local()
 
     def __init__(self, **values):
         self.values = values
 
     def __enter__(self):
-        for name, value in self.values.items():
-            check(lib().vs_set_thread_option(name.encode(), int(value)), "vs_set_thread_option(%s)" % name)
+        frames = getattr(self._stack, "frames", None)
+        if frames is None:
+            frames = self._stack.frames = []
+        frames.append(self.values)
+        try:
+            self._apply(frames)
+        except Exception:
+            frames.pop()            # a rejected value: the enclosing blocks' options stay in force
+            self._apply(frames)
+            raise
         return self
 
     def __exit__(self, *exc):
-        lib().vs_clear_thread_options()
+        frames = self._stack.frames
+        frames.pop()
+        self._apply(frames)
         return False
+
+    @staticmethod
+    def _apply(frames):
+        """The thread's options = the process-wide ones overridden by every open block, outermost first."""
+        lib().vs_clear_thread_options()
+        for values in frames:
+            for name, value in values.items():
+                check(lib().vs_set_thread_option(name.encode(), int(value)), "vs_set_thread_option(%s)" % name)

@@ -335,6 +335,13 @@ class SparseAttention:
         self._plans = {}
         self._rows = {}
 
+    def _parts_route_fits(self, d_v, heads):
+        """The SpMM of the three-operator route on row parts takes less than 2 GiB of partial tiles (the limit of
+        vs_wmma_spmm_f16_row_parts); larger masks or more heads take the other routes."""
+        parts = self.prob.row_parts(512)[0]
+        return spmm_row_parts_workspace_bytes(self.prob.vec_length, d_v, parts.n_split, parts.parts_max,
+                                              batch=heads) < 2 ** 31
+
     def union_rows(self, d_qk, d_v, heads=16):
         """Rows per workgroup for the single-launch kernel with these head widths and head count (cached)."""
         key = (int(d_qk), int(d_v), int(heads))
@@ -428,7 +435,8 @@ class SparseAttention:
         if fused is None:
             if kernel != "wmma":
                 fused = False
-            elif d % 8 == 0 and v.shape[2] % 4 == 0 and p.n * v.shape[2] < 2 ** 31 and p.row_parts(0)[0].n_split > 0:
+            elif (d % 8 == 0 and v.shape[2] % 4 == 0 and p.n * v.shape[2] < 2 ** 31 and p.row_parts(0)[0].n_split > 0
+                  and self._parts_route_fits(v.shape[2], heads)):
                 # rows far longer than the rest - global tokens: the three operators on the dispatch list of row
                 # parts (16 heads x 4096, d = 64, a +-32..128 band with 64-256 global tokens: 72-119 us against
                 # 145-160 us in one launch and 280-295 us for SDDMM + softmax-fused SpMM on whole rows)
