@@ -186,7 +186,7 @@ def test_attention_parts_route_respects_the_workspace_limit():
     import types
     layer = ops.SparseAttention.__new__(ops.SparseAttention)
     few = types.SimpleNamespace(n_split=8, parts_max=9)
-    many = types.SimpleNamespace(n_split=4000, parts_max=200)
+    many = types.SimpleNamespace(n_split=1000, parts_max=100)
     layer.prob = types.SimpleNamespace(vec_length=8, row_parts=lambda limit: [few])
     assert layer._parts_route_fits(64, 16)
     layer.prob = types.SimpleNamespace(vec_length=8, row_parts=lambda limit: [many])
