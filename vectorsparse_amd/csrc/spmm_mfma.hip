@@ -43,8 +43,7 @@ namespace vs {
 // the workgroup's fp32 tile goes to the workspace (`part_tiles`, tile of (split row, part, column tile)) and the
 // workgroup counts itself in on the row's arrival counter; the one that arrives last adds the parts in ascending
 // order - same bits whoever it is - writes the row and puts the counter back to zero.  Nobody waits for anybody.
-// The eight L2s of the chip do not see each other's lines within a launch, so the parts are written and read
-// with the device-coherence bits of the cache policy set (spmm_mfma_step.hpp).
+// How the parts reach the workgroup that adds them: PartMeeting in spmm_mfma_step.hpp.
 template <int V, int CPL, bool SOFTMAX, bool IDX32, typename OutT, bool RAGGED = false, int S = 1, bool TEAMS = false,
           bool PIPE = false, bool PARTS = false>
 __global__ void __launch_bounds__(S * CPL >= 32 ? 256 : (S * CPL >= 16 ? 512 : 1024))
@@ -256,21 +255,16 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row
 #pragma unroll
         for (int c4 = 0; c4 < CPL / 4; ++c4) {
             const float4_t t = {vals[4 * c4], vals[4 * c4 + 1], vals[4 * c4 + 2], vals[4 * c4 + 3]};
-            if (parts_meet_later)  // read by the next launch: an ordinary store
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, t), tile_area(part_tiles),
-                                                       at + 16u * c4, 0, 0);
+            if (parts_meet_later)  // read by the next launch
+                PartMeeting::store_plain(PartMeeting::area(part_tiles), at + 16u * c4, t);
             else
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, t), tile_area(part_tiles),
-                                                       at + 16u * c4, 0, kCoherent);
+                PartMeeting::store_part(PartMeeting::area(part_tiles), at + 16u * c4, t);
         }
     };
     auto arrive_and_finish = [&]() {  // one wave, all of its lanes; the workgroup's stores have completed
         int *counter = part_counters + ((size_t)part_split * n_tiles + tile) * kPartCounterStride;
-        int arrived = 0;
-        if (lane == 0) arrived = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        arrived = __builtin_amdgcn_readfirstlane(arrived);
-        if (arrived != part_count - 1) return;  // parts are still to come: whoever brings the last adds up
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // the parts are read after the count was seen
+        if (PartMeeting::arrive(counter, lane) != part_count - 1) return;  // parts are still to come: whoever brings the last adds up
+        PartMeeting::collect();
         for (int item = lane; item < V * 16; item += 64) {
             const int v = item >> 4;
             const int cs_at = item & 15;
@@ -283,8 +277,7 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row
                                     4u * (uint32_t)(v * TN + cs_at * CPL);
 #pragma unroll
                 for (int c4 = 0; c4 < CPL / 4; ++c4) {
-                    const float4_t x = __builtin_bit_cast(
-                        float4_t, __builtin_amdgcn_raw_buffer_load_b128(tile_area(part_tiles), at + 16u * c4, 0, kCoherent));
+                    const float4_t x = PartMeeting::load_part(PartMeeting::area(part_tiles), at + 16u * c4);
                     total[4 * c4] += x[0];
                     total[4 * c4 + 1] += x[1];
                     total[4 * c4 + 2] += x[2];
@@ -293,7 +286,7 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row
             }
             if (col < n_cols) store_converted<OutT, CPL>(out + ((size_t)row * V + v) * n_cols + col, total);
         }
-        if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+        PartMeeting::rearm(counter, lane);  // ready for the next launch
     };
     if constexpr (PIPE) {
         static_assert(S == 2 && IDX32 && !SOFTMAX && !RAGGED, "the pipelined walk exists for blocks of two steps");
@@ -381,9 +374,7 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row
                     }
                 }
                 if (parts_meet_later) return;
-                // the part's stores have completed (they go through to memory) before the count says so
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-                __builtin_amdgcn_s_waitcnt(0);
+                PartMeeting::publish();
                 arrive_and_finish();
                 return;
             }
@@ -455,8 +446,7 @@ spmm_mfma_kernel(int n_cols, int n_tiles, int shape, const int *__restrict__ row
     }
     if constexpr (PARTS) {
         if (part_info != 0 && !parts_meet_later) {  // (uniform over the workgroup; idle waves have left)
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-            __builtin_amdgcn_s_waitcnt(0);
+            PartMeeting::publish();
             if (V * 16 > 64) __syncthreads();  // the adding threads span two waves: both have stored
             if (wave == 0) arrive_and_finish();
         }

@@ -17,11 +17,9 @@
 //     ONE_LAUNCH (default): every wave that has written a part counts itself in on the row's arrival counter (the
 //     one of piece c0: at most one row starts in a piece and leaves it) and the wave that arrives last adds the
 //     parts, writes the output rows and puts the counter back to zero.  Nobody waits for anybody and the sum is
-//     the same whoever arrives last.  The eight L2s of the chip do not see each other's lines within a launch,
-//     so the parts are written and read with the device-coherence bits of the cache policy set (buffer accesses
-//     with sc0 sc1, tracked by the compiler; the same accesses as inline assembly lost their data registers to
-//     reuse before the stores had read them) - an L2-wide write-back and invalidate around the counter
-//     (__threadfence) cost 60 us per launch instead of 1.
+//     the same whoever arrives last.  How the parts reach the wave that adds them: PartMeeting in
+//     spmm_mfma_step.hpp (buffer accesses with the device-coherence bits set, tracked by the compiler; the same
+//     accesses as inline assembly lost their data registers to reuse before the stores had read them).
 //     Two launches: a second launch adds the parts; 1.5 to 2.5 us slower, no counters, and the route taken when
 //     the tiles would not fit 32-bit buffer offsets.
 // The zero rows of empty vector rows, which no wave's walk visits, are written by extra workgroups at the end of
@@ -88,9 +86,7 @@ __device__ __forceinline__ void tile_store_coherent(__amdgpu_buffer_rsrc_t tiles
 #pragma unroll
             for (int c4 = 0; c4 < CPL / 4; ++c4) {
                 const float4_t t = {acc[4 * c4][e], acc[4 * c4 + 1][e], acc[4 * c4 + 2][e], acc[4 * c4 + 3][e]};
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, t), tiles,
-                                                       tile_bytes + 4u * (uint32_t)(v * pitch + cs * CPL + 4 * c4), 0,
-                                                       kCoherent);
+                PartMeeting::store_part(tiles, tile_bytes + 4u * (uint32_t)(v * pitch + cs * CPL + 4 * c4), t);
             }
         }
     }
@@ -109,8 +105,7 @@ __device__ __forceinline__ void tile_add_coherent(__amdgpu_buffer_rsrc_t tiles, 
         for (int c4 = 0; c4 < CPL / 4; ++c4) {
             part[e][c4] = float4_t{0.f, 0.f, 0.f, 0.f};
             if (v < V)
-                part[e][c4] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(
-                                  tiles, tile_bytes + 4u * (uint32_t)(v * pitch + cs * CPL + 4 * c4), 0, kCoherent));
+                part[e][c4] = PartMeeting::load_part(tiles, tile_bytes + 4u * (uint32_t)(v * pitch + cs * CPL + 4 * c4));
         }
     }
 #pragma unroll
@@ -382,7 +377,7 @@ spmm_mfma_flat_kernel(int m_vec, int n_cols, int n_tiles, int nonzeros_vec, int 
         if (t_row_end <= ce) {  // the row ends inside the piece: this is all of it
             tile_to_output<V, CPL, OutT>(out, t_row, n_cols, col0, col_ok, g, acc, t_pos);
         } else if constexpr (ONE_LAUNCH) {
-            tile_store_coherent<V, CPL>(tile_area(ws_base), (uint32_t)(((size_t)2 * c + 1) * ws_tile + tile * TN) * 4u, ws_pitch,
+            tile_store_coherent<V, CPL>(PartMeeting::area(ws_base), (uint32_t)(((size_t)2 * c + 1) * ws_tile + tile * TN) * 4u, ws_pitch,
                                         cs, g, acc, t_pos);
             pending = true;
             p_row = t_row;
@@ -406,7 +401,7 @@ spmm_mfma_flat_kernel(int m_vec, int n_cols, int n_tiles, int nonzeros_vec, int 
                 const int last = (int)((stop - 1 - cb) / sub);
                 for (int w = 0; w <= last; ++w) tile_add<V, CPL>(f_tiles + (size_t)w * V * TN, TN, cs, g, sum);
                 if constexpr (ONE_LAUNCH) {
-                    tile_store_coherent<V, CPL>(tile_area(ws_base), (uint32_t)((size_t)2 * c * ws_tile + tile * TN) * 4u, ws_pitch,
+                    tile_store_coherent<V, CPL>(PartMeeting::area(ws_base), (uint32_t)((size_t)2 * c * ws_tile + tile * TN) * 4u, ws_pitch,
                                                 cs, g, sum);
                     pending = true;
                     p_row = f_row;
@@ -420,24 +415,19 @@ spmm_mfma_flat_kernel(int m_vec, int n_cols, int n_tiles, int nonzeros_vec, int 
         if constexpr (ONE_LAUNCH) {
             if (!pending) continue;
             int *counter = counters + (size_t)p_first * n_tiles + tile;
-            // the part's stores have completed (they go through to memory) before the count says so
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-            __builtin_amdgcn_s_waitcnt(0);
-            int arrived = 0;
-            if (lane == 0) arrived = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            arrived = __builtin_amdgcn_readfirstlane(arrived);
-            if (arrived != p_last - p_first) continue;  // parts are still to come: whoever brings the last adds up
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // the parts are read after the count was seen
+            PartMeeting::publish();
+            if (PartMeeting::arrive(counter, lane) != p_last - p_first) continue;  // parts are still to come: whoever brings the last adds up
+            PartMeeting::collect();
             float4_t total[CPL];
 #pragma unroll
             for (int q = 0; q < CPL; ++q) total[q] = float4_t{0.f, 0.f, 0.f, 0.f};
             // T of the first piece, then F of the others, in ascending order
             for (int pc = p_first; pc <= p_last; ++pc)
-                tile_add_coherent<V, CPL>(tile_area(ws_base),
+                tile_add_coherent<V, CPL>(PartMeeting::area(ws_base),
                                           (uint32_t)(((size_t)2 * pc + (pc == p_first ? 1 : 0)) * ws_tile + tile * TN) * 4u,
                                           ws_pitch, cs, g, total);
             tile_to_output<V, CPL, OutT>(out, p_row, n_cols, col0, col_ok, g, total);
-            if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+            PartMeeting::rearm(counter, lane);  // ready for the next launch
         }
     }
 }

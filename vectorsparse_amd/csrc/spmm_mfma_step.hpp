@@ -253,16 +253,72 @@ __device__ __forceinline__ void multiply_step(const RowChunk<CPL> (&chunk)[8], c
     }
 }
 
-// Partial tiles that waves on other CUs - and other XCDs, whose L2 is a different one - read within the same
-// launch go through a buffer descriptor over the tile area of a workspace (below 2^31 bytes, offsets in bytes)
-// with the device-coherence bits of the cache policy set: written through to memory, read past the caches.
+// ---------------------------------------------------------------------------------------------------------------
+// Meeting of partial tiles across workgroups within one launch (rows in parts, split rows).
+//
+// The parts of a row are computed by workgroups on different CUs - and different XCDs, whose L2s are not coherent
+// with each other inside a launch.  Each part leaves an fp32 tile in a workspace and counts itself in on the row's
+// arrival counter; whoever brings the count to the number of parts adds all tiles in ascending order, writes the row
+// and puts the counter back to zero.  Nobody waits for anybody, and the sum is the same whoever arrives last.
+//
+// What makes the last arriver read the other parts' data, in this order and with nothing else (an L2-wide write-back
+// and invalidate - __threadfence() - round the counter costs 60 us per launch instead of 1):
+//   1. store_part(): the tile is stored with the device-coherence bits of the cache policy (sc0 sc1) set: the store
+//      is written through the issuing CU's vector cache and its XCD's L2 to memory;
+//   2. publish(): s_waitcnt vmcnt(0) - the wave does not go on until every such store has been acknowledged by the
+//      memory side, i.e. is visible to any later access that bypasses the caches.  (The workgroup-scope release fence in
+//      front of it only keeps the compiler from moving the stores below this point.)  When several waves of the
+//      workgroup have stored, a workgroup barrier follows, so that all of them have passed their own publish();
+//   3. arrive(): one lane adds 1 to the counter with a relaxed agent-scope atomic, which is carried out at the memory
+//      side (L2 atomics of one address are ordered there, whichever XCD they come from): it is issued after the
+//      acknowledgements of step 2, so a workgroup that observes count == parts - 1 knows every other part's stores
+//      were acknowledged before its own add was performed;
+//   4. collect(): a workgroup-scope acquire fence (compiler ordering only: the loads below are issued after the
+//      atomic has returned its value), then load_part() reads every tile with sc0 sc1 set: past the vector cache and
+//      the L2, from the memory side that acknowledged the stores of step 2;
+//   5. rearm(): the counter goes back to zero with a relaxed agent-scope store; the next launch on the stream (a kernel
+//      boundary) finds it so.  Launches that overlap on one workspace race - the caller's contract.
+// The workspace area is addressed through a buffer descriptor (below 2^31 bytes, offsets in bytes).
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-constexpr int kCoherent = 1 | 16;  // cache policy bits: sc0, sc1
 
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_area(float *base)
-{
-    return __builtin_amdgcn_make_buffer_rsrc(base, 0, 0x7fffffff, 0x00020000);
-}
+struct PartMeeting {
+    static constexpr int kCoherent = 1 | 16;  // cache policy bits: sc0, sc1
+
+    static __device__ __forceinline__ __amdgpu_buffer_rsrc_t area(float *base)
+    {
+        return __builtin_amdgcn_make_buffer_rsrc(base, 0, 0x7fffffff, 0x00020000);
+    }
+    static __device__ __forceinline__ void store_part(__amdgpu_buffer_rsrc_t tiles, uint32_t byte_offset, const float4_t &x)
+    {
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, x), tiles, byte_offset, 0, kCoherent);
+    }
+    // (a store that the NEXT launch reads: an ordinary one, the kernel boundary makes it visible)
+    static __device__ __forceinline__ void store_plain(__amdgpu_buffer_rsrc_t tiles, uint32_t byte_offset, const float4_t &x)
+    {
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, x), tiles, byte_offset, 0, 0);
+    }
+    static __device__ __forceinline__ float4_t load_part(__amdgpu_buffer_rsrc_t tiles, uint32_t byte_offset)
+    {
+        return __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(tiles, byte_offset, 0, kCoherent));
+    }
+    static __device__ __forceinline__ void publish()
+    {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0);
+    }
+    // every lane of the wave gets the number of parts that had arrived before this one
+    static __device__ __forceinline__ int arrive(int *counter, int lane)
+    {
+        int arrived = 0;
+        if (lane == 0) arrived = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return __builtin_amdgcn_readfirstlane(arrived);
+    }
+    static __device__ __forceinline__ void collect() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup"); }
+    static __device__ __forceinline__ void rearm(int *counter, int lane)
+    {
+        if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+};
 
 // Last index i in [0, rows] with offsets[i] <= pos (of equal offsets, i.e. empty rows, the last one): the row
 // that holds nonzero `pos` when pos < offsets[rows].  64-ary search, one probe per lane and round (two dependent
