@@ -87,26 +87,6 @@ def time_graph(torch, fn, steps, warmup, replays=7):
     return walls[len(walls) // 2], events[len(events) // 2]
 
 
-def time_cold(torch, fn, samples=20):
-    """Device time of single launches with the caches thrashed in between: a 1 GiB fill evicts the 256 MB
-    Infinity Cache and the L2s before every timed launch (the reference measures with Nsight's
-    --cache-control all, i.e. flushed caches)."""
-    thrash = torch.empty(512 * 1024 * 1024, dtype=torch.float16, device="cuda")
-    times = []
-    for i in range(samples):
-        thrash.fill_(float(i))
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
-        e0.record()
-        fn()
-        e1.record()
-        torch.cuda.synchronize()
-        times.append(e0.elapsed_time(e1))
-    del thrash
-    times.sort()
-    return times[len(times) // 2]
-
-
 def kernel_source_tag(*names):
     """First 16 hex digits of the SHA-256 of the kernel sources a counter summary belongs to."""
     import hashlib
@@ -189,7 +169,7 @@ def cpu_baseline(pat, B, n_dense, flops, budget_s=12.0):
     }
 
 
-PMC_MODES = ["spmm", "spmm_largest", "spmm_slab_50", "spmm_slab_90", "spmm_dma", "spmm_split_rows", "spmm_row_parts", "sddmm", "attention",
+PMC_MODES = ["spmm", "spmm_largest", "spmm_slab_50", "spmm_slab_90", "spmm_valu_v1", "sddmm_valu_v1", "sddmm_k128", "spmm_dma", "spmm_split_rows", "spmm_row_parts", "sddmm", "attention",
              "attention_window"]
 
 
@@ -197,6 +177,129 @@ def largest_sweep_point(cv):
     """The largest single-GPU point of the ResNet-50-shaped sweep: M = 2048, K = 4608, N = 256, V = 8, 90 %."""
     pat = cv.random_values(cv.uniform_pattern(2048 // 8, 4608, 0.9, seed=3, vec_length=8), seed=4)
     return pat, cv.dense_uniform(4608, 256, seed=5)
+
+
+COLD_KERNELS = (("spmm_config2", "spmm_mfma_kernelILi8ELi4E"), ("spmm_largest", "spmm_mfma_kernelILi8ELi8E"),
+                ("sddmm_config4", "sddmm_mfma_kernel"), ("dense_gemm_config2", "Cijk_"), ("empty_kernel", "floor_probe_kernel"))
+COLD_PROFILE = os.path.join(ROOT, "profiles", "cold_cache_kernel_stats.txt")
+
+
+def cold_summary(stats_csv):
+    """Text of profiles/cold_cache_kernel_stats.txt from the kernel_stats.csv of
+    `rocprofv3 --kernel-trace --stats ... -- python3 bench.py --cold`."""
+    import csv
+    found = {}
+    with open(stats_csv) as f:
+        for r in csv.DictReader(f):
+            for key, needle in COLD_KERNELS:
+                if needle in r["Name"]:
+                    calls, total = found.get(key, (0, 0.0))
+                    found[key] = (calls + int(r["Calls"]), total + float(r["TotalDurationNs"]))
+    lines = ["Flushed-cache durations by the kernels' own timestamps (how the reference measures: Nsight --cache-control all,",
+             "ncu_profile.py:91): every timed launch follows a 1 GiB fill that evicts the L2s and the Infinity Cache.",
+             "",
+             "commands (`cd /tmp && export TMPDIR=/tmp` first, then from the repository root):",
+             "  rocprofv3 --kernel-trace --stats --output-format csv -d gpurun_out/prof/cold -o t -- python3 bench.py --cold",
+             "  python3 bench.py --cold-summary gpurun_out/prof/cold/t_kernel_stats.csv > profiles/cold_cache_kernel_stats.txt",
+             "",
+             "kernel_source_tag_spmm %s" % kernel_source_tag(*SPMM_SOURCES),
+             "kernel_source_tag_sddmm %s" % kernel_source_tag(*SDDMM_SOURCES),
+             "",
+             "mean kernel duration over the launches of the run (each right behind a fill), microseconds:"]
+    for key, _ in COLD_KERNELS:
+        if key in found:
+            calls, total = found[key]
+            lines.append("cold_us %-20s %8.2f   (%d launches)" % (key, total / calls * 1e-3, calls))
+    return "\n".join(lines)
+
+
+def read_cold_profile():
+    """({name: microseconds}, note) from the committed summary of a `--cold` run; figures of kernels whose sources
+    have changed since are dropped (the dense GEMM and the empty kernel are not ours and stay)."""
+    values, tags = {}, {}
+    try:
+        with open(COLD_PROFILE) as f:
+            for ln in f:
+                w = ln.split()
+                if len(w) >= 3 and w[0] == "cold_us":
+                    values[w[1]] = float(w[2])
+                elif len(w) == 2 and w[0].startswith("kernel_source_tag_"):
+                    tags[w[0][len("kernel_source_tag_"):]] = w[1]
+    except OSError:
+        return {}, "no summary at %s" % os.path.relpath(COLD_PROFILE, ROOT)
+    stale = []
+    if tags.get("spmm") != kernel_source_tag(*SPMM_SOURCES):
+        stale += [k for k in ("spmm_config2", "spmm_largest") if values.pop(k, None) is not None]
+    if tags.get("sddmm") != kernel_source_tag(*SDDMM_SOURCES):
+        stale += [k for k in ("sddmm_config4",) if values.pop(k, None) is not None]
+    note = "from %s" % os.path.relpath(COLD_PROFILE, ROOT)
+    if stale:
+        note += "; dropped as stale (kernel sources changed since the run): " + ", ".join(stale)
+    return values, note
+
+
+def fine_grained_spmm_point(cv):
+    """Where the fine-grained SpMM path is at home: V = 1, M = 2048, K = 4608, N = 256 at 90 % sparsity."""
+    pat = cv.random_values(cv.uniform_pattern(2048, 4608, 0.9, seed=13, vec_length=1), seed=14)
+    return pat, cv.dense_uniform(4608, 256, seed=15)
+
+
+def fine_grained_sddmm_mask(cv):
+    """The same for SDDMM: a 2048 x 2048 mask of single elements (V = 1) at 90 % sparsity (K = 64)."""
+    return cv.uniform_pattern(2048, 2048, 0.9, seed=16, vec_length=1)
+
+
+def sweep_v8(torch, cv, ops, iters=30):
+    """The north-star comparison on the ResNet-50-shaped grid: every (M, K) of the sweep at N = 256, V = 8, at 80 % and
+    90 % sparsity, through the reference-shaped entry point, each point verified (float64 product on a sample of rows,
+    as the sweep driver does) and timed beside hipBLASLt's dense fp16 product of the same shape (the comparison of
+    the reference's plot_spmm.py:43-58, per sparsity bucket)."""
+    import numpy as np
+    from vectorsparse_amd import sweep
+    from vectorsparse_amd.benchmark_common import time_launches
+    dense_us, dense_in, out_by_m, B_by_k = {}, {}, {}, {}
+    buckets = {}
+    unverified = 0
+    for s in (0.8, 0.9):
+        rows = []
+        for M in sweep.MS:
+            for K in sweep.KS:
+                pat = sweep.spmm_grid_pattern(M, K, s, 8)
+                if K not in B_by_k:
+                    host = cv.dense_uniform(K, sweep.N_DENSE, seed=11)
+                    B_by_k[K] = (host, torch.from_numpy(host).cuda())
+                B_host, B = B_by_k[K]
+                out = out_by_m.setdefault(M, torch.empty((M, sweep.N_DENSE), dtype=torch.float16, device="cuda"))
+                prob = ops.DeviceProblem(pat, sort=True)
+                out.fill_(float("nan"))
+                prob.spmm(B, kernel="wmma", out=out)
+                torch.cuda.synchronize()
+                ok, rel = sweep.verify_spmm(pat, B_host, out.cpu().numpy())
+                unverified += 0 if ok else 1
+                us = time_launches(torch, lambda: prob.spmm(B, kernel="wmma", out=out), iters, warmup=2, replays=3)
+                if (M, K) not in dense_us:
+                    A = torch.randn((M, K), dtype=torch.float16, device="cuda")
+                    dense_us[(M, K)] = time_launches(torch, lambda: torch.matmul(A, B, out=out), iters, warmup=2, replays=3)
+                    del A
+                rows.append({"M": M, "K": K, "us": us, "dense_us": dense_us[(M, K)], "speedup": dense_us[(M, K)] / us,
+                             "frac": sweep.spmm_bytes(pat, sweep.N_DENSE) / (us * 1e-6) * 1e-9 / HBM_PEAK_GBS,
+                             "max_rel_err": rel, "verified": ok})
+        worst = min(rows, key=lambda r: r["speedup"])
+        best = max(rows, key=lambda r: r["frac"])
+        fracs = sorted(r["frac"] for r in rows)
+        buckets["%g" % s] = {
+            "points": len(rows), "verified": sum(1 for r in rows if r["verified"]),
+            "geomean_speedup_vs_dense": sweep.geomean([r["speedup"] for r in rows]),
+            "worst_speedup_vs_dense": worst["speedup"], "worst_point": "M=%d K=%d" % (worst["M"], worst["K"]),
+            "points_slower_than_dense": sum(1 for r in rows if r["speedup"] < 1.0),
+            "max_frac": best["frac"], "max_frac_point": "M=%d K=%d (%.2f us)" % (best["M"], best["K"], best["us"]),
+            "median_frac": fracs[len(fracs) // 2],
+            "max_rel_err": max(r["max_rel_err"] for r in rows)}
+    if unverified:
+        raise SystemExit("sweep_v8: %d point(s) failed verification" % unverified)
+    return {"workload": "config 3 at V=8, N=256: M in %s x K in %s, uniform rows, vs_wmma_spmm_f16 with the sorted swizzle; "
+                        "frac = algorithmic bytes / launch time / 8 TB/s" % (list(sweep.MS), list(sweep.KS)),
+            "launches_per_replay": iters, "by_sparsity": buckets}
 
 
 def skewed_point(cv, np):
@@ -221,7 +324,17 @@ def main():
                          "(config 2), the largest sweep point (2048 x 4608 at 90 %%), the LDS-staged schedule on that shape at 50 %% and 90 %%, config 2 on the LDS-DMA gather "
                          "variant, the split-row SpMM and the SpMM with rows in parts on Pareto-distributed rows, the config-4 SDDMM, the config-5 "
                          "attention layer with its plan, or that layer with a plain 513-wide window mask")
+    ap.add_argument("--cold", action="store_true",
+                    help="flushed-cache mode for `rocprofv3 --kernel-trace --stats`: ten rounds of (1 GiB fill, ONE launch) "
+                         "for each of the config-2 SpMM, the largest sweep point, the config-4 SDDMM, the dense GEMM of "
+                         "config 2 and a kernel that does nothing; the kernels' own timestamps are the cold durations")
+    ap.add_argument("--cold-summary", metavar="KERNEL_STATS_CSV", default=None,
+                    help="turn the kernel_stats.csv of such a run into the text of profiles/cold_cache_kernel_stats.txt "
+                         "(printed; no GPU needed)")
     args = ap.parse_args()
+    if args.cold_summary:
+        print(cold_summary(args.cold_summary))
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU: the SpMM/SDDMM path has no multi-GPU leg (rows shard with no "
               "exchange step); run with --gpus 1", file=sys.stderr)
@@ -262,6 +375,28 @@ def main():
     def sddmm_step():
         sprob.sddmm(lhs, rhs, kernel="wmma", out=sout)
 
+    if args.cold:
+        import ctypes
+        probe_lib = ctypes.CDLL(os.path.join(ROOT, "vectorsparse_amd", "libvsprobe.so"))
+        probe_lib.vsprobe_empty_launch.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+        lpat, lB = largest_sweep_point(cv)
+        lprob = ops.DeviceProblem(lpat, sort=True)
+        lBd = torch.from_numpy(lB).cuda()
+        lout = torch.empty((lpat.m, 256), dtype=torch.float16, device="cuda")
+        Ad = torch.randn((M, K), dtype=torch.float16, device="cuda")
+        dense_out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+        launches = (step, lambda: lprob.spmm(lBd, kernel="wmma", out=lout), sddmm_step,
+                    lambda: torch.matmul(Ad, Bd, out=dense_out),
+                    lambda: probe_lib.vsprobe_empty_launch(256, 512, torch.cuda.current_stream().cuda_stream))
+        thrash = torch.empty(512 * 1024 * 1024, dtype=torch.float16, device="cuda")
+        for i in range(10):
+            for fn in launches:
+                thrash.fill_(float(i))
+                fn()
+            torch.cuda.synchronize()
+        print(json.dumps({"cold_mode": "10 rounds of (1 GiB fill, one launch) for %d kernels" % len(launches)}))
+        return
+
     if args.pmc:
         src = torch.zeros(32 * 1024 * 1024, dtype=torch.float16, device="cuda")   # 64 MiB read + 64 MiB written
         dst = torch.empty_like(src)
@@ -300,6 +435,34 @@ def main():
             info["algorithmic_bytes"] = spmm_algorithmic_bytes(lpat, 256)
             info["nonzero_vectors"] = int(lpat.nnz_vec)
             info["kernel_source_tag"] = kernel_source_tag("spmm_mfma_slab.hip", "spmm_mfma_step.hpp", "vs_common.hpp")
+        elif args.pmc == "spmm_valu_v1":
+            # the fine-grained SpMM on the shape it exists for: V = 1 (2048 x 4608 x 256 at 90 %)
+            vpat, vB = fine_grained_spmm_point(cv)
+            vprob = ops.DeviceProblem(vpat, sort=True)
+            vBd = torch.from_numpy(vB).cuda()
+            vout = torch.empty((vpat.m, 256), dtype=torch.float16, device="cuda")
+            for _ in range(10):
+                vprob.spmm(vBd, kernel="cuda", out=vout)
+            info["algorithmic_bytes"] = spmm_algorithmic_bytes(vpat, 256)
+            info["nonzero_vectors"] = int(vpat.nnz_vec)
+            info["kernel_source_tag"] = kernel_source_tag("spmm_valu.hip", "vs_common.hpp")
+        elif args.pmc == "sddmm_valu_v1":
+            # the fine-grained SDDMM at V = 1 (2048 x 2048 mask at 90 %, K = 64)
+            vmask = fine_grained_sddmm_mask(cv)
+            vsprob = ops.DeviceProblem(vmask)
+            vsout = torch.empty((vmask.nnz_vec, 1), dtype=torch.float16, device="cuda")
+            for _ in range(10):
+                vsprob.sddmm(lhs, rhs, kernel="cuda", out=vsout)
+            info["algorithmic_bytes"] = sddmm_algorithmic_bytes(vmask, 64)
+            info["nonzero_vectors"] = int(vmask.nnz_vec)
+            info["kernel_source_tag"] = kernel_source_tag("sddmm_valu.hip", "vs_common.hpp")
+        elif args.pmc == "sddmm_k128":
+            lhs128 = torch.from_numpy(cv.dense_normal(2048, 128, seed=15)).cuda()
+            rhs128 = torch.from_numpy(cv.dense_normal(2048, 128, seed=25)).cuda()
+            for _ in range(10):
+                sprob.sddmm(lhs128, rhs128, kernel="wmma", out=sout)
+            info["algorithmic_bytes"] = sddmm_algorithmic_bytes(mask, 128)
+            info["kernel_source_tag"] = kernel_source_tag(*SDDMM_SOURCES)
         elif args.pmc == "spmm_split_rows":
             kpat, kB = skewed_point(cv, np)
             kprob = ops.DeviceProblem(kpat, sort=True)
@@ -484,13 +647,44 @@ def main():
     if not global_diff < 2e-2:
         raise SystemExit("attention with global tokens: rows in parts and whole rows disagree: %g" % global_diff)
 
-    # ---- cold caches (how the reference measures: Nsight --cache-control all)
-    cold_ms = time_cold(torch, step)
-    cold_floor_ms = time_cold(torch, probe(512))  # what the same method reads for a kernel that does nothing
-    cold_dense_ms = time_cold(torch, lambda: torch.matmul(Ad, Bd, out=dense_out))
-    cold_large_ms = time_cold(torch, lambda: lprob.spmm(lBd, kernel="wmma", out=lout), samples=10)
-    cold_sddmm_ms = time_cold(torch, sddmm_step, samples=10)
-    cold_attn_ms = time_cold(torch, lambda: layer.forward(q, kk_, vv, scores=scores, out=ctx), samples=10)
+    # ---- cold caches (how the reference measures: Nsight --cache-control all): the kernels' own timestamps from a
+    # `rocprofv3 --kernel-trace` run of `bench.py --cold`, committed under profiles/ (HIP events round a single eager
+    # launch read 6 us for a kernel that does nothing, so they are not used for this)
+    cold, cold_note = read_cold_profile()
+
+    # ---- the fine-grained paths where they are at home: V = 1
+    vpat, vB = fine_grained_spmm_point(cv)
+    vprob = ops.DeviceProblem(vpat, sort=True)
+    vBd = torch.from_numpy(vB).cuda()
+    vout = torch.empty((vpat.m, 256), dtype=torch.float16, device="cuda")
+    fine_steps = max(20, dev_steps // 4)
+    _, v1_spmm_valu_ms = time_graph(torch, lambda: vprob.spmm(vBd, kernel="cuda", out=vout), fine_steps, 3)
+    _, v1_spmm_mfma_ms = time_graph(torch, lambda: vprob.spmm(vBd, kernel="wmma", out=vout), fine_steps, 3)
+    v1_spmm_bytes, v1_spmm_flops = spmm_algorithmic_bytes(vpat, 256), 2.0 * vpat.nnz * 256
+    vA = torch.randn((vpat.m, 4608), dtype=torch.float16, device="cuda")
+    _, v1_dense_ms = time_graph(torch, lambda: torch.matmul(vA, vBd, out=vout), fine_steps, 3)
+    vmask = fine_grained_sddmm_mask(cv)
+    vsprob = ops.DeviceProblem(vmask)
+    vsout = torch.empty((vmask.nnz_vec, 1), dtype=torch.float16, device="cuda")
+    _, v1_sddmm_valu_ms = time_graph(torch, lambda: vsprob.sddmm(lhs, rhs, kernel="cuda", out=vsout), fine_steps, 3)
+    _, v1_sddmm_mfma_ms = time_graph(torch, lambda: vsprob.sddmm(lhs, rhs, kernel="wmma", out=vsout, algorithm=1), fine_steps, 3)
+    v1_sddmm_bytes, v1_sddmm_flops = sddmm_algorithmic_bytes(vmask, 64), 2.0 * vmask.nnz * 64
+
+    # ---- config 4's other three points (K = 128, and 95 % sparsity)
+    sddmm_more = {}
+    for kk, sp, seed in ((128, 0.9, 4), (64, 0.95, 6), (128, 0.95, 6)):
+        m4 = mask if sp == 0.9 else cv.uniform_pattern(2048 // 8, 2048, sp, seed=seed, vec_length=8)
+        p4 = sprob if sp == 0.9 else ops.DeviceProblem(m4)
+        l4 = torch.from_numpy(cv.dense_normal(2048, kk, seed=14 + kk)).cuda()
+        r4 = torch.from_numpy(cv.dense_normal(2048, kk, seed=24 + kk)).cuda()
+        o4 = torch.empty((m4.nnz_vec, 8), dtype=torch.float16, device="cuda")
+        _, ms4 = time_graph(torch, lambda: p4.sddmm(l4, r4, kernel="wmma", out=o4), dev_steps, 3)
+        f4 = torch.empty((2048, 2048), dtype=torch.float16, device="cuda")
+        _, dense4 = time_graph(torch, lambda: torch.matmul(l4, r4.t(), out=f4), fine_steps, 3)
+        sddmm_more["k%d_s%g" % (kk, sp)] = (sddmm_algorithmic_bytes(m4, kk), ms4, 2.0 * m4.nnz * kk, dense4)
+
+    # ---- the sweep's V = 8 points at 80 % and 90 % beside hipBLASLt
+    sweep_block = sweep_v8(torch, cv, ops)
 
     achieved = alg_bytes / (ev_ms * 1e-3) * 1e-9
     traffic, traffic_note = measured_traffic(os.path.join(ROOT, "profiles", "spmm_mfma_config2_pmc.txt"), SPMM_SOURCES)
@@ -525,9 +719,10 @@ def main():
         "roofline": hbm(alg_bytes, ev_ms, traffic, kernel="spmm_mfma_kernel<V=8>", traffic_note=traffic_note,
                         caches="warm: the 3.2 MB working set stays in the Infinity Cache between launches (the L2s "
                                "start every launch cold); see extra.cold_cache",
-                        frac_cold=alg_bytes / (cold_ms * 1e-3) * 1e-9 / HBM_PEAK_GBS,
-                        frac_cold_note="from extra.cold_cache.spmm_config2_us, which contains the %.1f us the same "
-                                       "method reads for an empty kernel" % (cold_floor_ms * 1e3),
+                        frac_cold=(alg_bytes / (cold["spmm_config2"] * 1e-6) * 1e-9 / HBM_PEAK_GBS
+                                   if "spmm_config2" in cold else None),
+                        frac_cold_note="from extra.cold_cache.kernel_us.spmm_config2 (kernel timestamps of a launch "
+                                       "behind a 1 GiB fill; " + cold_note + ")",
                         ceiling_frac=alg_bytes / (floor_ms * 1e-3) * 1e-9 / HBM_PEAK_GBS,
                         ceiling_note="a kernel that does nothing on this launch's grid (256 workgroups of up to 1024 threads) "
                                      "takes extra.launch_floor.empty_grid_us: the HBM-roofline time of config 2 "
@@ -540,13 +735,13 @@ def main():
             "speedup_vs_dense_gemm": dense_ms / ev_ms,
             "launch_floor": {"empty_grid_us": floor_ms * 1e3, "empty_grid_one_wave_per_workgroup_us": floor_small_ms * 1e3,
                              "frac_of_floor": floor_ms / ev_ms},
-            "cold_cache": {"method": "HIP events round one eager launch that follows a 1 GiB fill; the same method reads "
-                                     "empty_kernel_us for a kernel that does nothing on config 2's grid, so only the "
-                                     "differences to it are kernel time",
-                           "empty_kernel_us": cold_floor_ms * 1e3,
-                           "spmm_config2_us": cold_ms * 1e3, "dense_gemm_config2_us": cold_dense_ms * 1e3,
-                           "spmm_largest_us": cold_large_ms * 1e3, "sddmm_config4_us": cold_sddmm_ms * 1e3,
-                           "attention_config5_us": cold_attn_ms * 1e3},
+            "cold_cache": {"method": "mean kernel duration by the kernels' own timestamps (rocprofv3 --kernel-trace --stats of "
+                                     "`bench.py --cold`: every launch right behind a 1 GiB fill), read from the committed "
+                                     "summary; null where the kernel sources have changed since",
+                           "source": cold_note, "kernel_us": cold,
+                           "speedup_vs_dense_gemm_config2": (cold["dense_gemm_config2"] / cold["spmm_config2"]
+                                                             if "dense_gemm_config2" in cold and "spmm_config2" in cold else None)},
+            "sweep_v8": sweep_block,
             "spmm_largest_sweep_point": dict(
                 hbm(large_bytes, large_ms, large_traffic),
                 workload="M=2048 K=4608 N=256 V=8 sparsity=0.9", tflops=2.0 * lpat.nnz * 256 / (large_ms * 1e-3) * 1e-12,
@@ -569,7 +764,23 @@ def main():
                 hbm(sddmm_bytes, sddmm_ms, sddmm_traffic, traffic_note=sddmm_note, kernel="sddmm_mfma_kernel<V=8>"),
                 ms=sddmm_ms, tflops=sddmm_flops / (sddmm_ms * 1e-3) * 1e-12, dense_product_us=sddmm_dense_ms * 1e3,
                 speedup_vs_dense=sddmm_dense_ms / sddmm_ms),
+            "sddmm_config4_other_points": {
+                name: dict(hbm(nb, ms4, kernel="sddmm_mfma_kernel<V=8>"), tflops=fl / (ms4 * 1e-3) * 1e-12,
+                           dense_product_us=d4 * 1e3, speedup_vs_dense=d4 / ms4)
+                for name, (nb, ms4, fl, d4) in sddmm_more.items()},
             "fine_grained_paths": {
+                "spmm_v1_2048x4608x256_s90": {
+                    "cuda_path": dict(hbm(v1_spmm_bytes, v1_spmm_valu_ms, kernel="spmm_valu_kernel<V=1>"),
+                                      tflops=v1_spmm_flops / (v1_spmm_valu_ms * 1e-3) * 1e-12),
+                    "wmma_path": dict(hbm(v1_spmm_bytes, v1_spmm_mfma_ms, kernel="spmm_mfma_kernel<V=1>"),
+                                      tflops=v1_spmm_flops / (v1_spmm_mfma_ms * 1e-3) * 1e-12),
+                    "dense_gemm_us": v1_dense_ms * 1e3, "cuda_over_wmma": v1_spmm_mfma_ms / v1_spmm_valu_ms},
+                "sddmm_v1_2048x2048_k64_s90": {
+                    "cuda_path": dict(hbm(v1_sddmm_bytes, v1_sddmm_valu_ms, kernel="sddmm_valu_kernel<V=1>"),
+                                      tflops=v1_sddmm_flops / (v1_sddmm_valu_ms * 1e-3) * 1e-12),
+                    "wmma_path": dict(hbm(v1_sddmm_bytes, v1_sddmm_mfma_ms, kernel="sddmm_mfma_kernel<V=1>"),
+                                      tflops=v1_sddmm_flops / (v1_sddmm_mfma_ms * 1e-3) * 1e-12),
+                    "cuda_over_wmma": v1_sddmm_mfma_ms / v1_sddmm_valu_ms},
                 "spmm_config2": dict(hbm(alg_bytes, valu_spmm_ms, kernel="spmm_valu_kernel<V=8>"),
                                      tflops=flops / (valu_spmm_ms * 1e-3) * 1e-12, speedup_vs_dense_gemm=dense_ms / valu_spmm_ms),
                 "sddmm_config4_k64": dict(hbm(sddmm_bytes, valu_sddmm_ms, kernel="sddmm_valu_kernel<V=8>"),
