@@ -9,6 +9,7 @@ import torch
 from vectorsparse_amd import _lib, ops
 from vectorsparse_amd import colvec_csr as cv
 from vectorsparse_amd.benchmark_common import time_launches
+from util import retired_variants_built
 
 pytestmark = pytest.mark.gpu
 
@@ -83,7 +84,8 @@ def test_thread_options_do_not_leak_between_threads_and_streams(gpu):
 
 
 def _best_of(fn, settings):
-    """(time of the automatic shape, best time over hand-picked shapes), each the minimum of three medians."""
+    """(time of the automatic shape, best time over hand-picked shapes), each the minimum of three medians; the
+    automatic shape is timed before and after the others, so that a clock still ramping up does not count against it."""
     def t():
         return min(time_launches(torch, fn, iters=100) for _ in range(3))
     auto = t()
@@ -91,7 +93,8 @@ def _best_of(fn, settings):
     for kw in settings:
         with _lib.thread_options(**kw):
             best = min(best, t())
-    return auto, best
+    auto = min(auto, t())
+    return auto, min(best, auto)
 
 
 def test_automatic_launch_shapes_are_close_to_the_best_on_the_headline_configs(gpu):
@@ -114,7 +117,8 @@ def test_automatic_launch_shapes_are_close_to_the_best_on_the_headline_configs(g
     for hint in (False, True):
         auto, best = _best_of(lambda: bprob.spmm(Bd, out=bout, row_length_hint=hint),
                               [dict(spmm_cols_per_lane=8, spmm_waves=w, spmm_steps=st, spmm_pipe=p)
-                               for w in (2, 4, 8) for st, p in ((2, 1), (2, 2), (4, 1))])
+                               for w in (2, 4, 8)
+                               for st, p in ((2, 1), (2, 2)) + (((4, 1),) if retired_variants_built() else ())])
         print("2048 x 4608 at 90 %%, hints %d: automatic %.2f us, best override %.2f us" % (hint, auto, best))
         assert auto <= 1.10 * best
 
@@ -128,3 +132,37 @@ def test_automatic_launch_shapes_are_close_to_the_best_on_the_headline_configs(g
                               [dict(sddmm_group=g, sddmm_slots=sl) for g in (1, 2, 4) for sl in (4, 8, 16)])
         print("config 4 SDDMM K=%d s=%g: automatic %.2f us, best override %.2f us" % (K, s, auto, best))
         assert auto <= 1.10 * best
+
+
+# (rows of 8, K, sparsity, vector length): points of the published sweep (N = 256), small to large, every vector
+# length, 50 % to 98 %
+SWEEP_POINTS = (
+    (2048, 4608, 0.5, 8), (2048, 4608, 0.8, 8), (1024, 2304, 0.7, 8), (512, 1152, 0.9, 8), (256, 576, 0.95, 8),
+    (64, 4608, 0.98, 8), (2048, 256, 0.8, 8), (128, 147, 0.5, 8),
+    (1024, 4608, 0.9, 4), (512, 1152, 0.8, 4), (2048, 576, 0.95, 4),
+    (2048, 2304, 0.9, 2), (256, 1152, 0.7, 2),
+    (2048, 4608, 0.95, 1), (512, 2304, 0.9, 1), (1024, 256, 0.8, 1),
+)
+
+
+@pytest.mark.parametrize("m,k,s,v", SWEEP_POINTS)
+def test_automatic_spmm_shape_is_close_to_the_best_on_sweep_points(gpu, m, k, s, v):
+    """SpMM on points of the sweep grid, against the best of sixteen hand-picked shapes (tile width x waves x
+    pipelined walk).  With the row lengths known (the batched entry with its hints) the automatic shape must be
+    within 10 % of the best.  The reference-shaped entry does not know the row lengths: where it launches more waves
+    than the hinted entry does - guard waves, which a row far longer than expected would spread over, and which end at
+    once on these uniform rows at about 0.1 us per thousand - the bound is 20 %, else 10 %."""
+    pat = cv.random_values(cv.uniform_pattern(m // v, k, s, seed=7, vec_length=v), seed=107)
+    Bd = torch.from_numpy(cv.dense_uniform(k, 256, seed=207)).cuda()
+    prob = ops.DeviceProblem(pat)
+    out = torch.empty((m, 256), dtype=torch.float16, device="cuda")
+    overrides = [dict(spmm_cols_per_lane=c, spmm_waves=w, spmm_pipe=p) for c in (4, 8) for w in (1, 2, 4, 8)
+                 for p in (1, 2)]
+    known = ops.spmm_launch_shape(m // v, v, 256, k, 1, pat.nnz_vec, prob.longest_row_vec, prob.long_rows)
+    blind = ops.spmm_launch_shape(m // v, v, 256, k)
+    for hint, shape in ((True, known), (False, blind)):
+        auto, best = _best_of(lambda: prob.spmm(Bd, out=out, row_length_hint=hint), overrides)
+        bound = 1.20 if not hint and blind["waves"] > known["waves"] else 1.10
+        print("%d x %d at %g, V=%d, hints %d (%d waves): automatic %.2f us, best override %.2f us"
+              % (m, k, s, v, hint, shape["waves"], auto, best))
+        assert auto <= bound * best

@@ -671,6 +671,11 @@ SpmmShape choose_spmm_shape(bool softmax, int m_vec, int vec_length, int k, int 
         const int resident = (registers >= 32 ? 2 : registers >= 16 ? 3 : 5) * 1024;   // waves the chip holds at once
         int room = 1;
         while (2LL * room * blocks <= resident) room <<= 1;
+        // Three and a half to four workgroups per CU: with one wave each every SIMD holds one wave and the launch is
+        // a single even round, which a second wave per row (and the sum through LDS it brings) only slows down - rows
+        // of 230 / 461 / 922 vectors, N = 256, on 896 and 1024 workgroups: V = 1 and 2 one wave 9-13 % ahead of two,
+        // V = 4 3-12 %, V = 8 2-7 %; from 1152 to 1536 workgroups two waves are 1-3 % ahead again.
+        if (blocks > 800 && blocks <= 1024) room = 1;
         waves = want < room ? want : room;
         // Row lengths unknown and the grid alone fills the chip: the workgroups still get a few waves, of which a
         // row of the expected length uses `room` (a wave takes want / room of its blocks); a row far longer than

@@ -33,11 +33,25 @@ __device__ __forceinline__ void load_values(uint32_t (&dst)[V > 1 ? V / 2 : 1], 
     }
 }
 
+// Sum of x over the 64 / LR lanes of a wave that hold the same columns (lane = group * LR + column lane): a butterfly
+// over the lane bits above LR; every lane ends up with the total.
+template <int LR>
+__device__ __forceinline__ float sum_over_groups(float x)
+{
+    if constexpr (LR <= 8) {
+        const int xi = __builtin_bit_cast(int, x);
+        x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, xi, 0x128, 0xF, 0xF, true));  // row_ror:8 = lane ^ 8
+    }
+    if constexpr (LR <= 16) x += partner<16>(x);
+    if constexpr (LR <= 32) x += partner<32>(x);
+    return x;
+}
+
 // RAGGED: the dense width is not a multiple of 8 (rows of the dense operand and of the output start at any 2-byte
 // boundary, the last chunk of a row is cut): chunks are fetched and stored half by half.
 template <int V, int LR, typename OutT, bool RAGGED = false>
 __global__ void __launch_bounds__(1024)
-spmm_valu_kernel(int n_cols, int n_tiles, int n_waves, const int *__restrict__ row_indices,
+spmm_valu_kernel(int n_cols, int n_tiles, int n_waves, uint32_t inv_waves, const int *__restrict__ row_indices,
                  const int *__restrict__ row_offsets, const int *__restrict__ column_indices,
                  const half_t *__restrict__ values, const half_t *__restrict__ rhs,
                  OutT *__restrict__ out, long long stride_values, long long stride_rhs, long long stride_out)
@@ -47,9 +61,14 @@ spmm_valu_kernel(int n_cols, int n_tiles, int n_waves, const int *__restrict__ r
         rhs += blockIdx.y * stride_rhs;
         out += blockIdx.y * stride_out;
     }
-    extern __shared__ float partial[];  // [W*G][V][TN]
+    extern __shared__ float partial[];  // [W * kTiles][V][TN] partial tiles, then the waves' staging slots
     constexpr int G = 64 / LR;
     constexpr int TN = 8 * LR;
+    // Short vectors: the groups of a wave add their partial sums up across the lanes (below) and the wave leaves one
+    // tile; V = 4 and 8 hold 32 and 64 accumulators per lane, for which that butterfly costs more than it saves
+    // (V = 8, 64 rows x 4608: 5.3 -> 6.3 us), so every group leaves a tile of its own.
+    constexpr bool kLaneSum = V <= 2;
+    constexpr int kTiles = kLaneSum ? 1 : G;  // partial tiles per wave
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int tile = blockIdx.x % n_tiles;
@@ -64,14 +83,26 @@ spmm_valu_kernel(int n_cols, int n_tiles, int n_waves, const int *__restrict__ r
         beg = row_offsets[row];
         end = row_offsets[row + 1];
     }
-    constexpr int U = 4;  // nonzero vectors per group and turn, so that U gathered rows are in flight per lane
-    // Group p starts at nonzero beg + p * U: on a short row only the first few groups have any.  Waves that have
-    // neither a group with nonzeros nor a share of the final sum (V * LR items, one per thread) end here: a
+    constexpr int U = V <= 4 ? 8 : 4;  // nonzero vectors per group and turn: U gathered rows in flight per lane
+    constexpr int kBlock = 64;   // nonzero vectors a wave fetches at once, at most: one column index and one vector per lane
+    constexpr int kWords = V > 1 ? V / 2 : 1;
+    // Wave w takes the blocks w, w + n_waves, .. of the row; inside a block group g takes the nonzeros
+    // (t * G + g) * U .. + U - 1 of turn t.  A block is 64 nonzeros, or fewer (whole turns) when the row is short
+    // enough for every wave to get one: a row of 115 nonzeros is eight blocks of 16 for eight waves, not two of 64.
+    // Waves that have neither a block nor a share of the final sum (V * LR items, one per thread) end here: a
     // workgroup barrier waits only for the waves that still run.
-    int n_partials = (end - beg + U - 1) / U;
-    n_partials = n_partials < 1 ? 1 : (n_partials > n_waves * G ? n_waves * G : n_partials);
     constexpr int kSumWaves = (V * LR + 63) / 64;
-    int alive_waves = (n_partials + G - 1) / G;
+    constexpr int kTurn = G * U < kBlock ? G * U : kBlock;  // nonzeros of a turn (a power of two)
+    // (inv_waves = 2^32 / n_waves + 1: the row's share per wave without a division, which costs a launch of
+    // short rows 0.5 us; an inexact quotient only moves the block size, any size gives the same coverage)
+    const int per_wave = (int)(((unsigned long long)(uint32_t)(end - beg + n_waves - 1) * inv_waves) >> 32);
+    int block = (per_wave + kTurn - 1) / kTurn * kTurn;
+    // (two turns a wave at least where the row has them: 512 rows of 115 nonzeros, V = 1, N = 256, eight waves launched:
+    // 4.1 us with a turn each, 3.7 us with four of them taking two turns and the others ending at once)
+    constexpr int kLeast = 2 * kTurn < kBlock ? 2 * kTurn : kBlock;
+    block = block < kLeast ? kLeast : (block > kBlock ? kBlock : block);
+    // waves with a block: all of them unless the blocks are at their smallest (a wave without one adds zeros)
+    int alive_waves = block == kLeast ? (end - beg + kLeast - 1) / kLeast : n_waves;
     alive_waves = alive_waves < kSumWaves ? kSumWaves : alive_waves;
     alive_waves = alive_waves < n_waves ? alive_waves : n_waves;
     if (wave >= alive_waves) return;
@@ -88,25 +119,37 @@ spmm_valu_kernel(int n_cols, int n_tiles, int n_waves, const int *__restrict__ r
 #pragma unroll
         for (int c = 0; c < 8; ++c) acc[v][c] = 0.f;
 
-    // (fetching the next turn's column indices and values a turn ahead costs 18 to 40 registers and measured 2-6 %
-    // slower over the ResNet-shaped grid when requested behind the gathered rows of the current turn, 3-5 % slower
-    // when requested ahead of them: with up to sixteen waves per workgroup the two round trips of a turn hide behind
-    // other waves)
-    for (int j0 = beg + (wave * G + g) * U; j0 < end; j0 += n_waves * G * U) {
-        int col[U];
-        uint32_t a[U][V > 1 ? V / 2 : 1];  // the vector's halves, two per word (V = 1: one half in the low bits)
+    // The wave's staging slot: 64 column indices, then the 64 vectors.  Every lane fetches one nonzero of the block - two coalesced
+    // requests per 64 nonzeros, the next block's under the current block's gathers - and the groups pick their
+    // four nonzeros of a turn from the slot with two LDS reads, where a request per nonzero and lane group
+    // (eight for a turn of two groups, each serving two distinct addresses) kept the address path as busy with
+    // indices as with gathered rows: large V = 1 problems ran at 19-21 TB/s of gather against the 24-28 TB/s of
+    // the MFMA kernel, whose waves have always fetched their indices this way.
+    constexpr int kSlotBytes = kBlock * (int)sizeof(int) + kBlock * V * (int)sizeof(half_t);
+    // (with a tile per group the slot lies in the wave's own tiles, 2048 V bytes that are written after its last block;
+    // a single tile of short vectors can be smaller than the slot, which then has room of its own behind the tiles)
+    unsigned char *slot_s = kLaneSum
+        ? reinterpret_cast<unsigned char *>(partial + (size_t)n_waves * V * TN) + (size_t)wave * kSlotBytes
+        : reinterpret_cast<unsigned char *>(partial + (size_t)wave * G * V * TN);
+    int *idx_s = reinterpret_cast<int *>(slot_s);
+    uint32_t *val_s = reinterpret_cast<uint32_t *>(slot_s + kBlock * sizeof(int));  // [64][V] halves
+    const int stride = n_waves * block;
+    int j0 = beg + wave * block;
+    int next_idx = 0;
+    uint32_t next_val[kWords];
+    auto fetch = [&](int from) {
+        const int j = from + lane;
+        const bool have = j < end && lane < block;
+        const int jc = have ? j : end - 1;  // slots past the row's end repeat its last vector with zero values
+        next_idx = column_indices[jc];
+        load_values<V>(next_val, values + (size_t)jc * V);
+        if (!have) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int j = j0 + u;
-            const bool valid = j < end;
-            const int jc = valid ? j : end - 1;  // padded slots repeat the last vector with zero values
-            col[u] = column_indices[jc];
-            load_values<V>(a[u], values + (size_t)jc * V);
-            if (!valid) {
-#pragma unroll
-                for (int i = 0; i < (V > 1 ? V / 2 : 1); ++i) a[u][i] = 0u;
-            }
+            for (int i = 0; i < kWords; ++i) next_val[i] = 0u;
         }
+    };
+    // U nonzeros of a group: gather their rows (all U requests before the first use), multiply and add.
+    auto consume = [&](const int (&col)[U], const uint32_t (&a)[U][kWords]) {
         uint4_t b[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -150,10 +193,86 @@ spmm_valu_kernel(int n_cols, int n_tiles, int n_waves, const int *__restrict__ r
                     for (int c = 0; c < 8; ++c) acc[v][c] = __builtin_amdgcn_fdot2(av[v], bv[c], acc[v][c], false);
             }
         }
+    };
+    if (end - beg <= kTurn) {
+        // A row of a single turn (wave 0 is the only one with a block): every group asks for its own nonzeros
+        // directly - the hop through the staging slot would be a third step in a chain of two round trips
+        // (2048 rows of 5 nonzeros, N = 256: 3.1 against 3.7 us).
+        const int first = beg + g * U;
+        if (wave == 0 && first < end) {
+            int col[U];
+            uint32_t a[U][kWords];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const bool have = first + u < end;
+                const int jc = have ? first + u : end - 1;
+                col[u] = column_indices[jc];
+                load_values<V>(a[u], values + (size_t)jc * V);
+                if (!have) {
+#pragma unroll
+                    for (int i = 0; i < kWords; ++i) a[u][i] = 0u;
+                }
+            }
+            consume(col, a);
+        }
+        j0 = end;
+    }
+    if (j0 < end) fetch(j0);
+    for (; j0 < end; j0 += stride) {
+        idx_s[lane] = next_idx;
+        if constexpr (V == 1) {
+            reinterpret_cast<uint16_t *>(val_s)[lane] = (uint16_t)next_val[0];
+        } else {
+#pragma unroll
+            for (int i = 0; i < kWords; ++i) val_s[lane * kWords + i] = next_val[i];
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        if (j0 + stride < end) fetch(j0 + stride);
+        const int count = end - j0 < block ? end - j0 : block;
+        const int turns = (count + kTurn - 1) / kTurn;
+        for (int t = 0; t < turns; ++t) {
+            const int first = (t * G + g) * U;  // the group's nonzeros of this turn: first .. first + U - 1 of the block
+            if (first >= count) continue;       // (the last turn of a row: groups past its end have nothing to add)
+            int col[U];
+#pragma unroll
+            for (int u4 = 0; u4 < U / 4; ++u4) {
+                const int4_t c4 = *reinterpret_cast<const int4_t *>(idx_s + first + 4 * u4);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) col[4 * u4 + u] = c4[u];
+            }
+            uint32_t a[U][kWords];  // the vectors' halves, two per word (V = 1: one half in the low bits)
+            if constexpr (V == 1) {
+#pragma unroll
+                for (int u2 = 0; u2 < U / 2; ++u2) {
+                    const uint32_t w = val_s[first / 2 + u2];  // (first is a multiple of U)
+                    a[2 * u2][0] = w & 0xffffu;
+                    a[2 * u2 + 1][0] = w >> 16;
+                }
+            } else {
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+#pragma unroll
+                    for (int i = 0; i < kWords; ++i) a[u][i] = val_s[(first + u) * kWords + i];
+            }
+            consume(col, a);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");  // the slot is read out before the next block lands in it
+        __builtin_amdgcn_wave_barrier();
     }
 
-    if (n_waves * G == 1) {  // (deciding this by the row's length at run time instead measured 0.5 us slower)
-        if (col_ok) {
+    // The groups of a wave hold partial sums of the same V x TN tile: added up across the lanes first (a butterfly
+    // of 64 / LR - 1 steps per accumulator), so that the workgroup sums one tile per wave through LDS instead of
+    // one per group - with eight groups of eight lanes (the narrow tiles of small problems) that was a chain of
+    // 64 tiles read by eight threads.
+    if constexpr (G > 1 && kLaneSum) {
+#pragma unroll
+        for (int v = 0; v < V; ++v)
+#pragma unroll
+            for (int c = 0; c < 8; ++c) acc[v][c] = sum_over_groups<LR>(acc[v][c]);
+    }
+    if (n_waves * kTiles == 1) {  // (deciding this by the row's length at run time instead measured 0.5 us slower)
+        if (col_ok && g == 0) {
 #pragma unroll
             for (int v = 0; v < V; ++v) {
                 if constexpr (RAGGED)
@@ -165,9 +284,9 @@ spmm_valu_kernel(int n_cols, int n_tiles, int n_waves, const int *__restrict__ r
         return;
     }
 
-    // only the partial tiles of the groups that had nonzeros are written and summed
-    if (wave * G + g < n_partials) {
-        float *mine = partial + (size_t)(wave * G + g) * V * TN;
+    // the tiles of the waves that are still running are written and summed (a wave without nonzeros writes zeros)
+    if (g < kTiles) {
+        float *mine = partial + (size_t)(wave * kTiles + g) * V * TN;
 #pragma unroll
         for (int v = 0; v < V; ++v) {
             float4_t lo = {acc[v][0], acc[v][1], acc[v][2], acc[v][3]};
@@ -185,7 +304,7 @@ spmm_valu_kernel(int n_cols, int n_tiles, int n_waves, const int *__restrict__ r
         float sum[8];
 #pragma unroll
         for (int c = 0; c < 8; ++c) sum[c] = 0.f;
-        for (int p = 0; p < n_partials; ++p) {
+        for (int p = 0; p < alive_waves * kTiles; ++p) {
             const float *src = partial + (size_t)p * V * TN + v * TN + cl2 * 8;
             const float4_t x = *reinterpret_cast<const float4_t *>(src);
             const float4_t y = *reinterpret_cast<const float4_t *>(src + 4);
@@ -209,13 +328,16 @@ static int launch_one(int m_vec, int k, int waves, const int *row_indices, const
     const int n_tiles = ceil_div(k, TN);
     const long long blocks = (long long)m_vec * n_tiles;
     if (blocks > 0x7fffffffLL) return hipErrorNotSupported;
-    // LDS for the partial tiles: waves * 64 lanes * V * 8 floats; stay within 64 KiB.
-    const int max_waves = (64 * 1024) / (64 * V * 8 * (int)sizeof(float));
+    // LDS per wave: one partial tile of V x TN floats and the staging slot (64 indices, 64 vectors) for V <= 2, a tile
+    // per group (the slot lies inside them) for V = 4 and 8; within 64 KiB.
+    constexpr int kPerWave = V <= 2 ? V * TN * (int)sizeof(float) + 64 * (int)sizeof(int) + 64 * V * (int)sizeof(half_t)
+                                    : G * V * TN * (int)sizeof(float);
+    const int max_waves = (64 * 1024) / kPerWave;
     if (waves > max_waves) waves = max_waves;
     if (waves < 1) waves = 1;
-    const size_t lds = (waves * G > 1) ? (size_t)waves * G * V * TN * sizeof(float) : 0;
+    const size_t lds = (size_t)waves * kPerWave;
     hipLaunchKernelGGL((spmm_valu_kernel<V, LR, OutT, RAGGED>), dim3((unsigned)blocks, (unsigned)batch.count),
-                       dim3(64 * waves), lds, stream, k, n_tiles, waves, row_indices, row_offsets, column_indices, values,
+                       dim3(64 * waves), lds, stream, k, n_tiles, waves, (uint32_t)((1ull << 32) / (unsigned)waves + 1u), row_indices, row_offsets, column_indices, values,
                        rhs, out, batch.stride_a, batch.stride_b, batch.stride_out);
     return (int)hipGetLastError();
 }
