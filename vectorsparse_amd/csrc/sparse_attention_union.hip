@@ -768,6 +768,19 @@ __device__ __forceinline__ int stream_v_pair_rank(int pair)
 // the transposed writes (lanes of a quad: columns 8 apart) nor the reads (lanes: columns CPL apart) collide.
 __device__ __forceinline__ int stream_v_offset(int col, int chunk) { return col * kStreamVPitch + ((chunk ^ ((col >> 3) & 7)) << 3); }
 
+// The per-row path as a function of its own: inlined into the streamed kernel it takes every register the launch
+// bounds leave, and the allocator then parks values of the streamed path in scratch memory around it.
+template <int V, int KS, int CPL>
+__device__ __noinline__ void per_row_block_call(int row_first, int row_last, int wave, int n_waves,
+                                                const int *__restrict__ row_offsets, const int *__restrict__ col_indices,
+                                                const half_t *__restrict__ q, const half_t *__restrict__ k,
+                                                const half_t *__restrict__ v, half_t *__restrict__ out, int d_qk,
+                                                int d_v, float s2, int c, int g, int col_off)
+{
+    per_row_block<V, KS, CPL>(row_first, row_last, wave, n_waves, row_offsets, col_indices, q, k, v, out, d_qk, d_v, s2,
+                              c, g, col_off);
+}
+
 template <int V, int KS, int CPL>
 __global__ void __launch_bounds__(512, union_wide(KS, CPL) ? 2 : 4)
 sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
@@ -819,8 +832,14 @@ sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
                          plan[8] == kStreamRounds && plan[9] == SS;
     const int *rec = plan + kPlanHeader + (size_t)(plan_ok ? bx : 0) * stride;
     const int n_union = plan_ok ? rec[0] : 0x7fffffff;
-    const int *masks = rec + 4;
-    const int *cols = rec + 4 + kStreamRounds * kMaskWords;
+    // The record, the K rows and the V rows are read through buffer descriptors: a scalar base and one 32-bit byte
+    // offset per thread and load, where a 64-bit pointer per thread and load used to take the registers that the
+    // launch bounds do not leave (n <= 2^20 columns of at most 128 halves: every offset is below 2^28).
+    const __amdgpu_buffer_rsrc_t rec_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<int *>(rec), 0, 0x7fffffff, 0x00020000);
+    const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t *>(k), 0, 0x7fffffff, 0x00020000);
+    const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t *>(v), 0, 0x7fffffff, 0x00020000);
+    constexpr unsigned kMasksAt = 4u * 4u;                                        // byte offsets inside the record
+    constexpr unsigned kColsAt = 4u * (4u + kStreamRounds * kMaskWords);
 
     // What a thread fetches per sub-round: NK slices of K rows (thread t takes slices t, t + 512, ...:
     // consecutive threads read consecutive 16 bytes of a row), NV times the same slice of the V rows of two
@@ -832,11 +851,14 @@ sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
     // column numbers of sub-round `round` < kStreamRounds (the plan lists 0 past the union: row 0, unused), which
     // do not wait for the union's size
     auto fetch_cols = [&](int round) {
+        const unsigned at = kColsAt + 4u * (unsigned)(round * SR);  // (uniform)
 #pragma unroll
-        for (int i = 0; i < NK; ++i) col_k[i] = cols[round * SR + ((tid + i * kThreads) >> kShiftK)];
+        for (int i = 0; i < NK; ++i)
+            col_k[i] = (int)__builtin_amdgcn_raw_buffer_load_b32(rec_rsrc, 4u * ((unsigned)(tid + i * kThreads) >> kShiftK), at, 0);
 #pragma unroll
         for (int i = 0; i < NV; ++i)
-            col_v[i] = *reinterpret_cast<const int2_t *>(cols + round * SR + stream_v_pair_rank((tid + i * kThreads) >> kShiftV));
+            col_v[i] = __builtin_bit_cast(int2_t, __builtin_amdgcn_raw_buffer_load_b64(
+                rec_rsrc, 4u * (unsigned)stream_v_pair_rank((tid + i * kThreads) >> kShiftV), at, 0));
     };
     // Requests only: nothing here reads what the loads return, so the wave goes on to the arithmetic at once.
     // Slices past the union or past d read the start of a valid row and are replaced by zeros in commit().
@@ -846,17 +868,23 @@ sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
             const int sidx = tid + i * kThreads;
             const int u = round * SR + (sidx >> kShiftK), sl = sidx & ((1 << kShiftK) - 1);
             const bool real = u < n_union && 8 * sl < d_qk;
-            stage_k[i] = *reinterpret_cast<const uint4_t *>(k + (size_t)col_k[i] * d_qk + (real ? 8 * sl : 0));
+            stage_k[i] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, 2u * ((unsigned)col_k[i] * (unsigned)d_qk + (real ? 8u * sl : 0u)), 0, 0);
         }
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int sidx = tid + i * kThreads;
             const int u = round * SR + stream_v_pair_rank(sidx >> kShiftV), sl = sidx & ((1 << kShiftV) - 1);
-            const int off = (u < n_union && 8 * sl < d_v) ? 8 * sl : 0;
-            stage_v[i][0] = *reinterpret_cast<const uint4_t *>(v + (size_t)col_v[i][0] * d_v + off);
-            stage_v[i][1] = *reinterpret_cast<const uint4_t *>(v + (size_t)col_v[i][1] * d_v + off);
+            const unsigned off = (u < n_union && 8 * sl < d_v) ? 8u * sl : 0u;
+            stage_v[i][0] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, 2u * ((unsigned)col_v[i][0] * (unsigned)d_v + off), 0, 0);
+            stage_v[i][1] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, 2u * ((unsigned)col_v[i][1] * (unsigned)d_v + off), 0, 0);
         }
-        if (tid < kRows * SS) stage_m = (unsigned)masks[round * kMaskWords + tid];
+        if (tid < kRows * SS) {
+            // (the offset is made anew in every sub-round: kept across the loop it is the one value the register
+            // allocator parks in scratch memory, and its reload waits for every gather requested just above)
+            unsigned word = (unsigned)tid;
+            asm volatile("" : "+v"(word));
+            stage_m = __builtin_amdgcn_raw_buffer_load_b32(rec_rsrc, 4u * word, kMasksAt + 4u * (unsigned)(round * kMaskWords), 0);
+        }
     };
     // The parked sub-round `round` into LDS; rows past the union and slices past d as zeros, so the arithmetic
     // never meets stale bits.  V goes in transposed: a thread holds 8 columns of two consecutive ranks and
@@ -890,8 +918,8 @@ sparse_attention_stream_kernel(int m_vec, int n, int d_qk, int d_v,
 
     fetch_cols(0);  // requested together with the union's size
     if (n_union > u_cap || d_v % 8 != 0) {
-        per_row_block<V, KS, CPL>(row_first, row_last, wave, 8, row_offsets, col_indices, q, k, v, out, d_qk, d_v, s2,
-                                  c, g, col_off);
+        per_row_block_call<V, KS, CPL>(row_first, row_last, wave, 8, row_offsets, col_indices, q, k, v, out, d_qk, d_v,
+                                       s2, c, g, col_off);
         return;
     }
     const int n_rounds = (n_union + SR - 1) / SR;
