@@ -249,7 +249,7 @@ def test_sweep_benchmark_selection(tmp_path):
 
 
 def test_plot_reads_the_sweep_result_file(tmp_path):
-    """Geometric means per (path, V, k, sparsity bucket) and a figure from the rows the sweep writes."""
+    """Geometric means per (path, V, k, sparsity bucket) from the rows the sweep writes."""
     import csv
     from vectorsparse_amd import plot
 
@@ -267,9 +267,8 @@ def test_plot_reads_the_sweep_result_file(tmp_path):
         w = csv.DictWriter(f, fieldnames=list(rows[0].keys()))
         w.writeheader()
         w.writerows(rows)
-    figure, geo = tmp_path / "speedup.png", tmp_path / "geo.csv"
-    assert plot.main(["--csv", str(result), "--out", str(figure), "--geo", str(geo)]) == 0
-    assert figure.stat().st_size > 1000
+    geo = tmp_path / "geo.csv"
+    assert plot.main(["--csv", str(result), "--geo", str(geo)]) == 0
     with open(geo) as f:
         table = list(csv.reader(f))
     assert table[0] == ["path", "V", "k", "0.7", "0.9"]

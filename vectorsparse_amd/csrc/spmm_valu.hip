@@ -10,6 +10,8 @@
 // of LR lanes, each group walks its own nonzero vectors and every lane owns 8 consecutive
 // columns (one 128-bit load per gathered row, four rows in flight per lane).  The W*G partial tiles
 // are summed through LDS in a fixed order.
+#include <type_traits>
+
 #include "vs_common.hpp"
 
 namespace vs {
@@ -49,8 +51,12 @@ __device__ __forceinline__ float sum_over_groups(float x)
 
 // RAGGED: the dense width is not a multiple of 8 (rows of the dense operand and of the output start at any 2-byte
 // boundary, the last chunk of a row is cut): chunks are fetched and stored half by half.
+// The second launch bound (waves per SIMD) is there for the launches of short rows: left to itself the compiler takes
+// 86 (V = 1) and 102 (V = 2) registers where 60 and 72 do without a spill, and a launch of short rows - waves that live for
+// one chain of round trips, three in four of them ending at once - then needs two rounds to seat its waves where one
+// would do (2048 rows of 1 to 6 nonzeros, N = 256, V = 2: 3.24 against 2.95 us).
 template <int V, int LR, typename OutT, bool RAGGED = false>
-__global__ void __launch_bounds__(1024)
+__global__ void __launch_bounds__(1024, RAGGED ? 4 : (V == 1 ? 8 : (V == 2 ? 7 : 4)))
 spmm_valu_kernel(int n_cols, int n_tiles, int n_waves, uint32_t inv_waves, const int *__restrict__ row_indices,
                  const int *__restrict__ row_offsets, const int *__restrict__ column_indices,
                  const half_t *__restrict__ values, const half_t *__restrict__ rhs,
@@ -103,6 +109,17 @@ spmm_valu_kernel(int n_cols, int n_tiles, int n_waves, uint32_t inv_waves, const
     block = block < kLeast ? kLeast : (block > kBlock ? kBlock : block);
     // waves with a block: all of them unless the blocks are at their smallest (a wave without one adds zeros)
     int alive_waves = block == kLeast ? (end - beg + kLeast - 1) / kLeast : n_waves;
+    // A row short enough for every group of the workgroup to take its nonzeros in one go, kDirect each, does so
+    // without the staging slot: one chain of two round trips (index, gathered row) on as many waves as the row has
+    // groups of kDirect nonzeros.  (One wave with eight nonzeros per group instead measured 11-28 % slower over the
+    // rows of 1 to 60 nonzeros of the sweep: every request of a wave, padded or not, takes the CU's address path
+    // 16 cycles, and eight workgroups per CU queue there.)
+    constexpr int kDirect = 4;
+    const bool direct = end - beg <= n_waves * G * kDirect;
+    if (direct) {
+        const int groups = (end - beg + kDirect - 1) / kDirect;
+        alive_waves = (groups + G - 1) / G;
+    }
     alive_waves = alive_waves < kSumWaves ? kSumWaves : alive_waves;
     alive_waves = alive_waves < n_waves ? alive_waves : n_waves;
     if (wave >= alive_waves) return;
@@ -149,10 +166,11 @@ spmm_valu_kernel(int n_cols, int n_tiles, int n_waves, uint32_t inv_waves, const
         }
     };
     // U nonzeros of a group: gather their rows (all U requests before the first use), multiply and add.
-    auto consume = [&](const int (&col)[U], const uint32_t (&a)[U][kWords]) {
-        uint4_t b[U];
+    auto consume = [&](auto count, const int (&col)[U], const uint32_t (&a)[U][kWords]) {
+        constexpr int N = decltype(count)::value;  // nonzeros taken: the first N entries of col and a
+        uint4_t b[N];
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
+        for (int u = 0; u < N; ++u) {
             if constexpr (RAGGED) {
                 RowChunk<8> chunk;
                 load_ragged<8>(chunk, rhs_col + (size_t)col[u] * n_cols, valid);
@@ -164,7 +182,7 @@ spmm_valu_kernel(int n_cols, int n_tiles, int n_waves, uint32_t inv_waves, const
         if constexpr (V == 1) {
             // one multiply-add per column and nonzero: nothing to pair up
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
+            for (int u = 0; u < N; ++u) {
                 const float av = (float)__builtin_bit_cast(half2_t, a[u][0])[0];
                 const half8_t bu = __builtin_bit_cast(half8_t, b[u]);
 #pragma unroll
@@ -175,7 +193,7 @@ spmm_valu_kernel(int n_cols, int n_tiles, int n_waves, uint32_t inv_waves, const
             // one instruction): the values of the two vectors and the two gathered rows are interleaved with
             // v_perm_b32 first - V + 8 shuffles buy 8 V instructions instead of 16 V.
 #pragma unroll
-            for (int u = 0; u < U; u += 2) {
+            for (int u = 0; u < N; u += 2) {
                 half2_t av[V], bv[8];
 #pragma unroll
                 for (int i = 0; i < V / 2; ++i) {
@@ -194,78 +212,13 @@ spmm_valu_kernel(int n_cols, int n_tiles, int n_waves, uint32_t inv_waves, const
             }
         }
     };
-    if (end - beg <= kTurn) {
-        // A row of a single turn (wave 0 is the only one with a block): every group asks for its own nonzeros
-        // directly - the hop through the staging slot would be a third step in a chain of two round trips
-        // (2048 rows of 5 nonzeros, N = 256: 3.1 against 3.7 us).
-        const int first = beg + g * U;
-        if (wave == 0 && first < end) {
-            int col[U];
-            uint32_t a[U][kWords];
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const bool have = first + u < end;
-                const int jc = have ? first + u : end - 1;
-                col[u] = column_indices[jc];
-                load_values<V>(a[u], values + (size_t)jc * V);
-                if (!have) {
-#pragma unroll
-                    for (int i = 0; i < kWords; ++i) a[u][i] = 0u;
-                }
-            }
-            consume(col, a);
-        }
-        j0 = end;
-    }
-    if (j0 < end) fetch(j0);
-    for (; j0 < end; j0 += stride) {
-        idx_s[lane] = next_idx;
-        if constexpr (V == 1) {
-            reinterpret_cast<uint16_t *>(val_s)[lane] = (uint16_t)next_val[0];
-        } else {
-#pragma unroll
-            for (int i = 0; i < kWords; ++i) val_s[lane * kWords + i] = next_val[i];
-        }
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        if (j0 + stride < end) fetch(j0 + stride);
-        const int count = end - j0 < block ? end - j0 : block;
-        const int turns = (count + kTurn - 1) / kTurn;
-        for (int t = 0; t < turns; ++t) {
-            const int first = (t * G + g) * U;  // the group's nonzeros of this turn: first .. first + U - 1 of the block
-            if (first >= count) continue;       // (the last turn of a row: groups past its end have nothing to add)
-            int col[U];
-#pragma unroll
-            for (int u4 = 0; u4 < U / 4; ++u4) {
-                const int4_t c4 = *reinterpret_cast<const int4_t *>(idx_s + first + 4 * u4);
-#pragma unroll
-                for (int u = 0; u < 4; ++u) col[4 * u4 + u] = c4[u];
-            }
-            uint32_t a[U][kWords];  // the vectors' halves, two per word (V = 1: one half in the low bits)
-            if constexpr (V == 1) {
-#pragma unroll
-                for (int u2 = 0; u2 < U / 2; ++u2) {
-                    const uint32_t w = val_s[first / 2 + u2];  // (first is a multiple of U)
-                    a[2 * u2][0] = w & 0xffffu;
-                    a[2 * u2 + 1][0] = w >> 16;
-                }
-            } else {
-#pragma unroll
-                for (int u = 0; u < U; ++u)
-#pragma unroll
-                    for (int i = 0; i < kWords; ++i) a[u][i] = val_s[(first + u) * kWords + i];
-            }
-            consume(col, a);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");  // the slot is read out before the next block lands in it
-        __builtin_amdgcn_wave_barrier();
-    }
-
+    // (a lambda, expanded at both of its calls: the short row's whole path then lies in one straight piece of code)
+    auto finish = [&](bool one_group) __attribute__((always_inline)) {
     // The groups of a wave hold partial sums of the same V x TN tile: added up across the lanes first (a butterfly
     // of 64 / LR - 1 steps per accumulator), so that the workgroup sums one tile per wave through LDS instead of
     // one per group - with eight groups of eight lanes (the narrow tiles of small problems) that was a chain of
     // 64 tiles read by eight threads.
-    if constexpr (G > 1 && kLaneSum) {
+    if (G > 1 && kLaneSum && !one_group) {  // (a row of one group's nonzeros: the other groups hold zeros)
 #pragma unroll
         for (int v = 0; v < V; ++v)
 #pragma unroll
@@ -316,6 +269,77 @@ spmm_valu_kernel(int n_cols, int n_tiles, int n_waves, uint32_t inv_waves, const
         else
             store_converted<OutT, 8>(out + ((size_t)row * V + v) * n_cols + col, sum);
     }
+    };
+    // (the short row's code comes first and runs straight through: the instruction cache starts every launch cold, and
+    // a jump across the staged loop's code costs a launch of short rows 0.2-0.4 us)
+    if (__builtin_expect(direct, 1)) {
+        const int first = beg + (wave * G + g) * kDirect;
+        if (first < end) {
+            int col[U];
+            uint32_t a[U][kWords];
+#pragma unroll
+            for (int u = 0; u < kDirect; ++u) {
+                const bool have = first + u < end;
+                const int jc = have ? first + u : end - 1;  // padded slots repeat the last vector with zero values
+                col[u] = column_indices[jc];
+                load_values<V>(a[u], values + (size_t)jc * V);
+                if (!have) {
+#pragma unroll
+                    for (int i = 0; i < kWords; ++i) a[u][i] = 0u;
+                }
+            }
+            consume(std::integral_constant<int, kDirect>(), col, a);
+        }
+        finish(end - beg <= kDirect);
+        return;
+    }
+    {
+    if (j0 < end) fetch(j0);
+    for (; j0 < end; j0 += stride) {
+        idx_s[lane] = next_idx;
+        if constexpr (V == 1) {
+            reinterpret_cast<uint16_t *>(val_s)[lane] = (uint16_t)next_val[0];
+        } else {
+#pragma unroll
+            for (int i = 0; i < kWords; ++i) val_s[lane * kWords + i] = next_val[i];
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        if (j0 + stride < end) fetch(j0 + stride);
+        const int count = end - j0 < block ? end - j0 : block;
+        const int turns = (count + kTurn - 1) / kTurn;
+        for (int t = 0; t < turns; ++t) {
+            const int first = (t * G + g) * U;  // the group's nonzeros of this turn: first .. first + U - 1 of the block
+            if (first >= count) continue;       // (the last turn of a row: groups past its end have nothing to add)
+            int col[U];
+#pragma unroll
+            for (int u4 = 0; u4 < U / 4; ++u4) {
+                const int4_t c4 = *reinterpret_cast<const int4_t *>(idx_s + first + 4 * u4);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) col[4 * u4 + u] = c4[u];
+            }
+            uint32_t a[U][kWords];  // the vectors' halves, two per word (V = 1: one half in the low bits)
+            if constexpr (V == 1) {
+#pragma unroll
+                for (int u2 = 0; u2 < U / 2; ++u2) {
+                    const uint32_t w = val_s[first / 2 + u2];  // (first is a multiple of U)
+                    a[2 * u2][0] = w & 0xffffu;
+                    a[2 * u2 + 1][0] = w >> 16;
+                }
+            } else {
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+#pragma unroll
+                    for (int i = 0; i < kWords; ++i) a[u][i] = val_s[(first + u) * kWords + i];
+            }
+            consume(std::integral_constant<int, U>(), col, a);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");  // the slot is read out before the next block lands in it
+        __builtin_amdgcn_wave_barrier();
+    }
+    }
+
+    finish(false);
 }
 
 template <int V, int LR, typename OutT, bool RAGGED = false>
