@@ -199,8 +199,8 @@ def cold_summary(stats_csv):
              "ncu_profile.py:91): every timed launch follows a 1 GiB fill that evicts the L2s and the Infinity Cache.",
              "",
              "commands (`cd /tmp && export TMPDIR=/tmp` first, then from the repository root):",
-             "  rocprofv3 --kernel-trace --stats --output-format csv -d gpurun_out/prof/cold -o t -- python3 bench.py --cold",
-             "  python3 bench.py --cold-summary gpurun_out/prof/cold/t_kernel_stats.csv > profiles/cold_cache_kernel_stats.txt",
+             "  rocprofv3 --kernel-trace --stats --output-format csv -d OUT -o t -- python3 bench.py --cold",
+             "  python3 bench.py --cold-summary OUT/t_kernel_stats.csv > profiles/cold_cache_kernel_stats.txt",
              "",
              "kernel_source_tag_spmm %s" % kernel_source_tag(*SPMM_SOURCES),
              "kernel_source_tag_sddmm %s" % kernel_source_tag(*SDDMM_SOURCES),
