@@ -7,9 +7,12 @@
 // first (src/spmm_utils/compute_utils.h:45); that rounding alone costs up to ~9e-2 of the
 // 1e-2 relative-error budget against the host loop on near-zero outputs, so it is not
 // reproduced.  Work item = (vector row, tile of TN = 8*LR dense columns); a wave is G = 64/LR groups
-// of LR lanes, each group walks its own nonzero vectors and every lane owns 8 consecutive
-// columns (one 128-bit load per gathered row, four rows in flight per lane).  The W*G partial tiles
-// are summed through LDS in a fixed order.
+// of LR lanes, every lane owns 8 consecutive columns (one 128-bit load per gathered row, U = 8 rows in flight per
+// lane, 4 for V = 8).  A wave fetches a block of up to 64 nonzeros with one coalesced load of indices and one of
+// values per lane and parks them in LDS, from where its groups take U nonzeros each per turn; rows short enough
+// for the workgroup's groups to take in one go, four nonzeros each, skip that hop.  The partial tiles (one per
+// wave for V <= 2, whose groups are summed across the lanes first; one per group else) are summed through LDS in
+// a fixed order.
 #include <type_traits>
 
 #include "vs_common.hpp"
@@ -138,7 +141,7 @@ spmm_valu_kernel(int n_cols, int n_tiles, int n_waves, uint32_t inv_waves, const
 
     // The wave's staging slot: 64 column indices, then the 64 vectors.  Every lane fetches one nonzero of the block - two coalesced
     // requests per 64 nonzeros, the next block's under the current block's gathers - and the groups pick their
-    // four nonzeros of a turn from the slot with two LDS reads, where a request per nonzero and lane group
+    // U nonzeros of a turn from the slot with a few LDS reads, where a request per nonzero and lane group
     // (eight for a turn of two groups, each serving two distinct addresses) kept the address path as busy with
     // indices as with gathered rows: large V = 1 problems ran at 19-21 TB/s of gather against the 24-28 TB/s of
     // the MFMA kernel, whose waves have always fetched their indices this way.
