@@ -40,6 +40,11 @@ def test_every_spmm_point_of_the_grid(gpu, M, V):
             hinted = torch.full((M, sweep.N_DENSE), float("nan"), dtype=torch.float16, device="cuda")
             prob.spmm(Bd, out=hinted, row_length_hint=True)     # the sweep's --hint route
             assert_parity(hinted.cpu().numpy(), ref, "spmm M%d K%d s%g V%d hinted" % (M, K, s, V))
+            # the schedule that stages the dense operand in LDS per block of eight vector rows (opt-in entry)
+            staged = torch.full((M, sweep.N_DENSE), float("nan"), dtype=torch.float16, device="cuda")
+            ops.spmm_slab(prob.m_vec, V, sweep.N_DENSE, K, prob.row_indices, prob.row_offsets, prob.column_indices,
+                          prob.values, Bd, staged)
+            assert_parity(staged.cpu().numpy(), ref, "spmm M%d K%d s%g V%d staged in LDS" % (M, K, s, V))
             points += 1
     assert points == len(sweep.KS) * len(sweep.SPARSITIES)
 
