@@ -603,7 +603,7 @@ SpmmShape choose_spmm_shape(bool softmax, int m_vec, int vec_length, int k, int 
 #endif
     if (use_dma) cpl = 8;
     const bool hinted = batch.nonzeros_vec >= 0;
-    const int mean_steps = hinted ? ceil_div(ceil_div(batch.nonzeros_vec, m_vec), kStep) : ceil_div(n, 4 * kStep);
+    int mean_steps = hinted ? ceil_div(ceil_div(batch.nonzeros_vec, m_vec), kStep) : ceil_div(n, 4 * kStep);
     const int longest_steps = ceil_div(batch.longest_row_vec > 0 ? batch.longest_row_vec : 0, kStep);
     // a few rows far longer than the mean (known only to the batched entry points)
     const bool skewed = hinted && longest_steps > 4 * mean_steps && longest_steps > 16;
@@ -618,6 +618,10 @@ SpmmShape choose_spmm_shape(bool softmax, int m_vec, int vec_length, int k, int 
     const bool ragged = k % 4 != 0;
     if (ragged) cpl = 4;
     const long long blocks = (long long)m_vec * ceil_div(k, 16 * cpl) * batch.count;
+    // Row lengths unknown on a grid of at most a workgroup per CU: the rows are taken to hold half of n rather than a
+    // quarter - there a wave that a shorter row leaves idle costs next to nothing, and a row of two blocks served by
+    // one wave 9 % (128 rows x 147 at 50 %, N = 256: 2.66 us with one wave, 2.44 us with two).
+    if (!hinted && blocks <= kTargetBlocks) mean_steps = ceil_div(n, 2 * kStep);
     // Steps of gathered rows a wave keeps in flight.  Two pay as soon as rows hold more than one step: the wave
     // waits once for 64 vectors instead of twice (ResNet-shaped grid, 16 to 2304 vectors per row, N = 64 and 256:
     // 5-20 % faster than one step at the best wave count of each; 3 % slower on rows of under 32 vectors).  Four
