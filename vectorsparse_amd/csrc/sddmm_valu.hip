@@ -11,6 +11,8 @@
 // partner's copy of that half, so after log2(V) stages each output sits in exactly one lane.
 // Partners are reached with DPP (quad_perm, row_half_mirror, row_mirror) inside a 16-lane row,
 // ds_swizzle across rows and ds_bpermute across the two 32-lane halves.
+#include <type_traits>
+
 #include "vs_common.hpp"
 
 namespace vs {
@@ -123,19 +125,35 @@ sddmm_valu_kernel(int m_vec, int K, int slots, int waves_per_block, const int *_
 
     // Every lane of the wave runs the same number of steps so the cross-lane exchanges below
     // always see all partners; padded slots gather the row's last vector and skip the store.
-    for (int grp = s; grp < n_groups; grp += slots) {
-        const int j = beg + grp * G + g;
-        const bool valid = j < end;
-        const int jc = valid ? j : end - 1;
-        const half_t *rhs_row = rhs + (size_t)col_indices[jc] * K;
-        float acc[V];
+    // A wave takes the groups s, s + slots, ... of its row, U of them per turn while it has that many left: their
+    // column indices are requested together and then their rhs rows, so that U gathered rows are in flight per lane
+    // instead of one; what is left goes one group per turn (no padded requests: each would take the CU's address
+    // path as long as a real one).
+    constexpr int U = SINGLE ? (V <= 2 ? 4 : 2) : 1;
+    auto turn = [&](auto count, int grp) {
+        constexpr int N = decltype(count)::value;
+        int j[N];
+        bool valid[N];
+        const half_t *rhs_row[N];
 #pragma unroll
-        for (int v = 0; v < V; ++v) acc[v] = 0.f;
+        for (int u = 0; u < N; ++u) {
+            j[u] = beg + (grp + u * slots) * G + g;
+            valid[u] = j[u] < end;
+            const int jc = valid[u] ? j[u] : end - 1;
+            rhs_row[u] = rhs + (size_t)col_indices[jc] * K;
+        }
+        float acc[N][V];
+#pragma unroll
+        for (int u = 0; u < N; ++u)
+#pragma unroll
+            for (int v = 0; v < V; ++v) acc[u][v] = 0.f;
         if constexpr (SINGLE) {
             const int off = cl * VEC;
-            half_t b[VEC];
-            load_slice<VEC>(b, rhs_row + off, off < K);
-            slice_dot<V, VEC>(acc, a0, b);
+            half_t b[N][VEC];
+#pragma unroll
+            for (int u = 0; u < N; ++u) load_slice<VEC>(b[u], rhs_row[u] + off, off < K);
+#pragma unroll
+            for (int u = 0; u < N; ++u) slice_dot<V, VEC>(acc[u], a0, b[u]);
         } else {
             for (int ch = 0; ch < n_chunks; ++ch) {
                 const int off = ch * CHUNK + cl * VEC;
@@ -144,23 +162,31 @@ sddmm_valu_kernel(int m_vec, int K, int slots, int waves_per_block, const int *_
                 half_t b[VEC];
 #pragma unroll
                 for (int v = 0; v < V; ++v) load_slice<VEC>(a[v], lhs_rows + (size_t)v * K + off, ok);
-                load_slice<VEC>(b, rhs_row + off, ok);
-                slice_dot<V, VEC>(acc, a, b);
+                load_slice<VEC>(b, rhs_row[0] + off, ok);
+                slice_dot<V, VEC>(acc[0], a, b);
             }
         }
-        reduce_group<LK, V>(acc, cl);
-        // After the butterfly: V >= LK -> lane cl holds outputs v = cl*(V/LK) + i, i < V/LK;
-        //                      V <  LK -> lanes with cl % (LK/V) == 0 hold output v = cl / (LK/V).
-        if (valid) {
-            if constexpr (V >= LK) {
-                constexpr int PER = V / LK;
-                store_converted<OutT, PER>(out + (size_t)j * V + cl * PER, acc);
-            } else {
-                constexpr int REP = LK / V;
-                if (cl % REP == 0) store_converted<OutT, 1>(out + (size_t)j * V + cl / REP, acc);
+#pragma unroll
+        for (int u = 0; u < N; ++u) {
+            reduce_group<LK, V>(acc[u], cl);
+            // After the butterfly: V >= LK -> lane cl holds outputs v = cl*(V/LK) + i, i < V/LK;
+            //                      V <  LK -> lanes with cl % (LK/V) == 0 hold output v = cl / (LK/V).
+            if (valid[u]) {
+                if constexpr (V >= LK) {
+                    constexpr int PER = V / LK;
+                    store_converted<OutT, PER>(out + (size_t)j[u] * V + cl * PER, acc[u]);
+                } else {
+                    constexpr int REP = LK / V;
+                    if (cl % REP == 0) store_converted<OutT, 1>(out + (size_t)j[u] * V + cl / REP, acc[u]);
+                }
             }
         }
+    };
+    int grp = s;
+    if constexpr (U > 1) {
+        for (; grp + (U - 1) * slots < n_groups; grp += U * slots) turn(std::integral_constant<int, U>(), grp);
     }
+    for (; grp < n_groups; grp += slots) turn(std::integral_constant<int, 1>(), grp);
 }
 
 template <int V, int LK, int VEC, bool SINGLE, typename OutT>
