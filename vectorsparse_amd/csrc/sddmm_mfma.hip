@@ -288,7 +288,6 @@ static int launch_one(int m_vec, int k, int nonzeros_vec, const int *row_indices
                       const int *col_indices, const half_t *lhs, const half_t *rhs, OutT *out, hipStream_t stream,
                       const Batch &batch)
 {
-    const int kWavesPerBlock = options().sddmm_block_waves > 0 ? options().sddmm_block_waves : 8;
     if constexpr (KS > 0) {
         if (batch.algorithm == 2 && !batch.row_parts) {
             // super-groups per wave: enough waves to fill the chip (~8192), at least `min_supers` of them per
@@ -309,6 +308,16 @@ static int launch_one(int m_vec, int k, int nonzeros_vec, const int *row_indices
     }
     const int slots = sddmm_auto_slots((long long)m_vec * batch.count, (long long)nonzeros_vec * batch.count, 16 * GRP, true);
     const long long waves = (long long)m_vec * slots;
+    // Waves per workgroup: eight on launches that fill the chip, fewer on smaller ones so that the launch still has two
+    // workgroups per CU - a wave's lhs slices and rhs rows then do not queue behind seven other waves' on one CU's
+    // address path while other CUs idle.  Measured (V = 8, K = 256, 512 / 1024 / 2048 rows at 98 %): 3.46 -> 2.38,
+    // 3.59 -> 2.41, 3.69 -> 2.69 us with one wave per workgroup; K = 128, 512 rows at 90 %: 2.57 -> 2.20 us; launches of 4096
+    // waves and more are the same or up to 8 % slower with narrow workgroups and keep eight.
+    int kWavesPerBlock = options().sddmm_block_waves;
+    if (kWavesPerBlock <= 0) {
+        kWavesPerBlock = 1;
+        while (kWavesPerBlock < 8 && waves * batch.count >= 512LL * 2 * kWavesPerBlock) kWavesPerBlock <<= 1;
+    }
     const long long blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks > 0x7fffffffLL || blocks * kWavesPerBlock > 0xffffffffLL) return hipErrorNotSupported;
     if (batch.row_parts) {  // m_vec counts the slots of the dispatch list that row_indices points to
